@@ -1,0 +1,756 @@
+// cabi.cpp -- the extern "C" boundary (include/cake_hip.h): argument checks,
+// host/device operand staging, workspace ownership, timing, kernel dispatch.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "blockdims.hpp"
+#include "cake_hip.h"
+#include "kernels.hpp"
+#include "planner.hpp"
+
+namespace {
+
+using namespace cake;
+
+thread_local std::string g_last_error;
+thread_local double g_family_seconds[5] = {0, 0, 0, 0, 0};
+
+int fail(int status, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return status;
+}
+
+#define HIP_TRY(expr)                                                                         \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess)                                                                 \
+            return fail(CAKE_HIP_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));     \
+    } while (0)
+
+// Grow-only device buffer.
+struct DeviceBuffer {
+    void* ptr = nullptr;
+    size_t cap = 0;
+    int reserve(size_t bytes)
+    {
+        if (bytes <= cap) return CAKE_HIP_OK;
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+        size_t want = bytes + (bytes >> 3) + 256;
+        if (hipMalloc(&ptr, want) != hipSuccess) {
+            (void)hipGetLastError();
+            ptr = nullptr;
+            return fail(CAKE_HIP_ERR_ALLOC, "device allocation of %zu bytes failed", want);
+        }
+        cap = want;
+        return CAKE_HIP_OK;
+    }
+    void release()
+    {
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+    }
+};
+
+enum { STAGE_SLOTS = 4 };
+
+struct Context {
+    bool ready = false;
+    int device = 0;
+    cake_hip_device_t info{};
+    DeviceModel model;
+    DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
+    DeviceBuffer splitk, gemv, conv, tables, unpacked;
+    hipEvent_t ev[2] = {nullptr, nullptr};
+    hipEvent_t fam[2] = {nullptr, nullptr};
+};
+
+Context g_ctx;
+std::mutex g_mutex;  // one compute call at a time: the workspaces are shared
+
+int ensure_init()
+{
+    if (g_ctx.ready) return CAKE_HIP_OK;
+    return cake_hip_init(0);
+}
+
+bool is_device_pointer(const void* p)
+{
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();  // plain host memory is reported as an error
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+// An operand as the kernels see it.  Host memory is mirrored in a staging slot.
+struct Operand {
+    float* dev = nullptr;
+    float* host = nullptr;  // non-null when staged
+    size_t bytes = 0;
+};
+
+int stage_in(const float* p, size_t bytes, int slot, bool copy, Operand* op)
+{
+    op->bytes = bytes;
+    if (bytes == 0 || is_device_pointer(p)) {
+        op->dev = const_cast<float*>(p);
+        op->host = nullptr;
+        return CAKE_HIP_OK;
+    }
+    int st = g_ctx.stage[slot].reserve(bytes);
+    if (st) return st;
+    op->dev = static_cast<float*>(g_ctx.stage[slot].ptr);
+    op->host = const_cast<float*>(p);
+    if (copy) HIP_TRY(hipMemcpy(op->dev, p, bytes, hipMemcpyHostToDevice));
+    return CAKE_HIP_OK;
+}
+
+int stage_out(const Operand& op, hipStream_t stream)
+{
+    if (!op.host) return CAKE_HIP_OK;
+    HIP_TRY(hipStreamSynchronize(stream));
+    HIP_TRY(hipMemcpy(op.host, op.dev, op.bytes, hipMemcpyDeviceToHost));
+    return CAKE_HIP_OK;
+}
+
+// Event bracket for `seconds`.
+struct Timer {
+    hipStream_t stream;
+    double* out;
+    bool on;
+    Timer(hipStream_t s, double* o) : stream(s), out(o), on(o != nullptr) {}
+    int start()
+    {
+        for (double& f : g_family_seconds) f = 0;
+        if (on) HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
+        return CAKE_HIP_OK;
+    }
+    int stop()
+    {
+        if (!on) return CAKE_HIP_OK;
+        HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));
+        HIP_TRY(hipEventSynchronize(g_ctx.ev[1]));
+        float ms = 0;
+        HIP_TRY(hipEventElapsedTime(&ms, g_ctx.ev[0], g_ctx.ev[1]));
+        *out = ms * 1e-3;
+        return CAKE_HIP_OK;
+    }
+    // time one kernel family when timing is on
+    template <class F>
+    int family(int which, F&& launch)
+    {
+        if (on) HIP_TRY(hipEventRecord(g_ctx.fam[0], stream));
+        hipError_t e = launch();
+        if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+        if (on) {
+            HIP_TRY(hipEventRecord(g_ctx.fam[1], stream));
+            HIP_TRY(hipEventSynchronize(g_ctx.fam[1]));
+            float ms = 0;
+            HIP_TRY(hipEventElapsedTime(&ms, g_ctx.fam[0], g_ctx.fam[1]));
+            g_family_seconds[which] += ms * 1e-3;
+        }
+        return CAKE_HIP_OK;
+    }
+};
+
+bool fits_int(double elems) { return elems < 2147483647.0; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+PackGeom make_geom(int M, int N, int K, int p, const cake_hip_blk_dims_t* d,
+                   const cake_hip_cpu_cntx_t* cx, int sched)
+{
+    PackGeom g;
+    g.d = *d;
+    g.M = M; g.N = N; g.K = K; g.p = p;
+    g.mr = cx->mr; g.nr = cx->nr;
+    g.sch = sched;
+    return g;
+}
+
+int check_geom(const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, int p, int sched)
+{
+    if (!d || !cx) return fail(CAKE_HIP_ERR_ARG, "block dims / cntx is NULL");
+    if (p <= 0 || cx->mr <= 0 || cx->nr <= 0 || d->m_c <= 0 || d->k_c <= 0 || d->n_c <= 0)
+        return fail(CAKE_HIP_ERR_ARG, "block dims are not initialised (p=%d mr=%d nr=%d m_c=%d k_c=%d n_c=%d)",
+                    p, cx->mr, cx->nr, d->m_c, d->k_c, d->n_c);
+    if (sched < CAKE_HIP_KMN || sched > CAKE_HIP_NKM) return fail(CAKE_HIP_ERR_ARG, "unknown schedule %d", sched);
+    return CAKE_HIP_OK;
+}
+
+// Device index tables for one packed operand, carved from g_ctx.tables at `at`.
+int build_tables(int which, const PackGeom& g, size_t* at, IndexTables* out, hipStream_t stream)
+{
+    const int Mp = padded_rows(g), Np = padded_cols(g);
+    const size_t nrows = (which == 1) ? g.K : Mp;
+    const size_t ncols = (which == 0) ? g.K : Np;
+    int4* base = reinterpret_cast<int4*>(static_cast<char*>(g_ctx.tables.ptr) + *at);
+    out->row = base;
+    out->col = base + nrows;
+    *at += (nrows + ncols) * sizeof(int4);
+    hipError_t e = launch_build_index_tables(which, g, base, base + nrows, stream);
+    if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "index table launch failed: %s", hipGetErrorString(e));
+    return CAKE_HIP_OK;
+}
+
+size_t tables_bytes(int which, const PackGeom& g)
+{
+    const size_t nrows = (which == 1) ? g.K : padded_rows(g);
+    const size_t ncols = (which == 0) ? g.K : padded_cols(g);
+    return (nrows + ncols) * sizeof(int4);
+}
+
+// The GEMM proper on device operands.
+int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
+             int sched, int accumulate, const int* tile_override, int a_mode, int b_mode,
+             IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer)
+{
+    const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
+    GemmPlan plan;
+    int st = plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);
+    if (st) return fail(st, "no tile matches the requested override");
+    if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
+        // packed loaders exist for a subset of the tiles
+        if (plan.tile_id != TILE_256x256x32_W128x64 && plan.tile_id != TILE_128x128x32_W64x64 &&
+            plan.tile_id != TILE_64x64x32_W32x32) {
+            const int forced[4] = {128, 128, 32, plan.pub.split_k};
+            st = plan_gemm(M, N, K, sched, forced, false, g_ctx.model, &plan);
+            if (st) return fail(st, "planner failed for packed operands");
+        }
+    }
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+    g.tiles_m = plan.pub.tiles_m; g.tiles_n = plan.pub.tiles_n;
+    g.split_k = plan.pub.split_k; g.k_per_split = plan.k_per_split;
+    g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
+    g.accumulate = accumulate;
+    g.a_tab = a_tab; g.b_tab = b_tab;
+    g.partial = nullptr;
+    if (plan.pub.split_k > 1) {
+        st = g_ctx.splitk.reserve((size_t)plan.pub.split_k * M * N * sizeof(float));
+        if (st) return st;
+        g.partial = static_cast<float*>(g_ctx.splitk.ptr);
+    }
+    st = timer.family(0, [&] { return launch_sgemm(plan.tile_id, a_mode, b_mode, g, plan.pub.grid, stream); });
+    if (st) return st;
+    if (plan.pub.split_k > 1)
+        st = timer.family(1, [&] {
+            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream);
+        });
+    return st;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cake_hip_strerror(int status)
+{
+    switch (status) {
+        case CAKE_HIP_OK: return "ok";
+        case CAKE_HIP_ERR_ARG: return "invalid argument";
+        case CAKE_HIP_ERR_NO_DEVICE: return "no usable HIP device";
+        case CAKE_HIP_ERR_HIP: return "HIP runtime error";
+        case CAKE_HIP_ERR_ALLOC: return "allocation failed";
+        case CAKE_HIP_ERR_RANGE: return "operand exceeds 32-bit element indexing";
+        case CAKE_HIP_ERR_ARCH: return "device is not gfx950";
+        default: return "unknown status";
+    }
+}
+
+const char* cake_hip_last_error(void) { return g_last_error.c_str(); }
+
+int cake_hip_init(int device)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_ctx.ready && g_ctx.device == device) return CAKE_HIP_OK;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(CAKE_HIP_ERR_NO_DEVICE, "hipGetDeviceCount found no device");
+    }
+    if (device < 0 || device >= count) return fail(CAKE_HIP_ERR_ARG, "device %d out of range (%d present)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(CAKE_HIP_ERR_ARCH, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    Context& c = g_ctx;
+    c.device = device;
+    c.info = cake_hip_device_t{};
+    c.info.device = device;
+    c.info.cus = prop.multiProcessorCount;
+    c.info.xcds = 8;
+    c.info.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+    c.info.l2_bytes = prop.l2CacheSize;
+    c.info.wavefront = prop.warpSize;
+    c.info.clock_khz = prop.clockRate;
+    c.info.hbm_bytes = prop.totalGlobalMem;
+    std::snprintf(c.info.arch, sizeof c.info.arch, "%s", prop.gcnArchName);
+    c.model = DeviceModel{};
+    if (c.info.cus > 0) c.model.cus = c.info.cus;
+    if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
+    for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
+        if (!*e) HIP_TRY(hipEventCreate(e));
+    c.ready = true;
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_shutdown(void)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!g_ctx.ready) return CAKE_HIP_OK;
+    (void)hipDeviceSynchronize();
+    for (DeviceBuffer& b : g_ctx.stage) b.release();
+    g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
+    g_ctx.tables.release(); g_ctx.unpacked.release();
+    for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1]}) {
+        if (*e) (void)hipEventDestroy(*e);
+        *e = nullptr;
+    }
+    g_ctx.ready = false;
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_device_info(cake_hip_device_t* out)
+{
+    if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
+    int st = ensure_init();
+    if (st) return st;
+    *out = g_ctx.info;
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_malloc(void** ptr, size_t bytes)
+{
+    if (!ptr) return fail(CAKE_HIP_ERR_ARG, "ptr is NULL");
+    int st = ensure_init();
+    if (st) return st;
+    *ptr = nullptr;
+    if (bytes == 0) return CAKE_HIP_OK;
+    if (hipMalloc(ptr, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(CAKE_HIP_ERR_ALLOC, "device allocation of %zu bytes failed", bytes);
+    }
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_free(void* ptr)
+{
+    if (!ptr) return CAKE_HIP_OK;
+    HIP_TRY(hipFree(ptr));
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_memcpy_h2d(void* dst, const void* src, size_t bytes)
+{
+    if (bytes && (!dst || !src)) return fail(CAKE_HIP_ERR_ARG, "NULL pointer");
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_memcpy_d2h(void* dst, const void* src, size_t bytes)
+{
+    if (bytes && (!dst || !src)) return fail(CAKE_HIP_ERR_ARG, "NULL pointer");
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_memset(void* dst, int value, size_t bytes)
+{
+    if (bytes && !dst) return fail(CAKE_HIP_ERR_ARG, "NULL pointer");
+    HIP_TRY(hipMemset(dst, value, bytes));
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_synchronize(void)
+{
+    HIP_TRY(hipDeviceSynchronize());
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake_hip_plan_t* out)
+{
+    if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
+    GemmPlan plan;
+    const DeviceModel model = g_ctx.ready ? g_ctx.model : DeviceModel{};
+    const bool vec = (K % 4 == 0) && (N % 4 == 0);
+    int st = plan_gemm(M, N, K, sched, tile_override, vec, model, &plan);
+    if (st) return fail(st, "cake_hip_plan: bad shape, schedule or tile override");
+    *out = plan.pub;
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx, int sched,
+                             int mcu, int kcu, int ncu, cake_hip_blk_dims_t* out)
+{
+    int st = init_block_dims(M, N, K, p, cntx, sched, mcu, kcu, ncu, out);
+    if (st) return fail(st, "cake_hip_init_block_dims: invalid argument");
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K, int sched,
+                   int accumulate, const int* tile_override, void* stream_, double* seconds)
+{
+    if (M < 0 || N < 0 || K < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (sched < 0 || sched > CAKE_HIP_NA) return fail(CAKE_HIP_ERR_ARG, "unknown schedule %d", sched);
+    if (seconds) *seconds = 0;
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (!A || !B || !C) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand a, b, c;
+    if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
+    if ((st = stage_in(B, (size_t)K * N * 4, 1, true, &b))) return st;
+    if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if (K == 0) {
+        // empty sum: C = 0 (or unchanged when accumulating); a fill kernel, not a memset node
+        if (!accumulate) {
+            hipError_t e = launch_splitk_reduce(nullptr, c.dev, M, N, N, 0, 0, stream);
+            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
+        }
+    } else {
+        const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(a.dev) && aligned16(b.dev);
+        const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
+        st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, tile_override, mode,
+                      mode, IndexTables{}, IndexTables{}, stream, timer);
+        if (st) return st;
+    }
+    if ((st = timer.stop())) return st;
+    return stage_out(c, stream);
+}
+
+size_t cake_hip_packed_a_size(int M, int K, int p, const cake_hip_blk_dims_t* d,
+                              const cake_hip_cpu_cntx_t* cx, int sched)
+{
+    if (check_geom(d, cx, p, sched)) return 0;
+    PackGeom g = make_geom(M, 0, K, p, d, cx, sched);
+    return (size_t)padded_rows(g) * (size_t)K * sizeof(float);
+}
+
+size_t cake_hip_packed_b_size(int K, int N, int p, const cake_hip_blk_dims_t* d,
+                              const cake_hip_cpu_cntx_t* cx)
+{
+    if (check_geom(d, cx, p, CAKE_HIP_KMN)) return 0;
+    PackGeom g = make_geom(0, N, K, p, d, cx, CAKE_HIP_KMN);
+    return (size_t)K * (size_t)padded_cols(g) * sizeof(float);
+}
+
+size_t cake_hip_packed_c_size(int M, int N, int p, const cake_hip_blk_dims_t* d,
+                              const cake_hip_cpu_cntx_t* cx, int sched)
+{
+    if (check_geom(d, cx, p, sched)) return 0;
+    PackGeom g = make_geom(M, N, 0, p, d, cx, sched);
+    return (size_t)padded_rows(g) * (size_t)padded_cols(g) * sizeof(float);
+}
+
+int64_t cake_hip_packed_offset(int which, int row, int col, int M, int N, int K, int p,
+                               const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, int sched)
+{
+    if (check_geom(d, cx, p, sched)) return -1;
+    PackGeom g = make_geom(M, N, K, p, d, cx, sched);
+    if (row < 0 || col < 0) return -1;
+    switch (which) {
+        case 0: return (row < padded_rows(g) && col < K) ? packed_a_offset(g, row, col) : -1;
+        case 1: return (row < K && col < padded_cols(g)) ? packed_b_offset(g, row, col) : -1;
+        case 2: return (row < padded_rows(g) && col < padded_cols(g)) ? packed_c_offset(g, row, col) : -1;
+        default: return -1;
+    }
+}
+
+// which: 0 A (rows M, cols K), 1 B (rows K, cols N), 2 C (rows M, cols N); dir: 0 pack, 1 unpack
+static int pack_common(int which, int dir, const float* src, float* dst, int M, int N, int K, int p,
+                       const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, int sched,
+                       void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int st = check_geom(d, cx, p, sched);
+    if (st) return st;
+    if (!src || !dst) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    PackGeom g = make_geom(M, N, K, p, d, cx, sched);
+    const int rows = (which == 1) ? K : M, cols = (which == 0) ? K : N;
+    const int rows_p = (which == 1) ? K : padded_rows(g), cols_p = (which == 0) ? K : padded_cols(g);
+    if (rows <= 0 || cols <= 0) return fail(CAKE_HIP_ERR_ARG, "empty operand");
+    if (!fits_int((double)rows_p * cols_p)) return fail(CAKE_HIP_ERR_RANGE, "packed operand exceeds 2^31 elements");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    const size_t plain_bytes = (size_t)rows * cols * 4, packed_bytes = (size_t)rows_p * cols_p * 4;
+    Operand in, out;
+    if ((st = stage_in(src, dir == 0 ? plain_bytes : packed_bytes, 0, true, &in))) return st;
+    // unpack writes only the real extent of C; a staged C must start from the caller's values
+    if ((st = stage_in(dst, dir == 0 ? packed_bytes : plain_bytes, 1, false, &out))) return st;
+    if ((st = g_ctx.tables.reserve(tables_bytes(which, g)))) return st;
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    size_t at = 0;
+    IndexTables tab;
+    if ((st = build_tables(which, g, &at, &tab, stream))) return st;
+    st = timer.family(4, [&] {
+        return dir == 0 ? launch_pack(in.dev, out.dev, rows, cols, cols, rows_p, cols_p, tab, stream)
+                        : launch_unpack(in.dev, out.dev, rows, cols, cols, tab, stream);
+    });
+    if (st) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(out, stream);
+}
+
+int cake_hip_pack_a(const float* A, float* A_p, int M, int K, int p, const cake_hip_blk_dims_t* d,
+                    const cake_hip_cpu_cntx_t* cx, int sched, void* stream, double* seconds)
+{
+    return pack_common(0, 0, A, A_p, M, 0, K, p, d, cx, sched, stream, seconds);
+}
+
+int cake_hip_pack_b(const float* B, float* B_p, int K, int N, int p, const cake_hip_blk_dims_t* d,
+                    const cake_hip_cpu_cntx_t* cx, int sched, void* stream, double* seconds)
+{
+    return pack_common(1, 0, B, B_p, 0, N, K, p, d, cx, sched, stream, seconds);
+}
+
+int cake_hip_pack_c(const float* C, float* C_p, int M, int N, int p, const cake_hip_blk_dims_t* d,
+                    const cake_hip_cpu_cntx_t* cx, int sched, void* stream, double* seconds)
+{
+    return pack_common(2, 0, C, C_p, M, N, 0, p, d, cx, sched, stream, seconds);
+}
+
+int cake_hip_unpack_c(float* C, const float* C_p, int M, int N, int p, const cake_hip_blk_dims_t* d,
+                      const cake_hip_cpu_cntx_t* cx, int sched, void* stream, double* seconds)
+{
+    return pack_common(2, 1, C_p, C, M, N, 0, p, d, cx, sched, stream, seconds);
+}
+
+int cake_hip_sgemm_packed(const float* A, const float* B, float* C, int M, int N, int K, int p,
+                          const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, int packedA,
+                          int packedB, int accumulate, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    if (!packedA && !packedB) return cake_hip_sgemm(A, B, C, M, N, K, d ? d->sch : CAKE_HIP_NA, accumulate, nullptr, stream_, seconds);
+    if (!d) return fail(CAKE_HIP_ERR_ARG, "block dims is NULL");
+    const int sched = d->sch;
+    int st = check_geom(d, cx, p, sched);
+    if (st) return st;
+    if (M <= 0 || N <= 0 || K <= 0) return fail(CAKE_HIP_ERR_ARG, "empty operand");
+    if (!A || !B || !C) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    PackGeom g = make_geom(M, N, K, p, d, cx, sched);
+    const size_t a_elems = packedA ? (size_t)padded_rows(g) * K : (size_t)M * K;
+    const size_t b_elems = packedB ? (size_t)K * padded_cols(g) : (size_t)K * N;
+    if (!fits_int((double)a_elems) || !fits_int((double)b_elems) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand exceeds 2^31 elements");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand a, b, c;
+    if ((st = stage_in(A, a_elems * 4, 0, true, &a))) return st;
+    if ((st = stage_in(B, b_elems * 4, 1, true, &b))) return st;
+    if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;
+    if ((st = g_ctx.tables.reserve((packedA ? tables_bytes(0, g) : 0) + (packedB ? tables_bytes(1, g) : 0)))) return st;
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    size_t at = 0;
+    IndexTables ta{}, tb{};
+    if (packedA && (st = build_tables(0, g, &at, &ta, stream))) return st;
+    if (packedB && (st = build_tables(1, g, &at, &tb, stream))) return st;
+    st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, nullptr,
+                  packedA ? LOAD_PACKED : LOAD_SCALAR, packedB ? LOAD_PACKED : LOAD_SCALAR, ta, tb,
+                  stream, timer);
+    if (st) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(c, stream);
+}
+
+int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K, int a_col_major,
+                   int accumulate, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    if (M < 0 || K < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (M == 0) return CAKE_HIP_OK;
+    if (!y || (K > 0 && (!A || !x))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (!fits_int((double)M * K)) return fail(CAKE_HIP_ERR_RANGE, "matrix of %dx%d exceeds 2^31 elements", M, K);
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand a, xv, yv;
+    if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
+    if ((st = stage_in(x, (size_t)K * 4, 1, true, &xv))) return st;
+    if ((st = stage_in(y, (size_t)M * 4, 2, accumulate != 0, &yv))) return st;
+    if (a_col_major && K > 0) {
+        st = g_ctx.gemv.reserve(sgemv_colmajor_scratch_floats(M, K, g_ctx.model.cus) * sizeof(float));
+        if (st) return st;
+    }
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if (K == 0) {
+        if (!accumulate) {
+            hipError_t e = launch_splitk_reduce(nullptr, yv.dev, M, 1, 1, 0, 0, stream);
+            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
+        }
+    } else {
+        st = timer.family(2, [&] {
+            return a_col_major ? launch_sgemv_colmajor(a.dev, xv.dev, yv.dev, M, K, accumulate,
+                                                       static_cast<float*>(g_ctx.gemv.ptr), g_ctx.model.cus, stream)
+                               : launch_sgemv_rowmajor(a.dev, xv.dev, yv.dev, M, K, accumulate, stream);
+        });
+        if (st) return st;
+    }
+    if ((st = timer.stop())) return st;
+    return stage_out(yv, stream);
+}
+
+static int conv_out_dims(int Hin, int Win, int Hf, int Wf, int stride, int pad, int* Hout, int* Wout)
+{
+    if (Hf <= 0 || Wf <= 0 || stride <= 0 || pad < 0) return 1;
+    if (Hin + 2 * pad < Hf || Win + 2 * pad < Wf) return 1;
+    *Hout = (Hin + 2 * pad - Hf) / stride + 1;
+    *Wout = (Win + 2 * pad - Wf) / stride + 1;
+    return 0;
+}
+
+int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win, int Hf,
+                    int Wf, int stride, int pad, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int Hout, Wout;
+    if (batch <= 0 || Cin <= 0 || Hin <= 0 || Win <= 0 || conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout))
+        return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
+    if (!in || !cols) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    const double krows = (double)Cin * Hf * Wf, ncols = (double)batch * Hout * Wout;
+    if (!fits_int(krows * ncols) || !fits_int((double)batch * Cin * Hin * Win) || krows > 65535)
+        return fail(CAKE_HIP_ERR_RANGE, "column matrix %gx%g out of range", krows, ncols);
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Operand i, o;
+    if ((st = stage_in(in, (size_t)batch * Cin * Hin * Win * 4, 0, true, &i))) return st;
+    if ((st = stage_in(cols, (size_t)(krows * ncols) * 4, 1, false, &o))) return st;
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    st = timer.family(3, [&] {
+        return launch_im2col(i.dev, o.dev, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad, stream);
+    });
+    if (st) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(o, stream);
+}
+
+size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout, int Hf, int Wf,
+                                 int stride, int pad)
+{
+    int Hout, Wout;
+    if (batch <= 0 || Cin <= 0 || Cout <= 0 || conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout)) return 0;
+    const size_t ncols = (size_t)batch * Hout * Wout;
+    // column matrix + a [Cout][ncols] product when the caller wants NCHW
+    return ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float) + 512;
+}
+
+int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
+                    int Win, int Cout, int Hf, int Wf, int stride, int pad, int out_nchw,
+                    void* workspace, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int Hout, Wout;
+    if (batch <= 0 || Cin <= 0 || Cout <= 0 || Hin <= 0 || Win <= 0 ||
+        conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout))
+        return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
+    if (!in || !weights || !out) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    const int K = Cin * Hf * Wf;
+    const double ncols_d = (double)batch * Hout * Wout;
+    if (!fits_int((double)K * ncols_d) || !fits_int((double)Cout * ncols_d) || K > 65535 ||
+        !fits_int((double)batch * Cin * Hin * Win))
+        return fail(CAKE_HIP_ERR_RANGE, "convolution lowers to a %dx%dx%g product that is out of range", Cout, K, ncols_d);
+    const int N = (int)ncols_d;
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand i, w, o;
+    if ((st = stage_in(in, (size_t)batch * Cin * Hin * Win * 4, 0, true, &i))) return st;
+    if ((st = stage_in(weights, (size_t)Cout * K * 4, 1, true, &w))) return st;
+    if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
+
+    char* ws = static_cast<char*>(workspace);
+    if (!ws) {
+        if ((st = g_ctx.conv.reserve(cake_hip_conv2d_workspace(batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)))) return st;
+        ws = static_cast<char*>(g_ctx.conv.ptr);
+    } else if (!is_device_pointer(ws)) {
+        return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
+    }
+    ws = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+    float* cols = reinterpret_cast<float*>(ws);
+    float* cn = cols + (size_t)K * N;  // [Cout][N] product, used only for NCHW output
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    st = timer.family(3, [&] {
+        return launch_im2col(i.dev, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad, stream);
+    });
+    if (st) return st;
+    float* prod = out_nchw ? cn : o.dev;
+    const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(w.dev) && aligned16(cols);
+    const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
+    st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode,
+                  IndexTables{}, IndexTables{}, stream, timer);
+    if (st) return st;
+    if (out_nchw) {
+        st = timer.family(3, [&] { return launch_cn_to_nchw(cn, o.dev, batch, Cout, Hout * Wout, stream); });
+        if (st) return st;
+    }
+    if ((st = timer.stop())) return st;
+    return stage_out(o, stream);
+}
+
+int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream_)
+{
+    if (n == 0) return CAKE_HIP_OK;
+    if (!dst) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Operand o;
+    if ((st = stage_in(dst, n * 4, 0, false, &o))) return st;
+    hipError_t e = launch_fill_uniform(o.dev, n, seed, stream);
+    if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "fill launch failed: %s", hipGetErrorString(e));
+    return stage_out(o, stream);
+}
+
+int cake_hip_last_kernel_seconds(double out[5])
+{
+    if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
+    for (int i = 0; i < 5; ++i) out[i] = g_family_seconds[i];
+    return CAKE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,91 @@
+// kernels.hpp -- launch interface between the host side of the library and the
+// gfx950 kernels.  Every launcher only enqueues on `stream` and returns the
+// hipError_t of the launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "blockdims.hpp"
+
+namespace cake {
+
+// One row (or column) of a packed operand's bilinear index map:
+//   offset(row, col) = R.x + C.x + R.y*C.y + R.z*C.z + R.w*C.w
+// which is the form every packed layout of the reference reduces to.
+struct IndexTables {
+    const int4* row;
+    const int4* col;
+};
+
+struct GemmArgs {
+    const float* A;
+    const float* B;
+    float* C;
+    float* partial;  // split-K slices [split][M][N], or nullptr
+    int M, N, K;
+    int lda, ldb, ldc;
+    int tiles_m, tiles_n;
+    int split_k, k_per_split;  // k_per_split is a multiple of the tile's BK
+    int group, group_along_n;  // CB-block raster
+    int accumulate;
+    IndexTables a_tab, b_tab;  // used by the packed-operand loaders only
+};
+
+// Macro-tile shapes the planner can choose from.
+enum TileId {
+    TILE_256x256x32_W128x64 = 0,  // 8 waves, 2 per SIMD: large compute-bound shapes
+    TILE_256x256x16_W128x128,     // 4 waves, 1 per SIMD, 16 accumulator tiles per wave
+    TILE_256x128x32_W64x64,       // 8 waves: N around 128 (tall-skinny)
+    TILE_128x256x32_W64x64,       // 8 waves: M around 128
+    TILE_128x128x32_W64x64,       // 4 waves: mid-size shapes, 2 workgroups per CU
+    TILE_64x64x32_W32x32,         // 4 waves: small shapes
+    TILE_COUNT
+};
+
+struct TileInfo {
+    int bm, bn, bk, wm, wn, threads, lds_bytes;
+};
+const TileInfo& tile_info(int tile_id);
+
+// Operand addressing of the macro-tile loaders.
+enum LoadMode {
+    LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
+    LOAD_SCALAR = 1, // row-major, any size/alignment
+    LOAD_PACKED = 2  // reference packed layout through IndexTables
+};
+
+hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
+                        hipStream_t stream);
+hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
+                                int accumulate, hipStream_t stream);
+
+hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
+                                 int accumulate, hipStream_t stream);
+// scratch: at least sgemv_colmajor_scratch_floats(M, K) floats
+size_t sgemv_colmajor_scratch_floats(int M, int K, int cus);
+hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,
+                                 int accumulate, float* scratch, int cus, hipStream_t stream);
+
+hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win,
+                         int Hf, int Wf, int Hout, int Wout, int stride, int pad,
+                         hipStream_t stream);
+// [Cout][batch*HW] -> [batch][Cout][HW]
+hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
+                             hipStream_t stream);
+
+hipError_t launch_fill_uniform(float* dst, size_t n, uint64_t seed, hipStream_t stream);
+
+// Packed layouts.  which: 0 = A, 1 = B, 2 = C.
+hipError_t launch_build_index_tables(int which, const PackGeom& g, int4* row_tab, int4* col_tab,
+                                     hipStream_t stream);
+// dst_packed[offset(r,c)] = (r,c) inside the matrix ? src[r*ld + c] : 0   over the padded extent
+hipError_t launch_pack(const float* src, float* dst_packed, int rows, int cols, int ld,
+                       int rows_padded, int cols_padded, IndexTables tab, hipStream_t stream);
+// dst[r*ld + c] = src_packed[offset(r,c)] over the real extent
+hipError_t launch_unpack(const float* src_packed, float* dst, int rows, int cols, int ld,
+                         IndexTables tab, hipStream_t stream);
+
+}  // namespace cake

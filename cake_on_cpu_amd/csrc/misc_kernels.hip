@@ -1,0 +1,345 @@
+// misc_kernels.hip -- im2col, layout change, seeded fill, and the reference's
+// packed layouts (index tables, pack, unpack).  All HBM-bound copies: one
+// thread per output element (or per 4), coalesced along the fastest dimension
+// of whichever side is written.
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+
+namespace cake {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------
+// im2col: im_2_col of examples/cake_conv.cpp:1178-1213 with batch, padding and
+// stride.  grid.y = row k of the column matrix (one (c, h, w) filter tap),
+// threads run along n = (b, ho, wo).
+// ---------------------------------------------------------------------------
+template <int VEC>
+__global__ void __launch_bounds__(256) im2col_kernel(const float* __restrict__ in,
+                                                     float* __restrict__ cols, int batch, int Cin,
+                                                     int Hin, int Win, int Hf, int Wf, int Hout,
+                                                     int Wout, int stride, int pad)
+{
+    const int k = blockIdx.y;
+    const int c = k / (Hf * Wf);
+    const int hw = k - c * (Hf * Wf);
+    const int h = hw / Wf, w = hw - h * Wf;
+    const int HW = Hout * Wout;
+    const size_t ncols = (size_t)batch * HW;
+    float* row = cols + (size_t)k * ncols;
+
+    for (size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC; n < ncols;
+         n += (size_t)gridDim.x * 256 * VEC) {
+        const int b = (int)(n / HW);
+        const int r = (int)(n - (size_t)b * HW);
+        const int ho = r / Wout, wo = r - ho * Wout;
+        const int hi = ho * stride + h - pad;
+        const float* src = in + (((size_t)b * Cin + c) * Hin + hi) * Win;
+        const bool hrow = hi >= 0 && hi < Hin;
+        float v[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const int wi = (wo + e) * stride + w - pad;  // VEC > 1 only when Wout % VEC == 0
+            v[e] = (hrow && wi >= 0 && wi < Win) ? src[wi] : 0.f;
+        }
+        if (VEC == 4) {
+            f32x4 o = {v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(row + n));
+        } else {
+            row[n] = v[0];
+        }
+    }
+}
+
+hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win, int Hf,
+                         int Wf, int Hout, int Wout, int stride, int pad, hipStream_t stream)
+{
+    const int krows = Cin * Hf * Wf;
+    const size_t ncols = (size_t)batch * Hout * Wout;
+    if (krows <= 0 || ncols == 0) return hipSuccess;
+    if (krows > 65535) return hipErrorInvalidValue;
+    const bool vec = (Wout % 4 == 0) && (reinterpret_cast<uintptr_t>(cols) % 16 == 0);
+    const size_t per_block = 256 * (vec ? 4 : 1);
+    size_t bx = (ncols + per_block - 1) / per_block;
+    if (bx > 4096) bx = 4096;
+    const dim3 grid((unsigned)bx, krows);
+    if (vec)
+        hipLaunchKernelGGL(im2col_kernel<4>, grid, dim3(256), 0, stream, in, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad);
+    else
+        hipLaunchKernelGGL(im2col_kernel<1>, grid, dim3(256), 0, stream, in, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad);
+    return hipGetLastError();
+}
+
+// [Cout][batch][HW] -> [batch][Cout][HW]
+__global__ void __launch_bounds__(256) cn_to_nchw_kernel(const float* __restrict__ src,
+                                                         float* __restrict__ dst, int batch,
+                                                         int Cout, int HW)
+{
+    const size_t total = (size_t)batch * Cout * HW;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int hw = (int)(i % HW);
+        const size_t t = i / HW;
+        const int co = (int)(t % Cout);
+        const int b = (int)(t / Cout);
+        dst[i] = src[((size_t)co * batch + b) * HW + hw];
+    }
+}
+
+hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
+                             hipStream_t stream)
+{
+    const size_t total = (size_t)batch * Cout * HW;
+    if (total == 0) return hipSuccess;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(cn_to_nchw_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, batch, Cout, HW);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Seeded uniform[-1,1): element i = 24 top bits of splitmix64(seed + (i+1)*G).
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) fill_uniform_kernel(float* __restrict__ dst, size_t n,
+                                                           uint64_t seed)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        uint64_t z = seed + (i + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        dst[i] = (float)(uint32_t)(z >> 40) * 0x1p-23f - 1.0f;
+    }
+}
+
+hipError_t launch_fill_uniform(float* dst, size_t n, uint64_t seed, hipStream_t stream)
+{
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_uniform_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dst, n, seed);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Packed layouts as bilinear index tables.
+//
+// Every packed layout of the reference places element (r, c) at
+//     R[r].x + C[c].x + R[r].y*C[c].y + R[r].z*C[c].z + R[r].w*C[c].w
+// where R depends only on the row and C only on the column: the CB-block walk
+// contributes (block start) x (block extent of the other dimension) products
+// and the m_r / n_r panels contribute (panel start) x (panel depth) products.
+// Building the two tables costs a handful of integer divisions per row and
+// per column; packing, unpacking and the GEMM loaders then address packed
+// data with two table reads and three multiply-adds per element.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ SplitPos split_m(const PackGeom& g, int row)
+{
+    return split_pos(row, g.p, g.d.m_c, g.d.Mb, g.d.m_pad, g.mr * g.d.mr_rem, g.d.m_c1, g.d.p_l,
+                     g.d.m_c1_last_core);
+}
+
+__device__ __forceinline__ SplitPos split_k(const PackGeom& g, int k)
+{
+    return split_pos(k, g.p, g.d.k_c, g.d.Kb, g.d.k_pad, g.d.k_rem, g.d.k_c1, g.d.p_l,
+                     g.d.k_c1_last_core);
+}
+
+// Row of C or A inside an M block of the K-split schedules.
+struct MPos { int mb, rows, panel, j; };
+
+__device__ __forceinline__ MPos m_block_pos(const PackGeom& g, int row)
+{
+    const int mspan = (g.sch == CAKE_HIP_MKN) ? g.d.m_c : g.p * g.d.m_c;
+    MPos r;
+    r.mb = row / mspan;
+    const int in = row - r.mb * mspan;
+    r.rows = (g.d.m_pad && r.mb == g.d.Mb - 1) ? g.d.m_c1 : mspan;
+    r.panel = in / g.mr;
+    r.j = in - r.panel * g.mr;
+    return r;
+}
+
+struct NPos { int nb, cols, panel, j; };
+
+__device__ __forceinline__ NPos n_block_pos(const PackGeom& g, int col)
+{
+    NPos r;
+    r.nb = col / g.d.n_c;
+    const int in = col - r.nb * g.d.n_c;
+    r.cols = (g.d.n_pad && r.nb == g.d.Nb - 1) ? g.d.n_c1 : g.d.n_c;
+    r.panel = in / g.nr;
+    r.j = in - r.panel * g.nr;
+    return r;
+}
+
+// K position of the K-first schedule (K not split over cores).
+struct KPos { int kb, kk, kc; };
+
+__device__ __forceinline__ KPos k_block_pos(const PackGeom& g, int k)
+{
+    KPos r;
+    r.kb = k / g.d.k_c;
+    r.kk = k - r.kb * g.d.k_c;
+    r.kc = (g.d.k_pad && r.kb == g.d.Kb - 1) ? g.d.k_c1 : g.d.k_c;
+    return r;
+}
+
+__global__ void __launch_bounds__(256) build_tables_kernel(int which, PackGeom g, int4* row_tab,
+                                                           int nrows, int4* col_tab, int ncols)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int mr = g.mr, nr = g.nr;
+    const int Mp = padded_rows(g), Np = padded_cols(g);
+    const int mspan = g.p * g.d.m_c, kspan = g.p * g.d.k_c;
+
+    if (i < nrows) {
+        int4 R = make_int4(0, 0, 0, 0);
+        if (which == 0) {  // A: rows are m
+            if (g.sch == CAKE_HIP_KMN) {
+                const SplitPos m = split_m(g, i);
+                const int panel = m.inner / mr, j = m.inner - panel * mr;
+                R = make_int4(m.block * mspan * g.K + j, m.span, m.core * m.slice + panel * mr, 0);
+            } else {
+                const MPos m = m_block_pos(g, i);
+                if (g.sch == CAKE_HIP_MKN) R = make_int4(m.j, m.mb * g.d.m_c, m.rows, m.panel * mr);
+                else R = make_int4(m.mb * mspan * g.K + m.j, m.rows, m.panel * mr, 0);
+            }
+        } else if (which == 1) {  // B: rows are k
+            if (g.sch == CAKE_HIP_KMN) {
+                const KPos k = k_block_pos(g, i);
+                R = make_int4(k.kk * nr, k.kb * g.d.k_c, k.kc, 0);
+            } else {
+                const SplitPos k = split_k(g, i);
+                if (g.sch == CAKE_HIP_MKN)
+                    R = make_int4(k.inner * nr, k.block * kspan + k.core * k.slice, k.length, 0);
+                else
+                    R = make_int4(k.block * kspan * Np + k.inner * nr, k.span, k.core * k.slice, k.length);
+            }
+        } else {  // C: rows are m
+            if (g.sch == CAKE_HIP_KMN) {
+                const SplitPos m = split_m(g, i);
+                const int pm = m.inner / mr, ii = m.inner - pm * mr;
+                R = make_int4(pm * mr * nr + ii * nr, m.block * mspan + m.core * m.slice, m.length, 0);
+            } else {
+                const MPos m = m_block_pos(g, i);
+                const int in = m.panel * mr * nr + m.j * nr;
+                if (g.sch == CAKE_HIP_MKN) R = make_int4(in, m.mb * g.d.m_c, m.rows, 0);
+                else R = make_int4(Np * m.mb * mspan + in, m.rows, 0, 0);
+            }
+        }
+        row_tab[i] = R;
+    }
+
+    if (i < ncols) {
+        int4 Cc = make_int4(0, 0, 0, 0);
+        if (which == 0) {  // A: columns are k
+            if (g.sch == CAKE_HIP_KMN) {
+                const KPos k = k_block_pos(g, i);
+                Cc = make_int4(k.kk * mr, k.kb * g.d.k_c, k.kc, 0);
+            } else {
+                const SplitPos k = split_k(g, i);
+                if (g.sch == CAKE_HIP_MKN)
+                    Cc = make_int4(k.block * Mp * kspan + k.inner * mr, k.span, k.core * k.slice, k.length);
+                else
+                    Cc = make_int4(k.inner * mr, k.block * kspan + k.core * k.slice, k.length, 0);
+            }
+        } else {  // B and C: columns are n
+            const NPos n = n_block_pos(g, i);
+            if (which == 1) {
+                if (g.sch == CAKE_HIP_NKM) Cc = make_int4(n.j, n.nb * g.d.n_c, n.cols, n.panel * nr);
+                else Cc = make_int4(n.nb * g.K * g.d.n_c + n.j, n.cols, n.panel * nr, 0);
+            } else {
+                if (g.sch == CAKE_HIP_KMN) Cc = make_int4(n.nb * g.d.n_c * Mp + n.j, n.cols, n.panel * nr, 0);
+                else if (g.sch == CAKE_HIP_MKN) Cc = make_int4(Mp * n.nb * g.d.n_c + n.j, n.cols, n.panel * nr, 0);
+                else Cc = make_int4(n.j, n.nb * g.d.n_c + n.panel * nr, 0, 0);
+            }
+        }
+        col_tab[i] = Cc;
+    }
+}
+
+hipError_t launch_build_index_tables(int which, const PackGeom& g, int4* row_tab, int4* col_tab,
+                                     hipStream_t stream)
+{
+    const int Mp = padded_rows(g), Np = padded_cols(g);
+    const int nrows = (which == 1) ? g.K : Mp;
+    const int ncols = (which == 0) ? g.K : Np;
+    const int n = nrows > ncols ? nrows : ncols;
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(build_tables_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, which, g,
+                       row_tab, nrows, col_tab, ncols);
+    return hipGetLastError();
+}
+
+__device__ __forceinline__ size_t table_offset(const int4 R, const int4 Cc)
+{
+    return (size_t)(R.x + Cc.x + R.y * Cc.y + R.z * Cc.z + R.w * Cc.w);
+}
+
+// pack_A / pack_B / pack_C (src/pack_helper.cpp:92-160): row-major -> packed,
+// zero in the padding (src/pack_ob.cpp:46-50).
+__global__ void __launch_bounds__(256) pack_kernel(const float* __restrict__ src,
+                                                   float* __restrict__ dst, int rows, int cols,
+                                                   int ld, int rows_p, int cols_p, IndexTables tab)
+{
+    const int r = blockIdx.y;
+    const int4 R = tab.row[r];
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < cols_p; c += gridDim.x * 256) {
+        const float v = (r < rows && c < cols) ? src[(size_t)r * ld + c] : 0.f;
+        dst[table_offset(R, tab.col[c])] = v;
+    }
+}
+
+// unpack_C (src/pack_helper.cpp:163-184, src/pack_ob.cpp:393-411): packed ->
+// row-major, real extent only, assignment.
+__global__ void __launch_bounds__(256) unpack_kernel(const float* __restrict__ src,
+                                                     float* __restrict__ dst, int rows, int cols,
+                                                     int ld, IndexTables tab)
+{
+    const int r = blockIdx.y;
+    const int4 R = tab.row[r];
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < cols; c += gridDim.x * 256)
+        dst[(size_t)r * ld + c] = src[table_offset(R, tab.col[c])];
+}
+
+static dim3 rowwise_grid(int rows, int cols)
+{
+    int bx = (cols + 255) / 256;
+    if (bx > 1024) bx = 1024;
+    return dim3(bx, rows);
+}
+
+hipError_t launch_pack(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
+                       int cols_p, IndexTables tab, hipStream_t stream)
+{
+    if (rows_p <= 0 || cols_p <= 0) return hipSuccess;
+    // grid.y is limited to 65535 rows per launch
+    for (int r0 = 0; r0 < rows_p; r0 += 65535) {
+        const int nr = rows_p - r0 < 65535 ? rows_p - r0 : 65535;
+        IndexTables t = {tab.row + r0, tab.col};
+        const int live = rows - r0 < 0 ? 0 : rows - r0;
+        hipLaunchKernelGGL(pack_kernel, rowwise_grid(nr, cols_p), dim3(256), 0, stream,
+                           src + (size_t)r0 * ld, dst, live, cols, ld, nr, cols_p, t);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_unpack(const float* src, float* dst, int rows, int cols, int ld, IndexTables tab,
+                         hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    for (int r0 = 0; r0 < rows; r0 += 65535) {
+        const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
+        IndexTables t = {tab.row + r0, tab.col};
+        hipLaunchKernelGGL(unpack_kernel, rowwise_grid(nr, cols), dim3(256), 0, stream, src,
+                           dst + (size_t)r0 * ld, nr, cols, ld, t);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace cake

@@ -1,0 +1,158 @@
+// planner.cpp -- see planner.hpp.
+#include "planner.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "kernels.hpp"
+
+namespace cake {
+
+namespace {
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Fraction of a CU's MFMA peak a workgroup of this shape sustains in the
+// middle of a long K walk (measured on MI355X; larger tiles amortise the
+// stage loads and the barrier over more matrix work).
+double tile_efficiency(int tile_id)
+{
+    switch (tile_id) {
+        case TILE_256x256x32_W128x64: return 0.80;
+        case TILE_256x256x16_W128x128: return 0.70;
+        case TILE_256x128x32_W64x64: return 0.70;
+        case TILE_128x256x32_W64x64: return 0.70;
+        case TILE_128x128x32_W64x64: return 0.60;
+        default: return 0.30;
+    }
+}
+
+struct Candidate {
+    int tile_id, split;
+    double seconds;
+};
+
+// Modelled time of one tile shape with one split factor.
+double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
+{
+    const TileInfo& t = tile_info(tile_id);
+    const int tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const long wgs = (long)tiles * split;
+    const int ksteps = ceil_div(ceil_div(K, split), t.bk);
+    // prologue (first stage load) and epilogue (C store) cost about two K steps
+    const double wg_flops = 2.0 * t.bm * t.bn * t.bk * (ksteps + 2);
+    const double cu_rate = dev.mfma_flops / dev.cus * tile_efficiency(tile_id);
+    const long per_cu = (wgs + dev.cus - 1) / dev.cus;
+    double s = per_cu * wg_flops / cu_rate;
+    // never faster than streaming the operands once
+    const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
+    s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
+    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 4e-6;
+    return s + 3e-6;  // launch
+}
+
+}  // namespace
+
+int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, const DeviceModel& dev,
+              GemmPlan* out)
+{
+    if (!out || M <= 0 || N <= 0 || K <= 0 || sched < 0 || sched > CAKE_HIP_NA) return CAKE_HIP_ERR_ARG;
+    std::memset(out, 0, sizeof *out);
+
+    int want_m = ov ? ov[0] : 0, want_n = ov ? ov[1] : 0, want_k = ov ? ov[2] : 0;
+    int want_split = ov ? ov[3] : 0;
+    if (want_m < 0 || want_n < 0 || want_k < 0 || want_split < 0) return CAKE_HIP_ERR_ARG;
+
+    Candidate best = {-1, 1, 1e30};
+    for (int id = 0; id < TILE_COUNT; ++id) {
+        const TileInfo& t = tile_info(id);
+        if (want_m && t.bm != want_m) continue;
+        if (want_n && t.bn != want_n) continue;
+        if (want_k && t.bk != want_k) continue;
+        if (t.lds_bytes > dev.lds_per_cu) continue;
+        // the single-wave-per-SIMD variant is only taken when asked for by its K depth
+        if (id == TILE_256x256x16_W128x128 && !want_k) continue;
+        const int max_split = std::max(1, K / (4 * t.bk));
+        for (int split = 1; split <= 64; split *= 2) {
+            if (want_split && split != want_split) continue;
+            if (!want_split && split > max_split) break;
+            const double s = model_seconds(M, N, K, id, split, dev);
+            if (s < best.seconds) best = {id, split, s};
+        }
+        if (want_split && (want_split & (want_split - 1))) {  // non power of two asked for
+            const double s = model_seconds(M, N, K, id, want_split, dev);
+            if (s < best.seconds) best = {id, want_split, s};
+        }
+    }
+    if (best.tile_id < 0) return CAKE_HIP_ERR_ARG;  // no tile matches the override
+
+    const TileInfo& t = tile_info(best.tile_id);
+    cake_hip_plan_t& p = out->pub;
+    out->tile_id = best.tile_id;
+    p.tile_m = t.bm; p.tile_n = t.bn; p.tile_k = t.bk;
+    p.wave_m = t.wm; p.wave_n = t.wn;
+    p.threads = t.threads;
+    p.lds_bytes = t.lds_bytes;
+    p.tiles_m = ceil_div(M, t.bm);
+    p.tiles_n = ceil_div(N, t.bn);
+    p.split_k = best.split;
+    out->k_per_split = ceil_div(ceil_div(K, best.split), t.bk) * t.bk;
+    // drop slices that would start past K
+    p.split_k = ceil_div(K, out->k_per_split);
+    p.grid = p.tiles_m * p.tiles_n * p.split_k;
+    p.vector_loads = vector_ok ? 1 : 0;
+    p.cus = dev.cus;
+    p.flops = 2.0 * M * N * (double)K;
+    p.min_bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
+
+    // Reuse order.  `resident` tiles run at the same time on one XCD and share
+    // its L2: a gm x gn block of them re-reads each A panel ceil(tiles_n/gn)
+    // times and each B panel ceil(tiles_m/gm) times from HBM.
+    const int slots = std::max(1, std::min(dev.lds_per_cu / t.lds_bytes, 2048 / t.threads));
+    const int resident = std::max(1, dev.cus / dev.xcds * slots);
+    auto traffic = [&](int gm, int gn) {
+        return 4.0 * ((double)M * K * ceil_div(p.tiles_n, gn) + (double)K * N * ceil_div(p.tiles_m, gm) +
+                      (double)M * N);
+    };
+    int gm, gn;
+    int resolved = sched;
+    if (sched == CAKE_HIP_NA) {
+        // pick the block shape with the least modelled traffic; name it after
+        // the reference schedule it corresponds to
+        double best_bytes = 1e300;
+        gm = 1; gn = resident;
+        for (int g = 1; g <= resident; g *= 2) {
+            const int cm = std::min(g, p.tiles_m), cn = std::min(std::max(1, resident / g), p.tiles_n);
+            const double b = traffic(cm, cn);
+            if (b < best_bytes) { best_bytes = b; gm = cm; gn = cn; }
+        }
+        if (gn == 1 && p.tiles_m > 1) resolved = CAKE_HIP_MKN;       // a column of tiles
+        else if (gm == 1 && p.tiles_n > 1) resolved = CAKE_HIP_NKM;  // a row of tiles
+        else resolved = CAKE_HIP_KMN;
+    }
+    if (resolved == CAKE_HIP_MKN) {          // M-first: walk down a tile column, B panel shared
+        out->group_along_n = 1;
+        p.group = 1;
+        gm = std::min(resident, p.tiles_m); gn = 1;
+    } else if (resolved == CAKE_HIP_NKM) {   // N-first: walk along a tile row, A panel shared
+        out->group_along_n = 0;
+        p.group = 1;
+        gm = 1; gn = std::min(resident, p.tiles_n);
+    } else {                                 // K-first with a compact CB block
+        if (sched != CAKE_HIP_NA) {
+            gm = std::max(1, (int)std::lround(std::sqrt((double)resident * t.bn / t.bm)));
+            int pow2 = 1;
+            while (pow2 * 2 <= gm) pow2 *= 2;
+            gm = std::min(pow2, p.tiles_m);
+            gn = std::min(std::max(1, resident / gm), p.tiles_n);
+        }
+        out->group_along_n = 0;
+        p.group = gm;
+    }
+    p.sched = resolved;
+    p.model_bytes = traffic(gm, gn);
+    return CAKE_HIP_OK;
+}
+
+}  // namespace cake

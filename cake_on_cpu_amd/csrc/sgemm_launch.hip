@@ -1,0 +1,69 @@
+// GEMM launch dispatch, tile table and the split-K reduction.
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
+hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
+hipError_t launch_sgemm_packed(int tile_id, int a_mode, int b_mode, const GemmArgs& a, int grid,
+                               hipStream_t s);
+
+template <class T>
+static constexpr TileInfo info_of()
+{
+    return TileInfo{T::BM, T::BN, T::BK, T::WM, T::WN, T::THREADS, T::LDS_BYTES};
+}
+
+const TileInfo& tile_info(int tile_id)
+{
+    static const TileInfo table[TILE_COUNT] = {
+        info_of<Tile256x256x32>(), info_of<Tile256x256x16>(), info_of<Tile256x128x32>(),
+        info_of<Tile128x256x32>(), info_of<Tile128x128x32>(), info_of<Tile64x64x32>(),
+    };
+    return table[tile_id < 0 || tile_id >= TILE_COUNT ? TILE_64x64x32_W32x32 : tile_id];
+}
+
+hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
+                        hipStream_t stream)
+{
+    if (grid <= 0) return hipSuccess;
+    if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
+        if (a_mode == LOAD_VEC4) a_mode = LOAD_SCALAR;
+        if (b_mode == LOAD_VEC4) b_mode = LOAD_SCALAR;
+        return launch_sgemm_packed(tile_id, a_mode, b_mode, args, grid, stream);
+    }
+    if (a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4) return launch_sgemm_vec(tile_id, args, grid, stream);
+    return launch_sgemm_scalar(tile_id, args, grid, stream);
+}
+
+// C = (accumulate ? C : 0) + sum over slices in ascending order: a fixed
+// summation order, so the split-K path is run-to-run deterministic like the
+// reference (one accumulation chain per element, no atomics).
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial,
+                                                            float* __restrict__ C, int M, int N,
+                                                            int ldc, int splits, int accumulate)
+{
+    const size_t total = (size_t)M * N;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const int row = (int)(i / N), col = (int)(i - (size_t)row * N);
+        float* dst = C + (size_t)row * ldc + col;
+        float acc = accumulate ? *dst : 0.f;
+        for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * total + i];
+        *dst = acc;
+    }
+}
+
+hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
+                                int accumulate, hipStream_t stream)
+{
+    const size_t total = (size_t)M * N;
+    if (total == 0) return hipSuccess;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
+                       M, N, ldc, splits, accumulate);
+    return hipGetLastError();
+}
+
+}  // namespace cake

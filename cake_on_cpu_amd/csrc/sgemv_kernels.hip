@@ -1,0 +1,189 @@
+// sgemv_kernels.hip -- bandwidth-bound fp32 matrix-vector kernels for gfx950.
+//
+// They replace cake_sgemv's schedule_mvm + cake_sgemv_haswell_8x8_col
+// (examples/cake_gemv.cpp:89-140,424-490).  A is read exactly once with
+// 16-byte, fully coalesced loads; x is small and is served from cache.
+//
+//   row-major  A[m*K + k]: one wavefront per 4 rows, lanes stride over k,
+//              64-lane butterfly reduction at the end.
+//   col-major  A[k*M + m] (the reference's layout): lanes own 4 consecutive m,
+//              K is cut into slices across workgroups and waves; slices are
+//              summed in a fixed order (no atomics), so results are
+//              run-to-run identical.
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+
+namespace cake {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// row-major
+// ---------------------------------------------------------------------------
+template <int ROWS, bool VEC>
+__global__ void __launch_bounds__(256) sgemv_rowmajor_kernel(const float* __restrict__ A,
+                                                             const float* __restrict__ x,
+                                                             float* __restrict__ y, int M, int K,
+                                                             int accumulate)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row0 = wave * ROWS;
+    if (row0 >= M) return;
+
+    float acc[ROWS];
+    const float* rowp[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        acc[r] = 0.f;
+        // rows past the end re-read the last row; their sums are dropped below
+        rowp[r] = A + (size_t)min(row0 + r, M - 1) * K;
+    }
+
+    if (VEC) {
+        const int K4 = K >> 2;
+        const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+#pragma unroll 4
+        for (int c = lane; c < K4; c += 64) {
+            const f32x4 xv = x4[c];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const f32x4 av = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(rowp[r]) + c);
+                acc[r] += av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
+            }
+        }
+    } else {
+#pragma unroll 4
+        for (int c = lane; c < K; c += 64) {
+            const float xv = x[c];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[r] += rowp[r][c] * xv;
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < M) y[row0 + r] = accumulate ? y[row0 + r] + s : s;
+    }
+}
+
+hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
+                                 int accumulate, hipStream_t stream)
+{
+    if (M <= 0) return hipSuccess;
+    constexpr int ROWS = 4;
+    const bool vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(x)) % 16 == 0);
+    const int waves = (M + ROWS - 1) / ROWS;
+    const int blocks = (waves + 3) / 4;
+    if (vec)
+        hipLaunchKernelGGL((sgemv_rowmajor_kernel<ROWS, true>), dim3(blocks), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+    else
+        hipLaunchKernelGGL((sgemv_rowmajor_kernel<ROWS, false>), dim3(blocks), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// column-major
+// ---------------------------------------------------------------------------
+static constexpr int COL_BLOCK_M = 256;  // columns of y per workgroup
+
+static int colmajor_slices(int M, int K, int cus)
+{
+    const int mblocks = (M + COL_BLOCK_M - 1) / COL_BLOCK_M;
+    int want = (8 * cus + mblocks - 1) / mblocks;  // ~8 workgroups per CU
+    int max_slices = (K + 63) / 64;                // at least 64 k per slice
+    if (want > max_slices) want = max_slices;
+    if (want < 1) want = 1;
+    return want;
+}
+
+size_t sgemv_colmajor_scratch_floats(int M, int K, int cus)
+{
+    return (size_t)colmajor_slices(M, K, cus) * (size_t)M;
+}
+
+// grid = (m blocks, k slices).  VEC: each wave covers all 256 columns of the
+// block with one 16-byte load per lane and takes a quarter of the slice's k
+// range; the four waves are summed through LDS in wave order.  Scalar: each
+// thread owns one column over the whole slice.
+template <bool VEC>
+__global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __restrict__ A,
+                                                             const float* __restrict__ x,
+                                                             float* __restrict__ out, int M, int K,
+                                                             int k_per_slice)
+{
+    __shared__ float red[4][COL_BLOCK_M];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kbeg = blockIdx.y * k_per_slice;
+    const int kend = min(K, kbeg + k_per_slice);
+    float* dst = out + (size_t)blockIdx.y * M;
+
+    if (VEC) {
+        const int m = blockIdx.x * COL_BLOCK_M + lane * 4;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (m < M) {
+            const int span = (kend - kbeg + 3) / 4;
+            const int k0 = kbeg + wave * span, k1 = min(kend, k0 + span);
+            const float* col = A + (size_t)k0 * M + m;
+#pragma unroll 8
+            for (int k = k0; k < k1; ++k, col += M) {
+                const f32x4 av = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(col));
+                const float xv = x[k];
+                acc.x += av.x * xv; acc.y += av.y * xv; acc.z += av.z * xv; acc.w += av.w * xv;
+            }
+        }
+        *reinterpret_cast<f32x4*>(&red[wave][lane * 4]) = acc;
+        __syncthreads();
+        const int mm = blockIdx.x * COL_BLOCK_M + tid;
+        if (mm < M) dst[mm] = ((red[0][tid] + red[1][tid]) + red[2][tid]) + red[3][tid];
+    } else {
+        const int m = blockIdx.x * COL_BLOCK_M + tid;
+        if (m >= M) return;
+        float acc = 0.f;
+        const float* col = A + (size_t)kbeg * M + m;
+#pragma unroll 8
+        for (int k = kbeg; k < kend; ++k, col += M) acc += *col * x[k];
+        dst[m] = acc;
+    }
+}
+
+__global__ void __launch_bounds__(256) sgemv_slice_reduce_kernel(const float* __restrict__ part,
+                                                                 float* __restrict__ y, int M,
+                                                                 int slices, int accumulate)
+{
+    const int m = blockIdx.x * 256 + threadIdx.x;
+    if (m >= M) return;
+    float acc = accumulate ? y[m] : 0.f;
+    for (int s = 0; s < slices; ++s) acc += part[(size_t)s * M + m];
+    y[m] = acc;
+}
+
+hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,
+                                 int accumulate, float* scratch, int cus, hipStream_t stream)
+{
+    if (M <= 0) return hipSuccess;
+    const int slices = colmajor_slices(M, K, cus);
+    int k_per_slice = (K + slices - 1) / slices;
+    k_per_slice = (k_per_slice + 3) & ~3;
+    const bool vec = (M % 4 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0);
+    const dim3 grid((M + COL_BLOCK_M - 1) / COL_BLOCK_M, slices);
+    if (vec)
+        hipLaunchKernelGGL((sgemv_colmajor_kernel<true>), grid, dim3(256), 0, stream, A, x, scratch, M, K, k_per_slice);
+    else
+        hipLaunchKernelGGL((sgemv_colmajor_kernel<false>), grid, dim3(256), 0, stream, A, x, scratch, M, K, k_per_slice);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 255) / 256), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
+    return hipGetLastError();
+}
+
+}  // namespace cake

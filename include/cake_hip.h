@@ -1,0 +1,218 @@
+/*
+ * cake_hip.h -- C-ABI of the MI355X (gfx950) implementation of CAKE's fp32
+ * GEMM hot path: cake_sgemm, cake_sgemv and the im2col -> GEMM convolution.
+ *
+ * Plain C: pointers, ints, sizes and status codes only.  This is the surface a
+ * foreign-function binding (ctypes, cgo, JNI, N-API) or the C++ drop-in
+ * library (include/cake.h) binds to.  Each entry point names the interface of
+ * vnatesh/CAKE_on_CPU it replaces.
+ *
+ * Pointers.  Every matrix/vector argument may be a device pointer (memory from
+ * cake_hip_malloc, hipMalloc or a torch ROCm tensor) or a plain host pointer.
+ * Host operands are staged through device buffers owned by the library and
+ * results copied back before the call returns.  `seconds`, when not NULL,
+ * receives the device time of the kernels alone (HIP events on the stream the
+ * kernels ran on); staging copies are not part of it.
+ *
+ * Streams.  `stream` is a hipStream_t passed as void*; NULL is the default
+ * stream.  With device operands and seconds == NULL a call only enqueues work.
+ *
+ * Every function returns CAKE_HIP_OK (0) or an error code; no function calls
+ * exit().  cake_hip_last_error() gives the text of the last failure on the
+ * calling thread.
+ */
+#ifndef CAKE_HIP_H
+#define CAKE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* enum sched of the reference (include/common.h:105), same values. */
+enum { CAKE_HIP_KMN = 0, CAKE_HIP_MKN = 1, CAKE_HIP_NKM = 2, CAKE_HIP_NA = 3 };
+
+enum {
+    CAKE_HIP_OK = 0,
+    CAKE_HIP_ERR_ARG = 1,       /* NULL pointer, negative size, unknown schedule */
+    CAKE_HIP_ERR_NO_DEVICE = 2, /* no usable gfx950 device                       */
+    CAKE_HIP_ERR_HIP = 3,       /* a HIP runtime call failed                     */
+    CAKE_HIP_ERR_ALLOC = 4,     /* device or host allocation failed              */
+    CAKE_HIP_ERR_RANGE = 5,     /* an operand does not fit 32-bit element indexing */
+    CAKE_HIP_ERR_ARCH = 6       /* device is not gfx950                          */
+};
+
+/* blk_dims_t of the reference (include/common.h:108-135): same fields, same order. */
+typedef struct cake_hip_blk_dims_t {
+    int m_c, k_c, n_c;
+    int m_c1, k_c1, n_c1;
+    int m_c1_last_core, n_c1_last_core, k_c1_last_core;
+    int mr_rem, nr_rem, k_rem;
+    int p_l, pm_l, pn_l, pm, pn;
+    int m_pad, k_pad, n_pad;
+    int Mb, Kb, Nb;
+    int M_padded, N_padded;
+    int sch;
+} cake_hip_blk_dims_t;
+
+/* The CPU-cache description the reference's block sizing reads from
+ * cake_cntx_t (include/common.h:138-151). */
+typedef struct cake_hip_cpu_cntx_t {
+    double alpha_n; /* written back by cake_hip_init_block_dims */
+    int mr, nr;
+    int L1, L2, L3;
+    int ncores;
+} cake_hip_cpu_cntx_t;
+
+/* What the GPU planner decided for one GEMM: the successor of
+ * get_cache_dims / derive_schedule (src/block_sizing.cpp:304-462). */
+typedef struct cake_hip_plan_t {
+    int sched;        /* resolved reuse order: KMN, MKN or NKM                   */
+    int tile_m, tile_n, tile_k; /* macro-tile held by one workgroup               */
+    int wave_m, wave_n;         /* sub-tile held by one 64-lane wavefront         */
+    int threads;      /* workgroup size                                           */
+    int split_k;      /* K slices reduced in a second, fixed-order pass (1 = none) */
+    int tiles_m, tiles_n;
+    int group;        /* CB-block edge in tiles: tiles that run together share panels */
+    int grid;         /* workgroups launched                                      */
+    int lds_bytes;    /* LDS per workgroup (double buffered)                      */
+    int vector_loads; /* 1: 16-byte global loads usable (K%4==0, N%4==0, aligned) */
+    int cus;          /* compute units the plan was made for                      */
+    double flops;     /* 2*M*N*K                                                  */
+    double min_bytes; /* compulsory traffic 4*(MK+KN+MN)                          */
+    double model_bytes; /* modelled HBM traffic of the chosen order and CB block  */
+} cake_hip_plan_t;
+
+typedef struct cake_hip_device_t {
+    int device;
+    int cus;
+    int xcds;
+    int lds_bytes_per_cu;
+    int l2_bytes;
+    int wavefront;
+    int clock_khz;
+    size_t hbm_bytes;
+    char arch[32];
+} cake_hip_device_t;
+
+/* ---- lifetime ---------------------------------------------------------- */
+/* Selects `device`, checks that it is gfx950 and creates the library context.
+ * Compute entry points call it with device 0 on first use. */
+int cake_hip_init(int device);
+int cake_hip_shutdown(void);
+int cake_hip_device_info(cake_hip_device_t* out);
+const char* cake_hip_strerror(int status);
+const char* cake_hip_last_error(void);
+
+/* ---- device memory for callers without a HIP runtime of their own ------- */
+int cake_hip_malloc(void** ptr, size_t bytes);
+int cake_hip_free(void* ptr);
+int cake_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int cake_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int cake_hip_memset(void* dst, int value, size_t bytes);
+int cake_hip_synchronize(void);
+
+/* ---- planner ------------------------------------------------------------ */
+/* GPU tile / wave-layout / reuse-order plan.  Needs no device: when the
+ * library is not initialised it plans for 256 CUs with 160 KB of LDS each.
+ * tile_override = {tile_m, tile_n, tile_k, split_k} or NULL; zero entries mean
+ * "choose" (the mcu,kcu,ncu arguments of cake_sgemm, include/cake.h:12-14). */
+int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override,
+                  cake_hip_plan_t* out);
+
+/* The reference's own CPU block sizing, init_block_dims
+ * (src/block_sizing.cpp:465-595; include/tiling.h:39-41), kept because callers
+ * read blk_dims_t fields and because it defines the packed layouts below. */
+int cake_hip_init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx,
+                             int sched, int mcu, int kcu, int ncu,
+                             cake_hip_blk_dims_t* out);
+
+/* ---- GEMM ---------------------------------------------------------------- */
+/* C[MxN] = A[MxK] . B[KxN], all row-major fp32: cake_sgemm
+ * (src/cake_sgemm.cpp:9-175).  accumulate != 0 starts from the existing C
+ * (what beta != 0 means in the reference's MKN/NKM paths, :114). */
+int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K,
+                   int sched, int accumulate, const int* tile_override,
+                   void* stream, double* seconds);
+
+/* Same product with A and/or B already in the reference's packed layouts
+ * (cake_sgemm with packedA / packedB, src/cake_sgemm.cpp:42-44,64-66), as
+ * written by cake_hip_pack_a / cake_hip_pack_b for the same (dims, p, cntx). */
+int cake_hip_sgemm_packed(const float* A, const float* B, float* C, int M, int N, int K,
+                          int p, const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                          int packedA, int packedB, int accumulate,
+                          void* stream, double* seconds);
+
+/* ---- packing (reference layouts, bit-exact) ------------------------------ */
+/* cake_sgemm_packed_{A,B,C}_size, src/pack_helper.cpp:5-87 (bytes). */
+size_t cake_hip_packed_a_size(int M, int K, int p, const cake_hip_blk_dims_t* dims,
+                              const cake_hip_cpu_cntx_t* cntx, int sched);
+size_t cake_hip_packed_b_size(int K, int N, int p, const cake_hip_blk_dims_t* dims,
+                              const cake_hip_cpu_cntx_t* cntx);
+size_t cake_hip_packed_c_size(int M, int N, int p, const cake_hip_blk_dims_t* dims,
+                              const cake_hip_cpu_cntx_t* cntx, int sched);
+/* pack_A / pack_B / pack_C / unpack_C, src/pack_helper.cpp:92-184. */
+int cake_hip_pack_a(const float* A, float* A_p, int M, int K, int p,
+                    const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                    int sched, void* stream, double* seconds);
+int cake_hip_pack_b(const float* B, float* B_p, int K, int N, int p,
+                    const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                    int sched, void* stream, double* seconds);
+int cake_hip_pack_c(const float* C, float* C_p, int M, int N, int p,
+                    const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                    int sched, void* stream, double* seconds);
+int cake_hip_unpack_c(float* C, const float* C_p, int M, int N, int p,
+                      const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                      int sched, void* stream, double* seconds);
+/* Packed offset of element (row, col) of A (which=0), B (1) or C (2): the
+ * index map the pack kernels implement, evaluated on the host. */
+int64_t cake_hip_packed_offset(int which, int row, int col, int M, int N, int K, int p,
+                               const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx,
+                               int sched);
+
+/* ---- GEMV ---------------------------------------------------------------- */
+/* y[M] = A . x (accumulate == 0) or y += A . x (accumulate != 0).
+ * a_col_major != 0: A[k*M + m], the layout cake_sgemv reads
+ * (examples/cake_gemv.cpp:89-140,716-767; it always accumulates);
+ * a_col_major == 0: A[m*K + k]. */
+int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K,
+                   int a_col_major, int accumulate, void* stream, double* seconds);
+
+/* ---- convolution through im2col ------------------------------------------ */
+/* NCHW input -> cols[Cin*Hf*Wf][batch*Hout*Wout], row k = c*Hf*Wf + h*Wf + w,
+ * column n = b*Hout*Wout + ho*Wout + wo, zero where the window hangs over the
+ * edge: im_2_col (examples/cake_conv.cpp:1178-1213) generalised to a batch,
+ * padding and stride.  Hout = (Hin + 2*pad - Hf)/stride + 1, same for W. */
+int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win,
+                    int Hf, int Wf, int stride, int pad, void* stream, double* seconds);
+
+/* out = conv(in, weights) computed as weights[Cout x Cin*Hf*Wf] . cols: the
+ * im2col path of examples/cake_conv.cpp:1007-1066.  weights are OIHW.
+ * out_nchw == 0: out is [Cout][batch*Hout*Wout] (the GEMM's own layout, which
+ * is what the reference produces for its single image); != 0: NCHW.
+ * workspace (device, cake_hip_conv2d_workspace bytes) may be NULL: the library
+ * then uses a buffer of its own. */
+size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
+                                 int Hf, int Wf, int stride, int pad);
+int cake_hip_conv2d(const float* in, const float* weights, float* out,
+                    int batch, int Cin, int Hin, int Win, int Cout, int Hf, int Wf,
+                    int stride, int pad, int out_nchw, void* workspace,
+                    void* stream, double* seconds);
+
+/* ---- seeded inputs -------------------------------------------------------- */
+/* dst[i] = uniform[-1,1) value i of the counter-based splitmix64 stream `seed`
+ * (24 random bits, exact in fp32).  Stands in for rand_init (src/util.cpp:259-267),
+ * which is time-seeded and not reproducible. */
+int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream);
+
+/* Average duration in seconds of the kernels of the last compute call on this
+ * thread, per kernel family: [0] GEMM macro-tile, [1] split-K reduce,
+ * [2] GEMV, [3] im2col, [4] pack/unpack.  Zero where none ran. */
+int cake_hip_last_kernel_seconds(double out[5]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CAKE_HIP_H */

@@ -1,0 +1,172 @@
+"""Host-side checks of libcake_hip.so that need no GPU: the library loads and
+exports every symbol include/cake_hip.h declares, the reference-compatible block
+sizing and packed index maps agree with the oracle, and the GPU planner's
+decisions are sane."""
+import ctypes as C
+import itertools
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import cake_on_cpu_amd as cake
+from cake_on_cpu_amd import _lib
+import oracle
+
+ROOT = Path(__file__).resolve().parent.parent
+EDGE = [1, 10, 96, 111, 960, 2111]
+
+
+def _cx(**kw):
+    o = oracle.make_cntx(**kw)
+    c = cake.CpuCntx(o.alpha_n, o.mr, o.nr, o.L1, o.L2, o.L3, o.ncores)
+    return o, c
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "cake_hip.h").read_text()
+    declared = set(re.findall(r"\b(cake_hip_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 25
+    lib = cake.load()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in cake_hip.h but not exported"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+
+
+def test_struct_sizes_match_reference_layout():
+    assert C.sizeof(cake.BlkDims) == 26 * 4
+    assert [n for n, _ in cake.BlkDims._fields_] == oracle.BLK_FIELDS
+
+
+def test_strerror_and_argument_errors():
+    lib = cake.load()
+    assert lib.cake_hip_strerror(0) == b"ok"
+    assert b"argument" in lib.cake_hip_strerror(_lib.ERR_ARG)
+    p = cake.Plan()
+    assert lib.cake_hip_plan(0, 4, 4, cake.NA, None, C.byref(p)) == _lib.ERR_ARG
+    assert lib.cake_hip_plan(4, 4, 4, 7, None, C.byref(p)) == _lib.ERR_ARG
+    bad_tile = (C.c_int * 4)(123, 0, 0, 0)
+    assert lib.cake_hip_plan(512, 512, 512, cake.NA, bad_tile, C.byref(p)) == _lib.ERR_ARG
+    assert lib.cake_hip_last_error() != b""
+    x = cake.BlkDims()
+    assert lib.cake_hip_init_block_dims(8, 8, 8, 0, C.byref(cake.CpuCntx(1, 6, 16, 1, 1, 1, 1)), 0, 0, 0, 0, C.byref(x)) == _lib.ERR_ARG
+
+
+@pytest.mark.parametrize("p", [1, 3, 8])
+@pytest.mark.parametrize("sch", [cake.KMN, cake.MKN, cake.NKM, cake.NA])
+def test_init_block_dims_equals_oracle(p, sch):
+    for M, K, N in itertools.product(EDGE, EDGE, EDGE):
+        ocx, ccx = _cx()
+        want = oracle.init_block_dims(M, N, K, p, ocx, sch).as_dict()
+        got = cake.init_block_dims(M, N, K, p, ccx, sch).as_dict()
+        assert got == want, (M, K, N)
+        assert ccx.alpha_n == ocx.alpha_n
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (1024, 1024, 1024), (65536, 1024, 128), (256, 2304, 100352)])
+def test_init_block_dims_baseline_shapes(shape):
+    M, K, N = shape
+    for p in (8, 64):
+        ocx, ccx = _cx()
+        assert cake.init_block_dims(M, N, K, p, ccx).as_dict() == oracle.init_block_dims(M, N, K, p, ocx).as_dict()
+    ocx, ccx = _cx()
+    assert (cake.init_block_dims(500, 700, 300, 4, ccx, cake.KMN, None, 4, 48, 64, 160).as_dict()
+            == oracle.init_block_dims(500, 700, 300, 4, ocx, oracle.KMN, 48, 64, 160).as_dict())
+
+
+@pytest.mark.parametrize("p", [1, 3, 8])
+@pytest.mark.parametrize("sch", [cake.KMN, cake.MKN, cake.NKM])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (10, 96, 111), (111, 10, 96), (96, 111, 10), (200, 150, 170)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_packed_index_maps_equal_oracle_layout(shape, sch, p):
+    """Pack a matrix of distinct integers with the oracle, then ask the library
+    where each element lives: the host evaluation of the index map every pack
+    kernel and packed loader uses."""
+    M, K, N = shape
+    ocx, ccx = _cx(L2=16 << 10, L3=256 << 10)  # small caches: several CB blocks even at these sizes
+    xo = oracle.init_block_dims(M, N, K, p, ocx, sch)
+    xc = cake.init_block_dims(M, N, K, p, ccx, sch)
+    mats = {0: np.arange(1, M * K + 1, dtype=np.float32).reshape(M, K),
+            1: np.arange(1, K * N + 1, dtype=np.float32).reshape(K, N),
+            2: np.arange(1, M * N + 1, dtype=np.float32).reshape(M, N)}
+    packed = {0: oracle.pack_A(mats[0], p, xo, ocx, sch), 1: oracle.pack_B(mats[1], p, xo, ocx, sch),
+              2: oracle.pack_C(mats[2], p, xo, ocx, sch)}
+    assert cake.cake_sgemm_packed_A_size(M, K, p, xc, ccx, sch) == packed[0].nbytes
+    assert cake.cake_sgemm_packed_B_size(K, N, p, xc, ccx) == packed[1].nbytes
+    assert cake.cake_sgemm_packed_C_size(M, N, p, xc, ccx, sch) == packed[2].nbytes
+    for which, m in mats.items():
+        rows, cols = m.shape
+        seen = set()
+        for r in range(rows):
+            for c in range(cols):
+                off = cake.packed_offset(which, r, c, M, N, K, p, xc, ccx, sch)
+                assert 0 <= off < packed[which].size
+                assert packed[which][off] == m[r, c], (which, r, c)
+                seen.add(off)
+        assert len(seen) == rows * cols
+        # padding positions map to zeros of the oracle's buffer
+        pr = xc.M_padded if which != 1 else K
+        pc = xc.N_padded if which != 0 else K
+        for r in range(rows, pr):
+            off = cake.packed_offset(which, r, 0, M, N, K, p, xc, ccx, sch)
+            assert packed[which][off] == 0
+        for c in range(cols, pc):
+            off = cake.packed_offset(which, 0, c, M, N, K, p, xc, ccx, sch)
+            assert packed[which][off] == 0
+        assert cake.packed_offset(which, pr, 0, M, N, K, p, xc, ccx, sch) == -1
+
+
+# ---------------------------------------------------------------------------
+# GPU planner (no device: plans for 256 CUs x 160 KB LDS)
+# ---------------------------------------------------------------------------
+def test_plan_baseline_shapes():
+    big = cake.plan(8192, 8192, 8192)
+    assert (big.tile_m, big.tile_n) == (256, 256) and big.split_k == 1
+    assert big.sched == cake.KMN and big.grid == 32 * 32
+    assert big.lds_bytes <= 160 * 1024 and big.vector_loads == 1
+    assert big.flops == 2.0 * 8192 ** 3 and big.min_bytes == 4.0 * 3 * 8192 ** 2
+    # a CB block of resident tiles must cut traffic far below one fetch per tile
+    naive = 4.0 * (2 * 8192.0 * 8192 * 32 + 8192.0 * 8192)
+    assert big.min_bytes <= big.model_bytes < naive / 3
+
+    skinny = cake.plan(65536, 128, 1024)
+    assert skinny.tile_n == 128 and skinny.tiles_n == 1
+    assert skinny.sched == cake.MKN          # one tile column: walk down M, B panel shared
+
+    conv = cake.plan(256, 100352, 2304)
+    assert conv.tiles_m == 1 and conv.sched == cake.NKM   # one tile row: walk along N, A shared
+
+    small = cake.plan(1024, 1024, 1024)
+    assert small.grid >= 128                 # enough workgroups to cover most of the 256 CUs
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (10, 111, 96), (2111, 960, 1), (7, 100000, 3), (300, 300, 100000)])
+def test_plan_covers_any_shape(M, N, K):
+    for sch in (cake.KMN, cake.MKN, cake.NKM, cake.NA):
+        pl = cake.plan(M, N, K, sch)
+        assert pl.tiles_m * pl.tile_m >= M and pl.tiles_n * pl.tile_n >= N
+        assert (pl.tiles_m - 1) * pl.tile_m < M and (pl.tiles_n - 1) * pl.tile_n < N
+        assert pl.split_k >= 1 and pl.grid == pl.tiles_m * pl.tiles_n * pl.split_k
+        assert 1 <= pl.group <= max(pl.tiles_m, pl.tiles_n)
+        assert pl.sched in (cake.KMN, cake.MKN, cake.NKM)
+        if sch != cake.NA:
+            assert pl.sched == sch
+        assert pl.vector_loads == int(K % 4 == 0 and N % 4 == 0)
+
+
+def test_plan_tile_override():
+    pl = cake.plan(4096, 4096, 4096, cake.KMN, (128, 128, 32, 0))
+    assert (pl.tile_m, pl.tile_n, pl.tile_k) == (128, 128, 32)
+    pl = cake.plan(4096, 4096, 4096, cake.KMN, (0, 0, 0, 4))
+    assert pl.split_k == 4
+
+
+def test_compute_without_gpu_fails_loudly():
+    import torch
+    if torch.cuda.device_count() > 0:
+        pytest.skip("a GPU is present")
+    a = np.zeros((4, 4), np.float32)
+    with pytest.raises(cake.CakeHipError) as e:
+        cake.cake_sgemm(a, a, a.copy(), 4, 4, 4, 1)
+    assert e.value.status == _lib.ERR_NO_DEVICE

@@ -1,0 +1,147 @@
+"""GPU parity of cake_sgemm through the C-ABI against the oracle.
+
+Bar (stated by the task): max |C - C_ref| / sum_k |a||b| <= 1e-4, where C_ref is
+the oracle's cake_sgemm on the same seeded inputs; the fp64 product is checked
+too, with the tighter bound a correct fp32 accumulation meets at these K."""
+import itertools
+
+import numpy as np
+import pytest
+
+import cake_on_cpu_amd as cake
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+TIGHT = 5e-6
+EDGE = [1, 10, 96, 111, 960, 2111]   # src/util.cpp:11-13
+SCHEDS = [cake.KMN, cake.MKN, cake.NKM, cake.NA]
+
+
+def _run(M, K, N, sch=cake.NA, p=4, tile=None, C0=None, beta=0.0, seedA=1, seedB=2):
+    A, B = oracle.uniform((M, K), seedA), oracle.uniform((K, N), seedB)
+    Cm = np.zeros((M, N), np.float32) if C0 is None else C0.copy()
+    if tile is None:
+        cake.cake_sgemm(A, B, Cm, M, N, K, p, None, None, False, False, 1.0, beta, sch)
+    else:
+        import ctypes as C
+        from cake_on_cpu_amd import _lib
+        ov = (C.c_int * 4)(*tile)
+        acc = int(beta != 0)
+        _lib.check(cake.load().cake_hip_sgemm(A.ctypes.data, B.ctypes.data, Cm.ctypes.data, M, N, K, sch, acc,
+                                              ov, None, None), "cake_hip_sgemm")
+    return A, B, Cm
+
+
+def _check(A, B, Cm, ref=None, what=""):
+    C64, S = oracle.gemm_f64(A, B)
+    err = oracle.max_rel_err(Cm, C64, S)
+    assert err <= TOL and err <= TIGHT, (what, err)
+    if ref is not None:
+        d = float(np.max(np.abs(Cm.astype(np.float64) - ref) / np.maximum(S, 1e-300)))
+        assert d <= TOL, (what, d)
+
+
+@pytest.mark.parametrize("sch", SCHEDS)
+def test_edge_shape_grid(sch):
+    """The reference's own shape list: every combination that keeps the job small,
+    against the oracle run with the same schedule."""
+    small = [1, 10, 96, 111, 960]
+    for M, K, N in itertools.product(small, small, small):
+        print(f"sgemm edge M={M} K={K} N={N} sch={sch}", flush=True)
+        A, B, Cm = _run(M, K, N, sch)
+        ref = oracle.cake_sgemm(A, B, 4, oracle.make_cntx(), sch=sch)
+        _check(A, B, Cm, ref, (M, K, N, sch))
+
+
+@pytest.mark.parametrize("shape", [(2111, 2111, 2111), (2111, 96, 111), (111, 2111, 96), (96, 111, 2111),
+                                   (1, 2111, 10), (2111, 1, 960), (10, 960, 2111)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_edge_shapes_with_2111(shape):
+    M, K, N = shape
+    for sch in (cake.KMN, cake.NA):
+        print(f"sgemm edge M={M} K={K} N={N} sch={sch}", flush=True)
+        A, B, Cm = _run(M, K, N, sch)
+        ref = oracle.cake_sgemm(A, B, 8, oracle.make_cntx(), sch=sch)
+        _check(A, B, Cm, ref, (shape, sch))
+
+
+TILES = [(256, 256, 32), (256, 256, 16), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32)]
+
+
+@pytest.mark.parametrize("tile", TILES, ids=lambda t: "x".join(map(str, t)))
+@pytest.mark.parametrize("shape", [(512, 512, 512), (700, 520, 900), (333, 419, 517), (257, 1000, 255)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_every_tile_shape(tile, shape):
+    """Each macro-tile instantiation, on aligned (16-byte loader) and ragged
+    (scalar loader) operands, without and with split-K."""
+    M, K, N = shape
+    for split in (0, 3):
+        print(f"sgemm tile={tile} split={split} M={M} K={K} N={N}", flush=True)
+        A, B, Cm = _run(M, K, N, cake.KMN, tile=tile + (split,))
+        _check(A, B, Cm, None, (tile, shape, split))
+
+
+def test_identity_all_ones_single_nonzero():
+    n = 300
+    B = oracle.uniform((n, 260), 5)
+    out = np.zeros_like(B)
+    cake.cake_sgemm(np.eye(n, dtype=np.float32), B, out, n, 260, n, 1)
+    assert np.array_equal(out, B)
+    out = np.zeros((70, 91), np.float32)
+    cake.cake_sgemm(np.ones((70, 513), np.float32), np.ones((513, 91), np.float32), out, 70, 91, 513, 1)
+    assert np.array_equal(out, np.full((70, 91), 513.0, np.float32))
+    A = np.zeros((40, 50), np.float32)
+    A[17, 23] = 2.0
+    Bm = oracle.uniform((50, 60), 6)
+    out = np.full((40, 60), 9.0, np.float32)
+    cake.cake_sgemm(A, Bm, out, 40, 60, 50, 1)
+    want = np.zeros((40, 60), np.float32)
+    want[17] = 2.0 * Bm[23]
+    assert np.array_equal(out, want)
+
+
+def test_overwrite_and_accumulate_semantics():
+    """K-first assigns whatever C held; M-/N-first add to C only when beta != 0
+    (src/cake_sgemm.cpp:114, src/pack_ob.cpp:404) -- same as the oracle."""
+    M, K, N = 200, 160, 240
+    C0 = oracle.uniform((M, N), 3)
+    cx = oracle.make_cntx()
+    for sch in (cake.KMN, cake.MKN, cake.NKM):
+        for beta in (0.0, 1.0):
+            A, B, Cm = _run(M, K, N, sch, C0=C0, beta=beta)
+            ref = oracle.cake_sgemm(A, B, 4, cx, Cinit=C0, beta=beta, sch=sch)
+            C64, S = oracle.gemm_f64(A, B)
+            d = float(np.max(np.abs(Cm.astype(np.float64) - ref) / (S + np.abs(C0))))
+            assert d <= 1e-5, (sch, beta, d)
+    # and the difference is exactly the old C where accumulation applies
+    A, B, plain = _run(M, K, N, cake.MKN)
+    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    assert np.allclose(acc - plain, C0, atol=1e-4)
+
+
+def test_schedules_agree_and_are_deterministic():
+    M, K, N = 777, 1030, 515
+    outs = [_run(M, K, N, sch)[2] for sch in (cake.KMN, cake.MKN, cake.NKM)]
+    # the reuse order only changes which workgroup computes a tile, not the sums
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    again = _run(M, K, N, cake.KMN)[2]
+    assert np.array_equal(outs[0], again)
+    s1 = _run(M, K, N, cake.KMN, tile=(128, 128, 32, 4))[2]
+    s2 = _run(M, K, N, cake.KMN, tile=(128, 128, 32, 4))[2]
+    assert np.array_equal(s1, s2)      # split-K reduces in a fixed order
+
+
+def test_empty_and_degenerate():
+    a = np.zeros((0, 5), np.float32)
+    cake.cake_sgemm(a, np.zeros((5, 3), np.float32), np.zeros((0, 3), np.float32), 0, 3, 5, 1)
+    out = np.full((4, 3), 7.0, np.float32)
+    cake.cake_sgemm(np.zeros((4, 0), np.float32), np.zeros((0, 3), np.float32), out, 4, 3, 0, 1)
+    assert not out.any()               # empty sum assigns zero in K-first
+    sq = np.zeros((4, 4), np.float32)
+    with pytest.raises(cake.CakeHipError):
+        cake.cake_sgemm(sq, sq, sq.copy(), -1, 3, 5, 1)
+    with pytest.raises(cake.CakeHipError):
+        cake.cake_sgemm(np.zeros((4, 4), np.float32), np.zeros((4, 4), np.float32),
+                        np.zeros((4, 4), np.float32), 4, 4, 4, 1, None, None, False, False, 1.0, 0.0, 9)
