@@ -406,6 +406,12 @@ int cake_hip_init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cn
     return CAKE_HIP_OK;
 }
 
+int cake_hip_derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_cpu_cntx_t* cntx)
+{
+    if (!cntx || p <= 0 || mc <= 0) return CAKE_HIP_KMN;
+    return derive_schedule(M, N, K, p, mc, cntx);
+}
+
 int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K, int sched,
                    int accumulate, const int* tile_override, void* stream_, double* seconds)
 {

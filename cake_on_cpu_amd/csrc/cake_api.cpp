@@ -1,0 +1,370 @@
+// cake_api.cpp -- libcake.so: the reference's C++ entry points for the fp32 GEMM
+// path, forwarding to the C-ABI of libcake_hip.so.
+//
+// Error behaviour follows the reference (src/cake_sgemm.cpp:49-52,
+// src/block_sizing.cpp:400-403): a failure prints a message and exit(1)s; there
+// are no return codes at this level.  Return values are wall-clock seconds of
+// the call, as in src/cake_sgemm.cpp:164-174.
+#include "cake.h"
+
+#include <math.h>
+#include <time.h>
+
+#include "cake_hip.h"
+
+namespace {
+
+double wall_seconds()
+{
+    struct timespec t;
+    clock_gettime(CLOCK_REALTIME, &t);
+    return (double)t.tv_sec + 1e-9 * (double)t.tv_nsec;
+}
+
+void die_on(int status, const char* where)
+{
+    if (status == CAKE_HIP_OK) return;
+    const char* detail = cake_hip_last_error();
+    printf("%s: %s (%s)\n", where, cake_hip_strerror(status), detail ? detail : "");
+    exit(1);
+}
+
+// blk_dims_t and cake_hip_blk_dims_t have the same 26 four-byte fields in the
+// same order; the enum is an int.
+static_assert(sizeof(blk_dims_t) == sizeof(cake_hip_blk_dims_t), "blk_dims_t layout");
+
+cake_hip_blk_dims_t to_abi(const blk_dims_t* x)
+{
+    cake_hip_blk_dims_t d;
+    memcpy(&d, x, sizeof d);
+    return d;
+}
+
+cake_hip_cpu_cntx_t to_abi(const cake_cntx_t* c)
+{
+    cake_hip_cpu_cntx_t r;
+    r.alpha_n = c->alpha_n;
+    r.mr = c->mr; r.nr = c->nr;
+    r.L1 = c->L1; r.L2 = c->L2; r.L3 = c->L3;
+    r.ncores = c->ncores;
+    return r;
+}
+
+long popen_number(const char* cmd)
+{
+    char buf[64] = {0};
+    FILE* fp = popen(cmd, "r");
+    if (!fp) return -1;
+    char* got = fgets(buf, sizeof buf, fp);
+    pclose(fp);
+    return got ? atol(buf) : -1;
+}
+
+// macro-tile override from the caller's mcu,kcu,ncu when such a tile exists
+const int* tile_from_user(int M, int N, int K, int sch, int mcu, int kcu, int ncu, int out[4])
+{
+    if (!(mcu && kcu && ncu)) return NULL;
+    out[0] = mcu; out[1] = ncu; out[2] = kcu; out[3] = 0;
+    cake_hip_plan_t probe;
+    return cake_hip_plan(M, N, K, sch, out, &probe) == CAKE_HIP_OK ? out : NULL;
+}
+
+double sgemm_common(float* A, float* B, float* C, int M, int N, int K, int p, cake_cntx_t* cntx,
+                    char* argv[], bool packedA, bool packedB, float beta, enum sched sch, int mcu,
+                    int kcu, int ncu)
+{
+    (void)argv;
+    if (cntx == NULL) cntx = cake_query_cntx();  // leaked, as in the reference (:14-16)
+    const double t0 = wall_seconds();
+    if (packedA || packedB) {
+        blk_dims_t x;
+        init_block_dims(M, N, K, p, &x, cntx, sch, argv, 4, mcu, kcu, ncu);
+        cake_hip_blk_dims_t d = to_abi(&x);
+        cake_hip_cpu_cntx_t cx = to_abi(cntx);
+        const int accumulate = (x.sch != KMN) && (beta != 0);
+        double dev_s = 0;
+        die_on(cake_hip_sgemm_packed(A, B, C, M, N, K, p, &d, &cx, packedA, packedB, accumulate, NULL, &dev_s),
+               "cake_sgemm");
+    } else {
+        int resolved = sch;
+        if (sch == NA && M > 0 && N > 0 && K > 0) {
+            cake_hip_plan_t plan;
+            die_on(cake_hip_plan(M, N, K, NA, NULL, &plan), "cake_sgemm");
+            resolved = plan.sched;
+        }
+        const int accumulate = (resolved != KMN) && (beta != 0);
+        int ov[4];
+        double dev_s = 0;
+        die_on(cake_hip_sgemm(A, B, C, M, N, K, sch, accumulate, tile_from_user(M, N, K, sch, mcu, kcu, ncu, ov),
+                              NULL, &dev_s),
+               "cake_sgemm");
+    }
+    return wall_seconds() - t0;
+}
+
+}  // namespace
+
+// ---- machine description ----------------------------------------------------
+
+int get_num_physical_cores()
+{
+    long logical = popen_number("grep -c ^processor /proc/cpuinfo");
+    long tpc = popen_number("lscpu | grep Thread -m 1 | tr -dc '0-9'");
+    long sockets = popen_number("lscpu | grep Socket -m 1 | tr -dc '0-9'");
+    if (logical <= 0) logical = 1;
+    if (tpc <= 0) tpc = 1;
+    if (sockets <= 0) sockets = 1;
+    long c = logical / (tpc * sockets);
+    return c > 0 ? (int)c : 1;
+}
+
+int get_cache_size(int level)
+{
+    char cmd[256], buf[64] = {0};
+    snprintf(cmd, sizeof cmd,
+             "lscpu --caches=NAME,%s | grep L%d | grep -Eo '[0-9]*M|[0-9]*K|[0-9]*G' | tr -d '\\n'",
+             level < 3 ? "ONE-SIZE" : "ALL-SIZE", level);
+    FILE* fp = popen(cmd, "r");
+    if (!fp) return 0;
+    char* got = fgets(buf, sizeof buf, fp);
+    pclose(fp);
+    size_t len = got ? strlen(buf) : 0;
+    if (len < 2) return level == 1 ? 32 << 10 : level == 2 ? 1 << 20 : 32 << 20;
+    int shift = buf[len - 1] == 'K' ? 10 : buf[len - 1] == 'M' ? 20 : 30;
+    buf[len - 1] = 0;
+    return atoi(buf) << shift;
+}
+
+cake_cntx_t* cake_query_cntx_torch(int L2, int L3)
+{
+    cake_cntx_t* c = (cake_cntx_t*)calloc(1, sizeof(cake_cntx_t));
+    c->alpha_n = 1.0;
+    c->mr = 6;
+    c->nr = 16;
+    c->L2 = L2;
+    c->L3 = L3;
+    c->ncores = get_num_physical_cores();
+    c->peak_dram_bw = 8.0e12;
+    c->peak_flops = 157.3e12;
+    return c;
+}
+
+cake_cntx_t* cake_query_cntx()
+{
+    cake_cntx_t* c = cake_query_cntx_torch(get_cache_size(2), get_cache_size(3));
+    c->L1 = get_cache_size(1);
+    return c;
+}
+
+void update_mr_nr(cake_cntx_t* cake_cntx, int m_r, int n_r)
+{
+    cake_cntx->mr = m_r;
+    cake_cntx->nr = n_r;
+    cake_cntx->m_map = 0;
+    cake_cntx->n_map = 0;
+}
+
+// ---- block sizing -------------------------------------------------------------
+
+void init_block_dims(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx,
+                     enum sched sch, char* argv[], float type_size, int mcu, int kcu, int ncu)
+{
+    (void)argv; (void)type_size;
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    cake_hip_blk_dims_t d;
+    int st = cake_hip_init_block_dims(M, N, K, p, &cx, sch, mcu, kcu, ncu, &d);
+    if (st != CAKE_HIP_OK) {
+        printf("unknown schedule\n");
+        exit(1);
+    }
+    memcpy(x, &d, sizeof d);
+    cake_cntx->alpha_n = cx.alpha_n;
+}
+
+cache_dims_t* get_cache_dims(int M, int N, int K, int p, cake_cntx_t* cake_cntx, enum sched sch,
+                             char* argv[], float type_size, int mcu, int kcu, int ncu)
+{
+    blk_dims_t x;
+    init_block_dims(M, N, K, p, &x, cake_cntx, sch, argv, type_size, mcu, kcu, ncu);
+    cache_dims_t* r = (cache_dims_t*)malloc(sizeof(cache_dims_t));
+    r->m_c = x.m_c; r->k_c = x.k_c; r->n_c = x.n_c; r->sch = x.sch;
+    return r;
+}
+
+enum sched derive_schedule(int M, int N, int K, int p, int mc_ret, cake_cntx_t* cake_cntx)
+{
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    return (enum sched)cake_hip_derive_schedule(M, N, K, p, mc_ret, &cx);
+}
+
+// ---- GEMM -----------------------------------------------------------------------
+
+double cake_sgemm(float* A, float* B, float* C, int M, int N, int K, int p, cake_cntx_t* cake_cntx,
+                  char* argv[], bool packedA, bool packedB, float alpha, float beta, enum sched sch,
+                  int mcu, int kcu, int ncu)
+{
+    (void)alpha;  // never read by the reference either
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
+}
+
+double cake_sgemm_online(float* A, float* B, float* C, int M, int N, int K, int p,
+                         cake_cntx_t* cake_cntx, char* argv[], bool packedA, bool packedB, float alpha,
+                         float beta, enum sched sch, int mcu, int kcu, int ncu)
+{
+    (void)alpha;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
+}
+
+double cake_sgemm_2d(float* A, float* B, float* C, int M, int N, int K, int p, cake_cntx_t* cake_cntx,
+                     char* argv[], bool packedA, bool packedB, float alpha, float beta, enum sched sch,
+                     int mcu, int kcu, int ncu)
+{
+    (void)alpha;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
+}
+
+double cake_sgemm_2d_small(float* A, float* B, float* C, int M, int N, int K, int p,
+                           cake_cntx_t* cake_cntx, char* argv[], bool packedA, bool packedB,
+                           float alpha, float beta, enum sched sch)
+{
+    (void)alpha;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, 0, 0, 0);
+}
+
+// ---- packing ----------------------------------------------------------------------
+
+size_t cake_sgemm_packed_A_size(int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    return cake_hip_packed_a_size(M, K, p, &d, &cx, sch);
+}
+
+size_t cake_sgemm_packed_B_size(int K, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    return cake_hip_packed_b_size(K, N, p, &d, &cx);
+}
+
+size_t cake_sgemm_packed_C_size(int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    return cake_hip_packed_c_size(M, N, p, &d, &cx, sch);
+}
+
+double pack_A(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    const double t0 = wall_seconds();
+    die_on(cake_hip_pack_a(A, A_p, M, K, p, &d, &cx, sch, NULL, NULL), "pack_A");
+    die_on(cake_hip_synchronize(), "pack_A");
+    return wall_seconds() - t0;
+}
+
+void pack_B(float* B, float* B_p, int K, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    die_on(cake_hip_pack_b(B, B_p, K, N, p, &d, &cx, sch, NULL, NULL), "pack_B");
+}
+
+void pack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    die_on(cake_hip_pack_c(C, C_p, M, N, p, &d, &cx, sch, NULL, NULL), "pack_C");
+}
+
+void unpack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    die_on(cake_hip_unpack_c(C, C_p, M, N, p, &d, &cx, sch, NULL, NULL), "unpack_C");
+}
+
+// ---- GEMV -------------------------------------------------------------------------
+
+double cake_sgemv(float* A, float* B, float* C, int M, int K, int p, cake_cntx_t* cake_cntx,
+                  char* argv[], bool packedA, float alpha, float beta, enum sched sch)
+{
+    (void)p; (void)cake_cntx; (void)argv; (void)packedA; (void)alpha; (void)beta; (void)sch;
+    const double t0 = wall_seconds();
+    double dev_s = 0;
+    // column-major A, accumulate into y: examples/cake_gemv.cpp:89-140
+    die_on(cake_hip_sgemv(A, B, C, M, K, 1, 1, NULL, &dev_s), "cake_sgemv");
+    return wall_seconds() - t0;
+}
+
+// ---- im2col -----------------------------------------------------------------------
+
+float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s)
+{
+    (void)Cout; (void)s;  // neither is used by the reference's im_2_col
+    if (Hout != Hin - Hf + 1 || Wout != Win - Wf + 1) {
+        printf("im_2_col: Hout/Wout must be Hin-Hf+1 / Win-Wf+1\n");
+        exit(1);
+    }
+    float* cols = (float*)malloc(sizeof(float) * (size_t)Cin * Hf * Wf * Hout * Wout);
+    if (!cols) {
+        printf("im_2_col: out of memory\n");
+        exit(1);
+    }
+    die_on(cake_hip_im2col(In, cols, 1, Cin, Hin, Win, Hf, Wf, 1, 0, NULL, NULL), "im_2_col");
+    return cols;
+}
+
+// ---- test helpers (host code) -------------------------------------------------------
+
+void rand_init(float* mat, int r, int c)
+{
+    for (size_t i = 0; i < (size_t)r * c; ++i) mat[i] = (float)rand() / (float)RAND_MAX * 2.0f - 1.0f;
+}
+
+bool mat_equals(float* C, float* C_check, int M, int N)
+{
+    const float eps = 1e-3f;  // util.cpp:144
+    long bad = 0;
+    for (size_t i = 0; i < (size_t)M * N; ++i)
+        if (fabsf(C_check[i] - C[i]) > eps) ++bad;
+    if (!bad) {
+        printf("CORRECT!\n");
+        return 0;
+    }
+    printf("WRONG!\n%ld\n", bad);
+    return 1;
+}
+
+bool cake_sgemm_checker(float* A, float* B, float* C, int N, int M, int K)
+{
+    float* ref = (float*)calloc((size_t)M * N, sizeof(float));
+    for (int m = 0; m < M; ++m)
+        for (int k = 0; k < K; ++k) {
+            const float a = A[(size_t)m * K + k];
+            const float* b = B + (size_t)k * N;
+            float* r = ref + (size_t)m * N;
+            for (int n = 0; n < N; ++n) r[n] += a * b[n];
+        }
+    bool ret = mat_equals(C, ref, M, N);
+    free(ref);
+    return ret;
+}
+
+void print_schedule(enum sched sch)
+{
+    static const char* names[] = {"KMN", "MKN", "NKM", "NA"};
+    printf("%s Cake Schedule\n", names[(int)sch & 3]);
+}
+
+void print_array(float* arr, int len)
+{
+    for (int i = 0; i < len; ++i) printf("%f ", arr[i]);
+    printf("\n");
+}
+
+void print_mat(float* arr, int r, int c)
+{
+    for (int i = 0; i < r; ++i) print_array(arr + (size_t)i * c, c);
+}

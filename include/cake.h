@@ -1,0 +1,128 @@
+// cake.h -- C++ interface of the fp32 GEMM path of CAKE, served by an MI355X.
+//
+// Source-compatible with the part of vnatesh/CAKE_on_CPU's include/cake.h,
+// include/common.h, include/tiling.h, include/packing.h and include/util.h that
+// the cake_sgemm / cake_sgemv / im2col-convolution path uses: same type names,
+// field order, function names, argument order and default arguments, so a
+// caller written against the reference recompiles against this header and
+// links libcake.so unchanged.  Underneath, every function forwards to the C-ABI
+// of libcake_hip.so (include/cake_hip.h); the product, the packing and im2col
+// all run on the GPU.  Only the test helpers at the end are host code, as an
+// independent checker has to be.
+//
+// Matrices are row-major float.  Pointers may be ordinary host memory (as in
+// the reference) or device memory.
+#pragma once
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+// ---- types (reference: include/common.h:105-159) ---------------------------
+
+enum sched { KMN, MKN, NKM, NA };
+
+typedef struct blk_dims_t {
+    int m_c, k_c, n_c;
+    int m_c1, k_c1, n_c1;
+    int m_c1_last_core, n_c1_last_core, k_c1_last_core;
+    int mr_rem, nr_rem, k_rem;
+    int p_l, pm_l, pn_l, pm, pn;
+    int m_pad, k_pad, n_pad;
+    int Mb, Kb, Nb;
+    int M_padded, N_padded;
+    enum sched sch;
+} blk_dims_t;
+
+typedef struct cake_cntx_t {
+    void* blis_cntx;      // unused here; kept so the layout matches
+    double alpha_n;
+    double peak_dram_bw;  // bytes/s of the device the library runs on
+    double peak_flops;    // fp32 matrix FLOP/s of that device
+    int mr, nr;           // register-tile shape that defines the packed layouts
+    int m_map, n_map;
+    int L1, L2, L3;       // host cache sizes: inputs of the CB-block sizing
+    int ncores;           // host physical cores
+} cake_cntx_t;
+
+typedef struct cache_dims_t {
+    int m_c, k_c, n_c;
+    enum sched sch;
+} cache_dims_t;
+
+#define cake_max(x, y) (((x) >= (y)) ? (x) : (y))
+#define cake_min(x, y) (((x) <= (y)) ? (x) : (y))
+
+// ---- machine description and block sizing (reference: include/tiling.h) -----
+
+cake_cntx_t* cake_query_cntx();                                    // block_sizing.cpp:40
+cake_cntx_t* cake_query_cntx_torch(int L2, int L3);                // block_sizing.cpp:10
+void update_mr_nr(cake_cntx_t* cake_cntx, int m_r, int n_r);        // block_sizing.cpp:78
+int get_cache_size(int level);                                     // block_sizing.cpp:148
+int get_num_physical_cores();                                      // block_sizing.cpp:91
+
+enum sched derive_schedule(int M, int N, int K, int p, int mc_ret, cake_cntx_t* cake_cntx);
+
+cache_dims_t* get_cache_dims(int M, int N, int K, int p, cake_cntx_t* cake_cntx, enum sched sch,
+                             char* argv[], float type_size = 4, int mcu = 0, int kcu = 0, int ncu = 0);
+
+void init_block_dims(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx,
+                     enum sched sch, char* argv[], float type_size = 4,
+                     int mcu = 0, int kcu = 0, int ncu = 0);
+
+// ---- GEMM (reference: include/cake.h:12-14,36-47) ---------------------------
+
+double cake_sgemm(float* A, float* B, float* C, int M, int N, int K, int p,
+                  cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0, bool packedB = 0,
+                  float alpha = 1, float beta = 0, enum sched sch = NA,
+                  int mcu = 0, int kcu = 0, int ncu = 0);
+
+// The pack-on-the-fly and 2-D core-grid entry points of the reference.  On the
+// GPU operands are always staged on the fly and the grid is the device's, so
+// these run the same kernel as cake_sgemm.
+double cake_sgemm_online(float* A, float* B, float* C, int M, int N, int K, int p,
+                         cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0,
+                         bool packedB = 0, float alpha = 1, float beta = 0, enum sched sch = NA,
+                         int mcu = 0, int kcu = 0, int ncu = 0);
+double cake_sgemm_2d(float* A, float* B, float* C, int M, int N, int K, int p,
+                     cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0,
+                     bool packedB = 0, float alpha = 1, float beta = 0, enum sched sch = NA,
+                     int mcu = 0, int kcu = 0, int ncu = 0);
+double cake_sgemm_2d_small(float* A, float* B, float* C, int M, int N, int K, int p,
+                           cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0,
+                           bool packedB = 0, float alpha = 1, float beta = 0, enum sched sch = NA);
+
+// ---- packing (reference: include/packing.h:6-13,70-72) ----------------------
+
+size_t cake_sgemm_packed_A_size(int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+size_t cake_sgemm_packed_B_size(int K, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx);
+size_t cake_sgemm_packed_C_size(int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+
+double pack_A(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+void pack_B(float* B, float* B_p, int K, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+void pack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+void unpack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);
+
+// ---- GEMV (reference: examples/cake_gemv.cpp:7-9) ---------------------------
+// y += A.x with A column-major, A[k*M + m].
+
+double cake_sgemv(float* A, float* B, float* C, int M, int K, int p, cake_cntx_t* cake_cntx,
+                  char* argv[] = NULL, bool packedA = 0, float alpha = 1, float beta = 0,
+                  enum sched sch = NA);
+
+// ---- convolution through im2col (reference: examples/cake_conv.cpp:24-25) ---
+// Returns a malloc'd [Cin*Hf*Wf][Hout*Wout] matrix; the caller frees it.
+
+float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
+                int Cin, int Cout, int s);
+
+// ---- test helpers (reference: include/util.h) -------------------------------
+
+void rand_init(float* mat, int r, int c);                          // util.cpp:259
+bool cake_sgemm_checker(float* A, float* B, float* C, int N, int M, int K);  // util.cpp:173
+bool mat_equals(float* C, float* C_check, int M, int N);           // util.cpp:139
+void print_schedule(enum sched sch);
+void print_mat(float* arr, int r, int c);
+void print_array(float* arr, int len);

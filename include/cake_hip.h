@@ -129,6 +129,10 @@ int cake_hip_init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cn
                              int sched, int mcu, int kcu, int ncu,
                              cake_hip_blk_dims_t* out);
 
+/* derive_schedule (src/block_sizing.cpp:434-462): the reference's IO-optimal
+ * reuse order for a CB block of side p*mc.  Returns KMN, MKN or NKM. */
+int cake_hip_derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_cpu_cntx_t* cntx);
+
 /* ---- GEMM ---------------------------------------------------------------- */
 /* C[MxN] = A[MxK] . B[KxN], all row-major fp32: cake_sgemm
  * (src/cake_sgemm.cpp:9-175).  accumulate != 0 starts from the existing C

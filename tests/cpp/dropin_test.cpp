@@ -1,0 +1,175 @@
+// dropin_test.cpp -- a caller written the way the reference's example mains are
+// (examples/cake_sgemm_test.cpp, examples/cake_gemv.cpp, examples/cake_conv.cpp:
+// query the context, rand_init, call, check against a naive host loop), compiled
+// against include/cake.h and linked to libcake.so only.  Prints one line per
+// case and "ALL PASS" at the end; exit status 0 only if every case passed.
+#include <math.h>
+
+#include "cake.h"
+
+static int failures = 0;
+
+static void report(const char* what, bool ok)
+{
+    printf("%-58s %s\n", what, ok ? "ok" : "FAILED");
+    fflush(stdout);
+    if (!ok) ++failures;
+}
+
+static bool close_to_naive(float* A, float* B, float* C, int M, int N, int K)
+{
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            double acc = 0, mag = 0;
+            for (int k = 0; k < K; ++k) {
+                acc += (double)A[(size_t)m * K + k] * B[(size_t)k * N + n];
+                mag += fabs((double)A[(size_t)m * K + k] * B[(size_t)k * N + n]);
+            }
+            if (fabs(acc - C[(size_t)m * N + n]) > 1e-4 * (mag > 0 ? mag : 1)) return false;
+        }
+    return true;
+}
+
+static void sgemm_case(int M, int K, int N, int p, enum sched sch, cake_cntx_t* cntx)
+{
+    float* A = (float*)malloc(sizeof(float) * M * K);
+    float* B = (float*)malloc(sizeof(float) * K * N);
+    float* C = (float*)calloc((size_t)M * N, sizeof(float));
+    rand_init(A, M, K);
+    rand_init(B, K, N);
+    double t = cake_sgemm(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, sch);
+    char what[128];
+    snprintf(what, sizeof what, "cake_sgemm M=%d K=%d N=%d p=%d sch=%d (%.4f s)", M, K, N, p, (int)sch, t);
+    report(what, close_to_naive(A, B, C, M, N, K));
+    free(A); free(B); free(C);
+}
+
+static void variants_case(cake_cntx_t* cntx)
+{
+    const int M = 111, K = 96, N = 213, p = 3;
+    float* A = (float*)malloc(sizeof(float) * M * K);
+    float* B = (float*)malloc(sizeof(float) * K * N);
+    rand_init(A, M, K);
+    rand_init(B, K, N);
+    float* C = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_sgemm_2d(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, KMN);
+    report("cake_sgemm_2d", close_to_naive(A, B, C, M, N, K));
+    memset(C, 0, sizeof(float) * M * N);
+    cake_sgemm_online(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, KMN);
+    report("cake_sgemm_online", close_to_naive(A, B, C, M, N, K));
+    memset(C, 0, sizeof(float) * M * N);
+    cake_sgemm(A, B, C, M, N, K, p, NULL);  // NULL context, all defaults
+    report("cake_sgemm default arguments, NULL context", !cake_sgemm_checker(A, B, C, N, M, K));
+    free(A); free(B); free(C);
+}
+
+// the packed path of examples/cake_conv.cpp:1007-1066
+static void conv_case(cake_cntx_t* cntx)
+{
+    const int Cin = 8, Cout = 20, Hf = 3, Wf = 3, Hout = 12, Wout = 10, Hin = Hout + 2, Win = Wout + 2, p = 4;
+    const int M = Cout, K = Cin * Hf * Wf, N = Hout * Wout;
+    float* F = (float*)malloc(sizeof(float) * M * K);
+    float* In = (float*)malloc(sizeof(float) * Cin * Hin * Win);
+    rand_init(F, M, K);
+    rand_init(In, Cin, Hin * Win);
+    float* Bm = im_2_col(In, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, 1);
+    bool cols_ok = true;
+    for (int c = 0; c < Cin && cols_ok; ++c)
+        for (int h = 0; h < Hf; ++h)
+            for (int w = 0; w < Wf; ++w)
+                for (int ho = 0; ho < Hout; ++ho)
+                    for (int wo = 0; wo < Wout; ++wo)
+                        if (Bm[(size_t)(c * Hf * Wf + h * Wf + w) * N + ho * Wout + wo] !=
+                            In[(size_t)c * Hin * Win + (ho + h) * Win + wo + w])
+                            cols_ok = false;
+    report("im_2_col layout", cols_ok);
+
+    enum sched sch = KMN;
+    blk_dims_t* x = (blk_dims_t*)malloc(sizeof(blk_dims_t));
+    init_block_dims(M, N, K, p, x, cntx, sch, NULL, 0);
+    float* A_p = (float*)malloc(cake_sgemm_packed_A_size(M, K, p, x, cntx, sch));
+    float* B_p = (float*)malloc(cake_sgemm_packed_B_size(K, N, p, x, cntx));
+    pack_A(F, A_p, M, K, p, x, cntx, sch);
+    pack_B(Bm, B_p, K, N, p, x, cntx, sch);
+    float* C = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_sgemm(A_p, B_p, C, M, N, K, p, cntx, NULL, 1, 1, 1, 0, KMN);
+    report("cake_sgemm(packedA=1, packedB=1) after pack_A/pack_B", close_to_naive(F, Bm, C, M, N, K));
+
+    // direct convolution as the independent answer
+    bool conv_ok = true;
+    for (int co = 0; co < Cout && conv_ok; ++co)
+        for (int ho = 0; ho < Hout; ++ho)
+            for (int wo = 0; wo < Wout; ++wo) {
+                double acc = 0;
+                for (int c = 0; c < Cin; ++c)
+                    for (int h = 0; h < Hf; ++h)
+                        for (int w = 0; w < Wf; ++w)
+                            acc += (double)F[(size_t)co * K + c * Hf * Wf + h * Wf + w] *
+                                   In[(size_t)c * Hin * Win + (ho + h) * Win + wo + w];
+                if (fabs(acc - C[(size_t)co * N + ho * Wout + wo]) > 1e-3) conv_ok = false;
+            }
+    report("im2col GEMM equals direct convolution", conv_ok);
+
+    // pack_C / unpack_C round trip
+    float* C_p = (float*)malloc(cake_sgemm_packed_C_size(M, N, p, x, cntx, sch));
+    float* C2 = (float*)calloc((size_t)M * N, sizeof(float));
+    pack_C(C, C_p, M, N, p, x, cntx, sch);
+    unpack_C(C2, C_p, M, N, p, x, cntx, sch);
+    report("unpack_C(pack_C(C)) == C", memcmp(C, C2, sizeof(float) * M * N) == 0);
+    free(F); free(In); free(Bm); free(x); free(A_p); free(B_p); free(C); free(C_p); free(C2);
+}
+
+// examples/cake_gemv.cpp main: column-major A, mr = 8, y accumulates
+static void gemv_case(cake_cntx_t* cntx, int M, int K)
+{
+    float* A = (float*)malloc(sizeof(float) * M * K);
+    float* x = (float*)malloc(sizeof(float) * K);
+    float* y = (float*)calloc(M, sizeof(float));
+    rand_init(A, M, K);
+    rand_init(x, K, 1);
+    cntx->mr = 8;
+    cake_sgemv(A, x, y, M, K, 4, cntx);
+    cake_sgemv(A, x, y, M, K, 4, cntx);  // second call doubles y
+    bool ok = true;
+    for (int m = 0; m < M && ok; ++m) {
+        double acc = 0, mag = 0;
+        for (int k = 0; k < K; ++k) {
+            acc += (double)A[(size_t)k * M + m] * x[k];
+            mag += fabs((double)A[(size_t)k * M + m] * x[k]);
+        }
+        if (fabs(2 * acc - y[m]) > 2e-4 * (mag > 0 ? mag : 1)) ok = false;
+    }
+    char what[96];
+    snprintf(what, sizeof what, "cake_sgemv M=%d K=%d (column-major, accumulating)", M, K);
+    report(what, ok);
+    cntx->mr = 6;
+    free(A); free(x); free(y);
+}
+
+int main()
+{
+    srand(1);
+    cake_cntx_t* cntx = cake_query_cntx();
+    printf("cntx: mr=%d nr=%d L2=%d L3=%d ncores=%d\n", cntx->mr, cntx->nr, cntx->L2, cntx->L3, cntx->ncores);
+    const int dims[] = {1, 10, 96, 111, 300};  // subset of src/util.cpp:11-13
+    for (int mi = 0; mi < 5; ++mi)
+        for (int ki = 0; ki < 5; ++ki)
+            for (int ni = 0; ni < 5; ++ni) {
+                enum sched sch = (enum sched)((mi + ki + ni) % 4);
+                sgemm_case(dims[mi], dims[ki], dims[ni], 2 + (mi + ni) % 3, sch, cntx);
+            }
+    sgemm_case(960, 2111, 333, 8, NA, cntx);
+    variants_case(cntx);
+    conv_case(cntx);
+    gemv_case(cntx, 1024, 777);
+    gemv_case(cntx, 37, 5);
+
+    blk_dims_t x;
+    init_block_dims(8192, 8192, 8192, 8, &x, cntx, NA, NULL);
+    report("init_block_dims fills blk_dims_t", x.m_c > 0 && x.k_c == x.m_c && x.Mb > 0 && x.M_padded >= 8192);
+    update_mr_nr(cntx, 8, 12);
+    report("update_mr_nr", cntx->mr == 8 && cntx->nr == 12);
+    free(cntx);
+    printf(failures ? "%d FAILED\n" : "ALL PASS\n", failures);
+    return failures ? 1 : 0;
+}

@@ -1,0 +1,223 @@
+"""GPU parity of cake_sgemv, im2col / conv2d, pack/unpack and the seeded fill
+through the C-ABI against the oracle.  Byte/index work (packing, im2col, fill)
+is bit-exact; floating-point results meet max |y - ref| / sum|a||x| <= 1e-4."""
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import cake_on_cpu_amd as cake
+from cake_on_cpu_amd import _lib
+import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+TIGHT = 5e-6
+
+
+# ---------------------------------------------------------------------------
+# seeded fill
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("n,seed", [(1, 0), (1000, 1), (65537, 2), (1 << 20, 12345678901234)])
+def test_fill_uniform_bit_exact(n, seed):
+    out = np.empty(n, np.float32)
+    cake.fill_uniform(out, seed)
+    assert np.array_equal(out, oracle.uniform(n, seed))
+    assert out.min() >= -1.0 and out.max() < 1.0
+
+
+# ---------------------------------------------------------------------------
+# GEMV
+# ---------------------------------------------------------------------------
+GEMV_SHAPES = [(1, 1), (8, 1), (13, 2111), (64, 7), (1000, 333), (1024, 1024), (4099, 517),
+               (2048, 3000), (300, 70000), (70000, 36)]
+
+
+@pytest.mark.parametrize("M,K", GEMV_SHAPES)
+def test_sgemv_column_major_matches_oracle(M, K):
+    """The reference's contract: A[k*M + m], y accumulates (examples/cake_gemv.cpp:89-140)."""
+    print(f"sgemv col-major M={M} K={K}", flush=True)
+    A, x, y0 = oracle.uniform(M * K, 41), oracle.uniform(K, 42), oracle.uniform(M, 43)
+    ref = oracle.cake_sgemv(A, x, 4, oracle.make_cntx(mr=8), y0=y0, M=M, K=K)
+    y64, S = oracle.gemv_f64(A, x, M, K, col_major=True)
+    y = y0.copy()
+    cake.cake_sgemv(A, x, y, M, K, 4)
+    S1 = S + np.abs(y0)
+    assert np.max(np.abs(y - ref) / S1) <= TOL
+    assert np.max(np.abs(y - (y64 + y0)) / S1) <= TIGHT
+    cake.cake_sgemv(A, x, y, M, K, 4)             # accumulates again
+    assert np.max(np.abs(y - (2 * y64 + y0)) / S1) <= 2 * TIGHT
+    z = np.full(M, 5.0, np.float32)
+    cake.cake_sgemv(A, x, z, M, K, 4, accumulate=False)
+    assert np.max(np.abs(z - y64) / np.maximum(S, 1e-30)) <= TIGHT
+
+
+@pytest.mark.parametrize("M,K", GEMV_SHAPES)
+def test_sgemv_row_major(M, K):
+    print(f"sgemv row-major M={M} K={K}", flush=True)
+    A, x = oracle.uniform(M * K, 44), oracle.uniform(K, 45)
+    y64, S = oracle.gemv_f64(A, x, M, K, col_major=False)
+    y = np.full(M, 3.0, np.float32)
+    cake.cake_sgemv(A, x, y, M, K, 1, row_major=True, accumulate=False)
+    assert np.max(np.abs(y - y64) / np.maximum(S, 1e-30)) <= TIGHT
+    cake.cake_sgemv(A, x, y, M, K, 1, row_major=True, accumulate=True)
+    assert np.max(np.abs(y - 2 * y64) / np.maximum(S, 1e-30)) <= 2 * TIGHT
+    # the same buffer read column-major is the transposed problem
+    if M == K and M > 1:
+        yc = np.zeros(M, np.float32)
+        cake.cake_sgemv(A, x, yc, M, K, 1, accumulate=False)
+        yT, ST = oracle.gemv_f64(A, x, M, K, col_major=True)
+        assert np.max(np.abs(yc - yT) / ST) <= TIGHT
+        assert np.max(np.abs(yc - y64)) > 1e-2
+
+
+def test_sgemv_unaligned_views():
+    """Operands that are not 16-byte aligned take the scalar-load kernels."""
+    M, K = 516, 1028
+    buf = oracle.uniform(M * K + 8, 46)
+    xb = oracle.uniform(K + 8, 47)
+    for off in (1, 3):
+        A, x = buf[off:off + M * K], xb[off:off + K]
+        for col in (True, False):
+            y64, S = oracle.gemv_f64(np.ascontiguousarray(A), np.ascontiguousarray(x), M, K, col_major=col)
+            y = np.zeros(M, np.float32)
+            secs = np.zeros(1)
+            st = cake.load().cake_hip_sgemv(A.ctypes.data, x.ctypes.data, y.ctypes.data, M, K, int(col), 0, None, None)
+            assert st == 0
+            assert np.max(np.abs(y - y64) / S) <= TIGHT
+
+
+def test_sgemv_deterministic():
+    M, K = 3000, 5000
+    A, x = oracle.uniform(M * K, 48), oracle.uniform(K, 49)
+    outs = []
+    for _ in range(3):
+        y = np.zeros(M, np.float32)
+        cake.cake_sgemv(A, x, y, M, K, 1, accumulate=False)
+        outs.append(y)
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+# ---------------------------------------------------------------------------
+# im2col and convolution
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("geom", [
+    (1, 3, 18, 18, 3, 3, 1, 0), (2, 5, 9, 13, 3, 3, 1, 1), (3, 4, 12, 12, 3, 3, 2, 1),
+    (1, 2, 6, 7, 1, 1, 1, 0), (2, 4, 8, 8, 5, 3, 1, 2), (4, 16, 14, 14, 3, 3, 1, 1), (1, 1, 7, 30, 3, 3, 3, 0),
+], ids=str)
+def test_im2col_bit_exact(geom):
+    Bn, Cin, Hin, Win, Hf, Wf, stride, pad = geom
+    inp = oracle.uniform((Bn, Cin, Hin, Win), 51)
+    want = oracle.im2col(inp, Hf, Wf, stride, pad)
+    got = np.full_like(want, np.nan)
+    cake.im2col(inp, got, Bn, Cin, Hin, Win, Hf, Wf, stride, pad)
+    assert np.array_equal(got, want)
+
+
+def test_im_2_col_reference_signature():
+    Cin, Hin, Win, Hf, Wf = 6, 20, 17, 3, 3
+    inp = oracle.uniform((Cin, Hin, Win), 52)
+    got = cake.im_2_col(inp, Wf, Hf, Win, Hin, Win - 2, Hin - 2, Cin, 4, 1)
+    assert np.array_equal(got, oracle.im_2_col(inp, Hf, Wf, Hin - 2, Win - 2))
+    with pytest.raises(ValueError):
+        cake.im_2_col(inp, Wf, Hf, Win, Hin, Win, Hin, Cin)
+
+
+@pytest.mark.parametrize("geom", [(2, 5, 10, 9, 7, 1, 1), (1, 8, 14, 12, 20, 1, 0), (3, 16, 12, 12, 32, 2, 1),
+                                  (2, 64, 28, 28, 96, 1, 1)], ids=str)
+@pytest.mark.parametrize("nchw", [False, True])
+def test_conv2d_matches_oracle(geom, nchw):
+    Bn, Cin, Hin, Win, Cout, stride, pad = geom
+    inp = oracle.uniform((Bn, Cin, Hin, Win), 54)
+    wt = oracle.uniform((Cout, Cin, 3, 3), 55)
+    ref64, S = oracle.conv_naive_f64(inp, wt, stride, pad)
+    _, _, Hout, Wout = ref64.shape
+    out = np.full((Bn, Cout, Hout, Wout) if nchw else (Cout, Bn * Hout * Wout), np.nan, np.float32)
+    cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, 3, 3, stride, pad, out_nchw=nchw)
+    got = out if nchw else out.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
+    assert np.max(np.abs(got - ref64) / S) <= TIGHT
+    # and against the oracle's own im2col -> cake_sgemm pipeline
+    cols = oracle.im2col(inp, 3, 3, stride, pad)
+    cpu = oracle.cake_sgemm(wt.reshape(Cout, -1), cols, 4, oracle.make_cntx(), sch=oracle.KMN)
+    cpu = cpu.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
+    assert np.max(np.abs(got - cpu) / S) <= TOL
+
+
+# ---------------------------------------------------------------------------
+# packed layouts
+# ---------------------------------------------------------------------------
+def _cx(**kw):
+    o = oracle.make_cntx(**kw)
+    return o, cake.CpuCntx(o.alpha_n, o.mr, o.nr, o.L1, o.L2, o.L3, o.ncores)
+
+
+PACK_SHAPES = [(1, 1, 1), (10, 96, 111), (111, 10, 96), (96, 111, 10), (960, 111, 96), (111, 960, 2111),
+               (2111, 96, 111), (500, 700, 300), (1030, 1500, 1000)]
+
+
+@pytest.mark.parametrize("p", [1, 3, 8])
+@pytest.mark.parametrize("sch", [cake.KMN, cake.MKN, cake.NKM])
+@pytest.mark.parametrize("shape", PACK_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_pack_unpack_bit_exact(shape, sch, p):
+    M, K, N = shape
+    print(f"pack M={M} K={K} N={N} sch={sch} p={p}", flush=True)
+    small = M * K * N < 10 ** 7
+    ocx, ccx = _cx(**({"L2": 32 << 10, "L3": 512 << 10} if small else {}))
+    xo = oracle.init_block_dims(M, N, K, p, ocx, sch)
+    xc = cake.init_block_dims(M, N, K, p, ccx, sch)
+    A, B, Cm = oracle.uniform((M, K), 11), oracle.uniform((K, N), 12), oracle.uniform((M, N), 13)
+
+    Ap = np.full(cake.cake_sgemm_packed_A_size(M, K, p, xc, ccx, sch) // 4, np.nan, np.float32)
+    cake.pack_A(A, Ap, M, K, p, xc, ccx, sch)
+    assert np.array_equal(Ap, oracle.pack_A(A, p, xo, ocx, sch))
+
+    Bp = np.full(cake.cake_sgemm_packed_B_size(K, N, p, xc, ccx) // 4, np.nan, np.float32)
+    cake.pack_B(B, Bp, K, N, p, xc, ccx, sch)
+    assert np.array_equal(Bp, oracle.pack_B(B, p, xo, ocx, sch))
+
+    Cp = np.full(cake.cake_sgemm_packed_C_size(M, N, p, xc, ccx, sch) // 4, np.nan, np.float32)
+    cake.pack_C(Cm, Cp, M, N, p, xc, ccx, sch)
+    assert np.array_equal(Cp, oracle.pack_C(Cm, p, xo, ocx, sch))
+
+    back = np.full((M, N), np.nan, np.float32)
+    cake.unpack_C(back, Cp, M, N, p, xc, ccx, sch)
+    assert np.array_equal(back, Cm)
+
+    # product straight from the packed operands, in every packed/plain combination
+    C64, S = oracle.gemm_f64(A, B)
+    for pa, pb in ((True, True), (True, False), (False, True)):
+        out = np.full((M, N), np.nan, np.float32)
+        st = cake.load().cake_hip_sgemm_packed((Ap if pa else A).ctypes.data, (Bp if pb else B).ctypes.data,
+                                               out.ctypes.data, M, N, K, p, xc, ccx, int(pa), int(pb), 0, None, None)
+        assert st == 0, cake.load().cake_hip_last_error()
+        assert oracle.max_rel_err(out, C64, S) <= TIGHT, (pa, pb)
+
+
+def test_packed_sgemm_through_reference_call_sequence():
+    """examples/cake_conv.cpp:1028-1055: init_block_dims -> pack_A, pack_B -> cake_sgemm(..., 1, 1, 1, 0, KMN)."""
+    M, K, N, p = 96, 8 * 9, 30 * 28, 10
+    ocx, ccx = _cx()
+    A, B = oracle.uniform((M, K), 61), oracle.uniform((K, N), 62)
+    x = cake.init_block_dims(M, N, K, p, ccx, cake.KMN)
+    Ap = np.empty(cake.cake_sgemm_packed_A_size(M, K, p, x, ccx, cake.KMN) // 4, np.float32)
+    Bp = np.empty(cake.cake_sgemm_packed_B_size(K, N, p, x, ccx) // 4, np.float32)
+    cake.pack_A(A, Ap, M, K, p, x, ccx, cake.KMN)
+    cake.pack_B(B, Bp, K, N, p, x, ccx, cake.KMN)
+    out = np.zeros((M, N), np.float32)
+    cake.cake_sgemm(Ap, Bp, out, M, N, K, p, ccx, None, True, True, 1.0, 0.0, cake.KMN)
+    ref = oracle.cake_sgemm(A, B, p, ocx, sch=oracle.KMN)
+    C64, S = oracle.gemm_f64(A, B)
+    assert np.max(np.abs(out - ref) / S) <= TOL
+    assert oracle.max_rel_err(out, C64, S) <= TIGHT
+
+
+# ---------------------------------------------------------------------------
+# the C++ drop-in library, driven the way the reference's example mains drive it
+# ---------------------------------------------------------------------------
+def test_cpp_dropin_program():
+    exe = _lib.LIB_DIR / "dropin_test"
+    assert exe.exists(), "build it with make -C cake_on_cpu_amd/csrc"
+    res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=600)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0 and "ALL PASS" in res.stdout
