@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the fp32 GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+
+A step is one cake_sgemm of BASELINE config 2 (M = K = N = 8192, row-major fp32,
+A and B uniform[-1,1) from seeds 1 and 2), operands resident in HBM, launched
+through the C-ABI on torch's current stream.  W untimed steps, then exactly K
+timed steps between two synchronisations.  Prints ONE JSON line:
+
+  value          whole-job TFLOP/s over the K steps (wall clock)
+  roofline       the GEMM macro-tile kernel: algorithmic FLOPs per launch
+                 (2*M*N*K) over its average launch duration, taken from HIP
+                 events recorded around every launch inside the timed region,
+                 against the 157.3 TFLOP/s fp32 matrix peak
+  cpu_baseline   the CPU restatement of the reference cake_sgemm (oracle/, kind
+                 "port") on this host's physical cores, same inputs, full 8192^3
+                 product once after a small warm-up
+  extras         the other BASELINE configs (not bench lines: reported for
+                 information, each with its own roofline figure)
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+METRIC = "fp32 GEMM TFLOP/s @8192^3 (% MFMA peak); GEMV GB/s (% HBM peak)"
+MFMA_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
+
+# HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script, each scaled by what the same counter reads for a plain 256 MiB
+# copy (FETCH_SIZE reads half the true size, WRITE_SIZE the true size).  The
+# summaries are kept under profiles/.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 3408154 * 1024, "sgemv_16384": None}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 256 MiB device copy kernel 3 times (reference point for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (single-GPU hot path); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import cake_on_cpu_amd as cake
+    from cake_on_cpu_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    lib = cake.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        src = torch.ones((64 << 20,), dtype=torch.float32, device=dev)   # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_each_way": src.numel() * 4, "launches": 3}))
+        return 0
+    info = cake.device_info()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def dev_uniform(shape, seed):
+        t = torch.empty(shape, dtype=torch.float32, device=dev)
+        cake.fill_uniform(t, seed)
+        return t
+
+    def time_steps(launch, steps, warmup):
+        """W warm-ups, then K launches between two synchronisations with an event pair per launch."""
+        for _ in range(warmup):
+            launch()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for a, b in evs:
+            a.record()
+            launch()
+            b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        kernel = [a.elapsed_time(b) * 1e-3 for a, b in evs]
+        return wall, float(np.mean(kernel)), float(np.min(kernel))
+
+    # ---------------------------------------------------------------- config 2
+    n = 8192
+    A, B = dev_uniform((n, n), 1), dev_uniform((n, n), 2)
+    Cm = torch.zeros((n, n), dtype=torch.float32, device=dev)
+    pa, pb, pc = A.data_ptr(), B.data_ptr(), Cm.data_ptr()
+
+    def sgemm_step():
+        _lib.check(lib.cake_hip_sgemm(pa, pb, pc, n, n, n, cake.NA, 0, None, stream, None), "cake_hip_sgemm")
+
+    wall, k_avg, k_min = time_steps(sgemm_step, args.steps, args.warmup)
+    flops = 2.0 * n * n * n
+    value = flops * args.steps / wall / 1e12
+    achieved = flops / k_avg / 1e12
+    plan = cake.plan(n, n, n)
+
+    # cheap guard against a fast wrong answer: a few rows against fp64
+    import oracle
+    rows = torch.tensor([0, 1, 4097, n - 1], device=dev)
+    C64, S = oracle.gemm_f64(np.ascontiguousarray(A[rows].cpu().numpy()), B.cpu().numpy())
+    check_err = oracle.max_rel_err(np.ascontiguousarray(Cm[rows].cpu().numpy()), C64, S)
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "cake_sgemm C=A*B, M=K=N=8192, row-major fp32, uniform[-1,1) seeds 1/2 (BASELINE configs[1])",
+            "tile": f"{plan.tile_m}x{plan.tile_n}x{plan.tile_k}",
+            "wave_tile": f"{plan.wave_m}x{plan.wave_n}",
+            "schedule": cake.SCHED_NAMES[plan.sched],
+            "split_k": plan.split_k,
+            "workgroups": plan.grid,
+            "device": info.arch.decode(),
+            "cus": info.cus,
+        },
+        "roofline": {
+            "kernel": "sgemm_tile_kernel<256x256x32, wave 128x64>",
+            "bound": "mfma",
+            "achieved": round(achieved, 3),
+            "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES["sgemm_8192"],
+            "algorithmic_flops_per_launch": flops,
+            "avg_launch_ms": round(k_avg * 1e3, 4),
+            "min_launch_ms": round(k_min * 1e3, 4),
+        },
+        "check": {"max_rel_err_sampled_rows": check_err, "tolerance": 1e-4},
+    }
+
+    # ------------------------------------------------------------ other configs
+    if not args.no_extras:
+        extras = []
+
+        def gemm_extra(name, M, N, K):
+            a, b = dev_uniform((M, K), 1), dev_uniform((K, N), 2)
+            c = torch.zeros((M, N), dtype=torch.float32, device=dev)
+            p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
+            _, avg, _ = time_steps(lambda: _lib.check(
+                lib.cake_hip_sgemm(p3[0], p3[1], p3[2], M, N, K, cake.NA, 0, None, stream, None), name), 20, 5)
+            pl = cake.plan(M, N, K)
+            fl = 2.0 * M * N * K
+            by = 4.0 * (M * K + K * N + M * N)
+            extras.append({"workload": name, "ms": round(avg * 1e3, 4), "tflops": round(fl / avg / 1e12, 2),
+                           "frac_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                           "compulsory_GBps": round(by / avg / 1e9, 1),
+                           "tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
+                           "schedule": cake.SCHED_NAMES[pl.sched]})
+
+        gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024)
+        gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024)
+
+        m = 16384
+        Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
+        yg = torch.zeros((m,), dtype=torch.float32, device=dev)
+        gbytes = 4.0 * (m * m + m + m)
+        for col, label in ((0, "row-major A (configs[3])"), (1, "column-major A (cake_sgemv's own layout)")):
+            _, avg, _ = time_steps(lambda: _lib.check(
+                lib.cake_hip_sgemv(Ag.data_ptr(), xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None), "sgemv"), 50, 10)
+            extras.append({"workload": f"sgemv 16384x16384 {label}", "us": round(avg * 1e6, 2),
+                           "GBps": round(gbytes / avg / 1e9, 1),
+                           "roofline": {"bound": "hbm", "achieved": round(gbytes / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
+                                        "unit": "GB/s", "frac": round(gbytes / avg / 1e9 / HBM_PEAK_GBPS, 4),
+                                        "traffic": MEASURED_TRAFFIC_BYTES["sgemv_16384"],
+                                        "algorithmic_bytes_per_launch": gbytes}})
+        del Ag
+
+        Bn, Cc, H = 32, 256, 56
+        inp, wt = dev_uniform((Bn, Cc, H, H), 5), dev_uniform((Cc, Cc, 3, 3), 4)
+        oc = torch.empty((Cc, Bn * H * H), dtype=torch.float32, device=dev)
+        ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
+        ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
+        _, avg, _ = time_steps(lambda: _lib.check(
+            lib.cake_hip_conv2d(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 0,
+                                ws.data_ptr(), stream, None), "conv2d"), 10, 3)
+        cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
+        extras.append({"workload": "conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 via im2col + sgemm (configs[4])",
+                       "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
+                       "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        out["extras"] = extras
+
+    # -------------------------------------------------------------- CPU baseline
+    if not args.no_cpu:
+        p = oracle.physical_cores()
+        cx = oracle.query_cntx()
+        Ah, Bh = oracle.uniform((n, n), 1), oracle.uniform((n, n), 2)
+        oracle.cake_sgemm(Ah[:2048, :2048].copy(), Bh[:2048, :2048].copy(), p, cx)   # warm-up
+        _, secs, dims = oracle.cake_sgemm(Ah, Bh, p, cx, return_time=True)
+        out["cpu_baseline"] = {
+            "value": round(flops / secs / 1e12, 4),
+            "unit": "TFLOP/s",
+            "cores": p,
+            "kind": "port",
+            "sample": f"one full 8192^3 cake_sgemm (plan+pack+compute+unpack, schedule "
+                      f"{oracle.SCHED_NAMES[dims.sch]}, m_c=k_c={dims.m_c}, n_c={dims.n_c}) after a 2048^3 warm-up; "
+                      f"{secs:.2f} s",
+        }
+    else:
+        out["cpu_baseline"] = None
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
