@@ -178,7 +178,7 @@ __device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
     }
 }
 
-// One LDS stage of MFMA work for a wave.
+// MFMA operands of one wave for a group of 8 consecutive k.
 //
 // v_mfma_f32_32x32x2_f32 takes A[i][kk] from lane i + 32*kk and B[kk][j] from
 // lane j + 32*kk.  The sum over k does not care which two k meet in one
@@ -186,28 +186,300 @@ __device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
 // lanes take k = 0..3 and the upper 32 lanes k = 4..7: each lane then fetches
 // its four A values with a single 16-byte LDS read.
 template <class T>
-__device__ __forceinline__ void mma_stage(const float* As, const float* Bs, int a_row, int b_col,
-                                          int lh, f32x16 (&acc)[T::TM][T::TN])
+struct Frag {
+    f32x4 a[T::TM];
+    float b[T::TN][4];
+};
+
+template <class T>
+__device__ __forceinline__ void load_frag(const float* As, const float* Bs, int a_row, int b_col,
+                                          int lh, int kg, Frag<T>& f)
+{
+    const int kk = kg * 8 + lh * 4;
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm)
+        f.a[tm] = *reinterpret_cast<const f32x4*>(As + (a_row + tm * 32) * T::LDA + kk);
+#pragma unroll
+    for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f.b[tn][i] = Bs[(kk + i) * T::LDB + b_col + tn * 32];
+}
+
+template <class T>
+__device__ __forceinline__ void mma_frag(const Frag<T>& f, f32x16 (&acc)[T::TM][T::TN])
 {
 #pragma unroll
-    for (int kg = 0; kg < T::BK / 8; ++kg) {
-        f32x4 a[T::TM];
-        float b[T::TN][4];
-        const int kk = kg * 8 + lh * 4;
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
-            a[tm] = *reinterpret_cast<const f32x4*>(As + (a_row + tm * 32) * T::LDA + kk);
 #pragma unroll
-        for (int tn = 0; tn < T::TN; ++tn)
+            for (int tn = 0; tn < T::TN; ++tn)
+                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[tm][i], f.b[tn][i], acc[tm][tn], 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------
+// 16-byte loader through buffer instructions.
+//
+// buffer_load_dwordx4 range-checks the byte offset against the resource's
+// num_records and returns zero when it is outside, so an element that must
+// read as zero (row >= M, column >= N, k >= kend) is requested at an offset
+// past num_records instead of being branched around.  The K walk of a
+// workgroup is therefore one straight-line basic block, which is what lets the
+// instruction scheduler interleave memory operations with MFMAs.
+// The resource is re-based every K step (tile origin + k0), so per-thread
+// offsets are constants and stay below 2^31 bytes for lda < 2M, ldb < 16M.
+// ---------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+static constexpr unsigned BUF_RECORDS = 0x80000000u;  // every legal offset is below, BUF_OOB is not
+static constexpr int BUF_OOB = (int)0x80000000u;
+
+__device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_offset)
+{
+    __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)BUF_RECORDS, 0x00020000);
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
+}
+
+template <class T>
+struct VecLoader {
+    int a_off[T::A_ITERS];  // byte offset from the A tile origin, or BUF_OOB for rows >= M
+    int a_k[T::A_ITERS];    // first k of the chunk inside a stage
+    int b_off[T::B_ITERS];  // byte offset from the B tile origin per stage, or BUF_OOB for cols >= N
+    int b_k[T::B_ITERS];    // k row of the chunk inside a stage
+    const float* a_base;    // A + m0*lda
+    const float* b_base;    // B + n0
+    int ldb;
+
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
+    {
+        a_base = g.A + (size_t)m0 * g.lda;
+        b_base = g.B + n0;
+        ldb = g.ldb;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[tn][i] = Bs[(kk + i) * T::LDB + b_col + tn * 32];
+        for (int it = 0; it < T::A_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            a_k[it] = (c % (T::BK / 4)) * 4;
+            a_off[it] = (m0 + r < g.M) ? (r * g.lda + a_k[it]) * 4 : BUF_OOB;
+        }
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int it = 0; it < T::B_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int col = (c % (T::BN / 4)) * 4;
+            b_k[it] = c / (T::BN / 4);
+            b_off[it] = (n0 + col < g.N) ? (b_k[it] * g.ldb + col) * 4 : BUF_OOB;
+        }
+    }
+
+    // chunk OP (A chunks first, then B chunks) of the stage starting at k0
+    template <int OP>
+    __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
+                                             f32x4 (&rb)[T::B_ITERS]) const
+    {
+        const int left = kend - k0;
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = buffer_load_f32x4(a_base + k0, a_k[OP] < left ? a_off[OP] : BUF_OOB);
+        else
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(b_base + (size_t)k0 * ldb,
+                                                    b_k[OP - T::A_ITERS] < left ? b_off[OP - T::A_ITERS] : BUF_OOB);
+    }
+
+    // stage starting at k0; k >= kend reads as zero
+    __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        const int left = kend - k0;
+        const float* a = a_base + k0;
+        const float* b = b_base + (size_t)k0 * ldb;
 #pragma unroll
-            for (int tm = 0; tm < T::TM; ++tm)
+        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = buffer_load_f32x4(a, a_k[it] < left ? a_off[it] : BUF_OOB);
 #pragma unroll
-                for (int tn = 0; tn < T::TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][i], b[tn][i], acc[tm][tn], 0, 0, 0);
+        for (int it = 0; it < T::B_ITERS; ++it) rb[it] = buffer_load_f32x4(b, b_k[it] < left ? b_off[it] : BUF_OOB);
+    }
+};
+
+// K walk for 16-byte-loadable operands.
+//
+// Per K step a wave issues 4*TM*TN*NKG MFMAs and a few dozen memory
+// instructions.  Two waves share a SIMD and run the same code in lockstep, so
+// memory instructions issued in a block stall BOTH waves' matrix work; spread
+// between MFMAs they ride in the shadow of the 64-cycle matrix instruction
+// instead.  Each group of 8 k is therefore cut into slots of a few MFMAs plus
+// ONE memory instruction, and __builtin_amdgcn_sched_barrier(0) after every
+// slot keeps the compiler from regrouping them:
+//     group 0      : LDS reads of group 1's operands, then the global loads of
+//                    step s+1 (they have the rest of the step to complete)
+//     groups 1..   : LDS reads of the next group's operands
+//     last group   : registers -> the other LDS buffer
+// then one barrier and the first operand group of the new stage.
+template <class T>
+struct Slots {
+    static constexpr int NKG = T::BK / 8;
+    static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
+    static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
+    static constexpr int GLOBAL_OPS = T::A_ITERS + T::B_ITERS;  // global loads (= LDS stores) per stage
+    // memory instructions riding in group kg
+    static constexpr int ops(int kg)
+    {
+        return (kg + 1 < NKG ? FRAG_OPS : 0) + (kg == 0 ? GLOBAL_OPS : 0) + (kg == NKG - 1 ? GLOBAL_OPS : 0);
+    }
+};
+
+// Everything a slot needs, so the recursive templates below stay readable.
+template <class T>
+struct WalkCtx {
+    const VecLoader<T>& ld;
+    int k_next, kend;
+    const float* Ac;
+    const float* Bc;
+    float* An;
+    float* Bn;
+    int tid, a_row, b_col, lh;
+    f32x4 (&ra)[T::A_ITERS];
+    f32x4 (&rb)[T::B_ITERS];
+};
+
+// Memory instruction number OP of group KG (compile-time indices, so every
+// register array access is static).
+template <class T, int KG, int OP>
+__device__ __forceinline__ void slot_op(const WalkCtx<T>& c, Frag<T>& next)
+{
+    using S = Slots<T>;
+    constexpr int N_FRAG = (KG + 1 < S::NKG) ? S::FRAG_OPS : 0;
+    constexpr int N_LOAD = (KG == 0) ? S::GLOBAL_OPS : 0;
+    if constexpr (OP < N_FRAG) {
+        const int kk = (KG + 1) * 8 + c.lh * 4;
+        if constexpr (OP < T::TM) {
+            next.a[OP] = *reinterpret_cast<const f32x4*>(c.Ac + (c.a_row + OP * 32) * T::LDA + kk);
+        } else {
+            constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
+            next.b[tn][i] = c.Bc[(kk + i) * T::LDB + c.b_col + tn * 32];
+        }
+    } else if constexpr (OP < N_FRAG + N_LOAD) {
+        c.ld.template load_one<OP - N_FRAG>(c.k_next, c.kend, c.ra, c.rb);
+    } else {
+        constexpr int W = OP - N_FRAG - N_LOAD;  // store number W of the stage
+        if constexpr (W < T::A_ITERS) {
+            const int ch = c.tid + W * T::THREADS;
+            *reinterpret_cast<f32x4*>(c.An + (ch / (T::BK / 4)) * T::LDA + (ch % (T::BK / 4)) * 4) = c.ra[W];
+        } else {
+            const int ch = c.tid + (W - T::A_ITERS) * T::THREADS;
+            *reinterpret_cast<f32x4*>(c.Bn + (ch / (T::BN / 4)) * T::LDB + (ch % (T::BN / 4)) * 4) = c.rb[W - T::A_ITERS];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Memory instruction OP of group KG is issued after MFMA number slot_of(OP)
+// of the group (0 = before the first): the ops are spread evenly over it.
+template <class T, int KG>
+constexpr int slot_of(int op)
+{
+    return ((op + 1) * Slots<T>::MFMA_PER_KG) / (Slots<T>::ops(KG) + 1);
+}
+
+template <class T, int KG, int SLOT, int OP = 0>
+__device__ __forceinline__ void issue_ops_of_slot(const WalkCtx<T>& c, Frag<T>& next)
+{
+    if constexpr (OP < Slots<T>::ops(KG)) {
+        if constexpr (slot_of<T, KG>(OP) == SLOT) slot_op<T, KG, OP>(c, next);
+        if constexpr (slot_of<T, KG>(OP) <= SLOT) issue_ops_of_slot<T, KG, SLOT, OP + 1>(c, next);
+    }
+}
+
+template <class T, int KG, int IDX = 0>
+__device__ __forceinline__ void mfma_group(const WalkCtx<T>& c, const Frag<T>& f, Frag<T>& next,
+                                           f32x16 (&acc)[T::TM][T::TN])
+{
+    if constexpr (IDX == 0) issue_ops_of_slot<T, KG, 0>(c, next);
+    if constexpr (IDX < Slots<T>::MFMA_PER_KG) {
+        constexpr int i = IDX / (T::TM * T::TN), tm = (IDX / T::TN) % T::TM, tn = IDX % T::TN;
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[tm][i], f.b[tn][i], acc[tm][tn], 0, 0, 0);
+        issue_ops_of_slot<T, KG, IDX + 1>(c, next);
+        mfma_group<T, KG, IDX + 1>(c, f, next, acc);
+    }
+}
+
+template <class T, int KG = 0>
+__device__ __forceinline__ void step_groups(const WalkCtx<T>& c, Frag<T> (&frag)[2],
+                                            f32x16 (&acc)[T::TM][T::TN])
+{
+    if constexpr (KG < Slots<T>::NKG) {
+        mfma_group<T, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
+        __builtin_amdgcn_sched_barrier(0);
+        step_groups<T, KG + 1>(c, frag, acc);
+    }
+}
+
+template <class T>
+__device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
+                                           int kbeg, int kend, int steps, int tid, int a_row,
+                                           int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
+{
+    VecLoader<T> ld;
+    ld.init(g, m0, n0, tid);
+    f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
+    Frag<T> frag[2];
+    if (steps <= 0) return;
+    ld.load(kbeg, kend, ra, rb);
+    store_stage<T>(As, Bs, tid, ra, rb);
+    __syncthreads();
+    load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
+
+    int cur = 0;
+    for (int s = 0; s < steps; ++s) {
+        // past the last step the loads fetch zeros into the idle buffer: no branch in the walk
+        const WalkCtx<T> c{ld, kbeg + (s + 1) * T::BK, kend,
+                           As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
+                           As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
+                           tid, a_row, b_col, lh, ra, rb};
+        __builtin_amdgcn_sched_barrier(0);
+        step_groups<T>(c, frag, acc);
+        __syncthreads();
+        cur ^= 1;
+        load_frag<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, a_row, b_col, lh, 0, frag[0]);
+    }
+}
+
+// K walk for operands that need per-element addressing (any alignment, or the
+// reference's packed layouts).  Same double-buffered pipeline with the loads of
+// the next stage issued first; correctness path, not tuned.
+template <class T, int A_MODE, int B_MODE>
+__device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
+                                               int kbeg, int kend, int steps, int tid, int a_row,
+                                               int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
+{
+    constexpr int NKG = T::BK / 8;
+    f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
+    Frag<T> frag[2];
+    if (steps > 0) {
+        load_a_stage<T, A_MODE>(g, m0, kbeg, kend, tid, ra);
+        load_b_stage<T, B_MODE>(g, n0, kbeg, kend, tid, rb);
+        store_stage<T>(As, Bs, tid, ra, rb);
+    }
+    __syncthreads();
+    if (steps > 0) load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
+
+    int cur = 0;
+    for (int s = 0; s < steps; ++s) {
+        const bool more = s + 1 < steps;
+        const float* Ac = As + cur * T::A_STAGE;
+        const float* Bc = Bs + cur * T::B_STAGE;
+        if (more) {
+            const int k0 = kbeg + (s + 1) * T::BK;
+            load_a_stage<T, A_MODE>(g, m0, k0, kend, tid, ra);
+            load_b_stage<T, B_MODE>(g, n0, k0, kend, tid, rb);
+        }
+#pragma unroll
+        for (int kg = 0; kg < NKG; ++kg) {
+            if (kg + 1 < NKG) load_frag<T>(Ac, Bc, a_row, b_col, lh, kg + 1, frag[(kg + 1) & 1]);
+            if (kg == NKG - 1 && more)
+                store_stage<T>(As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE, tid, ra, rb);
+            mma_frag<T>(frag[kg & 1], acc);
+        }
+        __syncthreads();
+        cur ^= 1;
+        if (more) load_frag<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, a_row, b_col, lh, 0, frag[0]);
     }
 }
 
@@ -239,27 +511,10 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
-    f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
-    if (steps > 0) {
-        load_a_stage<T, A_MODE>(g, m0, kbeg, kend, tid, ra);
-        load_b_stage<T, B_MODE>(g, n0, kbeg, kend, tid, rb);
-        store_stage<T>(As, Bs, tid, ra, rb);
-    }
-    __syncthreads();
-
-    int cur = 0;
-    for (int s = 0; s < steps; ++s) {
-        const bool more = s + 1 < steps;
-        if (more) {
-            const int k0 = kbeg + (s + 1) * T::BK;
-            load_a_stage<T, A_MODE>(g, m0, k0, kend, tid, ra);
-            load_b_stage<T, B_MODE>(g, n0, k0, kend, tid, rb);
-        }
-        mma_stage<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, wm0 + l32, wn0 + l32, lh, acc);
-        if (more) store_stage<T>(As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE, tid, ra, rb);
-        __syncthreads();
-        cur ^= 1;
-    }
+    if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4)
+        k_walk_vec<T>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+    else
+        k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32.

@@ -4,8 +4,11 @@
 // (examples/cake_gemv.cpp:89-140,424-490).  A is read exactly once with
 // 16-byte, fully coalesced loads; x is small and is served from cache.
 //
-//   row-major  A[m*K + k]: one wavefront per 4 rows, lanes stride over k,
-//              64-lane butterfly reduction at the end.
+//   row-major  A[m*K + k]: long rows (K >= 2048): one workgroup per 2 rows,
+//              all its lanes stride over k (each row is read as one
+//              sequential stream, which is what keeps the HBM pages open);
+//              short rows: one wavefront per 4 rows.  64-lane butterfly
+//              reduction at the end.
 //   col-major  A[k*M + m] (the reference's layout): lanes own 4 consecutive m,
 //              K is cut into slices across workgroups and waves; slices are
 //              summed in a fixed order (no atomics), so results are
@@ -76,6 +79,49 @@ __global__ void __launch_bounds__(256) sgemv_rowmajor_kernel(const float* __rest
     }
 }
 
+// Long rows: the whole workgroup walks ROWS rows front to back, so each row is
+// one sequential 16-byte-per-lane stream; wave sums meet in LDS in wave order.
+template <int ROWS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) sgemv_rowmajor_wg_kernel(const float* __restrict__ A,
+                                                                       const float* __restrict__ x,
+                                                                       float* __restrict__ y, int M,
+                                                                       int K, int accumulate)
+{
+    __shared__ float red[WAVES][ROWS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = blockIdx.x * ROWS;
+    float acc[ROWS];
+    const f32x4* rowp[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        acc[r] = 0.f;
+        rowp[r] = reinterpret_cast<const f32x4*>(A + (size_t)min(row0 + r, M - 1) * K);
+    }
+    const int K4 = K >> 2;
+    const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+#pragma unroll 4
+    for (int c = tid; c < K4; c += WAVES * 64) {
+        const f32x4 xv = x4[c];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const f32x4 av = __builtin_nontemporal_load(rowp[r] + c);
+            acc[r] += av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const float s = wave_sum(acc[r]);
+        if (lane == 0) red[wave][r] = s;
+    }
+    __syncthreads();
+    if (tid < ROWS && row0 + tid < M) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) s += red[w][tid];
+        y[row0 + tid] = accumulate ? y[row0 + tid] + s : s;
+    }
+}
+
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, hipStream_t stream)
 {
@@ -84,6 +130,14 @@ hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M
     const bool vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(x)) % 16 == 0);
     const int waves = (M + ROWS - 1) / ROWS;
     const int blocks = (waves + 3) / 4;
+    if (vec && K >= 8192) {
+        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2), dim3(512), 0, stream, A, x, y, M, K, accumulate);
+        return hipGetLastError();
+    }
+    if (vec && K >= 2048) {
+        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 4>), dim3((M + 1) / 2), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+        return hipGetLastError();
+    }
     if (vec)
         hipLaunchKernelGGL((sgemv_rowmajor_kernel<ROWS, true>), dim3(blocks), dim3(256), 0, stream, A, x, y, M, K, accumulate);
     else
@@ -99,7 +153,8 @@ static constexpr int COL_BLOCK_M = 256;  // columns of y per workgroup
 static int colmajor_slices(int M, int K, int cus)
 {
     const int mblocks = (M + COL_BLOCK_M - 1) / COL_BLOCK_M;
-    int want = (8 * cus + mblocks - 1) / mblocks;  // ~8 workgroups per CU
+    int want = (2 * cus + mblocks / 2) / mblocks;  // ~2 workgroups (8 waves) per CU: more concurrent
+                                                    // strided streams than that lose HBM page locality
     int max_slices = (K + 63) / 64;                // at least 64 k per slice
     if (want > max_slices) want = max_slices;
     if (want < 1) want = 1;
@@ -134,7 +189,7 @@ __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __rest
             const int span = (kend - kbeg + 3) / 4;
             const int k0 = kbeg + wave * span, k1 = min(kend, k0 + span);
             const float* col = A + (size_t)k0 * M + m;
-#pragma unroll 8
+#pragma unroll 16
             for (int k = k0; k < k1; ++k, col += M) {
                 const f32x4 av = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(col));
                 const float xv = x[k];
