@@ -37,7 +37,6 @@ struct GemmArgs {
 // Macro-tile shapes the planner can choose from.
 enum TileId {
     TILE_256x256x32_W128x64 = 0,  // 8 waves, 2 per SIMD: large compute-bound shapes
-    TILE_256x256x16_W128x128,     // 4 waves, 1 per SIMD, 16 accumulator tiles per wave
     TILE_256x128x32_W64x64,       // 8 waves: N around 128 (tall-skinny)
     TILE_128x256x32_W64x64,       // 8 waves: M around 128
     TILE_128x128x32_W64x64,       // 4 waves: mid-size shapes, 2 workgroups per CU

@@ -20,7 +20,6 @@ double tile_efficiency(int tile_id)
 {
     switch (tile_id) {
         case TILE_256x256x32_W128x64: return 0.80;
-        case TILE_256x256x16_W128x128: return 0.70;
         case TILE_256x128x32_W64x64: return 0.70;
         case TILE_128x256x32_W64x64: return 0.70;
         case TILE_128x128x32_W64x64: return 0.60;
@@ -71,8 +70,6 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
         if (want_n && t.bn != want_n) continue;
         if (want_k && t.bk != want_k) continue;
         if (t.lds_bytes > dev.lds_per_cu) continue;
-        // the single-wave-per-SIMD variant is only taken when asked for by its K depth
-        if (id == TILE_256x256x16_W128x128 && !want_k) continue;
         const int max_split = std::max(1, K / (4 * t.bk));
         for (int split = 1; split <= 64; split *= 2) {
             if (want_split && split != want_split) continue;

@@ -7,7 +7,6 @@ hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_
 {
     switch (tile_id) {
         case TILE_256x256x32_W128x64: return launch_tile<Tile256x256x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
-        case TILE_256x256x16_W128x128: return launch_tile<Tile256x256x16, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         case TILE_256x128x32_W64x64: return launch_tile<Tile256x128x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         case TILE_128x256x32_W64x64: return launch_tile<Tile128x256x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         case TILE_128x128x32_W64x64: return launch_tile<Tile128x128x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);

@@ -17,7 +17,7 @@ static constexpr TileInfo info_of()
 const TileInfo& tile_info(int tile_id)
 {
     static const TileInfo table[TILE_COUNT] = {
-        info_of<Tile256x256x32>(), info_of<Tile256x256x16>(), info_of<Tile256x128x32>(),
+        info_of<Tile256x256x32>(), info_of<Tile256x128x32>(),
         info_of<Tile128x256x32>(), info_of<Tile128x128x32>(), info_of<Tile64x64x32>(),
     };
     return table[tile_id < 0 || tile_id >= TILE_COUNT ? TILE_64x64x32_W32x32 : tile_id];

@@ -306,22 +306,30 @@ struct VecLoader {
 // between MFMAs they ride in the shadow of the 64-cycle matrix instruction
 // instead.  Each group of 8 k is therefore cut into slots of a few MFMAs plus
 // ONE memory instruction, and __builtin_amdgcn_sched_barrier(0) after every
-// slot keeps the compiler from regrouping them:
-//     group 0      : LDS reads of group 1's operands, then the global loads of
-//                    step s+1 (they have the rest of the step to complete)
-//     groups 1..   : LDS reads of the next group's operands
-//     last group   : registers -> the other LDS buffer
-// then one barrier and the first operand group of the new stage.
+// slot keeps the compiler from regrouping them.  With NKG = BK/8 groups:
+//     groups 0..    : LDS reads of the next group's operands
+//     group NKG-2   : ... + registers (stage s+1) -> the other LDS buffer
+//     ---- the step's one barrier ----
+//     group NKG-1   : LDS reads of the NEXT step's first operand group
+//                     + the global loads of stage s+2 into the registers just
+//                     freed, which gives every load NKG-1 groups to complete
+// The barrier sits before the last group on purpose: the last group's operands
+// are already in registers, so its MFMAs keep the matrix pipe busy while the
+// first operands of the new stage come in from LDS, instead of the pipe
+// draining after every barrier.  (By then nobody reads the current buffer any
+// more, and it is only overwritten a whole step later.)
 template <class T>
 struct Slots {
     static constexpr int NKG = T::BK / 8;
     static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
     static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
     static constexpr int GLOBAL_OPS = T::A_ITERS + T::B_ITERS;  // global loads (= LDS stores) per stage
-    // memory instructions riding in group kg
+    static constexpr int STORE_KG = NKG - 2;
+    static_assert(NKG >= 3, "the walk needs three operand groups per K step");
+    // memory instructions riding in group kg: operand reads, then loads, then stores
     static constexpr int ops(int kg)
     {
-        return (kg + 1 < NKG ? FRAG_OPS : 0) + (kg == 0 ? GLOBAL_OPS : 0) + (kg == NKG - 1 ? GLOBAL_OPS : 0);
+        return FRAG_OPS + (kg == NKG - 1 ? GLOBAL_OPS : 0) + (kg == STORE_KG ? GLOBAL_OPS : 0);
     }
 };
 
@@ -345,15 +353,19 @@ template <class T, int KG, int OP>
 __device__ __forceinline__ void slot_op(const WalkCtx<T>& c, Frag<T>& next)
 {
     using S = Slots<T>;
-    constexpr int N_FRAG = (KG + 1 < S::NKG) ? S::FRAG_OPS : 0;
-    constexpr int N_LOAD = (KG == 0) ? S::GLOBAL_OPS : 0;
+    constexpr int N_FRAG = S::FRAG_OPS;
+    constexpr int N_LOAD = (KG == S::NKG - 1) ? S::GLOBAL_OPS : 0;
     if constexpr (OP < N_FRAG) {
-        const int kk = (KG + 1) * 8 + c.lh * 4;
+        // operands of the next group; the last group reads group 0 of the next stage
+        constexpr bool wrap = (KG + 1 == S::NKG);
+        const float* A = wrap ? c.An : c.Ac;
+        const float* B = wrap ? c.Bn : c.Bc;
+        const int kk = (wrap ? 0 : KG + 1) * 8 + c.lh * 4;
         if constexpr (OP < T::TM) {
-            next.a[OP] = *reinterpret_cast<const f32x4*>(c.Ac + (c.a_row + OP * 32) * T::LDA + kk);
+            next.a[OP] = *reinterpret_cast<const f32x4*>(A + (c.a_row + OP * 32) * T::LDA + kk);
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
-            next.b[tn][i] = c.Bc[(kk + i) * T::LDB + c.b_col + tn * 32];
+            next.b[tn][i] = B[(kk + i) * T::LDB + c.b_col + tn * 32];
         }
     } else if constexpr (OP < N_FRAG + N_LOAD) {
         c.ld.template load_one<OP - N_FRAG>(c.k_next, c.kend, c.ra, c.rb);
@@ -405,6 +417,10 @@ __device__ __forceinline__ void step_groups(const WalkCtx<T>& c, Frag<T> (&frag)
                                             f32x16 (&acc)[T::TM][T::TN])
 {
     if constexpr (KG < Slots<T>::NKG) {
+        if constexpr (KG == Slots<T>::NKG - 1) {
+            __syncthreads();  // every wave has stored its share of the next stage
+            __builtin_amdgcn_sched_barrier(0);
+        }
         mfma_group<T, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
         __builtin_amdgcn_sched_barrier(0);
         step_groups<T, KG + 1>(c, frag, acc);
@@ -416,6 +432,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
                                            int kbeg, int kend, int steps, int tid, int a_row,
                                            int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
 {
+    static_assert(Slots<T>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
     VecLoader<T> ld;
     ld.init(g, m0, n0, tid);
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
@@ -423,21 +440,20 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     if (steps <= 0) return;
     ld.load(kbeg, kend, ra, rb);
     store_stage<T>(As, Bs, tid, ra, rb);
+    ld.load(kbeg + T::BK, kend, ra, rb);  // stage 1 waits in registers
     __syncthreads();
     load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
 
     int cur = 0;
     for (int s = 0; s < steps; ++s) {
-        // past the last step the loads fetch zeros into the idle buffer: no branch in the walk
-        const WalkCtx<T> c{ld, kbeg + (s + 1) * T::BK, kend,
+        // stages past the end are fetched as zeros and parked in the idle buffer: no branch in the walk
+        const WalkCtx<T> c{ld, kbeg + (s + 2) * T::BK, kend,
                            As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
                            As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
                            tid, a_row, b_col, lh, ra, rb};
         __builtin_amdgcn_sched_barrier(0);
         step_groups<T>(c, frag, acc);
-        __syncthreads();
         cur ^= 1;
-        load_frag<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, a_row, b_col, lh, 0, frag[0]);
     }
 }
 
@@ -553,7 +569,6 @@ inline hipError_t launch_tile(const GemmArgs& args, int grid, hipStream_t stream
 }
 
 using Tile256x256x32 = Tile<256, 256, 32, 128, 64>;
-using Tile256x256x16 = Tile<256, 256, 16, 128, 128>;
 using Tile256x128x32 = Tile<256, 128, 32, 64, 64>;
 using Tile128x256x32 = Tile<128, 256, 32, 64, 64>;
 using Tile128x128x32 = Tile<128, 128, 32, 64, 64>;
