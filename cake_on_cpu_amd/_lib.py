@@ -43,7 +43,7 @@ class CpuCntx(C.Structure):
 class Plan(C.Structure):
     _fields_ = [(n, C.c_int) for n in
                 ("sched", "tile_m", "tile_n", "tile_k", "wave_m", "wave_n", "threads", "split_k",
-                 "tiles_m", "tiles_n", "group", "grid", "lds_bytes", "vector_loads", "cus")] + \
+                 "tail_tiles", "tail_split", "tiles_m", "tiles_n", "group", "grid", "lds_bytes", "vector_loads", "cus")] + \
                [("flops", C.c_double), ("min_bytes", C.c_double), ("model_bytes", C.c_double)]
 
     def as_dict(self):

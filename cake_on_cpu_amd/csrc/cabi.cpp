@@ -243,6 +243,16 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.accumulate = accumulate;
     g.a_tab = a_tab; g.b_tab = b_tab;
     g.partial = nullptr;
+    g.tail_tiles = plan.pub.tail_tiles;
+    g.tail_split = plan.pub.tail_split;
+    g.tail_k_per_split = plan.tail_k_per_split;
+    g.tail_partial = nullptr;
+    if (plan.pub.tail_tiles > 0) {
+        st = g_ctx.splitk.reserve((size_t)plan.pub.tail_tiles * plan.pub.tail_split * plan.pub.tile_m *
+                                  plan.pub.tile_n * sizeof(float));
+        if (st) return st;
+        g.tail_partial = static_cast<float*>(g_ctx.splitk.ptr);
+    }
     if (plan.pub.split_k > 1) {
         st = g_ctx.splitk.reserve((size_t)plan.pub.split_k * M * N * sizeof(float));
         if (st) return st;
@@ -254,6 +264,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         st = timer.family(1, [&] {
             return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream);
         });
+    else if (plan.pub.tail_tiles > 0)
+        st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); });
     return st;
 }
 

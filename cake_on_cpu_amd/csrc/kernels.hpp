@@ -31,6 +31,12 @@ struct GemmArgs {
     int split_k, k_per_split;  // k_per_split is a multiple of the tile's BK
     int group, group_along_n;  // CB-block raster
     int accumulate;
+    // Tail splitting: the last `tail_tiles` tiles of the raster (the ones that
+    // would run as a thin final round) are cut into `tail_split` K slices each,
+    // written to tail_partial[slice][tail tile][BM x BN] and summed by
+    // launch_tail_reduce.  0 tail_tiles = off.  Not combined with split_k > 1.
+    int tail_tiles, tail_split, tail_k_per_split;
+    float* tail_partial;
     IndexTables a_tab, b_tab;  // used by the packed-operand loaders only
 };
 
@@ -58,6 +64,7 @@ enum LoadMode {
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
                         hipStream_t stream);
+hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
                                 int accumulate, hipStream_t stream);
 

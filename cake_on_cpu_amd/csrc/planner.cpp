@@ -19,11 +19,11 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 double tile_efficiency(int tile_id)
 {
     switch (tile_id) {
-        case TILE_256x256x32_W128x64: return 0.80;
-        case TILE_256x128x32_W64x64: return 0.70;
-        case TILE_128x256x32_W64x64: return 0.70;
-        case TILE_128x128x32_W64x64: return 0.60;
-        default: return 0.30;
+        case TILE_256x256x32_W128x64: return 0.92;
+        case TILE_256x128x32_W64x64: return 0.90;
+        case TILE_128x256x32_W64x64: return 0.90;
+        case TILE_128x128x32_W64x64: return 0.89;
+        default: return 0.60;  // 64x64: one wave per SIMD, 16 MFMAs between barriers
     }
 }
 
@@ -31,6 +31,16 @@ struct Candidate {
     int tile_id, split;
     double seconds;
 };
+
+// Tail splitting: when the tiles do not fill the last round of the machine, the
+// leftover tiles are cut along K so that the last round is short instead of
+// thin.  Returns the slice count for `rem` leftover tiles (1 = leave them whole).
+int tail_split_for(int rem, int ksteps, const DeviceModel& dev)
+{
+    if (rem <= 0 || rem > dev.cus / 2) return 1;
+    int split = std::min({8, dev.cus / rem, ksteps / 4});
+    return split >= 2 ? split : 1;
+}
 
 // Modelled time of one tile shape with one split factor.
 double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
@@ -42,12 +52,22 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     // prologue (first stage load) and epilogue (C store) cost about two K steps
     const double wg_flops = 2.0 * t.bm * t.bn * t.bk * (ksteps + 2);
     const double cu_rate = dev.mfma_flops / dev.cus * tile_efficiency(tile_id);
-    const long per_cu = (wgs + dev.cus - 1) / dev.cus;
-    double s = per_cu * wg_flops / cu_rate;
+    double rounds = (double)((wgs + dev.cus - 1) / dev.cus);
+    bool tail = false;
+    if (split == 1 && wgs > dev.cus) {
+        const int ts = tail_split_for((int)(wgs % dev.cus), ksteps, dev);
+        if (ts > 1) {
+            rounds = (double)(wgs / dev.cus) + (ceil_div(ksteps, ts) + 2.0) / (ksteps + 2.0);
+            tail = true;
+        }
+    }
+    double s = rounds * wg_flops / cu_rate;
     // never faster than streaming the operands once
     const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
-    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 4e-6;
+    // the slices are written, read back and summed by a second kernel
+    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 8e-6;
+    if (tail) s += 8e-6;
     return s + 3e-6;  // launch
 }
 
@@ -98,6 +118,21 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
     // drop slices that would start past K
     p.split_k = ceil_div(K, out->k_per_split);
     p.grid = p.tiles_m * p.tiles_n * p.split_k;
+    p.tail_tiles = 0;
+    p.tail_split = 1;
+    out->tail_k_per_split = 0;
+    const int tiles = p.tiles_m * p.tiles_n;
+    const bool tail_allowed = !(ov && ov[3]);  // an explicit split request is taken literally
+    if (p.split_k == 1 && tiles > dev.cus && tail_allowed) {
+        const int ksteps = ceil_div(K, t.bk);
+        const int ts = tail_split_for(tiles % dev.cus, ksteps, dev);
+        if (ts > 1) {
+            out->tail_k_per_split = ceil_div(ksteps, ts) * t.bk;
+            p.tail_split = ceil_div(K, out->tail_k_per_split);
+            p.tail_tiles = tiles % dev.cus;
+            p.grid = tiles - p.tail_tiles + p.tail_tiles * p.tail_split;
+        }
+    }
     p.vector_loads = vector_ok ? 1 : 0;
     p.cus = dev.cus;
     p.flops = 2.0 * M * N * (double)K;

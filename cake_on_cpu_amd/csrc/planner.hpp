@@ -26,6 +26,7 @@ struct GemmPlan {
     cake_hip_plan_t pub;   // what the C-ABI reports
     int tile_id;           // kernels.hpp TileId
     int k_per_split;       // multiple of tile_k
+    int tail_k_per_split;  // multiple of tile_k; meaningful when pub.tail_tiles > 0
     int group_along_n;
 };
 

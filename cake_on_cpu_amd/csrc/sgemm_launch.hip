@@ -36,6 +36,21 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
     return launch_sgemm_scalar(tile_id, args, grid, stream);
 }
 
+hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream)
+{
+    if (a.tail_tiles <= 0) return hipSuccess;
+    const dim3 grid(a.tail_tiles), block(256);
+    switch (tile_id) {
+        case TILE_256x256x32_W128x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile256x256x32>, grid, block, 0, stream, a); break;
+        case TILE_256x128x32_W64x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile256x128x32>, grid, block, 0, stream, a); break;
+        case TILE_128x256x32_W64x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile128x256x32>, grid, block, 0, stream, a); break;
+        case TILE_128x128x32_W64x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile128x128x32>, grid, block, 0, stream, a); break;
+        case TILE_64x64x32_W32x32: hipLaunchKernelGGL(tail_reduce_kernel<Tile64x64x32>, grid, block, 0, stream, a); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // C = (accumulate ? C : 0) + sum over slices in ascending order: a fixed
 // summation order, so the split-K path is run-to-run deterministic like the
 // reference (one accumulation chain per element, no atomics).

@@ -61,16 +61,8 @@ struct Tile {
 // the ~32 tiles an XCD holds at any moment cover a compact block of C and share
 // their A and B panels in L2.  group = tiles_m with group_along_n = 0 is a pure
 // M-first walk, group = tiles_n with group_along_n = 1 a pure N-first walk.
-__device__ __forceinline__ void decode_tile(const GemmArgs& g, int wg, int& tile_m, int& tile_n,
-                                            int& split)
+__device__ __forceinline__ void raster_tile(const GemmArgs& g, int t, int& tile_m, int& tile_n)
 {
-    const int tiles = g.tiles_m * g.tiles_n;
-    const int total = tiles * g.split_k;
-    const int q = total >> 3, r = total & 7;
-    const int xcd = wg & 7, idx = wg >> 3;
-    int lid = (xcd < r) ? xcd * (q + 1) + idx : r * (q + 1) + (xcd - r) * q + idx;
-    split = lid / tiles;
-    int t = lid - split * tiles;
     const int slow_n = g.group_along_n ? g.tiles_n : g.tiles_m;  // extent of the grouped dimension
     const int fast_n = g.group_along_n ? g.tiles_m : g.tiles_n;
     const int band_sz = g.group * fast_n;
@@ -82,6 +74,57 @@ __device__ __forceinline__ void decode_tile(const GemmArgs& g, int wg, int& tile
     const int slow = first + (rem - fast * gsz);
     tile_m = g.group_along_n ? fast : slow;
     tile_n = g.group_along_n ? slow : fast;
+}
+
+// Position in a sequence of `count` items of the item that workgroup `wg`
+// takes when each XCD is to own one contiguous run of the sequence.
+__device__ __forceinline__ int xcd_contiguous(int wg, int count)
+{
+    const int q = count >> 3, r = count & 7;
+    const int xcd = wg & 7, idx = wg >> 3;
+    return (xcd < r) ? xcd * (q + 1) + idx : r * (q + 1) + (xcd - r) * q + idx;
+}
+
+// Which tile and which K range a workgroup computes.
+struct WorkItem {
+    int tile_m, tile_n;
+    int kbeg, kend;
+    int slice;      // K slice number (split-K or tail), 0 otherwise
+    int tail_tile;  // >= 0: index among the tail tiles, result goes to tail_partial
+};
+
+__device__ __forceinline__ WorkItem decode_tile(const GemmArgs& g, int wg)
+{
+    const int tiles = g.tiles_m * g.tiles_n;
+    const int full = tiles - g.tail_tiles;
+    // Whole tiles first, then the (much shorter) tail slices, each set dealt
+    // evenly over the XCDs on its own so that every XCD gets the same work.
+    const int whole = g.tail_tiles ? full : tiles * g.split_k;
+    const int lid = wg < whole ? xcd_contiguous(wg, whole)
+                               : whole + xcd_contiguous(wg - whole, g.tail_tiles * g.tail_split);
+    WorkItem w;
+    int t, per;
+    if (g.tail_tiles && lid >= full) {
+        const int rr = lid - full;
+        w.tail_tile = rr / g.tail_split;
+        w.slice = rr - w.tail_tile * g.tail_split;
+        t = full + w.tail_tile;
+        per = g.tail_k_per_split;
+    } else if (g.tail_tiles) {
+        w.tail_tile = -1;
+        w.slice = 0;
+        t = lid;
+        per = g.K;
+    } else {
+        w.tail_tile = -1;
+        w.slice = lid / tiles;
+        t = lid - w.slice * tiles;
+        per = g.k_per_split;
+    }
+    w.kbeg = w.slice * per;
+    w.kend = min(g.K, w.kbeg + per);
+    raster_tile(g, t, w.tile_m, w.tile_n);
+    return w;
 }
 
 // ---------------------------------------------------------------------------
@@ -512,11 +555,9 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const int wm0 = (wave / T::WAVES_N) * T::WM;
     const int wn0 = (wave % T::WAVES_N) * T::WN;
 
-    int tile_m, tile_n, split;
-    decode_tile(g, blockIdx.x, tile_m, tile_n, split);
-    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
-    const int kbeg = split * g.k_per_split;
-    const int kend = min(g.K, kbeg + g.k_per_split);
+    const WorkItem w = decode_tile(g, blockIdx.x);
+    const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
+    const int kbeg = w.kbeg, kend = w.kend;
     const int steps = (kend - kbeg + T::BK - 1) / T::BK;
 
     f32x16 acc[T::TM][T::TN];
@@ -534,7 +575,19 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
 
     // Epilogue.  Accumulator register r of a 32x32 tile holds row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
-    float* out = g.partial ? g.partial + (size_t)split * g.M * g.N : g.C;
+    if (w.tail_tile >= 0) {
+        // a K slice of a tail tile: the whole BM x BN block, tile-local, no masking
+        float* out = g.tail_partial + ((size_t)w.slice * g.tail_tiles + w.tail_tile) * (T::BM * T::BN);
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    out[(wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3)) * T::BN + wn0 + tn * 32 + l32] = acc[tm][tn][r];
+        return;
+    }
+    float* out = g.partial ? g.partial + (size_t)w.slice * g.M * g.N : g.C;
     const int ldo = g.partial ? g.N : g.ldc;
     const bool add = (g.partial == nullptr) && g.accumulate;
 #pragma unroll
@@ -551,6 +604,26 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
                 }
             }
         }
+}
+
+// C tile = (accumulate ? C : 0) + sum over the K slices of a tail tile, in
+// ascending slice order.  One workgroup per tail tile.
+template <class T>
+__global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmArgs g)
+{
+    const int j = blockIdx.x;
+    int tile_m, tile_n;
+    raster_tile(g, g.tiles_m * g.tiles_n - g.tail_tiles + j, tile_m, tile_n);
+    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+    for (int e = threadIdx.x; e < T::BM * T::BN; e += 256) {
+        const int r = e / T::BN, c = e - r * T::BN;
+        if (m0 + r >= g.M || n0 + c >= g.N) continue;
+        float* dst = g.C + (size_t)(m0 + r) * g.ldc + n0 + c;
+        float acc = g.accumulate ? *dst : 0.f;
+        for (int s = 0; s < g.tail_split; ++s)
+            acc += g.tail_partial[((size_t)s * g.tail_tiles + j) * (T::BM * T::BN) + e];
+        *dst = acc;
+    }
 }
 
 template <class T, int A_MODE, int B_MODE>

@@ -74,6 +74,8 @@ typedef struct cake_hip_plan_t {
     int wave_m, wave_n;         /* sub-tile held by one 64-lane wavefront         */
     int threads;      /* workgroup size                                           */
     int split_k;      /* K slices reduced in a second, fixed-order pass (1 = none) */
+    int tail_tiles;   /* tiles of the thin last round that are cut along K instead (0 = none) */
+    int tail_split;   /* K slices per tail tile                                   */
     int tiles_m, tiles_n;
     int group;        /* CB-block edge in tiles: tiles that run together share panels */
     int grid;         /* workgroups launched                                      */

@@ -135,7 +135,10 @@ def test_plan_baseline_shapes():
     assert skinny.sched == cake.MKN          # one tile column: walk down M, B panel shared
 
     conv = cake.plan(256, 100352, 2304)
-    assert conv.tiles_m == 1 and conv.sched == cake.NKM   # one tile row: walk along N, A shared
+    assert conv.tiles_m <= 2 and conv.tiles_n >= 392      # a thin strip of tiles along N
+    assert conv.sched in (cake.NKM, cake.KMN)
+    strip = cake.plan(256, 100352, 2304, cake.NA, (256, 256, 32, 0))
+    assert strip.tiles_m == 1 and strip.sched == cake.NKM  # one tile row: walk along N, A shared
 
     small = cake.plan(1024, 1024, 1024)
     assert small.grid >= 128                 # enough workgroups to cover most of the 256 CUs
@@ -147,12 +150,26 @@ def test_plan_covers_any_shape(M, N, K):
         pl = cake.plan(M, N, K, sch)
         assert pl.tiles_m * pl.tile_m >= M and pl.tiles_n * pl.tile_n >= N
         assert (pl.tiles_m - 1) * pl.tile_m < M and (pl.tiles_n - 1) * pl.tile_n < N
-        assert pl.split_k >= 1 and pl.grid == pl.tiles_m * pl.tiles_n * pl.split_k
+        tiles = pl.tiles_m * pl.tiles_n
+        assert pl.split_k >= 1 and pl.tail_split >= 1 and 0 <= pl.tail_tiles < tiles
+        assert not (pl.split_k > 1 and pl.tail_tiles > 0)
+        assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
         assert 1 <= pl.group <= max(pl.tiles_m, pl.tiles_n)
         assert pl.sched in (cake.KMN, cake.MKN, cake.NKM)
         if sch != cake.NA:
             assert pl.sched == sch
         assert pl.vector_loads == int(K % 4 == 0 and N % 4 == 0)
+
+
+def test_plan_tail_split():
+    """A thin last round (few tiles left over after whole rounds of 256 CUs) is cut
+    along K instead: the convolution GEMM leaves 32 of 1568 tiles."""
+    conv = cake.plan(256, 100352, 2304)
+    assert (conv.tile_m, conv.tile_n) == (128, 128) and conv.split_k == 1
+    assert conv.tail_tiles == 1568 % 256 and conv.tail_split == 8
+    assert conv.grid == 1568 - 32 + 32 * 8
+    assert cake.plan(8192, 8192, 8192).tail_tiles == 0          # whole rounds: nothing to cut
+    assert cake.plan(256, 100352, 2304, cake.NA, (128, 128, 32, 1)).tail_tiles == 0   # explicit split is literal
 
 
 def test_plan_tile_override():

@@ -83,6 +83,24 @@ def test_every_tile_shape(tile, shape):
         _check(A, B, Cm, None, (tile, shape, split))
 
 
+@pytest.mark.parametrize("shape", [(1100, 520, 1100), (1100, 517, 1101), (2111, 2111, 2111), (4352, 256, 4096)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_tail_split_shapes(shape):
+    """Shapes whose tile count leaves a thin last round: the planner cuts those
+    tiles along K and a second kernel sums the slices in order."""
+    M, K, N = shape
+    pl = cake.plan(M, N, K)
+    assert pl.tail_tiles > 0 and pl.tail_split > 1, pl.as_dict()
+    print(f"sgemm tail M={M} K={K} N={N} plan={pl.as_dict()}", flush=True)
+    A, B, Cm = _run(M, K, N)
+    _check(A, B, Cm, None, shape)
+    C0 = oracle.uniform((M, N), 3)
+    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    assert np.allclose(acc - Cm, C0, atol=2e-4)
+    again = _run(M, K, N)[2]
+    assert np.array_equal(again, Cm)
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
