@@ -204,13 +204,15 @@ def main() -> int:
         oc = torch.empty((Cc, Bn * H * H), dtype=torch.float32, device=dev)
         ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
         ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
-        _, avg, _ = time_steps(lambda: _lib.check(
-            lib.cake_hip_conv2d(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 0,
-                                ws.data_ptr(), stream, None), "conv2d"), 10, 3)
         cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
-        extras.append({"workload": "conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 via im2col + sgemm (configs[4])",
-                       "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
-                       "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        for fn, label in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM"),
+                          (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps)")):
+            _, avg, _ = time_steps(lambda: _lib.check(
+                fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 0,
+                   ws.data_ptr(), stream, None), "conv2d"), 10, 3)
+            extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
+                           "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
+                           "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
         out["extras"] = extras
 
     # -------------------------------------------------------------- CPU baseline

@@ -98,6 +98,7 @@ SIGNATURES = {
     "cake_hip_im2col": (_i, [_fp, _fp, _i, _i, _i, _i, _i, _i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_conv2d_workspace": (C.c_size_t, [_i] * 9),
     "cake_hip_conv2d": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
+    "cake_hip_conv2d_im2col": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
     "cake_hip_fill_uniform": (_i, [_fp, C.c_size_t, C.c_uint64, C.c_void_p]),
     "cake_hip_last_kernel_seconds": (_i, [C.POINTER(C.c_double * 5)]),
 }

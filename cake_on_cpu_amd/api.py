@@ -272,9 +272,11 @@ def im_2_col(In, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout=0, s=1):
 
 
 def conv2d(inp, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride=1, pad=0,
-           out_nchw=False, workspace=None) -> float:
+           out_nchw=False, workspace=None, explicit_im2col=False) -> float:
     """weights[Cout x Cin*Hf*Wf] . im2col(inp): the im2col path of
-    examples/cake_conv.cpp:1007-1066.  out is [Cout][batch*Hout*Wout] or NCHW."""
+    examples/cake_conv.cpp:1007-1066.  out is [Cout][batch*Hout*Wout] or NCHW.
+    By default the column matrix is gathered inside the GEMM when the geometry
+    allows; explicit_im2col=True always materialises it first, as the reference does."""
     Hout = (Hin + 2 * pad - Hf) // stride + 1
     Wout = (Win + 2 * pad - Wf) // stride + 1
     _need(inp, batch * Cin * Hin * Win, "input")
@@ -286,7 +288,8 @@ def conv2d(inp, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride=1, pad=
         _need(workspace, (need + 3) // 4, "workspace")
         ws = _ptr(workspace, "workspace")
     secs = C.c_double(0.0)
-    check(load().cake_hip_conv2d(_ptr(inp, "input"), _ptr(weights, "weights"), _ptr(out, "out"),
+    fn = load().cake_hip_conv2d_im2col if explicit_im2col else load().cake_hip_conv2d
+    check(fn(_ptr(inp, "input"), _ptr(weights, "weights"), _ptr(out, "out"),
                                  batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, int(out_nchw), ws,
                                  _stream(inp, weights, out), C.byref(secs)), "conv2d")
     return secs.value

@@ -172,6 +172,14 @@ bool fits_int(double elems) { return elems < 2147483647.0; }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// The 16-byte loaders address a macro-tile with 32-bit byte offsets from its
+// origin: 256 rows of A (stride K) and 32 rows of B (stride N) must stay below 2^31.
+bool vec4_loadable(const float* A, const float* B, int K, int N)
+{
+    return (K % 4 == 0) && (N % 4 == 0) && aligned16(A) && aligned16(B) &&
+           (double)K * 256 * 4 < 2147483648.0 && (double)N * 32 * 4 < 2147483648.0;
+}
+
 PackGeom make_geom(int M, int N, int K, int p, const cake_hip_blk_dims_t* d,
                    const cake_hip_cpu_cntx_t* cx, int sched)
 {
@@ -218,7 +226,8 @@ size_t tables_bytes(int which, const PackGeom& g)
 // The GEMM proper on device operands.
 int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
              int sched, int accumulate, const int* tile_override, int a_mode, int b_mode,
-             IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer)
+             IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer,
+             const ConvGeom* conv = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
     GemmPlan plan;
@@ -242,6 +251,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
     g.accumulate = accumulate;
     g.a_tab = a_tab; g.b_tab = b_tab;
+    if (conv) g.conv = *conv;
+    const int nchw_hw = (conv && conv->out_nchw) ? conv->Hout * conv->Wout : 0;
     g.partial = nullptr;
     g.tail_tiles = plan.pub.tail_tiles;
     g.tail_split = plan.pub.tail_split;
@@ -262,7 +273,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     if (st) return st;
     if (plan.pub.split_k > 1)
         st = timer.family(1, [&] {
-            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream);
+            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream, nchw_hw);
         });
     else if (plan.pub.tail_tiles > 0)
         st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); });
@@ -453,7 +464,7 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
             if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
         }
     } else {
-        const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(a.dev) && aligned16(b.dev);
+        const bool vec = vec4_loadable(a.dev, b.dev, K, N);
         const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
         st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, tile_override, mode,
                       mode, IndexTables{}, IndexTables{}, stream, timer);
@@ -692,9 +703,13 @@ size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
     return ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float) + 512;
 }
 
-int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
-                    int Win, int Cout, int Hf, int Wf, int stride, int pad, int out_nchw,
-                    void* workspace, void* stream_, double* seconds)
+// ceil(2^32 / d), or 0 for d == 1 (the loaders then skip the division)
+static unsigned div_magic(unsigned d) { return d <= 1 ? 0u : (unsigned)(((1ull << 32) + d - 1) / d); }
+
+// explicit == 0: gather the column matrix inside the GEMM when the geometry allows it
+static int conv2d_common(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
+                         int Win, int Cout, int Hf, int Wf, int stride, int pad, int out_nchw,
+                         void* workspace, void* stream_, double* seconds, int explicit_cols)
 {
     if (seconds) *seconds = 0;
     int Hout, Wout;
@@ -702,22 +717,47 @@ int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch
         conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout))
         return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
     if (!in || !weights || !out) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
-    const int K = Cin * Hf * Wf;
+    const double K_d = (double)Cin * Hf * Wf;
     const double ncols_d = (double)batch * Hout * Wout;
-    if (!fits_int((double)K * ncols_d) || !fits_int((double)Cout * ncols_d) || K > 65535 ||
-        !fits_int((double)batch * Cin * Hin * Win))
-        return fail(CAKE_HIP_ERR_RANGE, "convolution lowers to a %dx%dx%g product that is out of range", Cout, K, ncols_d);
-    const int N = (int)ncols_d;
+    const double in_elems = (double)batch * Cin * Hin * Win;
+    if (!fits_int(K_d) || !fits_int(Cout * K_d) || !fits_int(Cout * ncols_d) || !fits_int(in_elems))
+        return fail(CAKE_HIP_ERR_RANGE, "convolution lowers to a %dx%gx%g product that is out of range", Cout, K_d, ncols_d);
+    const int K = (int)K_d, N = (int)ncols_d;
     int st = ensure_init();
     if (st) return st;
     std::lock_guard<std::mutex> lock(g_mutex);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     Operand i, w, o;
-    if ((st = stage_in(in, (size_t)batch * Cin * Hin * Win * 4, 0, true, &i))) return st;
+    if ((st = stage_in(in, (size_t)in_elems * 4, 0, true, &i))) return st;
     if ((st = stage_in(weights, (size_t)Cout * K * 4, 1, true, &w))) return st;
     if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
 
+    // The on-the-fly gather needs: 4 consecutive columns inside one output row,
+    // 16-byte loadable weights, byte offsets into the input below 2^31, and the
+    // multiply-high divisions by Hf*Wf and Wf exact (k * Hf*Wf < 2^32).
+    const bool implicit = !explicit_cols && (Wout % 4 == 0) && (K % 4 == 0) && aligned16(w.dev) &&
+                          in_elems * 4 < 2147483648.0 && K_d * Hf * Wf < 4294967296.0 &&
+                          (double)K * 256 * 4 < 2147483648.0;
+    Timer timer(stream, seconds);
+    if (implicit) {
+        ConvGeom cv{};
+        cv.in = i.dev;
+        cv.Cin = Cin; cv.Hin = Hin; cv.Win = Win; cv.Hf = Hf; cv.Wf = Wf;
+        cv.Hout = Hout; cv.Wout = Wout; cv.stride = stride; cv.pad = pad;
+        cv.div_hw_magic = div_magic((unsigned)(Hf * Wf));
+        cv.div_w_magic = div_magic((unsigned)Wf);
+        cv.out_nchw = out_nchw ? 1 : 0;
+        if ((st = timer.start())) return st;
+        st = run_gemm(w.dev, nullptr, o.dev, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
+                      LOAD_IM2COL, IndexTables{}, IndexTables{}, stream, timer, &cv);
+        if (st) return st;
+        if ((st = timer.stop())) return st;
+        return stage_out(o, stream);
+    }
+
+    if (!fits_int(K_d * ncols_d) || K > 65535)
+        return fail(CAKE_HIP_ERR_RANGE, "column matrix %gx%g out of range", K_d, ncols_d);
     char* ws = static_cast<char*>(workspace);
     if (!ws) {
         if ((st = g_ctx.conv.reserve(cake_hip_conv2d_workspace(batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)))) return st;
@@ -729,14 +769,13 @@ int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch
     float* cols = reinterpret_cast<float*>(ws);
     float* cn = cols + (size_t)K * N;  // [Cout][N] product, used only for NCHW output
 
-    Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
     st = timer.family(3, [&] {
         return launch_im2col(i.dev, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad, stream);
     });
     if (st) return st;
     float* prod = out_nchw ? cn : o.dev;
-    const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(w.dev) && aligned16(cols);
+    const bool vec = vec4_loadable(w.dev, cols, K, N);
     const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
     st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode,
                   IndexTables{}, IndexTables{}, stream, timer);
@@ -747,6 +786,22 @@ int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch
     }
     if ((st = timer.stop())) return st;
     return stage_out(o, stream);
+}
+
+int cake_hip_conv2d(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
+                    int Win, int Cout, int Hf, int Wf, int stride, int pad, int out_nchw,
+                    void* workspace, void* stream, double* seconds)
+{
+    return conv2d_common(in, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw,
+                         workspace, stream, seconds, 0);
+}
+
+int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out, int batch, int Cin,
+                           int Hin, int Win, int Cout, int Hf, int Wf, int stride, int pad,
+                           int out_nchw, void* workspace, void* stream, double* seconds)
+{
+    return conv2d_common(in, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw,
+                         workspace, stream, seconds, 1);
 }
 
 int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream_)

@@ -20,6 +20,18 @@ struct IndexTables {
     const int4* col;
 };
 
+// Geometry of a convolution whose column matrix B[k][n] is gathered on the fly:
+// k = c*Hf*Wf + h*Wf + w, n = b*Hout*Wout + ho*Wout + wo,
+// B[k][n] = in[b][c][ho*stride + h - pad][wo*stride + w - pad] or 0 outside the image.
+struct ConvGeom {
+    const float* in;
+    int Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad;
+    unsigned div_hw_magic;  // ceil(2^32 / (Hf*Wf)): k / (Hf*Wf) == mulhi(k, magic) for k*Hf*Wf < 2^32;
+                            // 0 when the divisor is 1
+    unsigned div_w_magic;   // ceil(2^32 / Wf)
+    int out_nchw;           // epilogue writes C as [batch][M][Hout*Wout] instead of [M][N]
+};
+
 struct GemmArgs {
     const float* A;
     const float* B;
@@ -38,6 +50,7 @@ struct GemmArgs {
     int tail_tiles, tail_split, tail_k_per_split;
     float* tail_partial;
     IndexTables a_tab, b_tab;  // used by the packed-operand loaders only
+    ConvGeom conv;             // used by the implicit-im2col loader only
 };
 
 // Macro-tile shapes the planner can choose from.
@@ -59,14 +72,16 @@ const TileInfo& tile_info(int tile_id);
 enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
-    LOAD_PACKED = 2  // reference packed layout through IndexTables
+    LOAD_PACKED = 2, // reference packed layout through IndexTables
+    LOAD_IM2COL = 3  // B only: column matrix of a convolution gathered from the NCHW input
 };
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
                         hipStream_t stream);
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
+// nchw_hw != 0: C is a convolution output written as [N / nchw_hw][M][nchw_hw]
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream);
+                                int accumulate, hipStream_t stream, int nchw_hw = 0);
 
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, hipStream_t stream);

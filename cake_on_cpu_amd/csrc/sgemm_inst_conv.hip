@@ -1,0 +1,20 @@
+// Macro-tile GEMM instantiations for convolution: A (the OIHW weights as a
+// Cout x Cin*Hf*Wf matrix) through 16-byte loads, B gathered from the NCHW input
+// on the fly, so the K x N column matrix never exists in memory.
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+hipError_t launch_sgemm_conv(int tile_id, const GemmArgs& a, int grid, hipStream_t s)
+{
+    switch (tile_id) {
+        case TILE_256x256x32_W128x64: return launch_tile<Tile256x256x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        case TILE_256x128x32_W64x64: return launch_tile<Tile256x128x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        case TILE_128x256x32_W64x64: return launch_tile<Tile128x256x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        case TILE_128x128x32_W64x64: return launch_tile<Tile128x128x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        case TILE_64x64x32_W32x32: return launch_tile<Tile64x64x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace cake

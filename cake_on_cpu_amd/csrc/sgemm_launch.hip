@@ -7,6 +7,7 @@ hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_
 hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_packed(int tile_id, int a_mode, int b_mode, const GemmArgs& a, int grid,
                                hipStream_t s);
+hipError_t launch_sgemm_conv(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 
 template <class T>
 static constexpr TileInfo info_of()
@@ -27,6 +28,10 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
                         hipStream_t stream)
 {
     if (grid <= 0) return hipSuccess;
+    if (b_mode == LOAD_IM2COL) {
+        if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
+        return launch_sgemm_conv(tile_id, args, grid, stream);
+    }
     if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
         if (a_mode == LOAD_VEC4) a_mode = LOAD_SCALAR;
         if (b_mode == LOAD_VEC4) b_mode = LOAD_SCALAR;
@@ -39,7 +44,8 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream)
 {
     if (a.tail_tiles <= 0) return hipSuccess;
-    const dim3 grid(a.tail_tiles), block(256);
+    const TileInfo& t = tile_info(tile_id);
+    const dim3 grid(a.tail_tiles, t.bm * t.bn / 1024), block(256);
     switch (tile_id) {
         case TILE_256x256x32_W128x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile256x256x32>, grid, block, 0, stream, a); break;
         case TILE_256x128x32_W64x64: hipLaunchKernelGGL(tail_reduce_kernel<Tile256x128x32>, grid, block, 0, stream, a); break;
@@ -56,13 +62,18 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream
 // reference (one accumulation chain per element, no atomics).
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial,
                                                             float* __restrict__ C, int M, int N,
-                                                            int ldc, int splits, int accumulate)
+                                                            int ldc, int splits, int accumulate,
+                                                            int nchw_hw)
 {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
         const int row = (int)(i / N), col = (int)(i - (size_t)row * N);
         float* dst = C + (size_t)row * ldc + col;
+        if (nchw_hw) {  // column (image b, pixel) of a convolution written as NCHW
+            const int b = col / nchw_hw;
+            dst = C + ((size_t)b * M + row) * nchw_hw + (col - b * nchw_hw);
+        }
         float acc = accumulate ? *dst : 0.f;
         for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * total + i];
         *dst = acc;
@@ -70,14 +81,14 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
 }
 
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream)
+                                int accumulate, hipStream_t stream, int nchw_hw)
 {
     const size_t total = (size_t)M * N;
     if (total == 0) return hipSuccess;
     size_t blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
-                       M, N, ldc, splits, accumulate);
+                       M, N, ldc, splits, accumulate, nchw_hw);
     return hipGetLastError();
 }
 

@@ -286,6 +286,7 @@ __device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_o
 
 template <class T>
 struct VecLoader {
+    static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;  // load instructions per stage
     int a_off[T::A_ITERS];  // byte offset from the A tile origin, or BUF_OOB for rows >= M
     int a_k[T::A_ITERS];    // first k of the chunk inside a stage
     int b_off[T::B_ITERS];  // byte offset from the B tile origin per stage, or BUF_OOB for cols >= N
@@ -341,6 +342,102 @@ struct VecLoader {
     }
 };
 
+__device__ __forceinline__ float buffer_load_f32(const float* base, int byte_offset)
+{
+    __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)BUF_RECORDS, 0x00020000);
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
+}
+
+// A through 16-byte buffer loads as in VecLoader; B = the column matrix of a
+// convolution, gathered element by element from the NCHW input ("implicit
+// im2col": examples/cake_conv.cpp:1178-1213 without the K x N intermediate).
+// A thread's B chunk is 4 consecutive n at one k; with Wout % 4 == 0 those are
+// 4 consecutive output pixels of one image row, so one (image, row, column)
+// triple per thread serves the whole K walk, and only the filter tap (c, h, w)
+// of each k has to be decoded per stage.  Window positions outside the image
+// are requested at an out-of-range buffer offset and read as zero.
+template <class T>
+struct ConvLoader {
+    static constexpr int NUM_LOADS = T::A_ITERS + 4 * T::B_ITERS;
+    int a_off[T::A_ITERS];
+    int a_k[T::A_ITERS];
+    int b_k[T::B_ITERS];  // k row of the chunk inside a stage
+    const float* a_base;
+    ConvGeom cv;
+    int pix;              // element offset of in[b][0][ho*s - pad][wo*s - pad] for the chunk's first n
+    int hs, ws;           // ho*s - pad, wo*s - pad
+    bool n_ok;
+
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
+    {
+        a_base = g.A + (size_t)m0 * g.lda;
+        cv = g.conv;
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            a_k[it] = (c % (T::BK / 4)) * 4;
+            a_off[it] = (m0 + r < g.M) ? (r * g.lda + a_k[it]) * 4 : BUF_OOB;
+        }
+#pragma unroll
+        for (int it = 0; it < T::B_ITERS; ++it) b_k[it] = (tid + it * T::THREADS) / (T::BN / 4);
+        static_assert(T::THREADS % (T::BN / 4) == 0, "a thread keeps the same 4 columns in every chunk");
+        const int n = n0 + (tid % (T::BN / 4)) * 4;
+        n_ok = n < g.N;
+        const int HW = cv.Hout * cv.Wout;
+        const int b = n / HW, r = n - b * HW;
+        const int ho = r / cv.Wout, wo = r - ho * cv.Wout;
+        hs = ho * cv.stride - cv.pad;
+        ws = wo * cv.stride - cv.pad;
+        pix = ((b * cv.Cin) * cv.Hin + hs) * cv.Win + ws;
+    }
+
+    // The filter tap of a chunk's k is decoded by the chunk's first load and
+    // kept for the other three (the loads of a chunk are issued in order).
+    mutable int tap_off[T::B_ITERS];  // byte offset of the tap's window start for n, or garbage when !tap_ok
+    mutable int tap_w[T::B_ITERS];    // ws + w
+    mutable bool tap_ok[T::B_ITERS];  // column, k and image row are all inside
+
+    template <int OP>
+    __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
+                                             f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS) {
+            ra[OP] = buffer_load_f32x4(a_base + k0, a_k[OP] < kend - k0 ? a_off[OP] : BUF_OOB);
+        } else {
+            constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
+            if constexpr (e == 0) {
+                const int k = k0 + b_k[it];
+                // ceil(2^32 / d) does not fit 32 bits for d == 1: a zero magic marks that case
+                const int c = cv.div_hw_magic ? (int)__umulhi((unsigned)k, cv.div_hw_magic) : k;
+                const int tap = k - c * (cv.Hf * cv.Wf);
+                const int h = cv.div_w_magic ? (int)__umulhi((unsigned)tap, cv.div_w_magic) : tap;
+                const int w = tap - h * cv.Wf;
+                tap_off[it] = (pix + (c * cv.Hin + h) * cv.Win + w) * 4;
+                tap_w[it] = ws + w;
+                tap_ok[it] = n_ok && k < kend && (unsigned)(hs + h) < (unsigned)cv.Hin;
+            }
+            const bool ok = tap_ok[it] && (unsigned)(tap_w[it] + e * cv.stride) < (unsigned)cv.Win;
+            rb[it][e] = buffer_load_f32(cv.in, ok ? tap_off[it] + e * cv.stride * 4 : BUF_OOB);
+        }
+    }
+
+    __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        load_all<0>(k0, kend, ra, rb);
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < NUM_LOADS) {
+            load_one<OP>(k0, kend, ra, rb);
+            load_all<OP + 1>(k0, kend, ra, rb);
+        }
+    }
+};
+
 // K walk for 16-byte-loadable operands.
 //
 // Per K step a wave issues 4*TM*TN*NKG MFMAs and a few dozen memory
@@ -361,25 +458,26 @@ struct VecLoader {
 // first operands of the new stage come in from LDS, instead of the pipe
 // draining after every barrier.  (By then nobody reads the current buffer any
 // more, and it is only overwritten a whole step later.)
-template <class T>
+template <class T, class L>
 struct Slots {
     static constexpr int NKG = T::BK / 8;
     static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
     static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
-    static constexpr int GLOBAL_OPS = T::A_ITERS + T::B_ITERS;  // global loads (= LDS stores) per stage
+    static constexpr int LOAD_OPS = L::NUM_LOADS;               // global load instructions per stage
+    static constexpr int STORE_OPS = T::A_ITERS + T::B_ITERS;   // 16-byte LDS stores per stage
     static constexpr int STORE_KG = NKG - 2;
     static_assert(NKG >= 3, "the walk needs three operand groups per K step");
     // memory instructions riding in group kg: operand reads, then loads, then stores
     static constexpr int ops(int kg)
     {
-        return FRAG_OPS + (kg == NKG - 1 ? GLOBAL_OPS : 0) + (kg == STORE_KG ? GLOBAL_OPS : 0);
+        return FRAG_OPS + (kg == NKG - 1 ? LOAD_OPS : 0) + (kg == STORE_KG ? STORE_OPS : 0);
     }
 };
 
 // Everything a slot needs, so the recursive templates below stay readable.
-template <class T>
+template <class T, class L>
 struct WalkCtx {
-    const VecLoader<T>& ld;
+    const L& ld;
     int k_next, kend;
     const float* Ac;
     const float* Bc;
@@ -392,12 +490,12 @@ struct WalkCtx {
 
 // Memory instruction number OP of group KG (compile-time indices, so every
 // register array access is static).
-template <class T, int KG, int OP>
-__device__ __forceinline__ void slot_op(const WalkCtx<T>& c, Frag<T>& next)
+template <class T, class L, int KG, int OP>
+__device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
 {
-    using S = Slots<T>;
+    using S = Slots<T, L>;
     constexpr int N_FRAG = S::FRAG_OPS;
-    constexpr int N_LOAD = (KG == S::NKG - 1) ? S::GLOBAL_OPS : 0;
+    constexpr int N_LOAD = (KG == S::NKG - 1) ? S::LOAD_OPS : 0;
     if constexpr (OP < N_FRAG) {
         // operands of the next group; the last group reads group 0 of the next stage
         constexpr bool wrap = (KG + 1 == S::NKG);
@@ -427,56 +525,56 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T>& c, Frag<T>& next)
 
 // Memory instruction OP of group KG is issued after MFMA number slot_of(OP)
 // of the group (0 = before the first): the ops are spread evenly over it.
-template <class T, int KG>
+template <class T, class L, int KG>
 constexpr int slot_of(int op)
 {
-    return ((op + 1) * Slots<T>::MFMA_PER_KG) / (Slots<T>::ops(KG) + 1);
+    return ((op + 1) * Slots<T, L>::MFMA_PER_KG) / (Slots<T, L>::ops(KG) + 1);
 }
 
-template <class T, int KG, int SLOT, int OP = 0>
-__device__ __forceinline__ void issue_ops_of_slot(const WalkCtx<T>& c, Frag<T>& next)
+template <class T, class L, int KG, int SLOT, int OP = 0>
+__device__ __forceinline__ void issue_ops_of_slot(const WalkCtx<T, L>& c, Frag<T>& next)
 {
-    if constexpr (OP < Slots<T>::ops(KG)) {
-        if constexpr (slot_of<T, KG>(OP) == SLOT) slot_op<T, KG, OP>(c, next);
-        if constexpr (slot_of<T, KG>(OP) <= SLOT) issue_ops_of_slot<T, KG, SLOT, OP + 1>(c, next);
+    if constexpr (OP < Slots<T, L>::ops(KG)) {
+        if constexpr (slot_of<T, L, KG>(OP) == SLOT) slot_op<T, L, KG, OP>(c, next);
+        if constexpr (slot_of<T, L, KG>(OP) <= SLOT) issue_ops_of_slot<T, L, KG, SLOT, OP + 1>(c, next);
     }
 }
 
-template <class T, int KG, int IDX = 0>
-__device__ __forceinline__ void mfma_group(const WalkCtx<T>& c, const Frag<T>& f, Frag<T>& next,
+template <class T, class L, int KG, int IDX = 0>
+__device__ __forceinline__ void mfma_group(const WalkCtx<T, L>& c, const Frag<T>& f, Frag<T>& next,
                                            f32x16 (&acc)[T::TM][T::TN])
 {
-    if constexpr (IDX == 0) issue_ops_of_slot<T, KG, 0>(c, next);
-    if constexpr (IDX < Slots<T>::MFMA_PER_KG) {
+    if constexpr (IDX == 0) issue_ops_of_slot<T, L, KG, 0>(c, next);
+    if constexpr (IDX < Slots<T, L>::MFMA_PER_KG) {
         constexpr int i = IDX / (T::TM * T::TN), tm = (IDX / T::TN) % T::TM, tn = IDX % T::TN;
         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[tm][i], f.b[tn][i], acc[tm][tn], 0, 0, 0);
-        issue_ops_of_slot<T, KG, IDX + 1>(c, next);
-        mfma_group<T, KG, IDX + 1>(c, f, next, acc);
+        issue_ops_of_slot<T, L, KG, IDX + 1>(c, next);
+        mfma_group<T, L, KG, IDX + 1>(c, f, next, acc);
     }
 }
 
-template <class T, int KG = 0>
-__device__ __forceinline__ void step_groups(const WalkCtx<T>& c, Frag<T> (&frag)[2],
+template <class T, class L, int KG = 0>
+__device__ __forceinline__ void step_groups(const WalkCtx<T, L>& c, Frag<T> (&frag)[2],
                                             f32x16 (&acc)[T::TM][T::TN])
 {
-    if constexpr (KG < Slots<T>::NKG) {
-        if constexpr (KG == Slots<T>::NKG - 1) {
+    if constexpr (KG < Slots<T, L>::NKG) {
+        if constexpr (KG == Slots<T, L>::NKG - 1) {
             __syncthreads();  // every wave has stored its share of the next stage
             __builtin_amdgcn_sched_barrier(0);
         }
-        mfma_group<T, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
+        mfma_group<T, L, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
         __builtin_amdgcn_sched_barrier(0);
-        step_groups<T, KG + 1>(c, frag, acc);
+        step_groups<T, L, KG + 1>(c, frag, acc);
     }
 }
 
-template <class T>
+template <class T, class L>
 __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
                                            int kbeg, int kend, int steps, int tid, int a_row,
                                            int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
 {
-    static_assert(Slots<T>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
-    VecLoader<T> ld;
+    static_assert(Slots<T, L>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
+    L ld;
     ld.init(g, m0, n0, tid);
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
     Frag<T> frag[2];
@@ -490,12 +588,12 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     int cur = 0;
     for (int s = 0; s < steps; ++s) {
         // stages past the end are fetched as zeros and parked in the idle buffer: no branch in the walk
-        const WalkCtx<T> c{ld, kbeg + (s + 2) * T::BK, kend,
+        const WalkCtx<T, L> c{ld, kbeg + (s + 2) * T::BK, kend,
                            As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
                            As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
                            tid, a_row, b_col, lh, ra, rb};
         __builtin_amdgcn_sched_barrier(0);
-        step_groups<T>(c, frag, acc);
+        step_groups<T, L>(c, frag, acc);
         cur ^= 1;
     }
 }
@@ -569,7 +667,9 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
     if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4)
-        k_walk_vec<T>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+        k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+    else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL)
+        k_walk_vec<T, ConvLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
     else
         k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
 
@@ -590,16 +690,26 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     float* out = g.partial ? g.partial + (size_t)w.slice * g.M * g.N : g.C;
     const int ldo = g.partial ? g.N : g.ldc;
     const bool add = (g.partial == nullptr) && g.accumulate;
+    // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
+    const bool nchw = (B_MODE == LOAD_IM2COL) && g.conv.out_nchw && g.partial == nullptr;
+    const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
 #pragma unroll
     for (int tm = 0; tm < T::TM; ++tm)
 #pragma unroll
         for (int tn = 0; tn < T::TN; ++tn) {
             const int col = n0 + wn0 + tn * 32 + l32;
+            size_t col_off = col;
+            size_t row_stride = ldo;
+            if (nchw) {
+                const int b = col / HW;
+                col_off = (size_t)b * g.M * HW + (col - b * HW);
+                row_stride = HW;
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
                 if (row < g.M && col < g.N) {
-                    float* dst = out + (size_t)row * ldo + col;
+                    float* dst = out + (size_t)row * row_stride + col_off;
                     *dst = add ? *dst + acc[tm][tn][r] : acc[tm][tn][r];
                 }
             }
@@ -607,23 +717,37 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
 }
 
 // C tile = (accumulate ? C : 0) + sum over the K slices of a tail tile, in
-// ascending slice order.  One workgroup per tail tile.
+// ascending slice order.  grid = (tail tiles, 1024-element chunks of a tile);
+// each thread sums 4 consecutive elements of a tile row.
 template <class T>
 __global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmArgs g)
 {
+    static_assert(T::BN % 4 == 0 && (T::BM * T::BN) % 1024 == 0, "tile is cut into float4 chunks");
     const int j = blockIdx.x;
     int tile_m, tile_n;
     raster_tile(g, g.tiles_m * g.tiles_n - g.tail_tiles + j, tile_m, tile_n);
-    const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
-    for (int e = threadIdx.x; e < T::BM * T::BN; e += 256) {
-        const int r = e / T::BN, c = e - r * T::BN;
-        if (m0 + r >= g.M || n0 + c >= g.N) continue;
-        float* dst = g.C + (size_t)(m0 + r) * g.ldc + n0 + c;
-        float acc = g.accumulate ? *dst : 0.f;
-        for (int s = 0; s < g.tail_split; ++s)
-            acc += g.tail_partial[((size_t)s * g.tail_tiles + j) * (T::BM * T::BN) + e];
-        *dst = acc;
+    const int e = (blockIdx.y * 256 + threadIdx.x) * 4;
+    const int r = e / T::BN, c = e - r * T::BN;
+    const int row = tile_m * T::BM + r, col = tile_n * T::BN + c;
+    if (row >= g.M || col >= g.N) return;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const float* src = g.tail_partial + (size_t)j * (T::BM * T::BN) + e;
+    const size_t slice_stride = (size_t)g.tail_tiles * (T::BM * T::BN);
+    float* dst = g.C + (size_t)row * g.ldc + col;
+    if (g.conv.in && g.conv.out_nchw) {  // 4 consecutive n stay inside one image row (Wout % 4 == 0)
+        const int HW = g.conv.Hout * g.conv.Wout, b = col / HW;
+        dst = g.C + ((size_t)b * g.M + row) * HW + (col - b * HW);
     }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        if (g.accumulate && col + q < g.N) acc[q] = dst[q];
+    for (int s = 0; s < g.tail_split; ++s) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(src + s * slice_stride);
+        acc += v;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        if (col + q < g.N) dst[q] = acc[q];
 }
 
 template <class T, int A_MODE, int B_MODE>

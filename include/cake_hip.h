@@ -198,14 +198,24 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * im2col path of examples/cake_conv.cpp:1007-1066.  weights are OIHW.
  * out_nchw == 0: out is [Cout][batch*Hout*Wout] (the GEMM's own layout, which
  * is what the reference produces for its single image); != 0: NCHW.
- * workspace (device, cake_hip_conv2d_workspace bytes) may be NULL: the library
- * then uses a buffer of its own. */
+ *
+ * cake_hip_conv2d gathers the column matrix inside the GEMM's B loader when the
+ * geometry allows it (Wout % 4 == 0, Cin*Hf*Wf % 4 == 0, input below 2 GiB), so
+ * the K x N intermediate is never written; otherwise it runs the two-step path.
+ * cake_hip_conv2d_im2col always runs the two steps the reference runs: im2col
+ * into a column matrix, then the GEMM.  Both give the same result.
+ * workspace (device, cake_hip_conv2d_workspace bytes; only the two-step path
+ * uses it) may be NULL: the library then uses a buffer of its own. */
 size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
                                  int Hf, int Wf, int stride, int pad);
 int cake_hip_conv2d(const float* in, const float* weights, float* out,
                     int batch, int Cin, int Hin, int Win, int Cout, int Hf, int Wf,
                     int stride, int pad, int out_nchw, void* workspace,
                     void* stream, double* seconds);
+int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
+                           int batch, int Cin, int Hin, int Win, int Cout, int Hf, int Wf,
+                           int stride, int pad, int out_nchw, void* workspace,
+                           void* stream, double* seconds);
 
 /* ---- seeded inputs -------------------------------------------------------- */
 /* dst[i] = uniform[-1,1) value i of the counter-based splitmix64 stream `seed`

@@ -99,6 +99,10 @@ def test_c5_conv_256x256x56x56_batch32_sampled():
     out = torch.empty((Cout, Bn * H * H), dtype=torch.float32, device="cuda:0")
     cake.conv2d(inp, wt, out, Bn, Cin, H, H, Cout, 3, 3, 1, 1)
     torch.cuda.synchronize()
+    # the reference's own two steps (column matrix first) give the same numbers
+    two_step = torch.empty_like(out)
+    cake.conv2d(inp, wt, two_step, Bn, Cin, H, H, Cout, 3, 3, 1, 1, explicit_im2col=True)
+    assert torch.equal(two_step, out)
     # two whole images (first and last) against the naive fp64 convolution
     wh = wt.cpu().numpy()
     for b in (0, Bn - 1):

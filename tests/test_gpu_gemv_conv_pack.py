@@ -124,24 +124,56 @@ def test_im_2_col_reference_signature():
         cake.im_2_col(inp, Wf, Hf, Win, Hin, Win, Hin, Cin)
 
 
-@pytest.mark.parametrize("geom", [(2, 5, 10, 9, 7, 1, 1), (1, 8, 14, 12, 20, 1, 0), (3, 16, 12, 12, 32, 2, 1),
-                                  (2, 64, 28, 28, 96, 1, 1)], ids=str)
+CONV_GEOMS = [
+    # batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad
+    (2, 5, 10, 9, 7, 3, 3, 1, 1),        # Wout = 9: two-step path only
+    (1, 8, 14, 12, 20, 3, 3, 1, 0),      # Wout = 10
+    (3, 16, 12, 12, 32, 3, 3, 2, 1),     # Wout = 6
+    (2, 64, 28, 28, 96, 3, 3, 1, 1),     # Wout = 28: gathered inside the GEMM
+    (2, 8, 16, 16, 24, 3, 3, 1, 1),      # Wout = 16
+    (3, 12, 18, 18, 40, 3, 3, 1, 0),     # Wout = 16, no padding
+    (2, 4, 17, 17, 300, 3, 3, 2, 1),     # Wout = 9 ... stride 2
+    (2, 4, 15, 16, 300, 3, 3, 2, 1),     # Wout = 8, stride 2, Cout over one tile
+    (1, 16, 9, 12, 10, 1, 1, 1, 0),      # 1x1 filter, Wout = 12
+    (2, 4, 12, 14, 9, 5, 3, 1, 2),       # 5x3 filter, pad 2, Wout = 16
+    (4, 32, 14, 8, 64, 3, 3, 1, 1),      # Wout = 8
+    (1, 4, 6, 8, 5, 3, 3, 3, 2),         # stride 3, pad 2, Wout = 4
+]
+
+
+@pytest.mark.parametrize("geom", CONV_GEOMS, ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
-def test_conv2d_matches_oracle(geom, nchw):
-    Bn, Cin, Hin, Win, Cout, stride, pad = geom
+@pytest.mark.parametrize("explicit", [False, True])
+def test_conv2d_matches_oracle(geom, nchw, explicit):
+    """Both convolution paths (column matrix materialised first, as the reference
+    does, or gathered inside the GEMM) against the naive fp64 convolution and
+    against the oracle's own im2col -> cake_sgemm pipeline."""
+    Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad = geom
+    print(f"conv2d geom={geom} nchw={nchw} explicit={explicit}", flush=True)
     inp = oracle.uniform((Bn, Cin, Hin, Win), 54)
-    wt = oracle.uniform((Cout, Cin, 3, 3), 55)
+    wt = oracle.uniform((Cout, Cin, Hf, Wf), 55)
     ref64, S = oracle.conv_naive_f64(inp, wt, stride, pad)
     _, _, Hout, Wout = ref64.shape
     out = np.full((Bn, Cout, Hout, Wout) if nchw else (Cout, Bn * Hout * Wout), np.nan, np.float32)
-    cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, 3, 3, stride, pad, out_nchw=nchw)
+    cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=nchw,
+                explicit_im2col=explicit)
     got = out if nchw else out.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
-    assert np.max(np.abs(got - ref64) / S) <= TIGHT
-    # and against the oracle's own im2col -> cake_sgemm pipeline
-    cols = oracle.im2col(inp, 3, 3, stride, pad)
+    assert np.max(np.abs(got - ref64) / np.maximum(S, 1e-30)) <= TIGHT
+    cols = oracle.im2col(inp, Hf, Wf, stride, pad)
     cpu = oracle.cake_sgemm(wt.reshape(Cout, -1), cols, 4, oracle.make_cntx(), sch=oracle.KMN)
     cpu = cpu.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
-    assert np.max(np.abs(got - cpu) / S) <= TOL
+    assert np.max(np.abs(got - cpu) / np.maximum(S, 1e-30)) <= TOL
+
+
+def test_conv2d_paths_agree_bitwise_layouts():
+    """Same sums in the same order whichever way the columns reach the GEMM."""
+    Bn, Cin, Hin, Win, Cout = 2, 32, 20, 20, 48
+    inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 56), oracle.uniform((Cout, Cin, 3, 3), 57)
+    a = np.empty((Cout, Bn * 400), np.float32)
+    b = np.empty_like(a)
+    cake.conv2d(inp, wt, a, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
+    cake.conv2d(inp, wt, b, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1, explicit_im2col=True)
+    assert np.array_equal(a, b)
 
 
 # ---------------------------------------------------------------------------
