@@ -86,11 +86,19 @@ def main() -> int:
         cake.fill_uniform(t, seed)
         return t
 
-    def time_steps(launch, steps, warmup):
-        """W warm-ups, then K launches between two synchronisations with an event pair per launch."""
+    def time_steps(launch, steps, warmup, settle_ms=0.0):
+        """W warm-ups, then K launches between two synchronisations with an event pair per launch.
+        settle_ms > 0 keeps launching warm-ups until that much GPU time has passed, so that a
+        sub-millisecond kernel is timed at settled clocks like the long ones are."""
         for _ in range(warmup):
             launch()
         torch.cuda.synchronize()
+        if settle_ms > 0:
+            t_end = time.perf_counter() + settle_ms * 1e-3
+            while time.perf_counter() < t_end:
+                for _ in range(20):
+                    launch()
+                torch.cuda.synchronize()
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -148,7 +156,7 @@ def main() -> int:
             "cus": info.cus,
         },
         "roofline": {
-            "kernel": "sgemm_tile_kernel<256x256x32, wave 128x64>",
+            "kernel": f"sgemm_tile_kernel<Tile<{plan.tile_m},{plan.tile_n},{plan.tile_k},{plan.wave_m},{plan.wave_n}>>",
             "bound": "mfma",
             "achieved": round(achieved, 3),
             "peak": MFMA_PEAK_TFLOPS,
@@ -171,7 +179,7 @@ def main() -> int:
             c = torch.zeros((M, N), dtype=torch.float32, device=dev)
             p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
             _, avg, _ = time_steps(lambda: _lib.check(
-                lib.cake_hip_sgemm(p3[0], p3[1], p3[2], M, N, K, cake.NA, 0, None, stream, None), name), 20, 5)
+                lib.cake_hip_sgemm(p3[0], p3[1], p3[2], M, N, K, cake.NA, 0, None, stream, None), name), 50, 5, 40.0)
             pl = cake.plan(M, N, K)
             fl = 2.0 * M * N * K
             by = 4.0 * (M * K + K * N + M * N)
@@ -190,7 +198,7 @@ def main() -> int:
         gbytes = 4.0 * (m * m + m + m)
         for col, label in ((0, "row-major A (configs[3])"), (1, "column-major A (cake_sgemv's own layout)")):
             _, avg, _ = time_steps(lambda: _lib.check(
-                lib.cake_hip_sgemv(Ag.data_ptr(), xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None), "sgemv"), 50, 10)
+                lib.cake_hip_sgemv(Ag.data_ptr(), xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None), "sgemv"), 50, 10, 40.0)
             extras.append({"workload": f"sgemv 16384x16384 {label}", "us": round(avg * 1e6, 2),
                            "GBps": round(gbytes / avg / 1e9, 1),
                            "roofline": {"bound": "hbm", "achieved": round(gbytes / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
@@ -209,7 +217,7 @@ def main() -> int:
                           (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps)")):
             _, avg, _ = time_steps(lambda: _lib.check(
                 fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 0,
-                   ws.data_ptr(), stream, None), "conv2d"), 10, 3)
+                   ws.data_ptr(), stream, None), "conv2d"), 20, 3, 40.0)
             extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
                            "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
                            "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})

@@ -32,9 +32,13 @@ namespace cake {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_>
+// REG_STAGES: how many K stages wait in registers between their global loads and
+// their LDS stores (the 16-byte loaders only).  2 gives every load a whole extra
+// K step to come back from HBM, for 6-8 more float4 registers per lane.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int REG_STAGES_ = 1>
 struct Tile {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr int REG_STAGES = REG_STAGES_;
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
     static constexpr int THREADS = WAVES_M * WAVES_N * 64;
     static constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 MFMA tiles per wave
@@ -574,27 +578,43 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
                                            int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
 {
     static_assert(Slots<T, L>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
+    constexpr int RS = T::REG_STAGES;
+    static_assert(RS == 1 || RS == 2, "one or two register stages");
     L ld;
     ld.init(g, m0, n0, tid);
-    f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
+    f32x4 ra[RS][T::A_ITERS], rb[RS][T::B_ITERS];
     Frag<T> frag[2];
     if (steps <= 0) return;
-    ld.load(kbeg, kend, ra, rb);
-    store_stage<T>(As, Bs, tid, ra, rb);
-    ld.load(kbeg + T::BK, kend, ra, rb);  // stage 1 waits in registers
+    ld.load(kbeg, kend, ra[0], rb[0]);
+    store_stage<T>(As, Bs, tid, ra[0], rb[0]);
+    // stage j waits in register set j % RS until step j-1 stores it
+    ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
+    if constexpr (RS == 2) ld.load(kbeg + 2 * T::BK, kend, ra[0], rb[0]);
     __syncthreads();
     load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
 
+    // One K step: stores stage s+1 from register set (s+1) % RS, then refills that
+    // set with stage s+1+RS.  Stages past the end are fetched as zeros and parked
+    // in the idle buffer, so the walk has no branch.
     int cur = 0;
-    for (int s = 0; s < steps; ++s) {
-        // stages past the end are fetched as zeros and parked in the idle buffer: no branch in the walk
-        const WalkCtx<T, L> c{ld, kbeg + (s + 2) * T::BK, kend,
-                           As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
-                           As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
-                           tid, a_row, b_col, lh, ra, rb};
+    auto step = [&](int s, f32x4 (&sa)[T::A_ITERS], f32x4 (&sb)[T::B_ITERS]) {
+        const WalkCtx<T, L> c{ld, kbeg + (s + 1 + RS) * T::BK, kend,
+                              As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
+                              As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
+                              tid, a_row, b_col, lh, sa, sb};
         __builtin_amdgcn_sched_barrier(0);
         step_groups<T, L>(c, frag, acc);
         cur ^= 1;
+    };
+    if constexpr (RS == 1) {
+        for (int s = 0; s < steps; ++s) step(s, ra[0], rb[0]);
+    } else {
+        int s = 0;
+        for (; s + 1 < steps; s += 2) {
+            step(s, ra[1], rb[1]);
+            step(s + 1, ra[0], rb[0]);
+        }
+        if (s < steps) step(s, ra[1], rb[1]);
     }
 }
 
@@ -766,9 +786,9 @@ inline hipError_t launch_tile(const GemmArgs& args, int grid, hipStream_t stream
 }
 
 using Tile256x256x32 = Tile<256, 256, 32, 128, 64>;
-using Tile256x128x32 = Tile<256, 128, 32, 64, 64>;
-using Tile128x256x32 = Tile<128, 256, 32, 64, 64>;
-using Tile128x128x32 = Tile<128, 128, 32, 64, 64>;
-using Tile64x64x32 = Tile<64, 64, 32, 32, 32>;
+using Tile256x128x32 = Tile<256, 128, 32, 64, 64, 2>;
+using Tile128x256x32 = Tile<128, 256, 32, 64, 64, 2>;
+using Tile128x128x32 = Tile<128, 128, 32, 64, 64, 2>;
+using Tile64x64x32 = Tile<64, 64, 32, 32, 32, 2>;
 
 }  // namespace cake
