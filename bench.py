@@ -40,7 +40,7 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # this script, each scaled by what the same counter reads for a plain 256 MiB
 # copy (FETCH_SIZE reads half the true size, WRITE_SIZE the true size).  The
 # summaries are kept under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": None}
+MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": (1049023 + 256) * 1024}
 
 
 def main() -> int:
