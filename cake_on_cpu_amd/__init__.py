@@ -1,15 +1,15 @@
 """MI355X-native implementation of CAKE's fp32 GEMM hot path.
 
 Host-side mirror of the reference's interface for this path (cake_sgemm,
-cake_sgemv, init_block_dims, pack_A/pack_B/unpack_C, im_2_col) over the
+cake_sgemv, init_block_dims, pack_A/pack_B/unpack_C, im_2_col, the linear layer) over the
 C-ABI of libcake_hip.so.  PyTorch is not required; torch ROCm tensors and numpy
 arrays are both accepted wherever a matrix is."""
 from ._lib import (KMN, MKN, NKM, NA, SCHED_NAMES, BlkDims, CakeHipError, CpuCntx, DeviceInfo,
                    Plan, load)
 from .api import (cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_size, cake_sgemm_packed_B_size,
                   cake_sgemm_packed_C_size, cake_sgemv, conv2d, device_info, fill_uniform, im2col,
-                  im_2_col, init_block_dims, last_kernel_seconds, pack_A, pack_B, pack_C,
-                  packed_offset, plan, unpack_C, update_mr_nr)
+                  im_2_col, init_block_dims, last_kernel_seconds, linear_backward, linear_forward, pack_A, pack_B, pack_C,
+                  packed_offset, plan, transpose_mat, unpack_C, update_mr_nr)
 
 __all__ = [
     "KMN", "MKN", "NKM", "NA", "SCHED_NAMES", "BlkDims", "CpuCntx", "Plan", "DeviceInfo",
@@ -17,5 +17,5 @@ __all__ = [
     "cake_sgemm", "cake_sgemv", "pack_A", "pack_B", "pack_C", "unpack_C",
     "cake_sgemm_packed_A_size", "cake_sgemm_packed_B_size", "cake_sgemm_packed_C_size",
     "packed_offset", "im2col", "im_2_col", "conv2d", "fill_uniform", "device_info",
-    "last_kernel_seconds",
+    "last_kernel_seconds", "transpose_mat", "linear_forward", "linear_backward",
 ]

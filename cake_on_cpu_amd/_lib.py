@@ -99,11 +99,36 @@ SIGNATURES = {
     "cake_hip_conv2d_workspace": (C.c_size_t, [_i] * 9),
     "cake_hip_conv2d": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
     "cake_hip_conv2d_im2col": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
+    "cake_hip_transpose": (_i, [_fp, _fp, _i, _i, C.c_void_p, _dp]),
+    "cake_hip_linear_forward": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),
+    "cake_hip_linear_backward": (_i, [_fp] * 6 + [_i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_fill_uniform": (_i, [_fp, C.c_size_t, C.c_uint64, C.c_void_p]),
     "cake_hip_last_kernel_seconds": (_i, [C.POINTER(C.c_double * 5)]),
 }
 
 _lib = None
+
+
+def _share_torch_hip_runtime() -> None:
+    """A process can hold one HIP runtime.  PyTorch-ROCm wheels bundle their own
+    libamdhip64.so (soname libamdhip64.so.7) and look it up by file name, so if
+    the system copy is already loaded under its soname torch loads a second
+    runtime, which then finds no GPU.  When such a wheel is installed, load its
+    copy first: libcake_hip.so's libamdhip64.so.7 dependency then resolves to it
+    whichever of the two packages is used first.  torch itself is not imported."""
+    import importlib.util
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return
+    if spec is None or not spec.origin:
+        return
+    bundled = Path(spec.origin).parent / "lib" / "libamdhip64.so"
+    if bundled.exists():
+        try:
+            C.CDLL(str(bundled), mode=C.RTLD_GLOBAL)
+        except OSError:
+            pass  # fall back to the system runtime
 
 
 def load() -> C.CDLL:
@@ -114,6 +139,7 @@ def load() -> C.CDLL:
             raise ImportError(
                 f"{LIB_PATH} is missing: build it with `make -C cake_on_cpu_amd/csrc` "
                 "(or __graft_entry__.build()); there is no CPU fallback")
+        _share_torch_hip_runtime()
         lib = C.CDLL(str(LIB_PATH))
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is not exported

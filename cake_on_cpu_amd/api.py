@@ -296,6 +296,54 @@ def conv2d(inp, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride=1, pad=
 
 
 # ----------------------------------------------------------------------------
+# transpose and the linear layer (include/util.h:32, src/linear.cpp:12-107)
+# ----------------------------------------------------------------------------
+def transpose_mat(A_old, At, K, N, Kt=0, Nt=0) -> float:
+    """At[n][k] = A_old[k][n] for a K x N matrix (src/transpose.cpp:5-29; the
+    blocking arguments Kt, Nt are accepted and unused).  Returns seconds."""
+    _need(A_old, K * N, "A_old")
+    _need(At, K * N, "At")
+    secs = C.c_double(0.0)
+    check(load().cake_hip_transpose(_ptr(A_old, "A_old"), _ptr(At, "At"), K, N, _stream(A_old, At),
+                                    C.byref(secs)), "transpose_mat")
+    return secs.value
+
+
+def _opt_ptr(a, what):
+    return None if a is None else _ptr(a, what)
+
+
+def linear_forward(x, w, bias, y, M, N, K) -> float:
+    """y[M][N] = x[M][K] . w[N][K]^T + bias[N] (bias may be None): linear_forward of
+    src/linear.cpp:12-50.  Returns seconds."""
+    _need(x, M * K, "x")
+    _need(w, N * K, "w")
+    _need(y, M * N, "y")
+    if bias is not None:
+        _need(bias, N, "bias")
+    secs = C.c_double(0.0)
+    check(load().cake_hip_linear_forward(_ptr(x, "x"), _ptr(w, "w"), _opt_ptr(bias, "bias"), _ptr(y, "y"),
+                                         M, N, K, _stream(x, w, y), C.byref(secs)), "linear_forward")
+    return secs.value
+
+
+def linear_backward(grad_y, x, w, grad_x, grad_w, grad_bias, M, N, K) -> float:
+    """grad_x = grad_y . w, grad_w = grad_y^T . x, grad_bias = column sums of grad_y
+    (src/linear.cpp:53-102).  Outputs passed as None are skipped.  Returns seconds."""
+    _need(grad_y, M * N, "grad_y")
+    for a, n, what in ((x, M * K, "x"), (w, N * K, "w"), (grad_x, M * K, "grad_x"),
+                       (grad_w, N * K, "grad_w"), (grad_bias, N, "grad_bias")):
+        if a is not None:
+            _need(a, n, what)
+    secs = C.c_double(0.0)
+    check(load().cake_hip_linear_backward(_ptr(grad_y, "grad_y"), _opt_ptr(x, "x"), _opt_ptr(w, "w"),
+                                          _opt_ptr(grad_x, "grad_x"), _opt_ptr(grad_w, "grad_w"),
+                                          _opt_ptr(grad_bias, "grad_bias"), M, N, K,
+                                          _stream(grad_y, x, w), C.byref(secs)), "linear_backward")
+    return secs.value
+
+
+# ----------------------------------------------------------------------------
 # utilities
 # ----------------------------------------------------------------------------
 def fill_uniform(dst, seed: int) -> None:

@@ -65,7 +65,7 @@ struct DeviceBuffer {
     }
 };
 
-enum { STAGE_SLOTS = 4 };
+enum { STAGE_SLOTS = 6 };
 
 struct Context {
     bool ready = false;
@@ -73,7 +73,7 @@ struct Context {
     cake_hip_device_t info{};
     DeviceModel model;
     DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
-    DeviceBuffer splitk, gemv, conv, tables, unpacked;
+    DeviceBuffer splitk, gemv, conv, tables, unpacked, linear;
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
 };
@@ -227,7 +227,7 @@ size_t tables_bytes(int which, const PackGeom& g)
 int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
              int sched, int accumulate, const int* tile_override, int a_mode, int b_mode,
              IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer,
-             const ConvGeom* conv = nullptr)
+             const ConvGeom* conv = nullptr, const float* col_bias = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
     GemmPlan plan;
@@ -250,6 +250,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.split_k = plan.pub.split_k; g.k_per_split = plan.k_per_split;
     g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
     g.accumulate = accumulate;
+    g.col_bias = col_bias;
     g.a_tab = a_tab; g.b_tab = b_tab;
     if (conv) g.conv = *conv;
     const int nchw_hw = (conv && conv->out_nchw) ? conv->Hout * conv->Wout : 0;
@@ -273,7 +274,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     if (st) return st;
     if (plan.pub.split_k > 1)
         st = timer.family(1, [&] {
-            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream, nchw_hw);
+            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream, nchw_hw,
+                                        col_bias);
         });
     else if (plan.pub.tail_tiles > 0)
         st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); });
@@ -343,7 +345,7 @@ int cake_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     for (DeviceBuffer& b : g_ctx.stage) b.release();
     g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
-    g_ctx.tables.release(); g_ctx.unpacked.release();
+    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release();
     for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1]}) {
         if (*e) (void)hipEventDestroy(*e);
         *e = nullptr;
@@ -802,6 +804,146 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out, in
 {
     return conv2d_common(in, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw,
                          workspace, stream, seconds, 1);
+}
+
+int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    if (rows < 0 || cols < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (rows == 0 || cols == 0) return CAKE_HIP_OK;
+    if (!src || !dst) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (src == dst) return fail(CAKE_HIP_ERR_ARG, "transpose in place is not supported");
+    if (!fits_int((double)rows * cols)) return fail(CAKE_HIP_ERR_RANGE, "matrix of %dx%d exceeds 2^31 elements", rows, cols);
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Operand in, out;
+    const size_t bytes = (size_t)rows * cols * 4;
+    if ((st = stage_in(src, bytes, 0, true, &in))) return st;
+    if ((st = stage_in(dst, bytes, 1, false, &out))) return st;
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    st = timer.family(4, [&] { return launch_transpose(in.dev, out.dev, rows, cols, stream); });
+    if (st) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(out, stream);
+}
+
+static int linear_dims_ok(int M, int N, int K)
+{
+    if (M < 0 || N < 0 || K < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
+    return CAKE_HIP_OK;
+}
+
+// C = A.B on device operands with the planner's choice of everything; K == 0 gives C = bias or 0.
+static int linear_gemm(const float* A, const float* B, float* C, int M, int N, int K, const float* col_bias,
+                       hipStream_t stream, Timer& timer)
+{
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (K == 0) {
+        hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream, 0, col_bias);
+        return e == hipSuccess ? CAKE_HIP_OK : fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
+    }
+    const int mode = vec4_loadable(A, B, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
+    return run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, IndexTables{}, IndexTables{},
+                    stream, timer, nullptr, col_bias);
+}
+
+int cake_hip_linear_forward(const float* x, const float* w, const float* bias, float* y, int M, int N,
+                            int K, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int st = linear_dims_ok(M, N, K);
+    if (st) return st;
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (!y || (K > 0 && (!x || !w))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand xo, wo, bo, yo;
+    if ((st = stage_in(x, (size_t)M * K * 4, 0, true, &xo))) return st;
+    if ((st = stage_in(w, (size_t)N * K * 4, 1, true, &wo))) return st;
+    if (bias && (st = stage_in(bias, (size_t)N * 4, 2, true, &bo))) return st;
+    if ((st = stage_in(y, (size_t)M * N * 4, 3, false, &yo))) return st;
+    // workspace: the weights as a K x N matrix (256-byte aligned so the 16-byte loader applies)
+    if ((st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
+    float* wt = static_cast<float*>(g_ctx.linear.ptr);
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if (K > 0) {
+        st = timer.family(4, [&] { return launch_transpose(wo.dev, wt, N, K, stream); });
+        if (st) return st;
+    }
+    if ((st = linear_gemm(xo.dev, wt, yo.dev, M, N, K, bias ? bo.dev : nullptr, stream, timer))) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(yo, stream);
+}
+
+int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w, float* grad_x,
+                             float* grad_w, float* grad_bias, int M, int N, int K, void* stream_,
+                             double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int st = linear_dims_ok(M, N, K);
+    if (st) return st;
+    if (!grad_y && M > 0 && N > 0) return fail(CAKE_HIP_ERR_ARG, "NULL grad_y");
+    if (grad_x && !w && N > 0) return fail(CAKE_HIP_ERR_ARG, "grad_x needs w");
+    if (grad_w && !x && M > 0) return fail(CAKE_HIP_ERR_ARG, "grad_w needs x");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand go, xo, wo, gxo, gwo, gbo;
+    if ((st = stage_in(grad_y, (size_t)M * N * 4, 0, true, &go))) return st;
+    if (grad_w && (st = stage_in(x, (size_t)M * K * 4, 1, true, &xo))) return st;
+    if (grad_x && (st = stage_in(w, (size_t)N * K * 4, 2, true, &wo))) return st;
+    if (grad_x && (st = stage_in(grad_x, (size_t)M * K * 4, 3, false, &gxo))) return st;
+    if (grad_w && (st = stage_in(grad_w, (size_t)N * K * 4, 4, false, &gwo))) return st;
+    if (grad_bias && (st = stage_in(grad_bias, (size_t)N * 4, 5, false, &gbo))) return st;
+    // workspace: grad_y transposed (N x M), then a vector of M ones, then the GEMV's slice partials
+    const size_t gt_floats = grad_w ? (((size_t)M * N + 63) & ~(size_t)63) : 0;
+    const size_t ones_floats = grad_bias ? (((size_t)M + 63) & ~(size_t)63) : 0;
+    const size_t gemv_floats = grad_bias && M > 0 && N > 0 ? sgemv_colmajor_scratch_floats(N, M, g_ctx.model.cus) : 0;
+    if ((st = g_ctx.linear.reserve((gt_floats + ones_floats + gemv_floats) * 4 + 256))) return st;
+    float* gt = static_cast<float*>(g_ctx.linear.ptr);
+    float* ones = gt + gt_floats;
+    float* gemv_scratch = ones + ones_floats;
+
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if (grad_x)  // grad_x[M][K] = grad_y[M][N] . w[N][K]   (src/linear.cpp:58-72)
+        if ((st = linear_gemm(go.dev, wo.dev, gxo.dev, M, K, N, nullptr, stream, timer))) return st;
+    if (grad_w) {  // grad_w[N][K] = grad_y^T[N][M] . x[M][K]   (src/linear.cpp:74-90)
+        if (M > 0 && N > 0) {
+            st = timer.family(4, [&] { return launch_transpose(go.dev, gt, M, N, stream); });
+            if (st) return st;
+        }
+        if ((st = linear_gemm(gt, xo.dev, gwo.dev, N, K, M, nullptr, stream, timer))) return st;
+    }
+    if (grad_bias && N > 0) {  // column sums of grad_y   (src/linear.cpp:92-93)
+        if (M == 0) {
+            hipError_t e = launch_fill_value(gbo.dev, (size_t)N, 0.f, stream);
+            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
+        } else {
+            // grad_y read as a column-major N x M matrix times a vector of ones
+            st = timer.family(2, [&] {
+                hipError_t e = launch_fill_value(ones, (size_t)M, 1.f, stream);
+                if (e != hipSuccess) return e;
+                return launch_sgemv_colmajor(go.dev, ones, gbo.dev, N, M, 0, gemv_scratch, g_ctx.model.cus, stream);
+            });
+            if (st) return st;
+        }
+    }
+    if ((st = timer.stop())) return st;
+    if (grad_x && (st = stage_out(gxo, stream))) return st;
+    if (grad_w && (st = stage_out(gwo, stream))) return st;
+    if (grad_bias && (st = stage_out(gbo, stream))) return st;
+    return CAKE_HIP_OK;
 }
 
 int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream_)

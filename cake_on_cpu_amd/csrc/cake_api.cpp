@@ -340,6 +340,7 @@ bool mat_equals(float* C, float* C_check, int M, int N)
 bool cake_sgemm_checker(float* A, float* B, float* C, int N, int M, int K)
 {
     float* ref = (float*)calloc((size_t)M * N, sizeof(float));
+#pragma omp parallel for schedule(static)
     for (int m = 0; m < M; ++m)
         for (int k = 0; k < K; ++k) {
             const float a = A[(size_t)m * K + k];
@@ -367,4 +368,89 @@ void print_array(float* arr, int len)
 void print_mat(float* arr, int r, int c)
 {
     for (int i = 0; i < r; ++i) print_array(arr + (size_t)i * c, c);
+}
+
+bool add_checker(float** C_arr, float* C, int M, int N, int p)
+{
+    const float eps = 1e-3f;
+    long bad = 0;
+    for (size_t i = 0; i < (size_t)M * N; ++i) {
+        float sum = 0.f;
+        for (int c = 0; c < p; ++c) sum += C_arr[c][i];
+        if (fabsf(sum - C[i]) > eps) ++bad;
+    }
+    if (!bad) {
+        printf("ADD CORRECT!\n");
+        return 0;
+    }
+    printf("ADD WRONG!\n%ld\n", bad);
+    return 1;
+}
+
+float rand_gen() { return ((float)rand() + 1.f) / ((float)RAND_MAX + 1.f); }
+
+float normalRandom()
+{
+    const float u = rand_gen(), v = rand_gen();
+    return cosf(2.f * 3.14159265358979323846f * v) * sqrtf(-2.f * logf(u));
+}
+
+void transpose_mat(float* A_old, float* At, int K, int N, int Kt, int Nt)
+{
+    (void)Kt; (void)Nt;
+    die_on(cake_hip_transpose(A_old, At, K, N, NULL, NULL), "transpose_mat");
+}
+
+// ---- the reference's self-test over the five entry points ---------------------------
+
+namespace {
+
+typedef double (*sgemm_entry)(float*, float*, float*, int, int, int, int, cake_cntx_t*, char**, bool, bool,
+                              float, float, enum sched, int, int, int);
+
+struct EntryCase {
+    const char* name;
+    sgemm_entry fn;
+    enum sched sch;
+};
+
+}  // namespace
+
+int run_tests()
+{
+    static const int dims[6] = {1, 10, 96, 111, 960, 2111};  // util.cpp:11-13
+    static const EntryCase entries[5] = {
+        {"2d K-first", cake_sgemm_2d, KMN},   {"M-first", cake_sgemm, MKN}, {"online K-first", cake_sgemm_online, KMN},
+        {"K-first", cake_sgemm, KMN},         {"N-first", cake_sgemm, NKM},
+    };
+    cake_cntx_t* cntx = cake_query_cntx();
+    const int ps[2] = {2, cntx->ncores > 2 ? cntx->ncores : 0};
+    int failed = 0;
+    srand((unsigned)time(NULL));
+    for (int pi = 0; pi < 2; ++pi) {
+        const int p = ps[pi];
+        if (p == 0) continue;
+        for (int mi = 0; mi < 6; ++mi)
+            for (int ki = 0; ki < 6; ++ki)
+                for (int ni = 0; ni < 6; ++ni) {
+                    const int M = dims[mi], K = dims[ki], N = dims[ni];
+                    float* A = (float*)malloc(sizeof(float) * (size_t)M * K);
+                    float* B = (float*)malloc(sizeof(float) * (size_t)K * N);
+                    float* C = (float*)malloc(sizeof(float) * (size_t)M * N);
+                    rand_init(A, M, K);
+                    rand_init(B, K, N);
+                    for (const EntryCase& e : entries) {
+                        memset(C, 0, sizeof(float) * (size_t)M * N);
+                        e.fn(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, e.sch, 0, 0, 0);
+                        if (cake_sgemm_checker(A, B, C, N, M, K)) {
+                            printf("TESTS FAILED on %s p=%d M=%d K=%d N=%d\n", e.name, p, M, K, N);
+                            ++failed;
+                        }
+                    }
+                    free(A); free(B); free(C);
+                }
+    }
+    free(cntx);
+    printf(failed ? "FAILED\n" : "ALL TESTS PASSED!\n");
+    return 0;
 }

@@ -43,6 +43,7 @@ struct GemmArgs {
     int split_k, k_per_split;  // k_per_split is a multiple of the tile's BK
     int group, group_along_n;  // CB-block raster
     int accumulate;
+    const float* col_bias;  // added to every row of the finished product (after accumulate), or nullptr
     // Tail splitting: the last `tail_tiles` tiles of the raster (the ones that
     // would run as a thin final round) are cut into `tail_split` K slices each,
     // written to tail_partial[slice][tail tile][BM x BN] and summed by
@@ -81,7 +82,8 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
 // nchw_hw != 0: C is a convolution output written as [N / nchw_hw][M][nchw_hw]
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream, int nchw_hw = 0);
+                                int accumulate, hipStream_t stream, int nchw_hw = 0,
+                                const float* col_bias = nullptr);
 
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, hipStream_t stream);
@@ -98,6 +100,9 @@ hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, 
                              hipStream_t stream);
 
 hipError_t launch_fill_uniform(float* dst, size_t n, uint64_t seed, hipStream_t stream);
+hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stream);
+// dst[c][r] = src[r][c], src rows x cols row-major; rows <= 64 * 65535
+hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t stream);
 
 // Packed layouts.  which: 0 = A, 1 = B, 2 = C.
 hipError_t launch_build_index_tables(int which, const PackGeom& g, int4* row_tab, int4* col_tab,

@@ -1,4 +1,4 @@
-// misc_kernels.hip -- im2col, layout change, seeded fill, and the reference's
+// misc_kernels.hip -- transpose, im2col, layout change, fills, and the reference's
 // packed layouts (index tables, pack, unpack).  All HBM-bound copies: one
 // thread per output element (or per 4), coalesced along the fastest dimension
 // of whichever side is written.
@@ -9,6 +9,55 @@
 namespace cake {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------
+// transpose: dst[c][r] = src[r][c] for a rows x cols row-major matrix
+// (transpose_mat of src/transpose.cpp:5-29).  64x64 tiles through LDS so both
+// the read and the write run along the contiguous dimension; the +1 padding
+// keeps the transposed LDS reads conflict-free.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) transpose_kernel(const float* __restrict__ src,
+                                                        float* __restrict__ dst, int rows, int cols)
+{
+    __shared__ float tile[64][65];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + ty + 4 * i, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + 4 * i][tx] = src[(size_t)r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int c = c0 + ty + 4 * i, r = r0 + tx;
+        if (r < rows && c < cols) dst[(size_t)c * rows + r] = tile[tx][ty + 4 * i];
+    }
+}
+
+hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    const unsigned gx = (cols + 63) / 64, gy = (rows + 63) / 64;
+    if (gy > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(transpose_kernel, dim3(gx, gy), dim3(256), 0, stream, src, dst, rows, cols);
+    return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) fill_value_kernel(float* __restrict__ dst, size_t n, float v)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = v;
+}
+
+hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stream)
+{
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(fill_value_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dst, n, value);
+    return hipGetLastError();
+}
 
 // ---------------------------------------------------------------------------
 // im2col: im_2_col of examples/cake_conv.cpp:1178-1213 with batch, padding and

@@ -63,7 +63,8 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial,
                                                             float* __restrict__ C, int M, int N,
                                                             int ldc, int splits, int accumulate,
-                                                            int nchw_hw)
+                                                            int nchw_hw,
+                                                            const float* __restrict__ col_bias)
 {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -76,19 +77,20 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
         }
         float acc = accumulate ? *dst : 0.f;
         for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * total + i];
+        if (col_bias) acc += col_bias[col];
         *dst = acc;
     }
 }
 
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream, int nchw_hw)
+                                int accumulate, hipStream_t stream, int nchw_hw, const float* col_bias)
 {
     const size_t total = (size_t)M * N;
     if (total == 0) return hipSuccess;
     size_t blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
-                       M, N, ldc, splits, accumulate, nchw_hw);
+                       M, N, ldc, splits, accumulate, nchw_hw, col_bias);
     return hipGetLastError();
 }
 

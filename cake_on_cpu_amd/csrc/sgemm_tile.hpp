@@ -710,6 +710,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     float* out = g.partial ? g.partial + (size_t)w.slice * g.M * g.N : g.C;
     const int ldo = g.partial ? g.N : g.ldc;
     const bool add = (g.partial == nullptr) && g.accumulate;
+    const float* bias = g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
     const bool nchw = (B_MODE == LOAD_IM2COL) && g.conv.out_nchw && g.partial == nullptr;
     const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
@@ -725,12 +726,15 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
                 col_off = (size_t)b * g.M * HW + (col - b * HW);
                 row_stride = HW;
             }
+            const float bias_v = (bias && col < g.N) ? bias[col] : 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
                 if (row < g.M && col < g.N) {
                     float* dst = out + (size_t)row * row_stride + col_off;
-                    *dst = add ? *dst + acc[tm][tn][r] : acc[tm][tn][r];
+                    float v = add ? *dst + acc[tm][tn][r] : acc[tm][tn][r];
+                    if (bias) v += bias_v;
+                    *dst = v;
                 }
             }
         }
@@ -767,7 +771,7 @@ __global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmArgs g)
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-        if (col + q < g.N) dst[q] = acc[q];
+        if (col + q < g.N) dst[q] = g.col_bias ? acc[q] + g.col_bias[col + q] : acc[q];
 }
 
 template <class T, int A_MODE, int B_MODE>

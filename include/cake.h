@@ -123,6 +123,18 @@ float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
 void rand_init(float* mat, int r, int c);                          // util.cpp:259
 bool cake_sgemm_checker(float* A, float* B, float* C, int N, int M, int K);  // util.cpp:173
 bool mat_equals(float* C, float* C_check, int M, int N);           // util.cpp:139
+bool add_checker(float** C_arr, float* C, int M, int N, int p);     // util.cpp:205
 void print_schedule(enum sched sch);
 void print_mat(float* arr, int r, int c);
 void print_array(float* arr, int len);
+float rand_gen();                                                  // util.cpp:251, uniform (0,1]
+float normalRandom();                                              // util.cpp:270, N(0,1) by Box-Muller
+// At[n][k] = A_old[k][n] for a K x N matrix, on the GPU; Kt, Nt (host blocking) are unused.
+void transpose_mat(float* A_old, float* At, int K, int N, int Kt, int Nt);  // transpose.cpp:5
+// The reference's self-test (util.cpp:3-136): every M, K, N in {1,10,96,111,960,2111}
+// through cake_sgemm_2d, cake_sgemm MKN, cake_sgemm_online, cake_sgemm KMN and
+// cake_sgemm NKM, each checked against a host loop.  p has no effect on the
+// device, so the sweep runs p = 2 and p = ncores (the two ends of the reference's
+// range) instead of every value between.  Prints "ALL TESTS PASSED!" or "FAILED";
+// returns 0 like the reference.
+int run_tests();

@@ -217,6 +217,30 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
                            int stride, int pad, int out_nchw, void* workspace,
                            void* stream, double* seconds);
 
+/* ---- transpose and the linear layer ---------------------------------------- */
+/* dst[c][r] = src[r][c] for a rows x cols row-major matrix; dst is cols x rows.
+ * Replaces transpose_mat (include/util.h:32, src/transpose.cpp:5-29; its blocking
+ * arguments Kt, Nt have no meaning here).  src and dst must not overlap. */
+int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* stream,
+                       double* seconds);
+
+/* y[M][N] = x[M][K] . w[N][K]^T (+ bias[N] on every row when bias != NULL).
+ * Replaces linear_forward (src/linear.cpp:12-50), which transposes the weights
+ * into a K x N matrix, calls cake_sgemm and adds the bias afterwards; here the
+ * transpose is a device kernel into a library workspace and the bias is added
+ * by the product's epilogue (same rounding: fl(fl(sum) + bias)). */
+int cake_hip_linear_forward(const float* x, const float* w, const float* bias, float* y, int M,
+                            int N, int K, void* stream, double* seconds);
+
+/* Gradients of the layer above for grad_y[M][N] (src/linear.cpp:53-102):
+ *   grad_x[M][K] = grad_y . w,   grad_w[N][K] = grad_y^T . x,
+ *   grad_bias[N] = column sums of grad_y (summed in a fixed order).
+ * Any of the three outputs may be NULL and is then skipped (x may be NULL when
+ * grad_w is, w when grad_x is). */
+int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w, float* grad_x,
+                             float* grad_w, float* grad_bias, int M, int N, int K, void* stream,
+                             double* seconds);
+
 /* ---- seeded inputs -------------------------------------------------------- */
 /* dst[i] = uniform[-1,1) value i of the counter-based splitmix64 stream `seed`
  * (24 random bits, exact in fp32).  Stands in for rand_init (src/util.cpp:259-267),
@@ -225,7 +249,7 @@ int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream);
 
 /* Average duration in seconds of the kernels of the last compute call on this
  * thread, per kernel family: [0] GEMM macro-tile, [1] split-K reduce,
- * [2] GEMV, [3] im2col, [4] pack/unpack.  Zero where none ran. */
+ * [2] GEMV, [3] im2col, [4] pack/unpack/transpose.  Zero where none ran. */
 int cake_hip_last_kernel_seconds(double out[5]);
 
 #ifdef __cplusplus

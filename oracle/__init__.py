@@ -2,7 +2,8 @@
 
 ctypes bindings over ``oracle/cake_oracle.c`` (a from-scratch C restatement of
 the reference algorithm: planner -> pack -> K/M/N-first snake schedule ->
-6x16 outer-product micro-kernel -> unpack, plus cake_sgemv and im_2_col) and
+6x16 outer-product micro-kernel -> unpack, plus cake_sgemv, im_2_col and the
+linear layer that calls cake_sgemm) and
 over the fp64 closed-form checkers that live in the same file.
 
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
@@ -247,6 +248,30 @@ def im_2_col(inp_chw, Hf, Wf, Hout, Wout) -> np.ndarray:
     out = np.empty((Cin * Hf * Wf, Hout * Wout), dtype=np.float32)
     lib().orc_im_2_col(_f(inp_chw), _f(out), Wf, Hf, Win, Hin, Wout, Hout, Cin)
     return out
+
+
+# ----------------------------------------------------------------------------
+# the linear layer of src/linear.cpp (caller of cake_sgemm; p = 10 there)
+# ----------------------------------------------------------------------------
+def linear_forward(x, w, bias=None, p=10, cx=None) -> np.ndarray:
+    """src/linear.cpp:12-50: weight.t() made contiguous (K x N), cake_sgemm with
+    default arguments, then the bias added to every row."""
+    wt = np.ascontiguousarray(w.T)
+    out = cake_sgemm(np.ascontiguousarray(x), wt, p, cx)
+    if bias is not None:
+        out = out + bias.astype(np.float32)[None, :]
+    return out
+
+
+def linear_backward(grad_y, x, w, bias=None, p=10, cx=None):
+    """src/linear.cpp:53-102: grad_input = cake_sgemm(grad_output, weight),
+    grad_weight = cake_sgemm(grad_output.t() contiguous, input), grad_bias =
+    grad_output.sum(0).  The bias sum is returned in fp64 (torch's summation order
+    is its own; callers compare within the bound any fp32 order meets)."""
+    gx = cake_sgemm(np.ascontiguousarray(grad_y), np.ascontiguousarray(w), p, cx)
+    gw = cake_sgemm(np.ascontiguousarray(grad_y.T), np.ascontiguousarray(x), p, cx)
+    gb = None if bias is None else grad_y.astype(np.float64).sum(axis=0)
+    return gx, gw, gb
 
 
 # ----------------------------------------------------------------------------

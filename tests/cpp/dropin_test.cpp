@@ -146,8 +146,25 @@ static void gemv_case(cake_cntx_t* cntx, int M, int K)
     free(A); free(x); free(y);
 }
 
-int main()
+static void transpose_case(int K, int N)
 {
+    float* A = (float*)malloc(sizeof(float) * K * N);
+    float* At = (float*)malloc(sizeof(float) * K * N);
+    rand_init(A, K, N);
+    transpose_mat(A, At, K, N, 8, 8);
+    bool ok = true;
+    for (int k = 0; k < K && ok; ++k)
+        for (int n = 0; n < N; ++n)
+            if (At[(size_t)n * K + k] != A[(size_t)k * N + n]) ok = false;
+    char what[64];
+    snprintf(what, sizeof what, "transpose_mat K=%d N=%d", K, N);
+    report(what, ok);
+    free(A); free(At);
+}
+
+int main(int argc, char** argv)
+{
+    if (argc > 1 && strcmp(argv[1], "run_tests") == 0) return run_tests();  // the reference's own sweep
     srand(1);
     cake_cntx_t* cntx = cake_query_cntx();
     printf("cntx: mr=%d nr=%d L2=%d L3=%d ncores=%d\n", cntx->mr, cntx->nr, cntx->L2, cntx->L3, cntx->ncores);
@@ -163,6 +180,8 @@ int main()
     conv_case(cntx);
     gemv_case(cntx, 1024, 777);
     gemv_case(cntx, 37, 5);
+    transpose_case(130, 77);
+    transpose_case(1, 1000);
 
     blk_dims_t x;
     init_block_dims(8192, 8192, 8192, 8, &x, cntx, NA, NULL);

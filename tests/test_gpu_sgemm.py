@@ -83,21 +83,28 @@ def test_every_tile_shape(tile, shape):
         _check(A, B, Cm, None, (tile, shape, split))
 
 
-@pytest.mark.parametrize("shape", [(1100, 520, 1100), (1100, 517, 1101), (2111, 2111, 2111), (4352, 256, 4096)],
-                         ids=lambda s: "x".join(map(str, s)))
-def test_tail_split_shapes(shape):
+TAIL_CASES = [  # (shape M,K,N; tile) -- tile count = a whole number of rounds plus a thin last one
+    ((1100, 520, 1100), (64, 64, 32)), ((1100, 517, 1101), (64, 64, 32)),
+    ((2111, 2111, 2111), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
+    ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)),
+]
+
+
+@pytest.mark.parametrize("case", TAIL_CASES, ids=lambda c: "x".join(map(str, c[0])) + "_t" + "x".join(map(str, c[1][:2])))
+def test_tail_split_shapes(case):
     """Shapes whose tile count leaves a thin last round: the planner cuts those
     tiles along K and a second kernel sums the slices in order."""
-    M, K, N = shape
-    pl = cake.plan(M, N, K)
+    (M, K, N), tile = case
+    tile = tile + (0,)
+    pl = cake.plan(M, N, K, cake.NA, tile)
     assert pl.tail_tiles > 0 and pl.tail_split > 1, pl.as_dict()
     print(f"sgemm tail M={M} K={K} N={N} plan={pl.as_dict()}", flush=True)
-    A, B, Cm = _run(M, K, N)
-    _check(A, B, Cm, None, shape)
+    A, B, Cm = _run(M, K, N, tile=tile)
+    _check(A, B, Cm, None, case)
     C0 = oracle.uniform((M, N), 3)
-    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    _, _, acc = _run(M, K, N, cake.MKN, tile=tile, C0=C0, beta=1.0)
     assert np.allclose(acc - Cm, C0, atol=2e-4)
-    again = _run(M, K, N)[2]
+    again = _run(M, K, N, tile=tile)[2]
     assert np.array_equal(again, Cm)
 
 
