@@ -221,6 +221,28 @@ def main() -> int:
             extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
                            "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
                            "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        del inp, oc, ws
+
+        # the linear layer (src/linear.cpp): batch 8192, 4096 -> 4096 features, with bias
+        Lm, Lk, Ln = 8192, 4096, 4096
+        lx, lw, lb = dev_uniform((Lm, Lk), 11), dev_uniform((Ln, Lk), 12), dev_uniform((Ln,), 13)
+        lg = dev_uniform((Lm, Ln), 14)
+        ly = torch.empty((Lm, Ln), dtype=torch.float32, device=dev)
+        lgx, lgw = torch.empty_like(lx), torch.empty_like(lw)
+        lgb = torch.empty_like(lb)
+        lfl = 2.0 * Lm * Ln * Lk
+        _, avg, _ = time_steps(lambda: _lib.check(
+            lib.cake_hip_linear_forward(lx.data_ptr(), lw.data_ptr(), lb.data_ptr(), ly.data_ptr(), Lm, Ln, Lk,
+                                        stream, None), "linear_forward"), 20, 3, 40.0)
+        extras.append({"workload": "linear forward, batch 8192, 4096->4096, bias (weight transpose + product)",
+                       "ms": round(avg * 1e3, 4), "tflops": round(lfl / avg / 1e12, 2),
+                       "frac_mfma_peak": round(lfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        _, avg, _ = time_steps(lambda: _lib.check(
+            lib.cake_hip_linear_backward(lg.data_ptr(), lx.data_ptr(), lw.data_ptr(), lgx.data_ptr(), lgw.data_ptr(),
+                                         lgb.data_ptr(), Lm, Ln, Lk, stream, None), "linear_backward"), 20, 3, 40.0)
+        extras.append({"workload": "linear backward, same layer (two products, one transpose, bias sums)",
+                       "ms": round(avg * 1e3, 4), "tflops": round(2 * lfl / avg / 1e12, 2),
+                       "frac_mfma_peak": round(2 * lfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
         out["extras"] = extras
 
     # -------------------------------------------------------------- CPU baseline
