@@ -6,10 +6,11 @@ C-ABI of libcake_hip.so.  PyTorch is not required; torch ROCm tensors and numpy
 arrays are both accepted wherever a matrix is."""
 from ._lib import (KMN, MKN, NKM, NA, SCHED_NAMES, BlkDims, CakeHipError, CpuCntx, DeviceInfo,
                    Plan, load)
-from .api import (cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_size, cake_sgemm_packed_B_size,
+from .api import (autotune, cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_size, cake_sgemm_packed_B_size,
                   cake_sgemm_packed_C_size, cake_sgemv, conv2d, device_info, fill_uniform, im2col,
                   im_2_col, init_block_dims, last_kernel_seconds, linear_backward, linear_forward, pack_A, pack_B, pack_C,
-                  packed_offset, plan, transpose_mat, unpack_C, update_mr_nr)
+                  packed_offset, plan, transpose_mat, tune_clear, tune_count, tune_load, tune_save, unpack_C,
+                  update_mr_nr)
 
 __all__ = [
     "KMN", "MKN", "NKM", "NA", "SCHED_NAMES", "BlkDims", "CpuCntx", "Plan", "DeviceInfo",
@@ -18,4 +19,5 @@ __all__ = [
     "cake_sgemm_packed_A_size", "cake_sgemm_packed_B_size", "cake_sgemm_packed_C_size",
     "packed_offset", "im2col", "im_2_col", "conv2d", "fill_uniform", "device_info",
     "last_kernel_seconds", "transpose_mat", "linear_forward", "linear_backward",
+    "autotune", "tune_save", "tune_load", "tune_clear", "tune_count",
 ]

@@ -102,6 +102,11 @@ SIGNATURES = {
     "cake_hip_transpose": (_i, [_fp, _fp, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_forward": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_backward": (_i, [_fp] * 6 + [_i, _i, _i, C.c_void_p, _dp]),
+    "cake_hip_autotune": (_i, [_i, _i, _i, C.c_double, C.POINTER(Plan), _dp, _dp]),
+    "cake_hip_tune_save": (_i, [C.c_char_p]),
+    "cake_hip_tune_load": (_i, [C.c_char_p, C.POINTER(_i)]),
+    "cake_hip_tune_clear": (_i, []),
+    "cake_hip_tune_count": (_i, []),
     "cake_hip_fill_uniform": (_i, [_fp, C.c_size_t, C.c_uint64, C.c_void_p]),
     "cake_hip_last_kernel_seconds": (_i, [C.POINTER(C.c_double * 5)]),
 }

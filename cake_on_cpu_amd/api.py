@@ -344,6 +344,37 @@ def linear_backward(grad_y, x, w, grad_x, grad_w, grad_bias, M, N, K) -> float:
 
 
 # ----------------------------------------------------------------------------
+# autotuner (successor of mcu,kcu,ncu + src/autotune_sa.cpp)
+# ----------------------------------------------------------------------------
+def autotune(M, N, K, budget_seconds=2.0):
+    """Measure the macro-tile / split-K candidates for an M x N x K product and keep the
+    fastest for later calls.  Returns (plan, best_seconds, default_seconds)."""
+    out = Plan()
+    best, base = C.c_double(0.0), C.c_double(0.0)
+    check(load().cake_hip_autotune(M, N, K, float(budget_seconds), C.byref(out), C.byref(best), C.byref(base)),
+          "autotune")
+    return out, best.value, base.value
+
+
+def tune_save(path) -> None:
+    check(load().cake_hip_tune_save(os.fsencode(path)), "tune_save")
+
+
+def tune_load(path) -> int:
+    n = C.c_int(0)
+    check(load().cake_hip_tune_load(os.fsencode(path), C.byref(n)), "tune_load")
+    return n.value
+
+
+def tune_clear() -> None:
+    check(load().cake_hip_tune_clear(), "tune_clear")
+
+
+def tune_count() -> int:
+    return load().cake_hip_tune_count()
+
+
+# ----------------------------------------------------------------------------
 # utilities
 # ----------------------------------------------------------------------------
 def fill_uniform(dst, seed: int) -> None:

@@ -4,7 +4,9 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <chrono>
 #include <mutex>
 #include <string>
 
@@ -227,11 +229,13 @@ size_t tables_bytes(int which, const PackGeom& g)
 int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
              int sched, int accumulate, const int* tile_override, int a_mode, int b_mode,
              IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer,
-             const ConvGeom* conv = nullptr, const float* col_bias = nullptr)
+             const ConvGeom* conv = nullptr, const float* col_bias = nullptr,
+             const TunedChoice* choice = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
     GemmPlan plan;
-    int st = plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);
+    int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec, g_ctx.model, &plan)
+                    : plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);
     if (st) return fail(st, "no tile matches the requested override");
     if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
         // packed loaders exist for a subset of the tiles
@@ -334,6 +338,7 @@ int cake_hip_init(int device)
     if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
     for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
         if (!*e) HIP_TRY(hipEventCreate(e));
+    if (const char* tuned = std::getenv("CAKE_HIP_TUNE_FILE")) (void)tune_load(tuned);  // optional
     c.ready = true;
     return CAKE_HIP_OK;
 }
@@ -945,6 +950,134 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
     if (grad_bias && (st = stage_out(gbo, stream))) return st;
     return CAKE_HIP_OK;
 }
+
+// ---- autotuner -----------------------------------------------------------------------
+
+int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_t* best_plan,
+                      double* best_seconds, double* default_seconds)
+{
+    if (best_seconds) *best_seconds = 0;
+    if (default_seconds) *default_seconds = 0;
+    if (M <= 0 || N <= 0 || K <= 0) return fail(CAKE_HIP_ERR_ARG, "autotune needs a non-empty product");
+    if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
+    if (!(budget_seconds > 0)) budget_seconds = 2.0;
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = nullptr;
+
+    // synthetic operands in the staging slots (what a host caller's operands would use)
+    if ((st = g_ctx.stage[0].reserve((size_t)M * K * 4))) return st;
+    if ((st = g_ctx.stage[1].reserve((size_t)K * N * 4))) return st;
+    if ((st = g_ctx.stage[2].reserve((size_t)M * N * 4))) return st;
+    float* A = static_cast<float*>(g_ctx.stage[0].ptr);
+    float* B = static_cast<float*>(g_ctx.stage[1].ptr);
+    float* C = static_cast<float*>(g_ctx.stage[2].ptr);
+    HIP_TRY(launch_fill_uniform(A, (size_t)M * K, 1, stream));
+    HIP_TRY(launch_fill_uniform(B, (size_t)K * N, 2, stream));
+    const bool vec = vec4_loadable(A, B, K, N);
+    const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
+
+    // time one explicit choice: a warm-up launch, then the average of a few back-to-back launches
+    auto measure = [&](const TunedChoice& c, double* secs) -> int {
+        Timer untimed(stream, nullptr);
+        double est = 0;
+        for (int pass = 0; pass < 2; ++pass) {
+            const int reps = pass == 0 ? 1 : (est < 2e-4 ? 20 : est < 5e-3 ? 5 : 2);
+            HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
+            for (int r = 0; r < reps; ++r) {
+                int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, IndexTables{},
+                                 IndexTables{}, stream, untimed, nullptr, nullptr, &c);
+                if (e) return e;
+            }
+            HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));
+            HIP_TRY(hipEventSynchronize(g_ctx.ev[1]));
+            float ms = 0;
+            HIP_TRY(hipEventElapsedTime(&ms, g_ctx.ev[0], g_ctx.ev[1]));
+            est = ms * 1e-3 / reps;
+        }
+        *secs = est;
+        return CAKE_HIP_OK;
+    };
+
+    // the model's own choice first: it is the baseline and the fallback
+    GemmPlan model_plan;
+    {
+        const int any[4] = {0, 0, 0, 0};
+        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, any, vec, g_ctx.model, &model_plan))) return st;
+    }
+    TunedChoice best{model_plan.tile_id, model_plan.pub.split_k, 1, 0.0};
+    if ((st = measure(best, &best.seconds))) return st;
+    if (default_seconds) *default_seconds = best.seconds;
+
+    const auto t0 = std::chrono::steady_clock::now();
+    auto spent = [&] { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count(); };
+    bool out_of_time = false;
+    for (int id = 0; id < TILE_COUNT && !out_of_time; ++id) {
+        const TileInfo& t = tile_info(id);
+        if (t.lds_bytes > g_ctx.model.lds_per_cu) continue;
+        const int max_split = std::max(1, K / (4 * t.bk));
+        for (int split = 1; split <= max_split && split <= 32; split *= 2) {
+            for (int tail = (split == 1 ? 1 : 0); tail >= 0; --tail) {
+                if (id == model_plan.tile_id && split == model_plan.pub.split_k && (tail == 1 || split > 1))
+                    continue;  // the baseline itself
+                if (spent() > budget_seconds) { out_of_time = true; break; }
+                TunedChoice c{id, split, tail, 0.0};
+                if (tail) {  // only a distinct candidate when the tile count leaves a thin round
+                    GemmPlan probe;
+                    if (plan_gemm_choice(M, N, K, CAKE_HIP_NA, c, vec, g_ctx.model, &probe) || probe.pub.tail_tiles == 0)
+                        continue;
+                }
+                // skip candidates the model already puts far behind: a split whose slices alone outweigh the product
+                if ((double)split * M * N * 4.0 > 64.0 * ((double)M * K + (double)K * N) * 4.0 && split > 1) continue;
+                double secs = 0;
+                if ((st = measure(c, &secs))) return st;
+                c.seconds = secs;
+                if (secs < best.seconds) best = c;
+            }
+            if (out_of_time) break;
+        }
+    }
+    tune_store(M, N, K, vec, best);
+    if (vec) {
+        // the same tile serves callers whose operands are not 16-byte loadable, unless measured separately
+        TunedChoice other;
+        if (!tune_lookup(M, N, K, false, &other)) tune_store(M, N, K, false, best);
+    }
+    if (best_seconds) *best_seconds = best.seconds;
+    if (best_plan) {
+        GemmPlan plan;
+        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
+        *best_plan = plan.pub;
+    }
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_tune_save(const char* path)
+{
+    if (!path) return fail(CAKE_HIP_ERR_ARG, "path is NULL");
+    const int st = tune_save(path);
+    return st ? fail(st, "cannot write %s", path) : CAKE_HIP_OK;
+}
+
+int cake_hip_tune_load(const char* path, int* entries)
+{
+    if (entries) *entries = 0;
+    if (!path) return fail(CAKE_HIP_ERR_ARG, "path is NULL");
+    const int n = tune_load(path);
+    if (n < 0) return fail(CAKE_HIP_ERR_ARG, "cannot read %s", path);
+    if (entries) *entries = n;
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_tune_clear(void)
+{
+    tune_clear();
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_tune_count(void) { return tune_count(); }
 
 int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream_)
 {

@@ -3,7 +3,11 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
 
 #include "kernels.hpp"
 
@@ -73,6 +77,106 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
 
 }  // namespace
 
+// ---- measured choices ------------------------------------------------------------
+namespace {
+
+struct TuneKey {
+    int M, N, K, vec;
+    bool operator<(const TuneKey& o) const
+    {
+        return std::tie(M, N, K, vec) < std::tie(o.M, o.N, o.K, o.vec);
+    }
+};
+
+std::map<TuneKey, TunedChoice> g_tuned;
+std::mutex g_tuned_mutex;
+
+}  // namespace
+
+bool tune_lookup(int M, int N, int K, bool vector_ok, TunedChoice* out)
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    auto it = g_tuned.find(TuneKey{M, N, K, vector_ok ? 1 : 0});
+    if (it == g_tuned.end()) return false;
+    if (out) *out = it->second;
+    return true;
+}
+
+void tune_store(int M, int N, int K, bool vector_ok, const TunedChoice& c)
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    g_tuned[TuneKey{M, N, K, vector_ok ? 1 : 0}] = c;
+}
+
+void tune_clear()
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    g_tuned.clear();
+}
+
+int tune_count()
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    return (int)g_tuned.size();
+}
+
+// One line per entry: M N K vec tile_m tile_n tile_k split_k tail_ok seconds
+int tune_save(const char* path)
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    FILE* f = std::fopen(path, "w");
+    if (!f) return CAKE_HIP_ERR_ARG;
+    std::fprintf(f, "# cake_hip tuned macro-tiles: M N K vec tile_m tile_n tile_k split_k tail_ok seconds\n");
+    for (const auto& kv : g_tuned) {
+        const TileInfo& t = tile_info(kv.second.tile_id);
+        std::fprintf(f, "%d %d %d %d %d %d %d %d %d %.9g\n", kv.first.M, kv.first.N, kv.first.K, kv.first.vec,
+                     t.bm, t.bn, t.bk, kv.second.split_k, kv.second.tail_ok, kv.second.seconds);
+    }
+    return std::fclose(f) == 0 ? CAKE_HIP_OK : CAKE_HIP_ERR_ARG;
+}
+
+// Entries naming a tile this build does not have, or malformed lines, are skipped.
+// Returns the number of entries taken, or -1 when the file cannot be read.
+int tune_load(const char* path)
+{
+    FILE* f = std::fopen(path, "r");
+    if (!f) return -1;
+    char line[256];
+    int taken = 0;
+    while (std::fgets(line, sizeof line, f)) {
+        if (line[0] == '#') continue;
+        int M, N, K, vec, bm, bn, bk, split, tail;
+        double secs;
+        if (std::sscanf(line, "%d %d %d %d %d %d %d %d %d %lf", &M, &N, &K, &vec, &bm, &bn, &bk, &split, &tail,
+                        &secs) != 10)
+            continue;
+        if (M <= 0 || N <= 0 || K <= 0 || split < 1 || split > ceil_div(K, bk > 0 ? bk : 1)) continue;
+        int id = -1;
+        for (int i = 0; i < TILE_COUNT; ++i) {
+            const TileInfo& t = tile_info(i);
+            if (t.bm == bm && t.bn == bn && t.bk == bk) id = i;
+        }
+        if (id < 0) continue;
+        tune_store(M, N, K, vec != 0, TunedChoice{id, split, tail != 0, secs});
+        ++taken;
+    }
+    std::fclose(f);
+    return taken;
+}
+
+static int finish_plan(int M, int N, int K, int sched, int tile_id, int split, bool tail_allowed,
+                       bool vector_ok, const DeviceModel& dev, GemmPlan* out);
+
+int plan_gemm_choice(int M, int N, int K, int sched, const TunedChoice& c, bool vector_ok,
+                     const DeviceModel& dev, GemmPlan* out)
+{
+    if (!out || M <= 0 || N <= 0 || K <= 0 || sched < 0 || sched > CAKE_HIP_NA) return CAKE_HIP_ERR_ARG;
+    if (c.tile_id < 0 || c.tile_id >= TILE_COUNT || c.split_k < 1) return CAKE_HIP_ERR_ARG;
+    if (tile_info(c.tile_id).lds_bytes > dev.lds_per_cu) return CAKE_HIP_ERR_ARG;
+    std::memset(out, 0, sizeof *out);
+    return finish_plan(M, N, K, sched, c.tile_id, c.split_k, c.tail_ok != 0, vector_ok, dev, out);
+}
+
 int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, const DeviceModel& dev,
               GemmPlan* out)
 {
@@ -82,6 +186,11 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
     int want_m = ov ? ov[0] : 0, want_n = ov ? ov[1] : 0, want_k = ov ? ov[2] : 0;
     int want_split = ov ? ov[3] : 0;
     if (want_m < 0 || want_n < 0 || want_k < 0 || want_split < 0) return CAKE_HIP_ERR_ARG;
+
+    // a measured choice for exactly this product wins over the model
+    TunedChoice tuned;
+    if (!ov && tune_lookup(M, N, K, vector_ok, &tuned) && tile_info(tuned.tile_id).lds_bytes <= dev.lds_per_cu)
+        return finish_plan(M, N, K, sched, tuned.tile_id, tuned.split_k, tuned.tail_ok != 0, vector_ok, dev, out);
 
     Candidate best = {-1, 1, 1e30};
     for (int id = 0; id < TILE_COUNT; ++id) {
@@ -103,7 +212,14 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
         }
     }
     if (best.tile_id < 0) return CAKE_HIP_ERR_ARG;  // no tile matches the override
+    const bool tail_allowed = !(ov && ov[3]);  // an explicit split request is taken literally
+    return finish_plan(M, N, K, sched, best.tile_id, best.split, tail_allowed, vector_ok, dev, out);
+}
 
+static int finish_plan(int M, int N, int K, int sched, int tile_id, int split, bool tail_allowed,
+                       bool vector_ok, const DeviceModel& dev, GemmPlan* out)
+{
+    const Candidate best = {tile_id, split, 0.0};
     const TileInfo& t = tile_info(best.tile_id);
     cake_hip_plan_t& p = out->pub;
     out->tile_id = best.tile_id;
@@ -122,7 +238,6 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
     p.tail_split = 1;
     out->tail_k_per_split = 0;
     const int tiles = p.tiles_m * p.tiles_n;
-    const bool tail_allowed = !(ov && ov[3]);  // an explicit split request is taken literally
     if (p.split_k == 1 && tiles > dev.cus && tail_allowed) {
         const int ksteps = ceil_div(K, t.bk);
         const int ts = tail_split_for(tiles % dev.cus, ksteps, dev);

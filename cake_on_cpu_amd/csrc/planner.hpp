@@ -36,4 +36,26 @@ struct GemmPlan {
 int plan_gemm(int M, int N, int K, int sched, const int* tile_override, bool vector_ok,
               const DeviceModel& dev, GemmPlan* out);
 
+// A measured choice for one product (the autotuner's result): which macro-tile,
+// how many K slices for every tile, and whether a thin last round may be cut.
+struct TunedChoice {
+    int tile_id;
+    int split_k;
+    int tail_ok;
+    double seconds;  // the measurement that won
+};
+
+// plan for an explicit choice (what the autotuner times)
+int plan_gemm_choice(int M, int N, int K, int sched, const TunedChoice& c, bool vector_ok,
+                     const DeviceModel& dev, GemmPlan* out);
+
+// Table of measured choices keyed by (M, N, K, vector_ok); plan_gemm consults it
+// when the caller gives no override.  Thread-safe.
+bool tune_lookup(int M, int N, int K, bool vector_ok, TunedChoice* out);
+void tune_store(int M, int N, int K, bool vector_ok, const TunedChoice& c);
+void tune_clear();
+int tune_count();
+int tune_save(const char* path);  // CAKE_HIP_* status
+int tune_load(const char* path);  // entries taken, or -1 when unreadable
+
 }  // namespace cake

@@ -35,10 +35,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // REG_STAGES: how many K stages wait in registers between their global loads and
 // their LDS stores (the 16-byte loaders only).  2 gives every load a whole extra
 // K step to come back from HBM, for 6-8 more float4 registers per lane.
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int REG_STAGES_ = 1>
+// STORE_LEAD: how many operand groups (of 8 k) before the step's barrier the
+// register -> LDS stores are issued.  1 puts them in the group that ends at the
+// barrier; 2 gives them a whole group to land first, which matters when a group
+// is only a few MFMAs long and nothing else would cover the wait at the barrier.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int REG_STAGES_ = 1, int STORE_LEAD_ = 1>
 struct Tile {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int REG_STAGES = REG_STAGES_;
+    static constexpr int STORE_LEAD = STORE_LEAD_;
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
     static constexpr int THREADS = WAVES_M * WAVES_N * 64;
     static constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 MFMA tiles per wave
@@ -469,7 +474,8 @@ struct Slots {
     static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
     static constexpr int LOAD_OPS = L::NUM_LOADS;               // global load instructions per stage
     static constexpr int STORE_OPS = T::A_ITERS + T::B_ITERS;   // 16-byte LDS stores per stage
-    static constexpr int STORE_KG = NKG - 2;
+    static constexpr int STORE_KG = NKG - 1 - T::STORE_LEAD;
+    static_assert(STORE_KG >= 0, "stores must follow the previous step's barrier");
     static_assert(NKG >= 3, "the walk needs three operand groups per K step");
     // memory instructions riding in group kg: operand reads, then loads, then stores
     static constexpr int ops(int kg)
@@ -579,7 +585,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
 {
     static_assert(Slots<T, L>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
     constexpr int RS = T::REG_STAGES;
-    static_assert(RS == 1 || RS == 2, "one or two register stages");
+    static_assert(RS == 1 || RS == 2 || RS == 4, "one, two or four register stages");
     L ld;
     ld.init(g, m0, n0, tid);
     f32x4 ra[RS][T::A_ITERS], rb[RS][T::B_ITERS];
@@ -589,7 +595,11 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     store_stage<T>(As, Bs, tid, ra[0], rb[0]);
     // stage j waits in register set j % RS until step j-1 stores it
     ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
-    if constexpr (RS == 2) ld.load(kbeg + 2 * T::BK, kend, ra[0], rb[0]);
+    if constexpr (RS >= 2) ld.load(kbeg + 2 * T::BK, kend, ra[2 % RS], rb[2 % RS]);
+    if constexpr (RS == 4) {
+        ld.load(kbeg + 3 * T::BK, kend, ra[3], rb[3]);
+        ld.load(kbeg + 4 * T::BK, kend, ra[0], rb[0]);
+    }
     __syncthreads();
     load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
 
@@ -608,13 +618,28 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     };
     if constexpr (RS == 1) {
         for (int s = 0; s < steps; ++s) step(s, ra[0], rb[0]);
-    } else {
+    } else if constexpr (RS == 2) {
         int s = 0;
         for (; s + 1 < steps; s += 2) {
             step(s, ra[1], rb[1]);
             step(s + 1, ra[0], rb[0]);
         }
         if (s < steps) step(s, ra[1], rb[1]);
+    } else {
+        int s = 0;
+        for (; s + 3 < steps; s += 4) {
+            step(s, ra[1], rb[1]);
+            step(s + 1, ra[2], rb[2]);
+            step(s + 2, ra[3], rb[3]);
+            step(s + 3, ra[0], rb[0]);
+        }
+        if (s < steps) {
+            step(s, ra[1], rb[1]);
+            if (s + 1 < steps) {
+                step(s + 1, ra[2], rb[2]);
+                if (s + 2 < steps) step(s + 2, ra[3], rb[3]);
+            }
+        }
     }
 }
 
@@ -793,6 +818,6 @@ using Tile256x256x32 = Tile<256, 256, 32, 128, 64>;
 using Tile256x128x32 = Tile<256, 128, 32, 64, 64, 2>;
 using Tile128x256x32 = Tile<128, 256, 32, 64, 64, 2>;
 using Tile128x128x32 = Tile<128, 128, 32, 64, 64, 2>;
-using Tile64x64x32 = Tile<64, 64, 32, 32, 32, 2>;
+using Tile64x64x32 = Tile<64, 64, 32, 32, 32, 2, 2>;
 
 }  // namespace cake

@@ -241,6 +241,30 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
                              float* grad_w, float* grad_bias, int M, int N, int K, void* stream,
                              double* seconds);
 
+/* ---- autotuner --------------------------------------------------------------- */
+/* Times macro-tile x split-K x tail-split candidates for an M x N x K product on
+ * the device (synthetic operands in library memory, default stream) for at most
+ * about budget_seconds (<= 0: 2 s), and records the fastest in a process-wide
+ * table keyed by (M, N, K).  From then on cake_hip_plan / cake_hip_sgemm and the
+ * other products use that choice whenever the caller gives no tile override.
+ * The planner's own choice is always measured first, so the result is never
+ * slower than the default by more than timing noise.  best_plan, best_seconds,
+ * default_seconds may be NULL.
+ * Successor of the reference's user-tile hook and stubbed simulated-annealing
+ * tuner (mcu,kcu,ncu of cake_sgemm, src/block_sizing.cpp:363-368;
+ * src/autotune_sa.cpp:36-81). */
+int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_t* best_plan,
+                      double* best_seconds, double* default_seconds);
+/* The table as a text file, one line per product:
+ *   M N K vec tile_m tile_n tile_k split_k tail_ok seconds
+ * Loading merges into the table (entries for tiles this build lacks are skipped)
+ * and needs no device.  cake_hip_init also loads the file named by the
+ * environment variable CAKE_HIP_TUNE_FILE when it is set and readable. */
+int cake_hip_tune_save(const char* path);
+int cake_hip_tune_load(const char* path, int* entries);
+int cake_hip_tune_clear(void);
+int cake_hip_tune_count(void);
+
 /* ---- seeded inputs -------------------------------------------------------- */
 /* dst[i] = uniform[-1,1) value i of the counter-based splitmix64 stream `seed`
  * (24 random bits, exact in fp32).  Stands in for rand_init (src/util.cpp:259-267),
