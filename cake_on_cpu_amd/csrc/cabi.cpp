@@ -75,7 +75,7 @@ struct Context {
     cake_hip_device_t info{};
     DeviceModel model;
     DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
-    DeviceBuffer splitk, gemv, conv, tables, unpacked, linear;
+    DeviceBuffer splitk, gemv, conv, conv_taps, tables, unpacked, linear;
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
 };
@@ -350,7 +350,7 @@ int cake_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     for (DeviceBuffer& b : g_ctx.stage) b.release();
     g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
-    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release();
+    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.conv_taps.release();
     for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1]}) {
         if (*e) (void)hipEventDestroy(*e);
         *e = nullptr;
@@ -706,12 +706,14 @@ size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
     int Hout, Wout;
     if (batch <= 0 || Cin <= 0 || Cout <= 0 || conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout)) return 0;
     const size_t ncols = (size_t)batch * Hout * Wout;
-    // column matrix + a [Cout][ncols] product when the caller wants NCHW
-    return ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float) + 512;
+    // two-step path: column matrix + a [Cout][ncols] product when the caller wants NCHW;
+    // gather path: a zero-padded copy of the input
+    const size_t two_step = ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float);
+    const size_t padded = (size_t)batch * Cin * (Hin + 2 * pad) * (Win + 2 * pad) * sizeof(float);
+    return (two_step > padded ? two_step : padded) + 512;
 }
 
 // ceil(2^32 / d), or 0 for d == 1 (the loaders then skip the division)
-static unsigned div_magic(unsigned d) { return d <= 1 ? 0u : (unsigned)(((1ull << 32) + d - 1) / d); }
 
 // explicit == 0: gather the column matrix inside the GEMM when the geometry allows it
 static int conv2d_common(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
@@ -741,23 +743,46 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
 
     // The on-the-fly gather needs: 4 consecutive columns inside one output row,
-    // 16-byte loadable weights, byte offsets into the input below 2^31, and the
-    // multiply-high divisions by Hf*Wf and Wf exact (k * Hf*Wf < 2^32).
+    // 16-byte loadable weights, byte offsets into the (padded) input below 2^31,
+    const int Hp = Hin + 2 * pad, Wp = Win + 2 * pad;
+    const double padded_elems = (double)batch * Cin * Hp * Wp;
     const bool implicit = !explicit_cols && (Wout % 4 == 0) && (K % 4 == 0) && aligned16(w.dev) &&
-                          in_elems * 4 < 2147483648.0 && K_d * Hf * Wf < 4294967296.0 &&
+                          padded_elems * 4 < 2147483648.0 &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
     if (implicit) {
+        const float* image = i.dev;
+        if (pad > 0) {  // a zero-padded copy, so that the gather has no edge cases
+            char* ws = static_cast<char*>(workspace);
+            if (!ws) {
+                if ((st = g_ctx.conv.reserve((size_t)padded_elems * 4 + 256))) return st;
+                ws = static_cast<char*>(g_ctx.conv.ptr);
+            } else if (!is_device_pointer(ws)) {
+                return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
+            }
+            image = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+        }
         ConvGeom cv{};
-        cv.in = i.dev;
-        cv.Cin = Cin; cv.Hin = Hin; cv.Win = Win; cv.Hf = Hf; cv.Wf = Wf;
-        cv.Hout = Hout; cv.Wout = Wout; cv.stride = stride; cv.pad = pad;
-        cv.div_hw_magic = div_magic((unsigned)(Hf * Wf));
-        cv.div_w_magic = div_magic((unsigned)Wf);
+        cv.in = image;
+        cv.Cin = Cin; cv.Hin = Hp; cv.Win = Wp; cv.Hf = Hf; cv.Wf = Wf;
+        cv.Hout = Hout; cv.Wout = Wout; cv.stride = stride;
+        if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
+        int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
+        cv.tap_table = taps;
         cv.out_nchw = out_nchw ? 1 : 0;
         if ((st = timer.start())) return st;
+        st = timer.family(3, [&] { return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, Hp, Wp, Hf, Wf, stream); });
+        if (st) return st;
+        if (pad > 0) {
+            st = timer.family(3, [&] {
+                return launch_pad_planes(i.dev, const_cast<float*>(image), (size_t)batch * Cin, Hin, Win, pad, stream);
+            });
+            if (st) return st;
+        }
+        // stride 1: 4 consecutive columns are one 16-byte load from an image row
+        const int b_mode = stride == 1 ? LOAD_IM2COL_ROW : LOAD_IM2COL;
         st = run_gemm(w.dev, nullptr, o.dev, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
-                      LOAD_IM2COL, IndexTables{}, IndexTables{}, stream, timer, &cv);
+                      b_mode, IndexTables{}, IndexTables{}, stream, timer, &cv);
         if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);

@@ -22,13 +22,12 @@ struct IndexTables {
 
 // Geometry of a convolution whose column matrix B[k][n] is gathered on the fly:
 // k = c*Hf*Wf + h*Wf + w, n = b*Hout*Wout + ho*Wout + wo,
-// B[k][n] = in[b][c][ho*stride + h - pad][wo*stride + w - pad] or 0 outside the image.
+// B[k][n] = in[b][c][ho*stride + h][wo*stride + w].  `in` carries its padding
+// already (Hin, Win include it), so every window position is inside the image.
 struct ConvGeom {
     const float* in;
-    int Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad;
-    unsigned div_hw_magic;  // ceil(2^32 / (Hf*Wf)): k / (Hf*Wf) == mulhi(k, magic) for k*Hf*Wf < 2^32;
-                            // 0 when the divisor is 1
-    unsigned div_w_magic;   // ceil(2^32 / Wf)
+    int Cin, Hin, Win, Hf, Wf, Hout, Wout, stride;
+    const int* tap_table;   // byte offset of tap k = (c, h, w) inside one image, K + CONV_TAP_TABLE_EXTRA entries
     int out_nchw;           // epilogue writes C as [batch][M][Hout*Wout] instead of [M][N]
 };
 
@@ -74,7 +73,8 @@ enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
     LOAD_PACKED = 2, // reference packed layout through IndexTables
-    LOAD_IM2COL = 3  // B only: column matrix of a convolution gathered from the NCHW input
+    LOAD_IM2COL = 3, // B only: column matrix of a convolution gathered from the NCHW input
+    LOAD_IM2COL_ROW = 4  // the same for stride 1: one 16-byte load per 4 columns
 };
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
@@ -95,6 +95,13 @@ hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M
 hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win,
                          int Hf, int Wf, int Hout, int Wout, int stride, int pad,
                          hipStream_t stream);
+// out[plane][y][x] = in[plane][y - pad][x - pad], zero in the border; out planes are (Hin+2pad) x (Win+2pad)
+hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
+                             hipStream_t stream);
+// table[k] = byte offset of filter tap k inside one image; `extra` zero entries follow
+enum { CONV_TAP_TABLE_EXTRA = 256 };
+hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win, int Hf, int Wf,
+                                 hipStream_t stream);
 // [Cout][batch*HW] -> [batch][Cout][HW]
 hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
                              hipStream_t stream);

@@ -60,6 +60,61 @@ hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stre
 }
 
 // ---------------------------------------------------------------------------
+// zero padding of image planes: the convolution's gather then needs no edge
+// tests.  One workgroup per plane, 64 lanes along a row, 4 rows at a time, so
+// no thread divides anything; reads and writes both run along image rows.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) pad_planes_kernel(const float* __restrict__ in,
+                                                         float* __restrict__ out, size_t planes,
+                                                         int Hin, int Win, int pad)
+{
+    const int Hp = Hin + 2 * pad, Wp = Win + 2 * pad;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (size_t plane = blockIdx.x; plane < planes; plane += gridDim.x) {
+        const float* src = in + plane * Hin * Win;
+        float* dst = out + plane * Hp * Wp;
+        for (int y = ty; y < Hp; y += 4) {
+            const int yi = y - pad;
+            const bool row_in = (unsigned)yi < (unsigned)Hin;
+            for (int x = tx; x < Wp; x += 64) {
+                const int xi = x - pad;
+                dst[y * Wp + x] = (row_in && (unsigned)xi < (unsigned)Win) ? src[yi * Win + xi] : 0.f;
+            }
+        }
+    }
+}
+
+hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
+                             hipStream_t stream)
+{
+    if (planes == 0) return hipSuccess;
+    const unsigned blocks = (unsigned)(planes < (1u << 20) ? planes : (1u << 20));
+    hipLaunchKernelGGL(pad_planes_kernel, dim3(blocks), dim3(256), 0, stream, in, out, planes, Hin, Win, pad);
+    return hipGetLastError();
+}
+
+// Byte offset of filter tap k = (c, h, w) inside one image of a convolution's
+// input: table[k] = ((c*Hin + h)*Win + w) * 4 for k < K, 0 for the `extra`
+// entries after it (the gather prefetches a few stages past the end).
+__global__ void __launch_bounds__(256) conv_tap_table_kernel(int* __restrict__ table, int K, int extra,
+                                                             int Hin, int Win, int Hf, int Wf)
+{
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= K + extra) return;
+    const int c = k / (Hf * Wf), tap = k - c * (Hf * Wf);
+    const int h = tap / Wf, w = tap - h * Wf;
+    table[k] = k < K ? ((c * Hin + h) * Win + w) * 4 : 0;
+}
+
+hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win, int Hf, int Wf,
+                                 hipStream_t stream)
+{
+    hipLaunchKernelGGL(conv_tap_table_kernel, dim3((K + extra + 255) / 256), dim3(256), 0, stream, table, K,
+                       extra, Hin, Win, Hf, Wf);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // im2col: im_2_col of examples/cake_conv.cpp:1178-1213 with batch, padding and
 // stride.  grid.y = row k of the column matrix (one (c, h, w) filter tap),
 // threads run along n = (b, ho, wo).

@@ -1,0 +1,19 @@
+// Macro-tile GEMM instantiations for stride-1 convolution: as sgemm_inst_conv.hip,
+// with the column matrix gathered 4 consecutive pixels per load.
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+hipError_t launch_sgemm_convrow(int tile_id, const GemmArgs& a, int grid, hipStream_t s)
+{
+    switch (tile_id) {
+        case TILE_256x256x32_W128x64: return launch_tile<Tile256x256x32, LOAD_VEC4, LOAD_IM2COL_ROW>(a, grid, s);
+        case TILE_256x128x32_W64x64: return launch_tile<Tile256x128x32, LOAD_VEC4, LOAD_IM2COL_ROW>(a, grid, s);
+        case TILE_128x256x32_W64x64: return launch_tile<Tile128x256x32, LOAD_VEC4, LOAD_IM2COL_ROW>(a, grid, s);
+        case TILE_128x128x32_W64x64: return launch_tile<Tile128x128x32, LOAD_VEC4, LOAD_IM2COL_ROW>(a, grid, s);
+        case TILE_64x64x32_W32x32: return launch_tile<Tile64x64x32, LOAD_VEC4, LOAD_IM2COL_ROW>(a, grid, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace cake

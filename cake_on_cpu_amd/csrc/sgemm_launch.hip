@@ -8,6 +8,7 @@ hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStre
 hipError_t launch_sgemm_packed(int tile_id, int a_mode, int b_mode, const GemmArgs& a, int grid,
                                hipStream_t s);
 hipError_t launch_sgemm_conv(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
+hipError_t launch_sgemm_convrow(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 
 template <class T>
 static constexpr TileInfo info_of()
@@ -28,9 +29,10 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
                         hipStream_t stream)
 {
     if (grid <= 0) return hipSuccess;
-    if (b_mode == LOAD_IM2COL) {
+    if (b_mode == LOAD_IM2COL || b_mode == LOAD_IM2COL_ROW) {
         if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
-        return launch_sgemm_conv(tile_id, args, grid, stream);
+        return b_mode == LOAD_IM2COL ? launch_sgemm_conv(tile_id, args, grid, stream)
+                                     : launch_sgemm_convrow(tile_id, args, grid, stream);
     }
     if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
         if (a_mode == LOAD_VEC4) a_mode = LOAD_SCALAR;

@@ -325,6 +325,8 @@ struct VecLoader {
         }
     }
 
+    __device__ __forceinline__ void prime(int) {}  // nothing to fetch ahead
+
     // chunk OP (A chunks first, then B chunks) of the stage starting at k0
     template <int OP>
     __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
@@ -361,11 +363,13 @@ __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_off
 // A through 16-byte buffer loads as in VecLoader; B = the column matrix of a
 // convolution, gathered element by element from the NCHW input ("implicit
 // im2col": examples/cake_conv.cpp:1178-1213 without the K x N intermediate).
+// The input the kernel sees has no padding left (the host hands over a
+// zero-padded copy when the convolution has one), so every window position is
+// inside the image and the gather needs no masks beyond the tile edges.
 // A thread's B chunk is 4 consecutive n at one k; with Wout % 4 == 0 those are
 // 4 consecutive output pixels of one image row, so one (image, row, column)
 // triple per thread serves the whole K walk, and only the filter tap (c, h, w)
-// of each k has to be decoded per stage.  Window positions outside the image
-// are requested at an out-of-range buffer offset and read as zero.
+// of each k has to be decoded per stage.
 template <class T>
 struct ConvLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + 4 * T::B_ITERS;
@@ -374,9 +378,12 @@ struct ConvLoader {
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
     const float* a_base;
     ConvGeom cv;
-    int pix;              // element offset of in[b][0][ho*s - pad][wo*s - pad] for the chunk's first n
-    int hs, ws;           // ho*s - pad, wo*s - pad
+    int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n
     bool n_ok;
+    // Byte offset of the filter tap of the chunk's k inside an image, for the
+    // stage the NEXT load call fetches.  It comes from a small table in memory,
+    // read one stage ahead so that its latency never sits in front of a gather.
+    mutable int tap_next[T::B_ITERS];
 
     __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
     {
@@ -397,16 +404,28 @@ struct ConvLoader {
         const int HW = cv.Hout * cv.Wout;
         const int b = n / HW, r = n - b * HW;
         const int ho = r / cv.Wout, wo = r - ho * cv.Wout;
-        hs = ho * cv.stride - cv.pad;
-        ws = wo * cv.stride - cv.pad;
-        pix = ((b * cv.Cin) * cv.Hin + hs) * cv.Win + ws;
+        pix4 = (((b * cv.Cin) * cv.Hin + ho * cv.stride) * cv.Win + wo * cv.stride) * 4;
     }
 
-    // The filter tap of a chunk's k is decoded by the chunk's first load and
-    // kept for the other three (the loads of a chunk are issued in order).
-    mutable int tap_off[T::B_ITERS];  // byte offset of the tap's window start for n, or garbage when !tap_ok
-    mutable int tap_w[T::B_ITERS];    // ws + w
-    mutable bool tap_ok[T::B_ITERS];  // column, k and image row are all inside
+    // before the first load: the stages are then fetched at k0, k0 + BK, k0 + 2 BK, ...
+    __device__ __forceinline__ void prime(int k0)
+    {
+#pragma unroll
+        for (int it = 0; it < T::B_ITERS; ++it) tap_next[it] = cv.tap_table[k0 + b_k[it]];
+    }
+
+    // byte offset of the window start of chunk `it` at stage k0, or BUF_OOB past the edges
+    __device__ __forceinline__ int tap_offset(int it, int k0, int kend) const
+    {
+        const int k = k0 + b_k[it];
+        const int off = (n_ok && k < kend) ? pix4 + tap_next[it] : BUF_OOB;
+        tap_next[it] = cv.tap_table[k + T::BK];  // the table has spare entries past K
+        return off;
+    }
+
+    // The chunk's offset is computed by its first load and kept for the other
+    // three (the loads of a chunk are issued in order).
+    mutable int tap_off[T::B_ITERS];
 
     template <int OP>
     __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
@@ -416,20 +435,43 @@ struct ConvLoader {
             ra[OP] = buffer_load_f32x4(a_base + k0, a_k[OP] < kend - k0 ? a_off[OP] : BUF_OOB);
         } else {
             constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
-            if constexpr (e == 0) {
-                const int k = k0 + b_k[it];
-                // ceil(2^32 / d) does not fit 32 bits for d == 1: a zero magic marks that case
-                const int c = cv.div_hw_magic ? (int)__umulhi((unsigned)k, cv.div_hw_magic) : k;
-                const int tap = k - c * (cv.Hf * cv.Wf);
-                const int h = cv.div_w_magic ? (int)__umulhi((unsigned)tap, cv.div_w_magic) : tap;
-                const int w = tap - h * cv.Wf;
-                tap_off[it] = (pix + (c * cv.Hin + h) * cv.Win + w) * 4;
-                tap_w[it] = ws + w;
-                tap_ok[it] = n_ok && k < kend && (unsigned)(hs + h) < (unsigned)cv.Hin;
-            }
-            const bool ok = tap_ok[it] && (unsigned)(tap_w[it] + e * cv.stride) < (unsigned)cv.Win;
-            rb[it][e] = buffer_load_f32(cv.in, ok ? tap_off[it] + e * cv.stride * 4 : BUF_OOB);
+            if constexpr (e == 0) tap_off[it] = tap_offset(it, k0, kend);
+            // BUF_OOB plus a few strides stays out of range
+            rb[it][e] = buffer_load_f32(cv.in, tap_off[it] + e * cv.stride * 4);
         }
+    }
+
+    __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        load_all<0>(k0, kend, ra, rb);
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < NUM_LOADS) {
+            load_one<OP>(k0, kend, ra, rb);
+            load_all<OP + 1>(k0, kend, ra, rb);
+        }
+    }
+};
+
+// ConvLoader for stride 1: the 4 consecutive n of a chunk are 4 consecutive
+// input pixels of one image row, so the chunk is ONE 16-byte load (4-byte
+// aligned, which buffer loads allow) instead of four 4-byte loads.
+template <class T>
+struct ConvRowLoader : ConvLoader<T> {
+    using Base = ConvLoader<T>;
+    static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
+
+    template <int OP>
+    __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
+                                             f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = buffer_load_f32x4(Base::a_base + k0, Base::a_k[OP] < kend - k0 ? Base::a_off[OP] : BUF_OOB);
+        else
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset(OP - T::A_ITERS, k0, kend));
     }
 
     __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
@@ -588,6 +630,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     static_assert(RS == 1 || RS == 2 || RS == 4, "one, two or four register stages");
     L ld;
     ld.init(g, m0, n0, tid);
+    ld.prime(kbeg);
     f32x4 ra[RS][T::A_ITERS], rb[RS][T::B_ITERS];
     Frag<T> frag[2];
     if (steps <= 0) return;
@@ -715,6 +758,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
         k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL)
         k_walk_vec<T, ConvLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+    else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
+        k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
     else
         k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
 
@@ -737,7 +782,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const bool add = (g.partial == nullptr) && g.accumulate;
     const float* bias = g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
-    const bool nchw = (B_MODE == LOAD_IM2COL) && g.conv.out_nchw && g.partial == nullptr;
+    const bool nchw = (B_MODE == LOAD_IM2COL || B_MODE == LOAD_IM2COL_ROW) && g.conv.out_nchw && g.partial == nullptr;
     const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
 #pragma unroll
     for (int tm = 0; tm < T::TM; ++tm)

@@ -200,12 +200,15 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * is what the reference produces for its single image); != 0: NCHW.
  *
  * cake_hip_conv2d gathers the column matrix inside the GEMM's B loader when the
- * geometry allows it (Wout % 4 == 0, Cin*Hf*Wf % 4 == 0, input below 2 GiB), so
- * the K x N intermediate is never written; otherwise it runs the two-step path.
+ * geometry allows it (Wout % 4 == 0, Cin*Hf*Wf % 4 == 0, padded input below
+ * 2 GiB), so the K x N intermediate is never written (with pad > 0 the input is
+ * first copied once into a zero-padded image, so that the gather has no edge
+ * cases); otherwise it runs the two-step path.
  * cake_hip_conv2d_im2col always runs the two steps the reference runs: im2col
  * into a column matrix, then the GEMM.  Both give the same result.
- * workspace (device, cake_hip_conv2d_workspace bytes; only the two-step path
- * uses it) may be NULL: the library then uses a buffer of its own. */
+ * workspace (device, cake_hip_conv2d_workspace bytes: the column matrix of the
+ * two-step path or the padded image of the gather path) may be NULL: the
+ * library then uses a buffer of its own. */
 size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
                                  int Hf, int Wf, int stride, int pad);
 int cake_hip_conv2d(const float* in, const float* weights, float* out,

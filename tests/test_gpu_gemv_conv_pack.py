@@ -138,6 +138,11 @@ CONV_GEOMS = [
     (2, 4, 12, 14, 9, 5, 3, 1, 2),       # 5x3 filter, pad 2, Wout = 16
     (4, 32, 14, 8, 64, 3, 3, 1, 1),      # Wout = 8
     (1, 4, 6, 8, 5, 3, 3, 3, 2),         # stride 3, pad 2, Wout = 4
+    (2, 6, 10, 12, 12, 7, 7, 1, 3),      # 7x7, pad 3: the 16-byte row gather shifts by up to 3 either way
+    (2, 8, 16, 16, 16, 5, 5, 1, 2),      # 5x5, pad 2, Wout = 16
+    (3, 5, 5, 4, 8, 3, 3, 1, 1),         # Win = 4: the row gather's narrowest image
+    (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
+    (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
 ]
 
 
