@@ -709,7 +709,7 @@ size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
     // two-step path: column matrix + a [Cout][ncols] product when the caller wants NCHW;
     // gather path: a zero-padded copy of the input
     const size_t two_step = ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float);
-    const size_t padded = (size_t)batch * Cin * (Hin + 2 * pad) * (Win + 2 * pad) * sizeof(float);
+    const size_t padded = (size_t)batch * Cin * (Hin + 2 * pad) * ((Win + 2 * pad + 3) & ~3) * sizeof(float);
     return (two_step > padded ? two_step : padded) + 512;
 }
 
@@ -744,7 +744,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
 
     // The on-the-fly gather needs: 4 consecutive columns inside one output row,
     // 16-byte loadable weights, byte offsets into the (padded) input below 2^31,
-    const int Hp = Hin + 2 * pad, Wp = Win + 2 * pad;
+    // (rows of the padded copy are a multiple of 4 floats apart, so it is written in 16-byte pieces)
+    const int Hp = Hin + 2 * pad, Wp = pad > 0 ? (Win + 2 * pad + 3) & ~3 : Win;
     const double padded_elems = (double)batch * Cin * Hp * Wp;
     const bool implicit = !explicit_cols && (Wout % 4 == 0) && (K % 4 == 0) && aligned16(w.dev) &&
                           padded_elems * 4 < 2147483648.0 &&
@@ -775,7 +776,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         if (st) return st;
         if (pad > 0) {
             st = timer.family(3, [&] {
-                return launch_pad_planes(i.dev, const_cast<float*>(image), (size_t)batch * Cin, Hin, Win, pad, stream);
+                return launch_pad_planes(i.dev, const_cast<float*>(image), (size_t)batch * Cin, Hin, Win, pad, Wp, stream);
             });
             if (st) return st;
         }

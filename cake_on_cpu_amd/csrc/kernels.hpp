@@ -95,9 +95,10 @@ hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M
 hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win,
                          int Hf, int Wf, int Hout, int Wout, int stride, int pad,
                          hipStream_t stream);
-// out[plane][y][x] = in[plane][y - pad][x - pad], zero in the border; out planes are (Hin+2pad) x (Win+2pad)
+// out[plane][y][x] = in[plane][y - pad][x - pad], zero in the border and in the row tail; out planes
+// are (Hin+2pad) rows of `pitch` floats (pitch % 4 == 0, pitch >= Win+2pad, out 16-byte aligned)
 hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                             hipStream_t stream);
+                             int pitch, hipStream_t stream);
 // table[k] = byte offset of filter tap k inside one image; `extra` zero entries follow
 enum { CONV_TAP_TABLE_EXTRA = 256 };
 hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win, int Hf, int Wf,

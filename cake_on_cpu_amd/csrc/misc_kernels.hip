@@ -61,35 +61,42 @@ hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stre
 
 // ---------------------------------------------------------------------------
 // zero padding of image planes: the convolution's gather then needs no edge
-// tests.  One workgroup per plane, 64 lanes along a row, 4 rows at a time, so
-// no thread divides anything; reads and writes both run along image rows.
+// tests.  Output rows are `pitch` floats apart (a multiple of 4, >= Win + 2 pad),
+// so every thread writes one aligned float4; reads run along image rows.  One
+// workgroup per plane: 16 lanes along a row, 16 rows at a time.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) pad_planes_kernel(const float* __restrict__ in,
                                                          float* __restrict__ out, size_t planes,
-                                                         int Hin, int Win, int pad)
+                                                         int Hin, int Win, int pad, int pitch)
 {
-    const int Hp = Hin + 2 * pad, Wp = Win + 2 * pad;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int Hp = Hin + 2 * pad;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     for (size_t plane = blockIdx.x; plane < planes; plane += gridDim.x) {
         const float* src = in + plane * Hin * Win;
-        float* dst = out + plane * Hp * Wp;
-        for (int y = ty; y < Hp; y += 4) {
+        float* dst = out + plane * Hp * pitch;
+        for (int y = ty; y < Hp; y += 16) {
             const int yi = y - pad;
             const bool row_in = (unsigned)yi < (unsigned)Hin;
-            for (int x = tx; x < Wp; x += 64) {
-                const int xi = x - pad;
-                dst[y * Wp + x] = (row_in && (unsigned)xi < (unsigned)Win) ? src[yi * Win + xi] : 0.f;
+            for (int x = tx * 4; x < pitch; x += 64) {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int xi = x + e - pad;
+                    v[e] = (row_in && (unsigned)xi < (unsigned)Win) ? src[yi * Win + xi] : 0.f;
+                }
+                *reinterpret_cast<f32x4*>(dst + y * pitch + x) = v;
             }
         }
     }
 }
 
 hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                             hipStream_t stream)
+                             int pitch, hipStream_t stream)
 {
     if (planes == 0) return hipSuccess;
+    if (pitch % 4 != 0 || pitch < Win + 2 * pad) return hipErrorInvalidValue;
     const unsigned blocks = (unsigned)(planes < (1u << 20) ? planes : (1u << 20));
-    hipLaunchKernelGGL(pad_planes_kernel, dim3(blocks), dim3(256), 0, stream, in, out, planes, Hin, Win, pad);
+    hipLaunchKernelGGL(pad_planes_kernel, dim3(blocks), dim3(256), 0, stream, in, out, planes, Hin, Win, pad, pitch);
     return hipGetLastError();
 }
 
