@@ -848,13 +848,11 @@ template <class T, int A_MODE, int B_MODE>
 inline hipError_t launch_tile(const GemmArgs& args, int grid, hipStream_t stream)
 {
     auto kern = sgemm_tile_kernel<T, A_MODE, B_MODE>;
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    // once per instantiation; the initialiser of a function-local static runs once even when
+    // several host threads launch at the same time
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+    if (attr != hipSuccess) return attr;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(T::THREADS), T::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
