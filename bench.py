@@ -156,7 +156,7 @@ def main() -> int:
             "cus": info.cus,
         },
         "roofline": {
-            "kernel": f"sgemm_tile_kernel<Tile<{plan.tile_m},{plan.tile_n},{plan.tile_k},{plan.wave_m},{plan.wave_n}>>",
+            "kernel": f"sgemm_tile_kernel<Tile<{plan.tile_m},{plan.tile_n},{plan.tile_k},{plan.wave_m},{plan.wave_n},...>,0,0>",
             "bound": "mfma",
             "achieved": round(achieved, 3),
             "peak": MFMA_PEAK_TFLOPS,
