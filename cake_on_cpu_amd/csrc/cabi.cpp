@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <chrono>
 #include <mutex>
 #include <string>
@@ -70,7 +71,7 @@ struct DeviceBuffer {
 enum { STAGE_SLOTS = 6 };
 
 struct Context {
-    bool ready = false;
+    std::atomic<bool> ready{false};
     int device = 0;
     cake_hip_device_t info{};
     DeviceModel model;
@@ -118,7 +119,12 @@ int stage_in(const float* p, size_t bytes, int slot, bool copy, Operand* op)
     if (st) return st;
     op->dev = static_cast<float*>(g_ctx.stage[slot].ptr);
     op->host = const_cast<float*>(p);
-    if (copy) HIP_TRY(hipMemcpy(op->dev, p, bytes, hipMemcpyHostToDevice));
+    if (copy) {
+        // an earlier call may have left kernels in flight that still read this slot (device
+        // outputs make a call asynchronous); hipMemcpy alone does not wait for non-blocking streams
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipMemcpy(op->dev, p, bytes, hipMemcpyHostToDevice));
+    }
     return CAKE_HIP_OK;
 }
 
