@@ -189,6 +189,38 @@ def test_compute_without_gpu_fails_loudly():
     assert e.value.status == _lib.ERR_NO_DEVICE
 
 
+def test_entry_points_reject_bad_arguments_before_touching_a_device():
+    """Argument and range checks come first, so they read the same with or without a GPU:
+    negative sizes, unknown schedules, NULL operands and operands of 2^31 elements or more
+    (all index arithmetic of the path is int, like the reference's)."""
+    lib = cake.load()
+    buf = np.zeros(16, np.float32)
+    ptr = buf.ctypes.data
+    sgemm = lambda M, N, K, sch=cake.NA, a=ptr: lib.cake_hip_sgemm(a, ptr, ptr, M, N, K, sch, 0, None, None, None)
+    assert sgemm(-1, 4, 4) == _lib.ERR_ARG
+    assert sgemm(4, 4, 4, sch=9) == _lib.ERR_ARG
+    assert sgemm(4, 4, 4, a=None) == _lib.ERR_ARG
+    assert sgemm(0, 4, 4) == _lib.OK and sgemm(4, 0, 4) == _lib.OK            # nothing to compute
+    assert sgemm(65536, 4, 32768) == _lib.ERR_RANGE                            # A has 2^31 elements
+    assert sgemm(46341, 46341, 4) == _lib.ERR_RANGE                            # C has more than 2^31 - 1
+    assert lib.cake_hip_sgemv(ptr, ptr, ptr, -1, 4, 1, 1, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_sgemv(ptr, ptr, ptr, 65536, 32768, 1, 1, None, None) == _lib.ERR_RANGE
+    assert lib.cake_hip_sgemv(None, ptr, ptr, 4, 4, 1, 1, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_transpose(ptr, ptr, 2, 2, None, None) == _lib.ERR_ARG  # in place
+    assert lib.cake_hip_transpose(ptr, None, 2, 2, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_transpose(ptr, ptr, 0, 5, None, None) == _lib.OK
+    assert lib.cake_hip_linear_forward(ptr, ptr, None, ptr, -2, 4, 4, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_linear_forward(ptr, ptr, None, None, 2, 4, 4, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_linear_forward(ptr, ptr, None, ptr, 65536, 4, 32768, None, None) == _lib.ERR_RANGE
+    assert lib.cake_hip_linear_backward(None, ptr, ptr, ptr, ptr, ptr, 2, 2, 2, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_conv2d(ptr, ptr, ptr, 1, 1, 2, 2, 1, 3, 3, 1, 0, 0, None, None, None) == _lib.ERR_ARG  # filter larger than image
+    assert lib.cake_hip_conv2d(ptr, ptr, ptr, 1, 1, 4, 4, 1, 3, 3, 0, 0, 0, None, None, None) == _lib.ERR_ARG  # stride 0
+    assert lib.cake_hip_conv2d(ptr, None, ptr, 1, 1, 4, 4, 1, 3, 3, 1, 0, 0, None, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_autotune(0, 4, 4, 1.0, None, None, None) == _lib.ERR_ARG
+    assert lib.cake_hip_tune_save(None) == _lib.ERR_ARG
+    assert lib.cake_hip_last_error() != b""
+
+
 # ---------------------------------------------------------------------------
 # the table of measured choices (no device needed to load, save or consult it)
 # ---------------------------------------------------------------------------
