@@ -25,6 +25,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernels.hpp"
 
 namespace cake {
@@ -32,9 +34,10 @@ namespace cake {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// REG_STAGES: how many K stages wait in registers between their global loads and
-// their LDS stores (the 16-byte loaders only).  2 gives every load a whole extra
-// K step to come back from HBM, for 6-8 more float4 registers per lane.
+// REG_STAGES: how many K stages' worth of registers sit between the global loads
+// and the LDS stores (the 16-byte loaders only).  With 2, a step's loads go into
+// the set the previous step emptied, so they can be issued anywhere in the step,
+// for 6-8 more float4 registers per lane.
 // STORE_LEAD: how many operand groups (of 8 k) before the step's barrier the
 // register -> LDS stores are issued.  1 puts them in the group that ends at the
 // barrier; 2 gives them a whole group to land first, which matters when a group
@@ -327,6 +330,16 @@ struct VecLoader {
 
     __device__ __forceinline__ void prime(int) {}  // nothing to fetch ahead
 
+    // the same for a stage that lies wholly below kend: no per-lane test, no vector ALU work
+    template <int OP>
+    __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = buffer_load_f32x4(a_base + k0, a_off[OP]);
+        else
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(b_base + (size_t)k0 * ldb, b_off[OP - T::A_ITERS]);
+    }
+
     // chunk OP (A chunks first, then B chunks) of the stage starting at k0
     template <int OP>
     __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
@@ -378,8 +391,8 @@ struct ConvLoader {
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
     const float* a_base;
     ConvGeom cv;
-    int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n
-    bool n_ok;
+    int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n; BUF_OOB for n >= N
+                          // (adding a tap offset, which is below 2^31, keeps it out of range)
     // Byte offset of the filter tap of the chunk's k inside an image, for the
     // stage the NEXT load call fetches.  It comes from a small table in memory,
     // read one stage ahead so that its latency never sits in front of a gather.
@@ -400,11 +413,10 @@ struct ConvLoader {
         for (int it = 0; it < T::B_ITERS; ++it) b_k[it] = (tid + it * T::THREADS) / (T::BN / 4);
         static_assert(T::THREADS % (T::BN / 4) == 0, "a thread keeps the same 4 columns in every chunk");
         const int n = n0 + (tid % (T::BN / 4)) * 4;
-        n_ok = n < g.N;
         const int HW = cv.Hout * cv.Wout;
         const int b = n / HW, r = n - b * HW;
         const int ho = r / cv.Wout, wo = r - ho * cv.Wout;
-        pix4 = (((b * cv.Cin) * cv.Hin + ho * cv.stride) * cv.Win + wo * cv.stride) * 4;
+        pix4 = n < g.N ? (((b * cv.Cin) * cv.Hin + ho * cv.stride) * cv.Win + wo * cv.stride) * 4 : BUF_OOB;
     }
 
     // before the first load: the stages are then fetched at k0, k0 + BK, k0 + 2 BK, ...
@@ -418,8 +430,16 @@ struct ConvLoader {
     __device__ __forceinline__ int tap_offset(int it, int k0, int kend) const
     {
         const int k = k0 + b_k[it];
-        const int off = (n_ok && k < kend) ? pix4 + tap_next[it] : BUF_OOB;
+        const int off = k < kend ? pix4 + tap_next[it] : BUF_OOB;
         tap_next[it] = cv.tap_table[k + T::BK];  // the table has spare entries past K
+        return off;
+    }
+
+    // the same for a stage that lies wholly below kend
+    __device__ __forceinline__ int tap_offset_inside(int it, int k0) const
+    {
+        const int off = pix4 + tap_next[it];
+        tap_next[it] = cv.tap_table[k0 + b_k[it] + T::BK];
         return off;
     }
 
@@ -437,6 +457,18 @@ struct ConvLoader {
             constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
             if constexpr (e == 0) tap_off[it] = tap_offset(it, k0, kend);
             // BUF_OOB plus a few strides stays out of range
+            rb[it][e] = buffer_load_f32(cv.in, tap_off[it] + e * cv.stride * 4);
+        }
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS) {
+            ra[OP] = buffer_load_f32x4(a_base + k0, a_off[OP]);
+        } else {
+            constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
+            if constexpr (e == 0) tap_off[it] = tap_offset_inside(it, k0);
             rb[it][e] = buffer_load_f32(cv.in, tap_off[it] + e * cv.stride * 4);
         }
     }
@@ -472,6 +504,15 @@ struct ConvRowLoader : ConvLoader<T> {
             ra[OP] = buffer_load_f32x4(Base::a_base + k0, Base::a_k[OP] < kend - k0 ? Base::a_off[OP] : BUF_OOB);
         else
             rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset(OP - T::A_ITERS, k0, kend));
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = buffer_load_f32x4(Base::a_base + k0, Base::a_off[OP]);
+        else
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset_inside(OP - T::A_ITERS, k0));
     }
 
     __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
@@ -519,10 +560,32 @@ struct Slots {
     static constexpr int STORE_KG = NKG - 1 - T::STORE_LEAD;
     static_assert(STORE_KG >= 0, "stores must follow the previous step's barrier");
     static_assert(NKG >= 3, "the walk needs three operand groups per K step");
-    // memory instructions riding in group kg: operand reads, then loads, then stores
-    static constexpr int ops(int kg)
+    // With two register stages the loads of a step fill the set that the PREVIOUS
+    // step stored, so they can go anywhere in the step and are dealt evenly over
+    // its groups: issued in one burst by all the waves at once they queue up at
+    // the memory pipe and hold back the MFMAs behind them.  With one register
+    // stage they have to follow the step's own stores.
+    static constexpr bool SPREAD_LOADS = T::REG_STAGES >= 2;
+    static constexpr int load_begin(int kg) { return SPREAD_LOADS ? kg * LOAD_OPS / NKG : 0; }
+    static constexpr int loads_in(int kg)
     {
-        return FRAG_OPS + (kg == NKG - 1 ? LOAD_OPS : 0) + (kg == STORE_KG ? STORE_OPS : 0);
+        return SPREAD_LOADS ? (kg + 1) * LOAD_OPS / NKG - kg * LOAD_OPS / NKG : (kg == NKG - 1 ? LOAD_OPS : 0);
+    }
+    // memory instructions riding in group kg: operand reads, then loads, then stores
+    static constexpr int ops(int kg) { return FRAG_OPS + loads_in(kg) + (kg == STORE_KG ? STORE_OPS : 0); }
+};
+
+// A loader seen through this wrapper fetches stages that lie wholly below kend,
+// which takes the per-lane "k < kend" tests (compares and selects between the
+// MFMAs) out of the bulk of the K walk.
+template <class L>
+struct InsideStages {
+    static constexpr int NUM_LOADS = L::NUM_LOADS;
+    const L& ld;
+    template <int OP, class RA, class RB>
+    __device__ __forceinline__ void load_one(int k0, int /*kend*/, RA& ra, RB& rb) const
+    {
+        ld.template load_one_inside<OP>(k0, ra, rb);
     }
 };
 
@@ -536,8 +599,10 @@ struct WalkCtx {
     float* An;
     float* Bn;
     int tid, a_row, b_col, lh;
-    f32x4 (&ra)[T::A_ITERS];
+    f32x4 (&ra)[T::A_ITERS];  // register stage that this step stores to LDS
     f32x4 (&rb)[T::B_ITERS];
+    f32x4 (&la)[T::A_ITERS];  // register stage that this step's global loads fill
+    f32x4 (&lb)[T::B_ITERS];
 };
 
 // Memory instruction number OP of group KG (compile-time indices, so every
@@ -547,7 +612,7 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
 {
     using S = Slots<T, L>;
     constexpr int N_FRAG = S::FRAG_OPS;
-    constexpr int N_LOAD = (KG == S::NKG - 1) ? S::LOAD_OPS : 0;
+    constexpr int N_LOAD = S::loads_in(KG);
     if constexpr (OP < N_FRAG) {
         // operands of the next group; the last group reads group 0 of the next stage
         constexpr bool wrap = (KG + 1 == S::NKG);
@@ -561,7 +626,7 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_col + tn * 32];
         }
     } else if constexpr (OP < N_FRAG + N_LOAD) {
-        c.ld.template load_one<OP - N_FRAG>(c.k_next, c.kend, c.ra, c.rb);
+        c.ld.template load_one<S::load_begin(KG) + OP - N_FRAG>(c.k_next, c.kend, c.la, c.lb);
     } else {
         constexpr int W = OP - N_FRAG - N_LOAD;  // store number W of the stage
         if constexpr (W < T::A_ITERS) {
@@ -627,7 +692,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
 {
     static_assert(Slots<T, L>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
     constexpr int RS = T::REG_STAGES;
-    static_assert(RS == 1 || RS == 2 || RS == 4, "one, two or four register stages");
+    static_assert(RS == 1 || RS == 2, "one or two register stages");
     L ld;
     ld.init(g, m0, n0, tid);
     ld.prime(kbeg);
@@ -636,53 +701,45 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     if (steps <= 0) return;
     ld.load(kbeg, kend, ra[0], rb[0]);
     store_stage<T>(As, Bs, tid, ra[0], rb[0]);
-    // stage j waits in register set j % RS until step j-1 stores it
     ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
-    if constexpr (RS >= 2) ld.load(kbeg + 2 * T::BK, kend, ra[2 % RS], rb[2 % RS]);
-    if constexpr (RS == 4) {
-        ld.load(kbeg + 3 * T::BK, kend, ra[3], rb[3]);
-        ld.load(kbeg + 4 * T::BK, kend, ra[0], rb[0]);
-    }
     __syncthreads();
     load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
 
-    // One K step: stores stage s+1 from register set (s+1) % RS, then refills that
-    // set with stage s+1+RS.  Stages past the end are fetched as zeros and parked
+    // One K step s: stage s is in LDS, stage s+1 waits in registers.  The step
+    // stores stage s+1 to the other LDS buffer and fetches stage s+2 -- with two
+    // register stages into the set the previous step emptied, with one into the
+    // set it has just stored.  Stages past the end are fetched as zeros and parked
     // in the idle buffer, so the walk has no branch.
     int cur = 0;
-    auto step = [&](int s, f32x4 (&sa)[T::A_ITERS], f32x4 (&sb)[T::B_ITERS]) {
-        const WalkCtx<T, L> c{ld, kbeg + (s + 1 + RS) * T::BK, kend,
-                              As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
-                              As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
-                              tid, a_row, b_col, lh, sa, sb};
+    const InsideStages<L> inside{ld};
+    auto step_with = [&](const auto& loader, int s, f32x4 (&sa)[T::A_ITERS], f32x4 (&sb)[T::B_ITERS],
+                         f32x4 (&fa)[T::A_ITERS], f32x4 (&fb)[T::B_ITERS]) {
+        using LD = std::remove_cv_t<std::remove_reference_t<decltype(loader)>>;
+        const WalkCtx<T, LD> c{loader, kbeg + (s + 2) * T::BK, kend,
+                               As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
+                               As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
+                               tid, a_row, b_col, lh, sa, sb, fa, fb};
         __builtin_amdgcn_sched_barrier(0);
-        step_groups<T, L>(c, frag, acc);
+        step_groups<T, LD>(c, frag, acc);
         cur ^= 1;
     };
+    // steps 0 .. bulk-1 fetch stages s+2 that end at or below kend
+    const int bulk = min(steps, max(0, (kend - kbeg) / T::BK - 2));
     if constexpr (RS == 1) {
-        for (int s = 0; s < steps; ++s) step(s, ra[0], rb[0]);
-    } else if constexpr (RS == 2) {
         int s = 0;
-        for (; s + 1 < steps; s += 2) {
-            step(s, ra[1], rb[1]);
-            step(s + 1, ra[0], rb[0]);
-        }
-        if (s < steps) step(s, ra[1], rb[1]);
+        for (; s < bulk; ++s) step_with(inside, s, ra[0], rb[0], ra[0], rb[0]);
+        for (; s < steps; ++s) step_with(ld, s, ra[0], rb[0], ra[0], rb[0]);
     } else {
         int s = 0;
-        for (; s + 3 < steps; s += 4) {
-            step(s, ra[1], rb[1]);
-            step(s + 1, ra[2], rb[2]);
-            step(s + 2, ra[3], rb[3]);
-            step(s + 3, ra[0], rb[0]);
+        for (; s + 1 < bulk; s += 2) {
+            step_with(inside, s, ra[1], rb[1], ra[0], rb[0]);
+            step_with(inside, s + 1, ra[0], rb[0], ra[1], rb[1]);
         }
-        if (s < steps) {
-            step(s, ra[1], rb[1]);
-            if (s + 1 < steps) {
-                step(s + 1, ra[2], rb[2]);
-                if (s + 2 < steps) step(s + 2, ra[3], rb[3]);
-            }
+        for (; s + 1 < steps; s += 2) {
+            step_with(ld, s, ra[1], rb[1], ra[0], rb[0]);
+            step_with(ld, s + 1, ra[0], rb[0], ra[1], rb[1]);
         }
+        if (s < steps) step_with(ld, s, ra[1], rb[1], ra[0], rb[0]);
     }
 }
 
