@@ -296,6 +296,15 @@ __device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_o
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
 }
 
+// 4-byte load at base + voffset (per lane) + soffset (same for the wave): the wave-uniform part of
+// an address rides in a scalar register and costs no vector ALU work
+__device__ __forceinline__ int buffer_load_i32(const int* base, int voffset_bytes, int soffset_bytes)
+{
+    __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(base), 0, (int)BUF_RECORDS, 0x00020000);
+    return __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset_bytes, soffset_bytes, 0);
+}
+
 template <class T>
 struct VecLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;  // load instructions per stage
@@ -389,6 +398,7 @@ struct ConvLoader {
     int a_off[T::A_ITERS];
     int a_k[T::A_ITERS];
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
+    int b_k4[T::B_ITERS]; // the same in bytes of the tap table
     const float* a_base;
     ConvGeom cv;
     int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n; BUF_OOB for n >= N
@@ -410,7 +420,10 @@ struct ConvLoader {
             a_off[it] = (m0 + r < g.M) ? (r * g.lda + a_k[it]) * 4 : BUF_OOB;
         }
 #pragma unroll
-        for (int it = 0; it < T::B_ITERS; ++it) b_k[it] = (tid + it * T::THREADS) / (T::BN / 4);
+        for (int it = 0; it < T::B_ITERS; ++it) {
+            b_k[it] = (tid + it * T::THREADS) / (T::BN / 4);
+            b_k4[it] = b_k[it] * 4;
+        }
         static_assert(T::THREADS % (T::BN / 4) == 0, "a thread keeps the same 4 columns in every chunk");
         const int n = n0 + (tid % (T::BN / 4)) * 4;
         const int HW = cv.Hout * cv.Wout;
@@ -423,7 +436,7 @@ struct ConvLoader {
     __device__ __forceinline__ void prime(int k0)
     {
 #pragma unroll
-        for (int it = 0; it < T::B_ITERS; ++it) tap_next[it] = cv.tap_table[k0 + b_k[it]];
+        for (int it = 0; it < T::B_ITERS; ++it) tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], k0 * 4);
     }
 
     // byte offset of the window start of chunk `it` at stage k0, or BUF_OOB past the edges
@@ -431,7 +444,7 @@ struct ConvLoader {
     {
         const int k = k0 + b_k[it];
         const int off = k < kend ? pix4 + tap_next[it] : BUF_OOB;
-        tap_next[it] = cv.tap_table[k + T::BK];  // the table has spare entries past K
+        tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], (k0 + T::BK) * 4);  // the table has spare entries past K
         return off;
     }
 
@@ -439,7 +452,7 @@ struct ConvLoader {
     __device__ __forceinline__ int tap_offset_inside(int it, int k0) const
     {
         const int off = pix4 + tap_next[it];
-        tap_next[it] = cv.tap_table[k0 + b_k[it] + T::BK];
+        tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], (k0 + T::BK) * 4);
         return off;
     }
 
