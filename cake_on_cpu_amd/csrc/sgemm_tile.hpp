@@ -289,11 +289,21 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 static constexpr unsigned BUF_RECORDS = 0x80000000u;  // every legal offset is below, BUF_OOB is not
 static constexpr int BUF_OOB = (int)0x80000000u;
 
-__device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_offset)
+__device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_offset,
+                                                   unsigned records = BUF_RECORDS)
 {
     __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)BUF_RECORDS, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)records, 0x00020000);
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
+}
+
+// Bytes of an operand that remain after `used`, as a buffer record count: loads are range-checked
+// per 4 bytes, so a 16-byte load that hangs over the end of the operand reads zeros there
+// instead of touching memory past the allocation.
+__device__ __forceinline__ unsigned records_left(long long total_bytes, long long used_bytes)
+{
+    const long long left = total_bytes - used_bytes;
+    return left <= 0 ? 0u : left >= (long long)BUF_RECORDS ? BUF_RECORDS : (unsigned)left;
 }
 
 // 4-byte load at base + voffset (per lane) + soffset (same for the wave): the wave-uniform part of
@@ -305,15 +315,29 @@ __device__ __forceinline__ int buffer_load_i32(const int* base, int voffset_byte
     return __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset_bytes, soffset_bytes, 0);
 }
 
+// Row-major operands through 16-byte buffer loads.  Only 4-byte alignment is
+// needed, so any K, N, leading dimension and base address qualify.  A chunk is
+// 4 consecutive k of one A row, or 4 consecutive n of one B row:
+//  * rows >= M of A, columns >= N of B (whole chunks) and k >= kend read as
+//    zero through an out-of-range offset;
+//  * an A chunk that straddles kend is loaded whole and its elements past kend
+//    are zeroed when the stage is stored to LDS (by then the data has arrived,
+//    so the test never waits on memory);
+//  * a B chunk that straddles N brings in values of the next row: they only
+//    reach columns >= N of the tile, which are never stored;
+//  * the record count of each load ends at the operand's last element.
 template <class T>
 struct VecLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;  // load instructions per stage
+    static constexpr bool MASK_A_STORES = true;
     int a_off[T::A_ITERS];  // byte offset from the A tile origin, or BUF_OOB for rows >= M
     int a_k[T::A_ITERS];    // first k of the chunk inside a stage
     int b_off[T::B_ITERS];  // byte offset from the B tile origin per stage, or BUF_OOB for cols >= N
     int b_k[T::B_ITERS];    // k row of the chunk inside a stage
     const float* a_base;    // A + m0*lda
     const float* b_base;    // B + n0
+    long long a_bytes;      // from a_base to the end of A
+    long long b_bytes;      // from b_base to the end of B
     int ldb;
 
     __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
@@ -321,6 +345,8 @@ struct VecLoader {
         a_base = g.A + (size_t)m0 * g.lda;
         b_base = g.B + n0;
         ldb = g.ldb;
+        a_bytes = ((long long)(g.M - 1 - m0) * g.lda + g.K) * 4;
+        b_bytes = ((long long)(g.K - 1) * g.ldb + g.N - n0) * 4;
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) {
             const int c = tid + it * T::THREADS;
@@ -339,41 +365,66 @@ struct VecLoader {
 
     __device__ __forceinline__ void prime(int) {}  // nothing to fetch ahead
 
-    // the same for a stage that lies wholly below kend: no per-lane test, no vector ALU work
+    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
+    {
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_bytes, (long long)k0 * 4));
+    }
+    __device__ __forceinline__ f32x4 load_b(int k0, int off) const
+    {
+        const long long skip = (long long)k0 * ldb;
+        return buffer_load_f32x4(b_base + skip, off, records_left(b_bytes, skip * 4));
+    }
+
+    // chunk OP (A chunks first, then B chunks) of a stage that lies wholly below
+    // kend: no per-lane test, no vector ALU work
     template <int OP>
     __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
         if constexpr (OP < T::A_ITERS)
-            ra[OP] = buffer_load_f32x4(a_base + k0, a_off[OP]);
+            ra[OP] = load_a(k0, a_off[OP]);
         else
-            rb[OP - T::A_ITERS] = buffer_load_f32x4(b_base + (size_t)k0 * ldb, b_off[OP - T::A_ITERS]);
+            rb[OP - T::A_ITERS] = load_b(k0, b_off[OP - T::A_ITERS]);
     }
 
-    // chunk OP (A chunks first, then B chunks) of the stage starting at k0
+    // chunk OP of the stage starting at k0; chunks that start at or past kend read as zero
     template <int OP>
     __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
                                              f32x4 (&rb)[T::B_ITERS]) const
     {
         const int left = kend - k0;
         if constexpr (OP < T::A_ITERS)
-            ra[OP] = buffer_load_f32x4(a_base + k0, a_k[OP] < left ? a_off[OP] : BUF_OOB);
+            ra[OP] = load_a(k0, a_k[OP] < left ? a_off[OP] : BUF_OOB);
         else
-            rb[OP - T::A_ITERS] = buffer_load_f32x4(b_base + (size_t)k0 * ldb,
-                                                    b_k[OP - T::A_ITERS] < left ? b_off[OP - T::A_ITERS] : BUF_OOB);
+            rb[OP - T::A_ITERS] = load_b(k0, b_k[OP - T::A_ITERS] < left ? b_off[OP - T::A_ITERS] : BUF_OOB);
     }
 
-    // stage starting at k0; k >= kend reads as zero
     __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
-        const int left = kend - k0;
-        const float* a = a_base + k0;
-        const float* b = b_base + (size_t)k0 * ldb;
-#pragma unroll
-        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = buffer_load_f32x4(a, a_k[it] < left ? a_off[it] : BUF_OOB);
-#pragma unroll
-        for (int it = 0; it < T::B_ITERS; ++it) rb[it] = buffer_load_f32x4(b, b_k[it] < left ? b_off[it] : BUF_OOB);
+        load_all<0>(k0, kend, ra, rb);
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < NUM_LOADS) {
+            load_one<OP>(k0, kend, ra, rb);
+            load_all<OP + 1>(k0, kend, ra, rb);
+        }
     }
 };
+
+// A chunk W of the stage that starts at k_stage, with the elements at or past kend zeroed.
+template <class T>
+__device__ __forceinline__ f32x4 a_chunk_below(const f32x4& v, int W, int tid, int k_stage, int kend)
+{
+    const int valid = kend - k_stage - ((tid + W * T::THREADS) % (T::BK / 4)) * 4;  // elements below kend
+    f32x4 r = v;
+    if (valid < 4) r[3] = 0.f;
+    if (valid < 3) r[2] = 0.f;
+    if (valid < 2) r[1] = 0.f;
+    if (valid < 1) r[0] = 0.f;
+    return r;
+}
 
 __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_offset)
 {
@@ -395,6 +446,7 @@ __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_off
 template <class T>
 struct ConvLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + 4 * T::B_ITERS;
+    static constexpr bool MASK_A_STORES = false;  // the host only takes this path when K % 4 == 0
     int a_off[T::A_ITERS];
     int a_k[T::A_ITERS];
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
@@ -594,6 +646,7 @@ struct Slots {
 template <class L>
 struct InsideStages {
     static constexpr int NUM_LOADS = L::NUM_LOADS;
+    static constexpr bool MASK_A_STORES = false;
     const L& ld;
     template <int OP, class RA, class RB>
     __device__ __forceinline__ void load_one(int k0, int /*kend*/, RA& ra, RB& rb) const
@@ -644,7 +697,10 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
         constexpr int W = OP - N_FRAG - N_LOAD;  // store number W of the stage
         if constexpr (W < T::A_ITERS) {
             const int ch = c.tid + W * T::THREADS;
-            *reinterpret_cast<f32x4*>(c.An + (ch / (T::BK / 4)) * T::LDA + (ch % (T::BK / 4)) * 4) = c.ra[W];
+            f32x4 v = c.ra[W];
+            // the stage stored here starts one K step before the one being fetched
+            if constexpr (L::MASK_A_STORES) v = a_chunk_below<T>(v, W, c.tid, c.k_next - T::BK, c.kend);
+            *reinterpret_cast<f32x4*>(c.An + (ch / (T::BK / 4)) * T::LDA + (ch % (T::BK / 4)) * 4) = v;
         } else {
             const int ch = c.tid + (W - T::A_ITERS) * T::THREADS;
             *reinterpret_cast<f32x4*>(c.Bn + (ch / (T::BN / 4)) * T::LDB + (ch % (T::BN / 4)) * 4) = c.rb[W - T::A_ITERS];
@@ -713,6 +769,10 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     Frag<T> frag[2];
     if (steps <= 0) return;
     ld.load(kbeg, kend, ra[0], rb[0]);
+    if constexpr (L::MASK_A_STORES) {
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[0][it] = a_chunk_below<T>(ra[0][it], it, tid, kbeg, kend);
+    }
     store_stage<T>(As, Bs, tid, ra[0], rb[0]);
     ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
     __syncthreads();

@@ -158,7 +158,7 @@ def test_plan_covers_any_shape(M, N, K):
         assert pl.sched in (cake.KMN, cake.MKN, cake.NKM)
         if sch != cake.NA:
             assert pl.sched == sch
-        assert pl.vector_loads == int(K % 4 == 0 and N % 4 == 0)
+        assert pl.vector_loads == 1   # the 16-byte loader needs 4-byte alignment only
 
 
 def test_plan_tail_split():

@@ -108,6 +108,46 @@ def test_tail_split_shapes(case):
     assert np.array_equal(again, Cm)
 
 
+@pytest.mark.parametrize("shape", [(257, 1001, 255), (130, 67, 131), (512, 30, 512), (1, 5, 3), (300, 4099, 2)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_operands_at_odd_addresses(shape):
+    """Device operands that start 4, 8 and 12 bytes off a 16-byte boundary, with sizes that are
+    not multiples of 4: the 16-byte loader only needs 4-byte alignment, masks the K tail when it
+    stores a stage, and must never read past the end of an operand."""
+    import torch
+    M, K, N = shape
+    dev = torch.device("cuda:0")
+    A, B = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+    C64, S = oracle.gemm_f64(A, B)
+    for shift in (1, 2, 3):
+        print(f"sgemm odd address M={M} K={K} N={N} shift={shift}", flush=True)
+        # each operand ends exactly at the end of its allocation
+        ta = torch.empty(M * K + shift, dtype=torch.float32, device=dev)
+        tb = torch.empty(K * N + shift, dtype=torch.float32, device=dev)
+        tc = torch.full((M * N + shift,), float("nan"), dtype=torch.float32, device=dev)
+        ta[shift:].copy_(torch.from_numpy(A).reshape(-1))
+        tb[shift:].copy_(torch.from_numpy(B).reshape(-1))
+        assert ta[shift:].data_ptr() % 16 == 4 * shift
+        cake.cake_sgemm(ta[shift:], tb[shift:], tc[shift:], M, N, K, 1)
+        torch.cuda.synchronize()
+        got = tc[shift:].cpu().numpy().reshape(M, N)
+        assert oracle.max_rel_err(got, C64, S) <= TIGHT
+        assert torch.isnan(tc[:shift]).all()      # nothing written in front of C
+
+
+def test_very_long_k_takes_the_element_loader():
+    """K so long that byte offsets inside a 256-row tile pass 2^31: the 16-byte loader does not
+    apply and the per-element loader computes the product."""
+    M, K, N = 8, 2_200_000, 8
+    A, B = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+    assert cake.plan(M, N, K).vector_loads == 0   # byte offsets inside a 256-row tile would pass 2^31
+    Cm = np.zeros((M, N), np.float32)
+    print(f"sgemm long K M={M} K={K} N={N}", flush=True)
+    cake.cake_sgemm(A, B, Cm, M, N, K, 1)
+    C64, S = oracle.gemm_f64(A, B)
+    assert oracle.max_rel_err(Cm, C64, S) <= TOL
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
