@@ -178,7 +178,6 @@ struct Timer {
 
 bool fits_int(double elems) { return elems < 2147483647.0; }
 
-bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // The 16-byte loaders address a macro-tile with 32-bit byte offsets from its
 // origin: 256 rows of A (stride K) and 32 rows of B (stride N) must stay below 2^31.
@@ -750,12 +749,12 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if ((st = stage_in(weights, (size_t)Cout * K * 4, 1, true, &w))) return st;
     if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
 
-    // The on-the-fly gather needs: 4 consecutive columns inside one output row,
-    // 16-byte loadable weights, byte offsets into the (padded) input below 2^31,
+    // The on-the-fly gather needs: 4 consecutive columns inside one output row and
+    // byte offsets into the (padded) input below 2^31
     // (rows of the padded copy are a multiple of 4 floats apart, so it is written in 16-byte pieces)
     const int Hp = Hin + 2 * pad, Wp = pad > 0 ? (Win + 2 * pad + 3) & ~3 : Win;
     const double padded_elems = (double)batch * Cin * Hp * Wp;
-    const bool implicit = !explicit_cols && (Wout % 4 == 0) && (K % 4 == 0) && aligned16(w.dev) &&
+    const bool implicit = !explicit_cols && (Wout % 4 == 0) &&
                           padded_elems * 4 < 2147483648.0 &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);

@@ -446,12 +446,13 @@ __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_off
 template <class T>
 struct ConvLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + 4 * T::B_ITERS;
-    static constexpr bool MASK_A_STORES = false;  // the host only takes this path when K % 4 == 0
+    static constexpr bool MASK_A_STORES = true;   // K need not be a multiple of 4 (see VecLoader)
     int a_off[T::A_ITERS];
     int a_k[T::A_ITERS];
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
     int b_k4[T::B_ITERS]; // the same in bytes of the tap table
     const float* a_base;
+    long long a_bytes;    // from a_base to the end of A
     ConvGeom cv;
     int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n; BUF_OOB for n >= N
                           // (adding a tap offset, which is below 2^31, keeps it out of range)
@@ -463,6 +464,7 @@ struct ConvLoader {
     __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
     {
         a_base = g.A + (size_t)m0 * g.lda;
+        a_bytes = ((long long)(g.M - 1 - m0) * g.lda + g.K) * 4;
         cv = g.conv;
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) {
@@ -482,6 +484,11 @@ struct ConvLoader {
         const int b = n / HW, r = n - b * HW;
         const int ho = r / cv.Wout, wo = r - ho * cv.Wout;
         pix4 = n < g.N ? (((b * cv.Cin) * cv.Hin + ho * cv.stride) * cv.Win + wo * cv.stride) * 4 : BUF_OOB;
+    }
+
+    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
+    {
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_bytes, (long long)k0 * 4));
     }
 
     // before the first load: the stages are then fetched at k0, k0 + BK, k0 + 2 BK, ...
@@ -517,7 +524,7 @@ struct ConvLoader {
                                              f32x4 (&rb)[T::B_ITERS]) const
     {
         if constexpr (OP < T::A_ITERS) {
-            ra[OP] = buffer_load_f32x4(a_base + k0, a_k[OP] < kend - k0 ? a_off[OP] : BUF_OOB);
+            ra[OP] = load_a(k0, a_k[OP] < kend - k0 ? a_off[OP] : BUF_OOB);
         } else {
             constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
             if constexpr (e == 0) tap_off[it] = tap_offset(it, k0, kend);
@@ -530,7 +537,7 @@ struct ConvLoader {
     __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
         if constexpr (OP < T::A_ITERS) {
-            ra[OP] = buffer_load_f32x4(a_base + k0, a_off[OP]);
+            ra[OP] = load_a(k0, a_off[OP]);
         } else {
             constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
             if constexpr (e == 0) tap_off[it] = tap_offset_inside(it, k0);
@@ -566,7 +573,7 @@ struct ConvRowLoader : ConvLoader<T> {
                                              f32x4 (&rb)[T::B_ITERS]) const
     {
         if constexpr (OP < T::A_ITERS)
-            ra[OP] = buffer_load_f32x4(Base::a_base + k0, Base::a_k[OP] < kend - k0 ? Base::a_off[OP] : BUF_OOB);
+            ra[OP] = Base::load_a(k0, Base::a_k[OP] < kend - k0 ? Base::a_off[OP] : BUF_OOB);
         else
             rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset(OP - T::A_ITERS, k0, kend));
     }
@@ -575,7 +582,7 @@ struct ConvRowLoader : ConvLoader<T> {
     __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
         if constexpr (OP < T::A_ITERS)
-            ra[OP] = buffer_load_f32x4(Base::a_base + k0, Base::a_off[OP]);
+            ra[OP] = Base::load_a(k0, Base::a_off[OP]);
         else
             rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset_inside(OP - T::A_ITERS, k0));
     }

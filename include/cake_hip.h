@@ -200,7 +200,7 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * is what the reference produces for its single image); != 0: NCHW.
  *
  * cake_hip_conv2d gathers the column matrix inside the GEMM's B loader when the
- * geometry allows it (Wout % 4 == 0, Cin*Hf*Wf % 4 == 0, padded input below
+ * geometry allows it (Wout % 4 == 0, padded input below
  * 2 GiB), so the K x N intermediate is never written (with pad > 0 the input is
  * first copied once into a zero-padded image, so that the gather has no edge
  * cases); otherwise it runs the two-step path.

@@ -143,6 +143,10 @@ CONV_GEOMS = [
     (3, 5, 5, 4, 8, 3, 3, 1, 1),         # Win = 4: the row gather's narrowest image
     (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
     (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
+    (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
+    (3, 5, 8, 8, 7, 1, 1, 1, 0),         # 1x1, K = 5
+    (2, 3, 17, 17, 33, 3, 3, 2, 1),      # stride 2, K = 27, Wout = 9 (two-step) ...
+    (2, 3, 15, 16, 33, 3, 3, 2, 1),      # ... and Wout = 8 (gathered, element loads)
 ]
 
 
