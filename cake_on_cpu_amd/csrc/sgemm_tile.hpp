@@ -297,13 +297,24 @@ __device__ __forceinline__ f32x4 buffer_load_f32x4(const float* base, int byte_o
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
 }
 
-// Bytes of an operand that remain after `used`, as a buffer record count: loads are range-checked
-// per 4 bytes, so a 16-byte load that hangs over the end of the operand reads zeros there
-// instead of touching memory past the allocation.
-__device__ __forceinline__ unsigned records_left(long long total_bytes, long long used_bytes)
+// Buffer record count (bytes) for a resource that starts `used` elements into an operand of
+// `total` elements: loads are range-checked per 4 bytes, so a 16-byte load that hangs over the
+// end of the operand reads zeros there instead of touching memory past the allocation.
+// 32-bit scalar arithmetic only: this sits between MFMAs in front of every load.
+__device__ __forceinline__ unsigned records_left(unsigned total_elems, unsigned used_elems)
 {
-    const long long left = total_bytes - used_bytes;
-    return left <= 0 ? 0u : left >= (long long)BUF_RECORDS ? BUF_RECORDS : (unsigned)left;
+    // used > total only happens for stages past K, whose lanes all ask for the out-of-range
+    // offset: the difference then wraps to a large count, which is as good as any.  (Written
+    // without a saturating subtraction on purpose: that only exists as a vector instruction,
+    // and a record count in a vector register makes the compiler loop over the load.)
+    return min(total_elems - used_elems, BUF_RECORDS / 4) * 4;
+}
+
+// element count as records_left takes it (operands here stay below 2^31 elements; larger counts
+// only need to stay "large")
+__device__ __forceinline__ unsigned clamp_elems(long long n)
+{
+    return n <= 0 ? 0u : n > 0xffffffffll ? 0xffffffffu : (unsigned)n;
 }
 
 // 4-byte load at base + voffset (per lane) + soffset (same for the wave): the wave-uniform part of
@@ -336,8 +347,8 @@ struct VecLoader {
     int b_k[T::B_ITERS];    // k row of the chunk inside a stage
     const float* a_base;    // A + m0*lda
     const float* b_base;    // B + n0
-    long long a_bytes;      // from a_base to the end of A
-    long long b_bytes;      // from b_base to the end of B
+    unsigned a_elems;       // from a_base to the end of A
+    unsigned b_elems;       // from b_base to the end of B
     int ldb;
 
     __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
@@ -345,8 +356,8 @@ struct VecLoader {
         a_base = g.A + (size_t)m0 * g.lda;
         b_base = g.B + n0;
         ldb = g.ldb;
-        a_bytes = ((long long)(g.M - 1 - m0) * g.lda + g.K) * 4;
-        b_bytes = ((long long)(g.K - 1) * g.ldb + g.N - n0) * 4;
+        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
+        b_elems = clamp_elems((long long)(g.K - 1) * g.ldb + g.N - n0);
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) {
             const int c = tid + it * T::THREADS;
@@ -367,12 +378,13 @@ struct VecLoader {
 
     __device__ __forceinline__ f32x4 load_a(int k0, int off) const
     {
-        return buffer_load_f32x4(a_base + k0, off, records_left(a_bytes, (long long)k0 * 4));
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
     }
     __device__ __forceinline__ f32x4 load_b(int k0, int off) const
     {
-        const long long skip = (long long)k0 * ldb;
-        return buffer_load_f32x4(b_base + skip, off, records_left(b_bytes, skip * 4));
+        const unsigned skip = (unsigned)k0 * (unsigned)ldb;  // below 2^32: K*ldb < 2^31 and the walk
+                                                             // runs a few stages of 32 rows past K
+        return buffer_load_f32x4(b_base + skip, off, records_left(b_elems, skip));
     }
 
     // chunk OP (A chunks first, then B chunks) of a stage that lies wholly below
@@ -452,7 +464,7 @@ struct ConvLoader {
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
     int b_k4[T::B_ITERS]; // the same in bytes of the tap table
     const float* a_base;
-    long long a_bytes;    // from a_base to the end of A
+    unsigned a_elems;     // from a_base to the end of A
     ConvGeom cv;
     int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n; BUF_OOB for n >= N
                           // (adding a tap offset, which is below 2^31, keeps it out of range)
@@ -464,7 +476,7 @@ struct ConvLoader {
     __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
     {
         a_base = g.A + (size_t)m0 * g.lda;
-        a_bytes = ((long long)(g.M - 1 - m0) * g.lda + g.K) * 4;
+        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
         cv = g.conv;
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) {
@@ -488,7 +500,7 @@ struct ConvLoader {
 
     __device__ __forceinline__ f32x4 load_a(int k0, int off) const
     {
-        return buffer_load_f32x4(a_base + k0, off, records_left(a_bytes, (long long)k0 * 4));
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
     }
 
     // before the first load: the stages are then fetched at k0, k0 + BK, k0 + 2 BK, ...
