@@ -184,9 +184,9 @@ bool fits_int(double elems) { return elems < 2147483647.0; }
 bool vec4_loadable(const float* A, const float* B, int K, int N)
 {
     // the 16-byte buffer loads need 4-byte alignment only; what limits them is the 32-bit byte
-    // offset inside a tile (256 rows of A, 32 rows of B)
+    // offset inside a tile (up to 256 rows of A, 64 rows of B)
     (void)A; (void)B;
-    return (double)K * 256 * 4 < 2147483648.0 && (double)N * 32 * 4 < 2147483648.0;
+    return (double)K * 256 * 4 < 2147483648.0 && (double)N * 64 * 4 < 2147483648.0;
 }
 
 PackGeom make_geom(int M, int N, int K, int p, const cake_hip_blk_dims_t* d,
@@ -247,7 +247,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
         // packed loaders exist for a subset of the tiles
         if (plan.tile_id != TILE_256x256x32_W128x64 && plan.tile_id != TILE_128x128x32_W64x64 &&
-            plan.tile_id != TILE_64x64x32_W32x32) {
+            plan.tile_id != TILE_64x64x32_W32x32 && plan.tile_id != TILE_64x64x64_W32x32) {
             const int forced[4] = {128, 128, 32, plan.pub.split_k};
             st = plan_gemm(M, N, K, sched, forced, false, g_ctx.model, &plan);
             if (st) return fail(st, "planner failed for packed operands");

@@ -59,7 +59,8 @@ enum TileId {
     TILE_256x128x32_W64x64,       // 8 waves: N around 128 (tall-skinny)
     TILE_128x256x32_W64x64,       // 8 waves: M around 128
     TILE_128x128x32_W64x64,       // 4 waves: mid-size shapes, 2 workgroups per CU
-    TILE_64x64x32_W32x32,         // 4 waves: small shapes
+    TILE_64x64x32_W32x32,         // 4 waves: small shapes with several workgroups per CU
+    TILE_64x64x64_W32x32,         // 8 waves, two per 32x32 block of C (one per K half): small shapes, one workgroup per CU
     TILE_COUNT
 };
 

@@ -27,7 +27,8 @@ double tile_efficiency(int tile_id)
         case TILE_256x128x32_W64x64: return 0.94;
         case TILE_128x256x32_W64x64: return 0.94;
         case TILE_128x128x32_W64x64: return 0.93;
-        default: return 0.85;  // 64x64: one wave per SIMD per workgroup, 16 MFMAs between barriers
+        case TILE_64x64x32_W32x32: return 0.85;  // one wave per SIMD per workgroup, 16 MFMAs between barriers
+        default: return 0.80;  // 64x64x64 with two waves per block of C: see model_seconds
     }
 }
 
@@ -53,15 +54,20 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     const int tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
     const long wgs = (long)tiles * split;
     const int ksteps = ceil_div(ceil_div(K, split), t.bk);
-    // prologue (first stage load) and epilogue (C store) cost about two K steps
-    const double wg_flops = 2.0 * t.bm * t.bn * t.bk * (ksteps + 2);
-    const double cu_rate = dev.mfma_flops / dev.cus * tile_efficiency(tile_id);
+    const double extra = 64.0 / t.bk;  // prologue and epilogue cost about as much as 64 k of the walk
+    const double wg_flops = 2.0 * t.bm * t.bn * t.bk * (ksteps + extra);
+    double eff = tile_efficiency(tile_id);
+    // The K-split 64x64 tile pays off when the grid leaves a CU with a single workgroup: its two
+    // waves per SIMD hide each other's latencies.  With more workgroups than that the plain
+    // 64x64 tile does the same with half the LDS, so four of them share a CU.
+    if (tile_id == TILE_64x64x64_W32x32 && wgs <= dev.cus) eff = 0.88;
+    const double cu_rate = dev.mfma_flops / dev.cus * eff;
     double rounds = (double)((wgs + dev.cus - 1) / dev.cus);
     bool tail = false;
     if (split == 1 && wgs > dev.cus) {
         const int ts = tail_split_for((int)(wgs % dev.cus), ksteps, dev);
         if (ts > 1) {
-            rounds = (double)(wgs / dev.cus) + (ceil_div(ksteps, ts) + 2.0) / (ksteps + 2.0);
+            rounds = (double)(wgs / dev.cus) + (ceil_div(ksteps, ts) + extra) / (ksteps + extra);
             tail = true;
         }
     }

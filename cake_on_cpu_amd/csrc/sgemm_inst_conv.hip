@@ -13,6 +13,7 @@ hipError_t launch_sgemm_conv(int tile_id, const GemmArgs& a, int grid, hipStream
         case TILE_128x256x32_W64x64: return launch_tile<Tile128x256x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
         case TILE_128x128x32_W64x64: return launch_tile<Tile128x128x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
         case TILE_64x64x32_W32x32: return launch_tile<Tile64x64x32, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
+        case TILE_64x64x64_W32x32: return launch_tile<Tile64x64x64, LOAD_VEC4, LOAD_IM2COL>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }

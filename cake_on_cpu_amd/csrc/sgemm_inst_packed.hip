@@ -21,6 +21,7 @@ hipError_t launch_sgemm_packed(int tile_id, int a_mode, int b_mode, const GemmAr
         case TILE_256x256x32_W128x64: return by_mode<Tile256x256x32>(a_mode, b_mode, a, grid, s);
         case TILE_128x128x32_W64x64: return by_mode<Tile128x128x32>(a_mode, b_mode, a, grid, s);
         case TILE_64x64x32_W32x32: return by_mode<Tile64x64x32>(a_mode, b_mode, a, grid, s);
+        case TILE_64x64x64_W32x32: return by_mode<Tile64x64x64>(a_mode, b_mode, a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }

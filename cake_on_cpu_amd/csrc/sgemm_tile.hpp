@@ -42,13 +42,20 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // register -> LDS stores are issued.  1 puts them in the group that ends at the
 // barrier; 2 gives them a whole group to land first, which matters when a group
 // is only a few MFMAs long and nothing else would cover the wait at the barrier.
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int REG_STAGES_ = 1, int STORE_LEAD_ = 1>
+// KSPLIT: how many waves share each WM x WN block of C, each taking its own
+// BK / KSPLIT slice of every K stage (summed once through LDS after the walk).
+// A 32x32 wave tile has only 16 MFMAs per 32 k, too few to hide its own LDS and
+// barrier latencies when it is alone on its SIMD; with KSPLIT = 2 every SIMD
+// holds two waves of the workgroup even when the grid is one workgroup per CU.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int REG_STAGES_ = 1, int STORE_LEAD_ = 1, int KSPLIT_ = 1>
 struct Tile {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int REG_STAGES = REG_STAGES_;
     static constexpr int STORE_LEAD = STORE_LEAD_;
+    static constexpr int KSPLIT = KSPLIT_;
+    static constexpr int WAVE_BK = BK / KSPLIT;        // k extent of a stage that one wave multiplies
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
-    static constexpr int THREADS = WAVES_M * WAVES_N * 64;
+    static constexpr int THREADS = WAVES_M * WAVES_N * KSPLIT * 64;
     static constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 MFMA tiles per wave
     static constexpr int LDA = BK + 4;                 // floats; 16-byte reads of 8 consecutive rows hit 8 distinct bank quads
     static constexpr int LDB = BN + 8;                 // floats; rows k and k+4 land 32 banks apart
@@ -60,7 +67,8 @@ struct Tile {
     static constexpr int A_ITERS = A_CHUNKS / THREADS;
     static constexpr int B_ITERS = B_CHUNKS / THREADS;
     static_assert(BM % WM == 0 && BN % WN == 0 && WM % 32 == 0 && WN % 32 == 0, "wave tiling");
-    static_assert(BK % 8 == 0, "K step is consumed 8 deep");
+    static_assert(BK % KSPLIT == 0 && WAVE_BK % 8 == 0, "K step is consumed 8 deep");
+    static_assert(KSPLIT == 1 || BM * BN * 4 <= LDS_BYTES, "the K halves are summed through the stage memory");
     static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "stage loaders");
 };
 
@@ -247,17 +255,20 @@ struct Frag {
 };
 
 template <class T>
-__device__ __forceinline__ void load_frag(const float* As, const float* Bs, int a_row, int b_col,
+// a_lane / b_lane: where the lane's operands start inside a stage (floats):
+// its row of A (times LDA) and its column of B, plus the wave's K slice of the
+// stage when several waves share a block of C.
+__device__ __forceinline__ void load_frag(const float* As, const float* Bs, int a_lane, int b_lane,
                                           int lh, int kg, Frag<T>& f)
 {
     const int kk = kg * 8 + lh * 4;
 #pragma unroll
     for (int tm = 0; tm < T::TM; ++tm)
-        f.a[tm] = *reinterpret_cast<const f32x4*>(As + (a_row + tm * 32) * T::LDA + kk);
+        f.a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + kk);
 #pragma unroll
     for (int tn = 0; tn < T::TN; ++tn)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) f.b[tn][i] = Bs[(kk + i) * T::LDB + b_col + tn * 32];
+        for (int i = 0; i < 4; ++i) f.b[tn][i] = Bs[(kk + i) * T::LDB + b_lane + tn * 32];
 }
 
 template <class T>
@@ -622,7 +633,7 @@ struct ConvRowLoader : ConvLoader<T> {
 // between MFMAs they ride in the shadow of the 64-cycle matrix instruction
 // instead.  Each group of 8 k is therefore cut into slots of a few MFMAs plus
 // ONE memory instruction, and __builtin_amdgcn_sched_barrier(0) after every
-// slot keeps the compiler from regrouping them.  With NKG = BK/8 groups:
+// slot keeps the compiler from regrouping them.  With NKG = WAVE_BK/8 groups:
 //     groups 0..    : LDS reads of the next group's operands
 //     group NKG-2   : ... + registers (stage s+1) -> the other LDS buffer
 //     ---- the step's one barrier ----
@@ -636,7 +647,7 @@ struct ConvRowLoader : ConvLoader<T> {
 // more, and it is only overwritten a whole step later.)
 template <class T, class L>
 struct Slots {
-    static constexpr int NKG = T::BK / 8;
+    static constexpr int NKG = T::WAVE_BK / 8;      // operand groups of 8 k a wave walks per stage
     static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
     static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
     static constexpr int LOAD_OPS = L::NUM_LOADS;               // global load instructions per stage
@@ -683,7 +694,7 @@ struct WalkCtx {
     const float* Bc;
     float* An;
     float* Bn;
-    int tid, a_row, b_col, lh;
+    int tid, a_lane, b_lane, lh;
     f32x4 (&ra)[T::A_ITERS];  // register stage that this step stores to LDS
     f32x4 (&rb)[T::B_ITERS];
     f32x4 (&la)[T::A_ITERS];  // register stage that this step's global loads fill
@@ -705,10 +716,10 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
         const float* B = wrap ? c.Bn : c.Bc;
         const int kk = (wrap ? 0 : KG + 1) * 8 + c.lh * 4;
         if constexpr (OP < T::TM) {
-            next.a[OP] = *reinterpret_cast<const f32x4*>(A + (c.a_row + OP * 32) * T::LDA + kk);
+            next.a[OP] = *reinterpret_cast<const f32x4*>(A + c.a_lane + OP * 32 * T::LDA + kk);
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
-            next.b[tn][i] = B[(kk + i) * T::LDB + c.b_col + tn * 32];
+            next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
         }
     } else if constexpr (OP < N_FRAG + N_LOAD) {
         c.ld.template load_one<S::load_begin(KG) + OP - N_FRAG>(c.k_next, c.kend, c.la, c.lb);
@@ -775,8 +786,8 @@ __device__ __forceinline__ void step_groups(const WalkCtx<T, L>& c, Frag<T> (&fr
 
 template <class T, class L>
 __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
-                                           int kbeg, int kend, int steps, int tid, int a_row,
-                                           int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
+                                           int kbeg, int kend, int steps, int tid, int a_lane,
+                                           int b_lane, int lh, f32x16 (&acc)[T::TM][T::TN])
 {
     static_assert(Slots<T, L>::NKG % 2 == 0, "operand double buffer must come back to slot 0 every step");
     constexpr int RS = T::REG_STAGES;
@@ -795,7 +806,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     store_stage<T>(As, Bs, tid, ra[0], rb[0]);
     ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
     __syncthreads();
-    load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
+    load_frag<T>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
 
     // One K step s: stage s is in LDS, stage s+1 waits in registers.  The step
     // stores stage s+1 to the other LDS buffer and fetches stage s+2 -- with two
@@ -810,7 +821,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
         const WalkCtx<T, LD> c{loader, kbeg + (s + 2) * T::BK, kend,
                                As + cur * T::A_STAGE, Bs + cur * T::B_STAGE,
                                As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE,
-                               tid, a_row, b_col, lh, sa, sb, fa, fb};
+                               tid, a_lane, b_lane, lh, sa, sb, fa, fb};
         __builtin_amdgcn_sched_barrier(0);
         step_groups<T, LD>(c, frag, acc);
         cur ^= 1;
@@ -840,10 +851,10 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
 // the next stage issued first; correctness path, not tuned.
 template <class T, int A_MODE, int B_MODE>
 __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
-                                               int kbeg, int kend, int steps, int tid, int a_row,
-                                               int b_col, int lh, f32x16 (&acc)[T::TM][T::TN])
+                                               int kbeg, int kend, int steps, int tid, int a_lane,
+                                               int b_lane, int lh, f32x16 (&acc)[T::TM][T::TN])
 {
-    constexpr int NKG = T::BK / 8;
+    constexpr int NKG = T::WAVE_BK / 8;
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
     Frag<T> frag[2];
     if (steps > 0) {
@@ -852,7 +863,7 @@ __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, flo
         store_stage<T>(As, Bs, tid, ra, rb);
     }
     __syncthreads();
-    if (steps > 0) load_frag<T>(As, Bs, a_row, b_col, lh, 0, frag[0]);
+    if (steps > 0) load_frag<T>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
 
     int cur = 0;
     for (int s = 0; s < steps; ++s) {
@@ -866,14 +877,14 @@ __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, flo
         }
 #pragma unroll
         for (int kg = 0; kg < NKG; ++kg) {
-            if (kg + 1 < NKG) load_frag<T>(Ac, Bc, a_row, b_col, lh, kg + 1, frag[(kg + 1) & 1]);
+            if (kg + 1 < NKG) load_frag<T>(Ac, Bc, a_lane, b_lane, lh, kg + 1, frag[(kg + 1) & 1]);
             if (kg == NKG - 1 && more)
                 store_stage<T>(As + (cur ^ 1) * T::A_STAGE, Bs + (cur ^ 1) * T::B_STAGE, tid, ra, rb);
             mma_frag<T>(frag[kg & 1], acc);
         }
         __syncthreads();
         cur ^= 1;
-        if (more) load_frag<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, a_row, b_col, lh, 0, frag[0]);
+        if (more) load_frag<T>(As + cur * T::A_STAGE, Bs + cur * T::B_STAGE, a_lane, b_lane, lh, 0, frag[0]);
     }
 }
 
@@ -887,8 +898,13 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int wm0 = (wave / T::WAVES_N) * T::WM;
-    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    // waves that share a block of C sit WAVES_M * WAVES_N apart, i.e. on the same SIMD
+    const int ks = wave / (T::WAVES_M * T::WAVES_N);
+    const int wblk = wave % (T::WAVES_M * T::WAVES_N);
+    const int wm0 = (wblk / T::WAVES_N) * T::WM;
+    const int wn0 = (wblk % T::WAVES_N) * T::WN;
+    const int a_lane = (wm0 + l32) * T::LDA + ks * T::WAVE_BK;
+    const int b_lane = wn0 + l32 + ks * T::WAVE_BK * T::LDB;
 
     const WorkItem w = decode_tile(g, blockIdx.x);
     const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
@@ -904,16 +920,41 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
     if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4)
-        k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+        k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL)
-        k_walk_vec<T, ConvLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+        k_walk_vec<T, ConvLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
-        k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+        k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else
-        k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, wm0 + l32, wn0 + l32, lh, acc);
+        k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
 
-    // Epilogue.  Accumulator register r of a 32x32 tile holds row
-    // 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // Accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    if constexpr (T::KSPLIT > 1) {
+        // sum the K slices of each block of C in slice order, through the stage memory
+        static_assert(T::KSPLIT == 2, "two waves per block of C");
+        __syncthreads();  // nobody reads operands any more
+        float* red = smem + ((wm0 + 4 * lh) * T::BN + wn0 + l32);
+        if (ks == 1) {
+#pragma unroll
+            for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        red[(tm * 32 + 8 * (r >> 2) + (r & 3)) * T::BN + tn * 32] = acc[tm][tn][r];
+        }
+        __syncthreads();
+        if (ks == 1) return;
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[tm][tn][r] += red[(tm * 32 + 8 * (r >> 2) + (r & 3)) * T::BN + tn * 32];
+    }
+
+    // Epilogue.
     if (w.tail_tile >= 0) {
         // a K slice of a tail tile: the whole BM x BN block, tile-local, no masking
         float* out = g.tail_partial + ((size_t)w.slice * g.tail_tiles + w.tail_tile) * (T::BM * T::BN);
@@ -1011,5 +1052,6 @@ using Tile256x128x32 = Tile<256, 128, 32, 64, 64, 2>;
 using Tile128x256x32 = Tile<128, 256, 32, 64, 64, 2>;
 using Tile128x128x32 = Tile<128, 128, 32, 64, 64, 2>;
 using Tile64x64x32 = Tile<64, 64, 32, 32, 32, 2, 2>;
+using Tile64x64x64 = Tile<64, 64, 64, 32, 32, 2, 2, 2>;
 
 }  // namespace cake

@@ -80,7 +80,7 @@ typedef struct cake_hip_plan_t {
     int group;        /* CB-block edge in tiles: tiles that run together share panels */
     int grid;         /* workgroups launched                                      */
     int lds_bytes;    /* LDS per workgroup (double buffered)                      */
-    int vector_loads; /* 1: 16-byte global loads usable (K below 2M and N below 16M floats) */
+    int vector_loads; /* 1: 16-byte global loads usable (K below 2M and N below 8M floats) */
     int cus;          /* compute units the plan was made for                      */
     double flops;     /* 2*M*N*K                                                  */
     double min_bytes; /* compulsory traffic 4*(MK+KN+MN)                          */

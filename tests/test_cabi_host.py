@@ -231,10 +231,10 @@ def test_tune_table_load_lookup_save_clear(tmp_path):
         src = tmp_path / "tuned.txt"
         src.write_text("# comment\n"
                        "4096 4096 4096 1 128 128 32 2 0 0.001\n"      # taken
-                       "4096 4096 4096 0 64 64 32 1 1 0.002\n"        # taken (operands not 16-byte loadable)
+                       "4096 4096 4096 0 64 64 64 1 1 0.002\n"        # taken (operands not 16-byte loadable)
                        "this line is not an entry\n"
                        "10 10 10 1 96 96 32 1 0 1.0\n"                # no such tile: skipped
-                       "64 64 64 1 64 64 32 9 0 1.0\n")               # more slices than K steps: skipped
+                       "64 64 64 1 64 64 64 9 0 1.0\n")               # more slices than K steps: skipped
         assert cake.tune_load(src) == 2 and cake.tune_count() == 2
         tuned = cake.plan(4096, 4096, 4096).as_dict()
         assert (tuned["tile_m"], tuned["tile_n"], tuned["split_k"], tuned["tail_tiles"]) == (128, 128, 2, 0)
@@ -245,7 +245,7 @@ def test_tune_table_load_lookup_save_clear(tmp_path):
         dst = tmp_path / "saved.txt"
         cake.tune_save(dst)
         rows = [l.split() for l in dst.read_text().splitlines() if not l.startswith("#")]
-        assert sorted(r[:9] for r in rows) == [["4096", "4096", "4096", "0", "64", "64", "32", "1", "1"],
+        assert sorted(r[:9] for r in rows) == [["4096", "4096", "4096", "0", "64", "64", "64", "1", "1"],
                                                ["4096", "4096", "4096", "1", "128", "128", "32", "2", "0"]]
         cake.tune_clear()
         assert cake.tune_count() == 0 and cake.plan(4096, 4096, 4096).as_dict() == default
