@@ -235,7 +235,7 @@ size_t tables_bytes(int which, const PackGeom& g)
 // The GEMM proper on device operands.
 int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
              int sched, int accumulate, const int* tile_override, int a_mode, int b_mode,
-             IndexTables a_tab, IndexTables b_tab, hipStream_t stream, Timer& timer,
+             hipStream_t stream, Timer& timer,
              const ConvGeom* conv = nullptr, const float* col_bias = nullptr,
              const TunedChoice* choice = nullptr)
 {
@@ -244,15 +244,6 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec, g_ctx.model, &plan)
                     : plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);
     if (st) return fail(st, "no tile matches the requested override");
-    if (a_mode == LOAD_PACKED || b_mode == LOAD_PACKED) {
-        // packed loaders exist for a subset of the tiles
-        if (plan.tile_id != TILE_256x256x32_W128x64 && plan.tile_id != TILE_128x128x32_W64x64 &&
-            plan.tile_id != TILE_64x64x32_W32x32 && plan.tile_id != TILE_64x64x64_W32x32) {
-            const int forced[4] = {128, 128, 32, plan.pub.split_k};
-            st = plan_gemm(M, N, K, sched, forced, false, g_ctx.model, &plan);
-            if (st) return fail(st, "planner failed for packed operands");
-        }
-    }
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C;
     g.M = M; g.N = N; g.K = K;
@@ -262,7 +253,6 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
     g.accumulate = accumulate;
     g.col_bias = col_bias;
-    g.a_tab = a_tab; g.b_tab = b_tab;
     if (conv) g.conv = *conv;
     const int nchw_hw = (conv && conv->out_nchw) ? conv->Hout * conv->Wout : 0;
     g.partial = nullptr;
@@ -481,7 +471,7 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
         const bool vec = vec4_loadable(a.dev, b.dev, K, N);
         const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
         st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, tile_override, mode,
-                      mode, IndexTables{}, IndexTables{}, stream, timer);
+                      mode, stream, timer);
         if (st) return st;
     }
     if ((st = timer.stop())) return st;
@@ -615,16 +605,31 @@ int cake_hip_sgemm_packed(const float* A, const float* B, float* C, int M, int N
     if ((st = stage_in(B, b_elems * 4, 1, true, &b))) return st;
     if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;
     if ((st = g_ctx.tables.reserve((packedA ? tables_bytes(0, g) : 0) + (packedB ? tables_bytes(1, g) : 0)))) return st;
+    // A packed operand is first copied back to row-major order (one pass at HBM speed through
+    // the index tables); the product then runs on the row-major kernel, which is several times
+    // faster than gathering packed elements inside the K walk.
+    const size_t ua_floats = packedA ? (((size_t)M * K + 63) & ~(size_t)63) : 0;
+    const size_t ub_floats = packedB ? (size_t)K * N : 0;
+    if ((st = g_ctx.unpacked.reserve((ua_floats + ub_floats) * sizeof(float)))) return st;
+    float* ua = static_cast<float*>(g_ctx.unpacked.ptr);
+    float* ub = ua + ua_floats;
 
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
     size_t at = 0;
     IndexTables ta{}, tb{};
-    if (packedA && (st = build_tables(0, g, &at, &ta, stream))) return st;
-    if (packedB && (st = build_tables(1, g, &at, &tb, stream))) return st;
-    st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, nullptr,
-                  packedA ? LOAD_PACKED : LOAD_SCALAR, packedB ? LOAD_PACKED : LOAD_SCALAR, ta, tb,
-                  stream, timer);
+    if (packedA) {
+        if ((st = build_tables(0, g, &at, &ta, stream))) return st;
+        if ((st = timer.family(4, [&] { return launch_unpack(a.dev, ua, M, K, K, ta, stream); }))) return st;
+    }
+    if (packedB) {
+        if ((st = build_tables(1, g, &at, &tb, stream))) return st;
+        if ((st = timer.family(4, [&] { return launch_unpack(b.dev, ub, K, N, N, tb, stream); }))) return st;
+    }
+    const float* ga = packedA ? ua : a.dev;
+    const float* gb = packedB ? ub : b.dev;
+    const int mode = vec4_loadable(ga, gb, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
+    st = run_gemm(ga, gb, c.dev, M, N, K, K, N, N, sched, accumulate, nullptr, mode, mode, stream, timer);
     if (st) return st;
     if ((st = timer.stop())) return st;
     return stage_out(c, stream);
@@ -790,7 +795,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         // stride 1: 4 consecutive columns are one 16-byte load from an image row
         const int b_mode = stride == 1 ? LOAD_IM2COL_ROW : LOAD_IM2COL;
         st = run_gemm(w.dev, nullptr, o.dev, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
-                      b_mode, IndexTables{}, IndexTables{}, stream, timer, &cv);
+                      b_mode, stream, timer, &cv);
         if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);
@@ -818,7 +823,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const bool vec = vec4_loadable(w.dev, cols, K, N);
     const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
     st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode,
-                  IndexTables{}, IndexTables{}, stream, timer);
+                  stream, timer);
     if (st) return st;
     if (out_nchw) {
         st = timer.family(3, [&] { return launch_cn_to_nchw(cn, o.dev, batch, Cout, Hout * Wout, stream); });
@@ -886,7 +891,7 @@ static int linear_gemm(const float* A, const float* B, float* C, int M, int N, i
         return e == hipSuccess ? CAKE_HIP_OK : fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
     }
     const int mode = vec4_loadable(A, B, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
-    return run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, IndexTables{}, IndexTables{},
+    return run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode,
                     stream, timer, nullptr, col_bias);
 }
 
@@ -1021,8 +1026,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
             const int reps = pass == 0 ? 1 : (est < 2e-4 ? 20 : est < 5e-3 ? 5 : 2);
             HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
             for (int r = 0; r < reps; ++r) {
-                int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, IndexTables{},
-                                 IndexTables{}, stream, untimed, nullptr, nullptr, &c);
+                int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, stream, untimed, nullptr, nullptr, &c);
                 if (e) return e;
             }
             HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));

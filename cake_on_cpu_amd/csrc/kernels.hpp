@@ -49,7 +49,6 @@ struct GemmArgs {
     // launch_tail_reduce.  0 tail_tiles = off.  Not combined with split_k > 1.
     int tail_tiles, tail_split, tail_k_per_split;
     float* tail_partial;
-    IndexTables a_tab, b_tab;  // used by the packed-operand loaders only
     ConvGeom conv;             // used by the implicit-im2col loader only
 };
 
@@ -73,7 +72,6 @@ const TileInfo& tile_info(int tile_id);
 enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
-    LOAD_PACKED = 2, // reference packed layout through IndexTables
     LOAD_IM2COL = 3, // B only: column matrix of a convolution gathered from the NCHW input
     LOAD_IM2COL_ROW = 4  // the same for stride 1: one 16-byte load per 4 columns
 };

@@ -165,22 +165,12 @@ __device__ __forceinline__ void load_a_stage(const GemmArgs& g, int m0, int k0, 
         if (MODE == LOAD_VEC4) {
             if (row < g.M && col < kend)
                 v = *reinterpret_cast<const f32x4*>(g.A + (size_t)row * g.lda + col);
-        } else if (MODE == LOAD_SCALAR) {
+        } else {
             if (row < g.M) {
                 const float* src = g.A + (size_t)row * g.lda + col;
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (col + e < kend) v[e] = src[e];
-            }
-        } else {
-            if (row < g.M) {
-                const int4 R = g.a_tab.row[row];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (col + e < kend) {
-                        const int4 Cc = g.a_tab.col[col + e];
-                        v[e] = g.A[(size_t)(R.x + Cc.x + R.y * Cc.y + R.z * Cc.z + R.w * Cc.w)];
-                    }
             }
         }
         ra[it] = v;
@@ -201,22 +191,12 @@ __device__ __forceinline__ void load_b_stage(const GemmArgs& g, int n0, int k0, 
         if (MODE == LOAD_VEC4) {
             if (row < kend && col < g.N)
                 v = *reinterpret_cast<const f32x4*>(g.B + (size_t)row * g.ldb + col);
-        } else if (MODE == LOAD_SCALAR) {
+        } else {
             if (row < kend) {
                 const float* src = g.B + (size_t)row * g.ldb + col;
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (col + e < g.N) v[e] = src[e];
-            }
-        } else {
-            if (row < kend) {
-                const int4 R = g.b_tab.row[row];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (col + e < g.N) {
-                        const int4 Cc = g.b_tab.col[col + e];
-                        v[e] = g.B[(size_t)(R.x + Cc.x + R.y * Cc.y + R.z * Cc.z + R.w * Cc.w)];
-                    }
             }
         }
         rb[it] = v;
@@ -847,7 +827,7 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
 }
 
 // K walk for operands that need per-element addressing (any alignment, or the
-// reference's packed layouts).  Same double-buffered pipeline with the loads of
+// K far beyond the 16-byte loader.s reach).  Same double-buffered pipeline with the loads of
 // the next stage issued first; correctness path, not tuned.
 template <class T, int A_MODE, int B_MODE>
 __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, float* Bs, int m0, int n0,
