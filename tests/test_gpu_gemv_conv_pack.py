@@ -185,6 +185,27 @@ def test_conv2d_paths_agree_bitwise_layouts():
     assert np.array_equal(a, b)
 
 
+def test_conv2d_with_a_caller_workspace_on_device_tensors():
+    """Device operands and a caller-owned workspace of cake_hip_conv2d_workspace bytes, offset so it
+    is not 256-byte aligned: both paths must give what they give with the library's own buffer."""
+    import torch
+    dev = torch.device("cuda:0")
+    Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad = 3, 12, 18, 20, 40, 3, 3, 1, 1
+    inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 58), oracle.uniform((Cout, Cin, Hf, Wf), 59)
+    want = np.empty((Bn, Cout, Hin, Win), np.float32)
+    cake.conv2d(inp, wt, want, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=True)
+    need = cake.load().cake_hip_conv2d_workspace(Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)
+    assert need >= 4 * Cin * 9 * Bn * Hin * Win
+    ws = torch.empty((need + 3) // 4 + 1, dtype=torch.float32, device=dev)[1:]
+    ti, tw = torch.from_numpy(inp).to(dev), torch.from_numpy(wt).to(dev)
+    for explicit in (False, True):
+        out = torch.full((Bn, Cout, Hin, Win), float("nan"), dtype=torch.float32, device=dev)
+        cake.conv2d(ti, tw, out, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=True,
+                    workspace=ws, explicit_im2col=explicit)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want)
+
+
 # ---------------------------------------------------------------------------
 # packed layouts
 # ---------------------------------------------------------------------------
