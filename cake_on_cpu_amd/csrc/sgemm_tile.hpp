@@ -33,6 +33,7 @@ namespace cake {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));  // 16 bytes at any 4-byte address
 
 // REG_STAGES: how many K stages' worth of registers sit between the global loads
 // and the LDS stores (the 16-byte loaders only).  With 2, a step's loads go into
@@ -954,30 +955,64 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
     const bool nchw = (B_MODE == LOAD_IM2COL || B_MODE == LOAD_IM2COL_ROW) && g.conv.out_nchw && g.partial == nullptr;
     const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
+    // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
+    // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
+    // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
+    // quarter of the store instructions, and rows written in runs of WN floats.
+    constexpr int PITCH = T::WN + 4;            // floats between rows of the wave's staging block
+    constexpr int CH = T::WN / 4;               // 16-byte pieces per row
+    constexpr int ROWS = 64 / CH;               // rows one wave-wide 16-byte read covers
+    static_assert(T::WAVES_M * T::WAVES_N * 32 * PITCH * 4 <= T::LDS_BYTES, "staging blocks fit the stage memory");
+    __syncthreads();  // nobody reads operand stages any more
+    float* wbuf = smem + wblk * (32 * PITCH);
+    const int rd_row = lane / CH, rd_col = (lane % CH) * 4;
+    const int col = n0 + wn0 + rd_col;          // first of the lane's 4 columns
+    size_t col_off = col;
+    size_t row_stride = ldo;
+    if (nchw) {  // 4 consecutive n stay inside one image (Hout*Wout % 4 == 0 on this path)
+        const int b = col / HW;
+        col_off = (size_t)b * g.M * HW + (col - b * HW);
+        row_stride = HW;
+    }
+    f32x4 bias_v = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
 #pragma unroll
-    for (int tm = 0; tm < T::TM; ++tm)
+        for (int e = 0; e < 4; ++e)
+            if (col + e < g.N) bias_v[e] = bias[col + e];
+    }
+    const bool whole = col + 3 < g.N;
 #pragma unroll
-        for (int tn = 0; tn < T::TN; ++tn) {
-            const int col = n0 + wn0 + tn * 32 + l32;
-            size_t col_off = col;
-            size_t row_stride = ldo;
-            if (nchw) {
-                const int b = col / HW;
-                col_off = (size_t)b * g.M * HW + (col - b * HW);
-                row_stride = HW;
-            }
-            const float bias_v = (bias && col < g.N) ? bias[col] : 0.f;
+    for (int tm = 0; tm < T::TM; ++tm) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                if (row < g.M && col < g.N) {
-                    float* dst = out + (size_t)row * row_stride + col_off;
-                    float v = add ? *dst + acc[tm][tn][r] : acc[tm][tn][r];
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                wbuf[(8 * (r >> 2) + 4 * lh + (r & 3)) * PITCH + tn * 32 + l32] = acc[tm][tn][r];
+        // LDS serves a wave's requests in order, so the reads below see the writes above
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS; ++pass) {
+            const int lr = pass * ROWS + rd_row;
+            const int row = m0 + wm0 + tm * 32 + lr;
+            f32x4 v = *reinterpret_cast<const f32x4*>(wbuf + lr * PITCH + rd_col);
+            if (row < g.M && col < g.N) {
+                float* dst = out + (size_t)row * row_stride + col_off;
+                if (whole) {
+                    f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst);
+                    if (add) v += *d4;
                     if (bias) v += bias_v;
-                    *dst = v;
+                    *d4 = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < g.N) {
+                            float x = add ? dst[e] + v[e] : v[e];
+                            if (bias) x += bias_v[e];
+                            dst[e] = x;
+                        }
                 }
             }
         }
+    }
 }
 
 // C tile = (accumulate ? C : 0) + sum over the K slices of a tail tile, in
