@@ -189,6 +189,27 @@ def test_compute_without_gpu_fails_loudly():
     assert e.value.status == _lib.ERR_NO_DEVICE
 
 
+def test_missing_library_fails_loudly(tmp_path):
+    """No CPU fallback: without libcake_hip.so the package refuses to load, in a fresh
+    interpreter so that this process keeps its own library."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, pathlib\n"
+        "sys.path.insert(0, %r)\n"
+        "from cake_on_cpu_amd import _lib\n"
+        "_lib.LIB_PATH = pathlib.Path(%r) / 'libcake_hip.so'\n"
+        "import cake_on_cpu_amd as cake\n"
+        "try:\n"
+        "    cake.plan(8, 8, 8)\n"
+        "except ImportError as e:\n"
+        "    print('ImportError', 'no CPU fallback' in str(e))\n"
+        "else:\n"
+        "    print('loaded something')\n" % (str(Path(__file__).resolve().parents[1]), str(tmp_path)))
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert res.stdout.strip() == "ImportError True", (res.stdout, res.stderr[-500:])
+
+
 def test_entry_points_reject_bad_arguments_before_touching_a_device():
     """Argument and range checks come first, so they read the same with or without a GPU:
     negative sizes, unknown schedules, NULL operands and operands of 2^31 elements or more
