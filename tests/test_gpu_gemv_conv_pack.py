@@ -283,3 +283,48 @@ def test_cpp_dropin_program():
     res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=600)
     print(res.stdout[-3000:], res.stderr[-2000:])
     assert res.returncode == 0 and "ALL PASS" in res.stdout
+
+
+# ---------------------------------------------------------------------------
+# committed outputs of the reference's own compiled code (tests/golden/reference_vectors.npz)
+# ---------------------------------------------------------------------------
+def test_device_kernels_against_reference_golden_vectors():
+    """pack_A/B/C, unpack_C, im_2_col bit for bit and cake_sgemv within tolerance against what
+    the reference's own pack_*.cpp, unpack_*.cpp, im_2_col and schedule_mvm produced."""
+    from tests import golden_vectors
+    meta, Z = golden_vectors.load()
+    seed = meta["seeds"]
+    ocx, ccx = _cx()
+    for i, (M, K, N, p, sch) in enumerate(meta["pack"]):
+        print(f"golden pack M={M} K={K} N={N} p={p} sch={sch}", flush=True)
+        xc = cake.init_block_dims(M, N, K, p, ccx, sch)
+        assert [getattr(xc, n) for n in oracle.BLK_FIELDS] == Z[f"pack{i}_dims"].tolist()
+        xo = golden_vectors.blk_dims(Z[f"pack{i}_dims"])
+        A, B, Cm = oracle.uniform((M, K), seed["A"]), oracle.uniform((K, N), seed["B"]), oracle.uniform((M, N), seed["C"])
+        Ap = np.full(cake.cake_sgemm_packed_A_size(M, K, p, xc, ccx, sch) // 4, np.nan, np.float32)
+        cake.pack_A(A, Ap, M, K, p, xc, ccx, sch)
+        assert np.array_equal(Ap, Z[f"pack{i}_A"])
+        Bp = np.full(cake.cake_sgemm_packed_B_size(K, N, p, xc, ccx) // 4, np.nan, np.float32)
+        cake.pack_B(B, Bp, K, N, p, xc, ccx, sch)
+        real = oracle.pack_B(np.ones((K, N), np.float32), p, xo, ocx, sch) != 0
+        assert np.array_equal(Bp[real], Z[f"pack{i}_B"][real]) and not Bp[~real].any()
+        Cp = oracle.uniform(cake.cake_sgemm_packed_C_size(M, N, p, xc, ccx, sch) // 4, seed["Cp"])
+        back = np.full((M, N), 7.0, np.float32)
+        cake.unpack_C(back, Cp, M, N, p, xc, ccx, sch)
+        assert np.array_equal(back, Z[f"pack{i}_Cunpacked"])
+        if not (sch == cake.NKM and xc.m_pad):
+            Cpk = np.full(Cp.size, np.nan, np.float32)
+            cake.pack_C(Cm, Cpk, M, N, p, xc, ccx, sch)
+            assert np.array_equal(Cpk, Z[f"pack{i}_Cpacked"])
+    for (M, K, p) in meta["gemv"]:
+        print(f"golden gemv M={M} K={K}", flush=True)
+        A, xv, y = oracle.uniform(M * K, seed["gemv_A"]), oracle.uniform(K, seed["gemv_x"]), oracle.uniform(M, seed["gemv_y"]).copy()
+        cake.cake_sgemv(A, xv, y, M, K, p)
+        ref = Z[f"gemv_{M}_{K}_{p}"]
+        _, S = oracle.gemv_f64(A, xv, M, K, True)
+        assert np.max(np.abs(y - ref) / np.maximum(S + 1.0, 1e-30)) <= 1e-6
+    for (Cin, Hin, Win, Hf, Wf) in meta["im2col"]:
+        print(f"golden im_2_col Cin={Cin} {Hin}x{Win} filter {Hf}x{Wf}", flush=True)
+        inp = oracle.uniform((Cin, Hin, Win), seed["image"])
+        cols = cake.im_2_col(inp, Wf, Hf, Win, Hin, Win - Wf + 1, Hin - Hf + 1, Cin)
+        assert np.array_equal(cols, Z[f"im2col_{Cin}_{Hin}_{Win}_{Hf}_{Wf}"])

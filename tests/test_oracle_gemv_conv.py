@@ -21,9 +21,13 @@ def test_sgemv_matches_reference_sources(M, K, p):
     xv = oracle.uniform(K, 42)
     y0 = oracle.uniform(M, 43)
     mine = oracle.cake_sgemv(A, xv, p, cx, y0=y0, M=M, K=K)
-    ref = y0.copy()
-    L.ref_schedule_mvm(refparts.f(A), refparts.f(xv), refparts.f(ref), M, K, p, refparts.dims_array(x), 8)
-    assert np.array_equal(mine, ref)
+    def slack(a):  # the reference's 8-row kernel may touch a little past its arrays
+        buf = np.zeros(a.size + 256, np.float32)
+        buf[:a.size] = a
+        return buf
+    ref = slack(y0)
+    L.ref_schedule_mvm(refparts.f(slack(A)), refparts.f(slack(xv)), refparts.f(ref), M, K, p, refparts.dims_array(x), 8)
+    assert np.array_equal(mine, ref[:M])
 
 
 @pytest.mark.parametrize("M,K,p", [(1024, 1024, 8), (1000, 333, 3), (13, 2111, 2), (1, 1, 1), (4099, 517, 8)])

@@ -19,6 +19,14 @@ def _mats(M, K, N):
     return oracle.uniform((M, K), 11), oracle.uniform((K, N), 12), oracle.uniform((M, N), 13)
 
 
+def _slack(a, fill=0.0, extra=256):
+    """A copy of `a` with room behind it: the reference's packing loops read (and for partial
+    panels write) a little past the arrays they are given."""
+    buf = np.full(a.size + extra, fill, np.float32)
+    buf[:a.size] = a.ravel()
+    return buf
+
+
 @pytest.mark.parametrize("p", [1, 3, 8])
 @pytest.mark.parametrize("sch", SCHEDS)
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -35,9 +43,10 @@ def test_pack_matches_reference_sources(shape, sch, p):
     assert L.ref_packed_C_size(M, N, p, dims, cx.mr, cx.nr, sch) == oracle.packed_C_size(M, N, p, x, cx, sch)
 
     Ap = oracle.pack_A(A, p, x, cx, sch)
-    Ar = np.full_like(Ap, np.nan)
-    L.ref_pack_A(refparts.f(A), refparts.f(Ar), M, K, p, dims, cx.mr, cx.nr, sch)
-    assert np.array_equal(Ap, Ar)
+    Ar = _slack(Ap, np.nan)
+    Ar[:Ap.size] = np.nan
+    L.ref_pack_A(refparts.f(_slack(A)), refparts.f(Ar), M, K, p, dims, cx.mr, cx.nr, sch)
+    assert np.array_equal(Ap, Ar[:Ap.size])
 
     # MKN/NKM pack_B in the reference bounds-checks the N padding only in the
     # last core of the last K block (pack_m_first.cpp:128-139 passes a K-derived
@@ -45,10 +54,10 @@ def test_pack_matches_reference_sources(shape, sch, p):
     # instead of zeros.  Those columns never reach C.  Compare real data
     # everywhere and the padding only for KMN; give the reference slack to read.
     Bp = oracle.pack_B(B, p, x, cx, sch)
-    Bslack = np.zeros(K * N + 64, dtype=np.float32)
-    Bslack[:K * N] = B.ravel()
-    Br = np.full_like(Bp, np.nan)
-    L.ref_pack_B(refparts.f(Bslack), refparts.f(Br), K, N, p, dims, cx.mr, cx.nr, sch)
+    Br = _slack(Bp, np.nan)
+    Br[:Bp.size] = np.nan
+    L.ref_pack_B(refparts.f(_slack(B)), refparts.f(Br), K, N, p, dims, cx.mr, cx.nr, sch)
+    Br = Br[:Bp.size]
     if sch == oracle.KMN:
         assert np.array_equal(Bp, Br)
     else:
@@ -60,17 +69,18 @@ def test_pack_matches_reference_sources(shape, sch, p):
     # unpack: the reference writes only the in-range part of C
     Cp = oracle.uniform(oracle.packed_C_size(M, N, p, x, cx, sch) // 4, 14)
     Cu = oracle.unpack_C(Cp, M, N, p, x, cx, sch, into=np.full((M, N), 7.0, np.float32))
-    Cr = np.full((M, N), 7.0, np.float32)
-    L.ref_unpack_C(refparts.f(Cr), refparts.f(Cp), M, N, p, dims, cx.mr, cx.nr, sch)
-    assert np.array_equal(Cu, Cr)
+    Cr = _slack(np.full((M, N), 7.0, np.float32))
+    L.ref_unpack_C(refparts.f(Cr), refparts.f(_slack(Cp)), M, N, p, dims, cx.mr, cx.nr, sch)
+    assert np.array_equal(Cu, Cr[:M * N].reshape(M, N))
 
     # pack_C: identical to the reference except NKM with a partial last M block,
     # where the reference's own offset disagrees with its unpack and schedule
     Cpk = oracle.pack_C(Cm, p, x, cx, sch)
     if not (sch == oracle.NKM and x.m_pad):
-        Cpr = np.full_like(Cpk, np.nan)
-        L.ref_pack_C(refparts.f(Cm), refparts.f(Cpr), M, N, p, dims, cx.mr, cx.nr, sch)
-        assert np.array_equal(Cpk, Cpr)
+        Cpr = _slack(Cpk, np.nan)
+        Cpr[:Cpk.size] = np.nan
+        L.ref_pack_C(refparts.f(_slack(Cm)), refparts.f(Cpr), M, N, p, dims, cx.mr, cx.nr, sch)
+        assert np.array_equal(Cpk, Cpr[:Cpk.size])
 
 
 @pytest.mark.parametrize("p", [2, 8])
