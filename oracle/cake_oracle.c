@@ -30,6 +30,12 @@
  *   orc_im_2_col / orc_im2col
  *       - bit-exact against the reference's im_2_col (oracle/_ref), brute-force
  *         definition, naive 7-loop convolution.
+ *   The outputs of the compiled reference parts on seeded inputs are also
+ *   committed (tests/golden/reference_vectors.npz), so the packing, kernel, gemv
+ *   and im_2_col comparisons run where the reference sources are absent too.
+ *   The linear layer (oracle/__init__.py, a caller of orc_cake_sgemm) is pinned
+ *   against torch.nn.functional.linear and its autograd in fp64.
+ *   No function here is "parity unpinned".
  */
 #define _GNU_SOURCE
 #include <immintrin.h>
