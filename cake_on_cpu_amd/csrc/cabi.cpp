@@ -652,9 +652,10 @@ int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K, int a
     if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
     if ((st = stage_in(x, (size_t)K * 4, 1, true, &xv))) return st;
     if ((st = stage_in(y, (size_t)M * 4, 2, accumulate != 0, &yv))) return st;
-    if (a_col_major && K > 0) {
-        st = g_ctx.gemv.reserve(sgemv_colmajor_scratch_floats(M, K, g_ctx.model.cus) * sizeof(float));
-        if (st) return st;
+    if (K > 0) {
+        const size_t floats = a_col_major ? sgemv_colmajor_scratch_floats(M, K, g_ctx.model.cus)
+                                          : sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus);
+        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
     }
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
@@ -667,7 +668,8 @@ int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K, int a
         st = timer.family(2, [&] {
             return a_col_major ? launch_sgemv_colmajor(a.dev, xv.dev, yv.dev, M, K, accumulate,
                                                        static_cast<float*>(g_ctx.gemv.ptr), g_ctx.model.cus, stream)
-                               : launch_sgemv_rowmajor(a.dev, xv.dev, yv.dev, M, K, accumulate, stream);
+                               : launch_sgemv_rowmajor(a.dev, xv.dev, yv.dev, M, K, accumulate,
+                                                       static_cast<float*>(g_ctx.gemv.ptr), g_ctx.model.cus, stream);
         });
         if (st) return st;
     }

@@ -84,8 +84,10 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, in
                                 int accumulate, hipStream_t stream, int nchw_hw = 0,
                                 const float* col_bias = nullptr);
 
+// scratch: at least sgemv_rowmajor_scratch_floats(M, K, cus) floats (0 for most shapes), or nullptr
+size_t sgemv_rowmajor_scratch_floats(int M, int K, int cus);
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
-                                 int accumulate, hipStream_t stream);
+                                 int accumulate, float* scratch, int cus, hipStream_t stream);
 // scratch: at least sgemv_colmajor_scratch_floats(M, K) floats
 size_t sgemv_colmajor_scratch_floats(int M, int K, int cus);
 hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,

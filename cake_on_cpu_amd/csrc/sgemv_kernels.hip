@@ -85,11 +85,15 @@ template <int ROWS, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) sgemv_rowmajor_wg_kernel(const float* __restrict__ A,
                                                                        const float* __restrict__ x,
                                                                        float* __restrict__ y, int M,
-                                                                       int K, int accumulate)
+                                                                       int K, int accumulate,
+                                                                       int k4_per_slice)
 {
+    // grid.y > 1: few rows and very long ones -- each workgroup takes a slice of k and writes
+    // its sums to y[slice][M] (a scratch array that sgemv_slice_reduce_kernel adds up in order)
     __shared__ float red[WAVES][ROWS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = blockIdx.x * ROWS;
+    y += (size_t)blockIdx.y * M;
     float acc[ROWS];
     const f32x4* rowp[ROWS];
 #pragma unroll
@@ -97,10 +101,11 @@ __global__ void __launch_bounds__(WAVES * 64) sgemv_rowmajor_wg_kernel(const flo
         acc[r] = 0.f;
         rowp[r] = reinterpret_cast<const f32x4*>(A + (size_t)min(row0 + r, M - 1) * K);
     }
-    const int K4 = K >> 2;
+    const int c_begin = blockIdx.y * k4_per_slice;
+    const int c_end = min(K >> 2, c_begin + k4_per_slice);
     const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
 #pragma unroll 4
-    for (int c = tid; c < K4; c += WAVES * 64) {
+    for (int c = c_begin + tid; c < c_end; c += WAVES * 64) {
         const f32x4 xv = x4[c];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
@@ -122,20 +127,78 @@ __global__ void __launch_bounds__(WAVES * 64) sgemv_rowmajor_wg_kernel(const flo
     }
 }
 
+// Very short rows (K <= 32): a thread per row.  Neighbouring threads read neighbouring rows, so a
+// wave still touches one contiguous piece of A, and the few loads of a row hit the same lines.
+template <bool VEC>
+__global__ void __launch_bounds__(256) sgemv_rowmajor_thread_kernel(const float* __restrict__ A,
+                                                                    const float* __restrict__ x,
+                                                                    float* __restrict__ y, int M, int K,
+                                                                    int accumulate)
+{
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= M) return;
+    const float* a = A + (size_t)row * K;
+    float acc = 0.f;
+    if (VEC) {
+        for (int k = 0; k < K; k += 4) {
+            const f32x4 av = *reinterpret_cast<const f32x4*>(a + k);
+            acc += av.x * x[k] + av.y * x[k + 1] + av.z * x[k + 2] + av.w * x[k + 3];
+        }
+    } else {
+        for (int k = 0; k < K; ++k) acc += a[k] * x[k];
+    }
+    y[row] = accumulate ? y[row] + acc : acc;
+}
+
+__global__ void sgemv_slice_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int M,
+                                          int slices, int accumulate);
+
+// K slices for the long-row kernel when the rows alone do not fill the device.
+static int rowmajor_slices(int M, int K, int cus)
+{
+    const int wgs = (M + 1) / 2;
+    if (K < 16384 || wgs >= cus) return 1;
+    int want = (2 * cus + wgs - 1) / wgs;
+    const int max_slices = K / 8192;  // at least 8192 k per slice
+    return want < max_slices ? want : max_slices;
+}
+
+size_t sgemv_rowmajor_scratch_floats(int M, int K, int cus)
+{
+    const int s = rowmajor_slices(M, K, cus);
+    return s > 1 ? (size_t)s * M : 0;
+}
+
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
-                                 int accumulate, hipStream_t stream)
+                                 int accumulate, float* scratch, int cus, hipStream_t stream)
 {
     if (M <= 0) return hipSuccess;
     constexpr int ROWS = 4;
     const bool vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(x)) % 16 == 0);
     const int waves = (M + ROWS - 1) / ROWS;
     const int blocks = (waves + 3) / 4;
+    if (K <= 32) {
+        if (vec)
+            hipLaunchKernelGGL((sgemv_rowmajor_thread_kernel<true>), dim3((M + 255) / 256), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+        else
+            hipLaunchKernelGGL((sgemv_rowmajor_thread_kernel<false>), dim3((M + 255) / 256), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+        return hipGetLastError();
+    }
     if (vec && K >= 8192) {
-        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2), dim3(512), 0, stream, A, x, y, M, K, accumulate);
+        const int slices = scratch ? rowmajor_slices(M, K, cus) : 1;
+        if (slices > 1) {
+            const int k4_per = ((K / 4 + slices - 1) / slices + 511) & ~511;  // whole sweeps of the workgroup
+            hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2, slices), dim3(512), 0, stream, A, x, scratch, M, K, 0, k4_per);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 255) / 256), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
+            return hipGetLastError();
+        }
+        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2), dim3(512), 0, stream, A, x, y, M, K, accumulate, K / 4);
         return hipGetLastError();
     }
     if (vec && K >= 2048) {
-        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 4>), dim3((M + 1) / 2), dim3(256), 0, stream, A, x, y, M, K, accumulate);
+        hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 4>), dim3((M + 1) / 2), dim3(256), 0, stream, A, x, y, M, K, accumulate, K / 4);
         return hipGetLastError();
     }
     if (vec)
@@ -211,9 +274,8 @@ __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __rest
     }
 }
 
-__global__ void __launch_bounds__(256) sgemv_slice_reduce_kernel(const float* __restrict__ part,
-                                                                 float* __restrict__ y, int M,
-                                                                 int slices, int accumulate)
+__global__ void sgemv_slice_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int M,
+                                          int slices, int accumulate)
 {
     const int m = blockIdx.x * 256 + threadIdx.x;
     if (m >= M) return;

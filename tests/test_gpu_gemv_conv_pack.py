@@ -31,7 +31,9 @@ def test_fill_uniform_bit_exact(n, seed):
 # GEMV
 # ---------------------------------------------------------------------------
 GEMV_SHAPES = [(1, 1), (8, 1), (13, 2111), (64, 7), (1000, 333), (1024, 1024), (4099, 517),
-               (2048, 3000), (300, 70000), (70000, 36)]
+               (2048, 3000), (300, 70000), (70000, 36),
+               (6, 200000), (9, 65536),        # few long rows: the row-major path cuts K into slices
+               (50000, 8), (4097, 20), (333, 31)]  # very short rows: a thread per row
 
 
 @pytest.mark.parametrize("M,K", GEMV_SHAPES)
