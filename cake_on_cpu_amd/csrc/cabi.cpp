@@ -467,6 +467,18 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
             hipError_t e = launch_splitk_reduce(nullptr, c.dev, M, N, N, 0, 0, stream);
             if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
         }
+    } else if ((M == 1 || N == 1) && !tile_override) {
+        // A product with a single row or column is a matrix-vector product: C[M] = A[M][K] . B[K]
+        // reads A row-major; C[N] = A[K] . B[K][N] is B read as a column-major N x K matrix.
+        const size_t floats = N == 1 ? sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus)
+                                     : sgemv_colmajor_scratch_floats(N, K, g_ctx.model.cus);
+        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
+        float* scratch = static_cast<float*>(g_ctx.gemv.ptr);
+        st = timer.family(2, [&] {
+            return N == 1 ? launch_sgemv_rowmajor(a.dev, b.dev, c.dev, M, K, accumulate, scratch, g_ctx.model.cus, stream)
+                          : launch_sgemv_colmajor(b.dev, a.dev, c.dev, N, K, accumulate, scratch, g_ctx.model.cus, stream);
+        });
+        if (st) return st;
     } else {
         const bool vec = vec4_loadable(a.dev, b.dev, K, N);
         const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
@@ -1059,7 +1071,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
         const TileInfo& t = tile_info(id);
         if (t.lds_bytes > g_ctx.model.lds_per_cu) continue;
         const int max_split = std::max(1, K / (4 * t.bk));
-        for (int split = 1; split <= max_split && split <= 32; split *= 2) {
+        for (int split = 1; split <= max_split && split <= 1024; split *= 2) {
             for (int tail = (split == 1 ? 1 : 0); tail >= 0; --tail) {
                 if (id == model_plan.tile_id && split == model_plan.pub.split_k && (tail == 1 || split > 1))
                     continue;  // the baseline itself

@@ -206,7 +206,7 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
         if (want_k && t.bk != want_k) continue;
         if (t.lds_bytes > dev.lds_per_cu) continue;
         const int max_split = std::max(1, K / (4 * t.bk));
-        for (int split = 1; split <= 64; split *= 2) {
+        for (int split = 1; split <= 1024; split *= 2) {
             if (want_split && split != want_split) continue;
             if (!want_split && split > max_split) break;
             const double s = model_seconds(M, N, K, id, split, dev);
