@@ -240,6 +240,20 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
              const TunedChoice* choice = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
+    if (vec && !conv && !choice && !tile_override && fewrows_applies(M, N, K)) {
+        // a few rows of A against a wide B: bound by reading B, served by the streaming kernel
+        const int slices = fewrows_slices(N, K, g_ctx.model.cus);
+        float* partial = nullptr;
+        if (slices > 1) {
+            int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
+            if (st2) return st2;
+            partial = static_cast<float*>(g_ctx.splitk.ptr);
+        }
+        return timer.family(0, [&] {
+            return launch_sgemm_fewrows(A, B, C, partial, M, N, K, lda, ldb, ldc, accumulate, col_bias,
+                                        g_ctx.model.cus, stream);
+        });
+    }
     GemmPlan plan;
     int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec, g_ctx.model, &plan)
                     : plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);

@@ -86,6 +86,13 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, in
 
 // scratch: at least sgemv_rowmajor_scratch_floats(M, K, cus) floats (0 for most shapes), or nullptr
 size_t sgemv_rowmajor_scratch_floats(int M, int K, int cus);
+// Products with at most 16 rows of A (bound by streaming B): see sgemm_fewrows.hip.
+bool fewrows_applies(int M, int N, int K);
+int fewrows_slices(int N, int K, int cus);
+hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float* partial, int M, int N,
+                                int K, int lda, int ldb, int ldc, int accumulate, const float* col_bias,
+                                int cus, hipStream_t stream);
+
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, float* scratch, int cus, hipStream_t stream);
 // scratch: at least sgemv_colmajor_scratch_floats(M, K) floats

@@ -148,6 +148,23 @@ def test_very_long_k_takes_the_element_loader():
     assert oracle.max_rel_err(Cm, C64, S) <= TOL
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 512), (3, 300, 1000), (5, 1000, 4096), (8, 4096, 4097), (13, 777, 2050),
+                                   (16, 2111, 16384), (16, 16384, 1024), (1, 100, 600), (9, 65, 515),
+                                   (17, 300, 1000), (32, 1000, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_few_rows_times_wide_matrix(shape):
+    """M <= 16 against a wide B: the streaming kernel (B read once, 16-row MFMAs; 17 and 32 rows take the tile kernel),
+    with K slices summed in order, ragged N and K, accumulation, and run-to-run identical sums."""
+    M, K, N = shape
+    print(f"sgemm few rows M={M} K={K} N={N}", flush=True)
+    A, B, Cm = _run(M, K, N)
+    _check(A, B, Cm, oracle.cake_sgemm(A, B, 4, oracle.make_cntx()).astype(np.float64), shape)
+    C0 = oracle.uniform((M, N), 3)
+    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    assert np.allclose(acc - Cm, C0, atol=2e-4)
+    assert np.array_equal(_run(M, K, N)[2], Cm)
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
