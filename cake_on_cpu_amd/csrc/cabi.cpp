@@ -240,7 +240,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
              const TunedChoice* choice = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
-    if (vec && !conv && !choice && !tile_override && fewrows_applies(M, N, K)) {
+    if (vec && !conv && !choice && !tile_override && fewrows_applies(M, N, K, lda, ldb)) {
         // a few rows of A against a wide B: bound by reading B, served by the streaming kernel
         const int slices = fewrows_slices(N, K, g_ctx.model.cus);
         float* partial = nullptr;
@@ -252,6 +252,20 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         return timer.family(0, [&] {
             return launch_sgemm_fewrows(A, B, C, partial, M, N, K, lda, ldb, ldc, accumulate, col_bias,
                                         g_ctx.model.cus, stream);
+        });
+    }
+    if (vec && !conv && !choice && !tile_override && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
+        // a tall A against a few columns of B: the same with A streamed along its rows
+        const int slices = fewrows_nt_slices(M, K, g_ctx.model.cus);
+        float* partial = nullptr;
+        if (slices > 1) {
+            int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
+            if (st2) return st2;
+            partial = static_cast<float*>(g_ctx.splitk.ptr);
+        }
+        return timer.family(0, [&] {
+            return launch_sgemm_fewrows_nt(B, A, C, partial, N, M, K, ldb, lda, ldc, true, true, accumulate,
+                                           col_bias, g_ctx.model.cus, stream);
         });
     }
     GemmPlan plan;
@@ -941,11 +955,28 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
     if (bias && (st = stage_in(bias, (size_t)N * 4, 2, true, &bo))) return st;
     if ((st = stage_in(y, (size_t)M * N * 4, 3, false, &yo))) return st;
     // workspace: the weights as a K x N matrix (256-byte aligned so the 16-byte loader applies)
-    if ((st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
+    const bool small_batch = fewrows_nt_applies(M, N, K, K, K, false);
+    if (!small_batch && (st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
     float* wt = static_cast<float*>(g_ctx.linear.ptr);
 
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
+    if (small_batch) {
+        // a small batch: y = x w^T with w streamed once as it lies, no transposed copy
+        const int slices = fewrows_nt_slices(N, K, g_ctx.model.cus);
+        float* partial = nullptr;
+        if (slices > 1) {
+            if ((st = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float)))) return st;
+            partial = static_cast<float*>(g_ctx.splitk.ptr);
+        }
+        st = timer.family(0, [&] {
+            return launch_sgemm_fewrows_nt(xo.dev, wo.dev, yo.dev, partial, M, N, K, K, K, N, false, false, 0,
+                                           bias ? bo.dev : nullptr, g_ctx.model.cus, stream);
+        });
+        if (st) return st;
+        if ((st = timer.stop())) return st;
+        return stage_out(yo, stream);
+    }
     if (K > 0) {
         st = timer.family(4, [&] { return launch_transpose(wo.dev, wt, N, K, stream); });
         if (st) return st;

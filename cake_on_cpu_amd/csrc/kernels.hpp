@@ -86,12 +86,18 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, in
 
 // scratch: at least sgemv_rowmajor_scratch_floats(M, K, cus) floats (0 for most shapes), or nullptr
 size_t sgemv_rowmajor_scratch_floats(int M, int K, int cus);
-// Products with at most 16 rows of A (bound by streaming B): see sgemm_fewrows.hip.
-bool fewrows_applies(int M, int N, int K);
+// Products in which one operand has at most 16 rows or columns (bound by streaming the other
+// one): see sgemm_fewrows.hip.
+bool fewrows_applies(int M, int N, int K, int lda, int ldb);
 int fewrows_slices(int N, int K, int cus);
 hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float* partial, int M, int N,
                                 int K, int lda, int ldb, int ldc, int accumulate, const float* col_bias,
                                 int cus, hipStream_t stream);
+bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor);
+int fewrows_nt_slices(int N, int K, int cus);
+hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, float* partial, int M, int N,
+                                   int K, int ldx, int ldw, int ldc, bool x_kmajor, bool c_is_n_by_m,
+                                   int accumulate, const float* bias, int cus, hipStream_t stream);
 
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, float* scratch, int cus, hipStream_t stream);

@@ -1,26 +1,37 @@
-// sgemm_fewrows.hip -- C[M][N] = A[M][K] . B[K][N] for M <= 16 ("a few vectors
-// times a matrix": small-batch linear layers, blocks of matrix-vector products).
+// sgemm_fewrows.hip -- products in which one operand has at most 16 rows or
+// columns ("a few vectors times a matrix": small-batch linear layers, blocks of
+// matrix-vector products).
 //
-// Such a product is bound by reading B once from HBM, not by arithmetic, and a
-// 64-row macro-tile would waste most of the matrix pipe on zero rows while
-// reading B in 256-byte pieces.  Here B is streamed the way the column-major
-// matrix-vector kernel streams its operand: a workgroup owns 256 consecutive
-// columns and a slice of k; each of its four waves takes a quarter of every k
-// chunk and reads whole 1 KB row pieces, 64 bytes per lane.  The arithmetic
-// runs on v_mfma_f32_16x16x4_f32, whose 16 rows fit the problem: the 16 columns
-// a lane loads feed 16 MFMAs, A comes from a
-// k-major copy of the current chunk in LDS.  Wave sums meet in LDS in wave
-// order and K slices are summed by splitk_reduce_kernel in slice order, so
-// results are run-to-run identical.
+// Such a product is bound by reading the large operand once from HBM, not by
+// arithmetic, and a 64-row macro-tile would spend most of the matrix pipe on
+// zero rows while reading the large operand in short pieces.  The kernels here
+// stream the large operand straight from global memory into the operand
+// registers of v_mfma_f32_16x16x4_f32, whose 16 rows fit the problem: no LDS
+// and no barrier inside the k loop, so every wave keeps its loads in flight on
+// its own.  The small operand comes from L2 with one load per 4 to 16 loads of
+// the large one.
+//
+//   sgemm_fewrows_nn_kernel   C[M<=16][N] = A[M][K] . B[K][N]      streams B (n contiguous)
+//   sgemm_fewrows_nt_kernel   C'[i<=16][n] = sum_k X[i][k] W[n][k]  streams W (k contiguous):
+//                             the linear layer y = x w^T for a small batch without
+//                             transposing w, and C[M][N<=16] = A.B with W = A, X = B^T
+//
+// A workgroup owns 256 columns of B (64 rows of W) and a slice of k; its four
+// waves take a quarter of the slice each and add their sums in LDS in wave
+// order; K slices are summed by splitk_reduce_kernel in slice order, so results
+// are run-to-run identical.
 //
 // Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l % 16][l / 16]
 // and B[l / 16][l % 16]; result register r of lane l is C[4 * (l / 16) + r][l % 16].
+// The order of k inside a product is free as long as both operands agree, so a
+// lane that loads 4 consecutive k of its row (16 bytes) feeds them to 4
+// successive MFMAs: MFMA e of a group of 16 k works on k = 4 (l / 16) + e.
 #include "sgemm_tile.hpp"
 
 namespace cake {
 
-// 16-byte load marked non-temporal: B is read once and should not push A or the partial sums
-// out of the caches on its way through
+// 16-byte load marked non-temporal: the large operand is read once and should not push the small
+// one or the partial sums out of the caches on its way through
 __device__ __forceinline__ f32x4 stream_load_f32x4(const float* base, int byte_offset, unsigned records)
 {
     __amdgpu_buffer_rsrc_t rsrc =
@@ -28,86 +39,131 @@ __device__ __forceinline__ f32x4 stream_load_f32x4(const float* base, int byte_o
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, /*nt*/ 2));
 }
 
-static constexpr int FR_COLS = 256;   // columns per workgroup
-static constexpr int FR_KC = 1024;    // k per LDS chunk of A (a quarter per wave)
-static constexpr int FR_PITCH = 17;   // floats per k in the LDS copy of A: odd, so staging writes spread over banks
-
-__global__ void __launch_bounds__(256) sgemm_fewrows_kernel(const float* __restrict__ A,
-                                                            const float* __restrict__ B,
-                                                            float* __restrict__ out, int M, int N, int K,
-                                                            int lda, int ldb, int k_per_slice,
-                                                            int out_ld, size_t out_slice_stride,
-                                                            int accumulate, const float* __restrict__ col_bias)
+__device__ __forceinline__ float load_f32(const float* base, int byte_offset, unsigned records)
 {
-    __shared__ __align__(16) float smem[FR_KC * FR_PITCH];   // At[k][m] while walking, then the wave sums
-    static_assert(FR_KC * FR_PITCH >= 16 * FR_COLS, "the reduction buffer fits the A chunk's memory");
-    float* At = smem;
+    __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)records, 0x00020000);
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
+}
+
+static constexpr int FR_COLS = 256;     // nn: columns of B per workgroup
+static constexpr int FR_ROWS = 64;      // nt: rows of W per workgroup
+static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave and loop step
+
+// The part of [kbeg, kend) that wave `wave` of 4 walks: quarters rounded up to 16 k
+__device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0, int& kw1)
+{
+    const int part = (((kend - kbeg + 3) >> 2) + 15) & ~15;
+    kw0 = min(kend, kbeg + wave * part);
+    kw1 = min(kend, kw0 + part);
+}
+
+__global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float* __restrict__ out, int M, int N, int K,
+                                                               int lda, int ldb, int k_per_slice,
+                                                               int out_ld, size_t out_slice_stride,
+                                                               int accumulate, const float* __restrict__ col_bias)
+{
+    __shared__ __align__(16) float red[16 * FR_COLS];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
     const int n0 = blockIdx.x * FR_COLS;
     const int kbeg = blockIdx.y * k_per_slice;
     const int kend = min(K, kbeg + k_per_slice);
+    int kw0, kw1;
+    wave_part(kbeg, kend, wave, kw0, kw1);
+
+    const unsigned a_elems = clamp_elems((long long)(M - 1) * lda + K);
     const unsigned b_elems = clamp_elems((long long)(K - 1) * ldb + N - n0);
-    // The lane's four 16-byte pieces of its row of B: piece j is columns 64 j + 4 li .. + 3, so that
-    // the 16 lanes of a row read 256 contiguous bytes per load instruction.
+    // A: row li, k = 4 lq .. 4 lq + 3 of the group.  B: rows 4 lq + e of the group (e = 0..3 by
+    // moving the base), and of each row four 16-byte pieces: piece j is columns 64 j + 4 li .. + 3,
+    // so that the 16 lanes of a row read 256 contiguous bytes per load instruction.
+    const int a_off = li < M ? (li * lda + 4 * lq) * 4 : BUF_OOB;
     int b_off[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b_off[j] = n0 + 64 * j + 4 * li < N ? (64 * j + 4 * li + lq * ldb) * 4 : BUF_OOB;
+    for (int j = 0; j < 4; ++j)
+        b_off[j] = n0 + 64 * j + 4 * li < N ? (4 * lq * ldb + 64 * j + 4 * li) * 4 : BUF_OOB;
 
     f32x4 acc[16];
 #pragma unroll
     for (int c = 0; c < 16; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int k0 = kbeg; k0 < kend; k0 += FR_KC) {
-        __syncthreads();  // the previous chunk has been consumed
-        for (int kt = tid; kt < FR_KC; kt += 256) {
-            const int k = k0 + kt;
+    // Groups of 16 k that lie wholly below kw1 <= K: every row asked for exists, so the record
+    // counts are exact (records_left must not be asked about a start past the end of an operand:
+    // its difference would wrap to "everything in range").  Half a group (8 loads of B) is in
+    // flight while the other half is multiplied.
+    auto load_a = [&](int k) { return buffer_load_f32x4(A + k, a_off, records_left(a_elems, (unsigned)k)); };
+    auto load_half = [&](int k, int h, f32x4 (&b)[2][4]) {
 #pragma unroll
-            for (int m = 0; m < 16; ++m)
-                At[kt * FR_PITCH + m] = (m < M && k < kend) ? A[(size_t)m * lda + k] : 0.f;
+        for (int e = 0; e < 2; ++e) {
+            const unsigned skip = (unsigned)(k + 2 * h + e) * (unsigned)ldb;
+            const unsigned rec = records_left(b_elems, skip);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[e][j] = stream_load_f32x4(B + n0 + (size_t)skip, b_off[j], rec);
         }
-        __syncthreads();
-        // This wave's quarter of the chunk, as far as it lies below kend.  The groups of 4 rows
-        // start below kend <= K, so their record counts are exact (records_left must not be asked
-        // about a start past the end of B: its difference would wrap to "everything in range");
-        // rows of the last group that reach past K are outside those records and read as zero,
-        // rows between kend and K meet zeros of A.
-        const int kw = k0 + wave * (FR_KC / 4);
-        const int kk_end = min(FR_KC / 4, kend - kw);
-        // U groups of 4 rows of B against 4 k of A each: all the loads first, so that 4 U loads of
-        // 16 bytes are in flight per lane before the first MFMA needs one
-        auto groups = [&](int kk, auto u_count) {
-            constexpr int U = decltype(u_count)::value;
-            f32x4 b[U][4];
-            float a[U];
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
+    };
+    auto mma_half = [&](const f32x4& a, int h, const f32x4 (&b)[2][4]) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const unsigned skip = (unsigned)(kw + kk + 4 * u) * (unsigned)ldb;
-                const unsigned rec = records_left(b_elems, skip);
+        for (int e = 0; e < 2; ++e)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) b[u][j] = stream_load_f32x4(B + n0 + (size_t)skip, b_off[j], rec);
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    acc[4 * j + c] =
+                        __builtin_amdgcn_mfma_f32_16x16x4f32(a[2 * h + e], b[e][j][c], acc[4 * j + c], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int k = kw0;
+    {
+        f32x4 a_cur = {0.f, 0.f, 0.f, 0.f}, a_nxt = a_cur;
+        f32x4 b0[2][4], b1[2][4];
+        if (k + 16 <= kw1) {
+            a_cur = load_a(k);
+            load_half(k, 0, b0);
+            // no branch inside the loop body: the wait counts in front of the MFMAs are exact
+            for (; k + 32 <= kw1; k += 16) {
+                load_half(k, 1, b1);
+                mma_half(a_cur, 0, b0);
+                a_nxt = load_a(k + 16);
+                load_half(k + 16, 0, b0);
+                mma_half(a_cur, 1, b1);
+                a_cur = a_nxt;
             }
+            load_half(k, 1, b1);
+            mma_half(a_cur, 0, b0);
+            mma_half(a_cur, 1, b1);
+            k += 16;
+        }
+    }
+    if (k < kw1) {
+        // the last 1..15 k of the wave's part, element by element: k at or past kw1 reads as zero
+        // on both sides (rows of B between kw1 and K belong to another wave or slice)
+#pragma nounroll
+        for (int e = 0; e < 4; ++e) {
+            const bool below = k + 4 * lq + e < kw1;
+            const float a = buffer_load_f32(A + k, below && li < M ? (li * lda + 4 * lq + e) * 4 : BUF_OOB);
+            const float* row = B + n0 + (size_t)(k + e) * ldb;
 #pragma unroll
-            for (int u = 0; u < U; ++u) a[u] = At[(wave * (FR_KC / 4) + kk + 4 * u + lq) * FR_PITCH + li];
+            for (int j = 0; j < 4; ++j) {
+                const bool col = n0 + 64 * j + 4 * li < N;
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        acc[4 * j + e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u][j][e], acc[4 * j + e], 0, 0, 0);
-        };
-        int kk = 0;
-        for (; kk + 16 <= kk_end; kk += 16) groups(kk, std::integral_constant<int, 4>{});
-        for (; kk < kk_end; kk += 4) groups(kk, std::integral_constant<int, 1>{});
+                for (int c = 0; c < 4; ++c) {
+                    // element loads: a 16-byte load of the last row could hang over the end of B
+                    const bool ok = below && col && n0 + 64 * j + 4 * li + c < N;
+                    const float b = buffer_load_f32(row, ok ? b_off[j] + 4 * c : BUF_OOB);
+                    acc[4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[4 * j + c], 0, 0, 0);
+                }
+            }
+        }
     }
 
-    // register r of MFMA 4j+e holds C[4*lq + r][n0 + 64 j + 4 li + e].  Wave sums meet in LDS in
+    // register r of MFMA 4j+c holds C[4*lq + r][n0 + 64 j + 4 li + c].  Wave sums meet in LDS in
     // wave order: red[row][column].
-    float* red = smem;
     for (int w = 0; w < 4; ++w) {
-        __syncthreads();
+        if (w) __syncthreads();
         if (wave == w) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -132,19 +188,208 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_kernel(const float* __restr
     }
 }
 
-int fewrows_slices(int N, int K, int cus)
+// out[i * ld_i + n * ld_n] = sum_k X(i, k) W[n][k] for i < M <= 16, n < N.
+// X_KMAJOR: X(i, k) = X[k * ldx + i] (the B of a product with few columns), else X[i * ldx + k].
+//
+// The MFMA wants lane (lq, li) to hold 4 consecutive k of row li: loaded that way, the four
+// lanes of every quad would touch four different rows, and the texture path serves a quad per
+// cycle only when its lanes fall into one cache line.  So the wave loads with its lanes along k
+// (8 rows x 128 bytes per instruction), passes the data through an LDS area of its own and reads
+// it back in MFMA order: no barrier, LDS operations of one wave complete in order.  The waves
+// of a workgroup take the steps of 32 k in turn, so together they read 512 contiguous bytes of
+// every row at a time.
+static constexpr int NT_STEP = 32;                               // k per step of a wave
+static constexpr int NT_PITCH = 36;                              // floats per staged row: 16-byte reads of 16 rows spread over all banks
+static constexpr int NT_WAVE_FLOATS = (FR_ROWS + 16) * NT_PITCH; // 64 rows of W and 16 of X
+
+__device__ __forceinline__ f32x4 keep_below(f32x4 v, int valid)  // zero the elements at and past `valid`
 {
-    const int nblocks = (N + FR_COLS - 1) / FR_COLS;
-    int want = (2 * cus + nblocks - 1) / nblocks;
-    const int max_slices = (K + FR_KC - 1) / FR_KC;  // at least one chunk per slice
+    if (valid < 4) v[3] = 0.f;
+    if (valid < 3) v[2] = 0.f;
+    if (valid < 2) v[1] = 0.f;
+    if (valid < 1) v[0] = 0.f;
+    return v;
+}
+
+template <bool X_KMAJOR>
+__global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __restrict__ X,
+                                                               const float* __restrict__ W,
+                                                               float* __restrict__ out, int M, int N, int K,
+                                                               int ldx, int ldw, int k_per_slice,
+                                                               long long ld_i, long long ld_n,
+                                                               size_t out_slice_stride, int accumulate,
+                                                               const float* __restrict__ bias_n,
+                                                               const float* __restrict__ bias_i)
+{
+    __shared__ __align__(16) float smem[4 * NT_WAVE_FLOATS];
+    static_assert(4 * NT_WAVE_FLOATS >= 16 * FR_ROWS, "the reduction buffer fits the staging memory");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lq = lane >> 4;   // MFMA order: row li, k = 4 lq .. + 3 of a group of 16
+    const int lr = lane >> 3, lc = lane & 7;    // load order: row lr of 8, k = 4 lc .. + 3 of the step
+    const int n0 = blockIdx.x * FR_ROWS;
+    const int kbeg = blockIdx.y * k_per_slice;
+    const int kend = min(K, kbeg + k_per_slice);
+    float* Ws = smem + wave * NT_WAVE_FLOATS;   // [64][NT_PITCH]
+    float* Xs = Ws + FR_ROWS * NT_PITCH;        // [16][NT_PITCH]
+
+    const float* Wb = W + (size_t)n0 * ldw;
+    const int rows_left = N - n0;
+    const unsigned w_elems = clamp_elems((long long)(rows_left - 1) * ldw + K);
+    const unsigned x_elems = clamp_elems(X_KMAJOR ? (long long)(K - 1) * ldx + M : (long long)(M - 1) * ldx + K);
+    const int w_off = (lr * ldw + 4 * lc) * 4;
+    const int x_off = X_KMAJOR ? (lq * ldx + li) * 4 : (lr * ldx + 4 * lc) * 4;
+
+    f32x4 acc[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Rows at and past N (or M) are not masked: what they bring only reaches results that are
+    // never written.  Their addresses are kept inside the operands by exact record counts, and
+    // a group of 8 rows that starts past the end gets a count of 0 (records_left must not be asked
+    // about a start past the end: its difference would wrap to "everything in range").
+    // TAIL: the last, partial step of the slice; k at and past kend reads as zero on both sides.
+    auto load_step = [&](int k, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2], float (&gk)[8]) {
+        constexpr bool TAIL = decltype(tail)::value;
+        const int below = kend - (k + 4 * lc);   // of this lane's 4 k, how many lie below kend
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const unsigned used = (unsigned)(8 * t) * (unsigned)ldw + (unsigned)k;
+            const unsigned rec = 8 * t < rows_left ? records_left(w_elems, used) : 0u;
+            gw[t] = stream_load_f32x4(Wb + (size_t)(8 * t) * ldw + k, TAIL && below <= 0 ? BUF_OOB : w_off, rec);
+            if (TAIL) gw[t] = keep_below(gw[t], below);
+        }
+        if constexpr (!X_KMAJOR) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const unsigned used = (unsigned)(8 * t) * (unsigned)ldx + (unsigned)k;
+                const unsigned rec = 8 * t < M ? records_left(x_elems, used) : 0u;
+                gx[t] = buffer_load_f32x4(X + (size_t)(8 * t) * ldx + k, TAIL && below <= 0 ? BUF_OOB : x_off, rec);
+                if (TAIL) gx[t] = keep_below(gx[t], below);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {   // k = 4 t + lq of the step, i = li
+                const unsigned used = (unsigned)(k + 4 * t) * (unsigned)ldx;
+                const unsigned rec = (!TAIL || k + 4 * t < kend) ? records_left(x_elems, used) : 0u;
+                gk[t] = load_f32(X + (size_t)(k + 4 * t) * ldx, TAIL && k + 4 * t + lq >= kend ? BUF_OOB : x_off, rec);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
+    };
+    auto store_step = [&](const f32x4 (&gw)[8], const f32x4 (&gx)[2], const float (&gk)[8]) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(Ws + (8 * t + lr) * NT_PITCH + 4 * lc) = gw[t];
+        if constexpr (!X_KMAJOR) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) *reinterpret_cast<f32x4*>(Xs + (8 * t + lr) * NT_PITCH + 4 * lc) = gx[t];
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) Xs[li * NT_PITCH + 4 * t + lq] = gk[t];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto compute_step = [&]() {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(Xs + li * NT_PITCH + 16 * u + 4 * lq);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 w = *reinterpret_cast<const f32x4*>(Ws + (16 * g + li) * NT_PITCH + 16 * u + 4 * lq);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], w[e], acc[g], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    {
+        f32x4 gw[8], gx[2];
+        float gk[8];
+        const int full = (kend - kbeg) / NT_STEP;
+        int s = wave;
+        if (s < full) {
+            load_step(kbeg + NT_STEP * s, std::false_type{}, gw, gx, gk);
+            // no branch inside the loop body: the wait counts in front of the stores are exact
+            for (; s + 4 < full; s += 4) {
+                store_step(gw, gx, gk);
+                load_step(kbeg + NT_STEP * (s + 4), std::false_type{}, gw, gx, gk);
+                compute_step();
+            }
+            store_step(gw, gx, gk);
+            compute_step();
+        }
+        if (((kend - kbeg) & (NT_STEP - 1)) && wave == (full & 3)) {
+            load_step(kbeg + NT_STEP * full, std::true_type{}, gw, gx, gk);
+            store_step(gw, gx, gk);
+            compute_step();
+        }
+    }
+
+    // register r of acc[g] holds C'[4 lq + r][n0 + 16 g + li]; wave sums meet in LDS in wave order
+    float* red = smem;
+    for (int w = 0; w < 4; ++w) {
+        __syncthreads();  // the first: every wave is done with its staging area
+        if (wave == w) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float* p = red + (4 * lq + r) * FR_ROWS + 16 * g + li;
+                    *p = w == 0 ? acc[g][r] : *p + acc[g][r];
+                }
+        }
+    }
+    __syncthreads();
+    const int n = n0 + (tid & 63);
+    if (n >= N) return;
+    float* dst = out + (size_t)blockIdx.y * out_slice_stride + (long long)n * ld_n;
+    const float bn = bias_n ? bias_n[n] : 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int i = 4 * (tid >> 6) + r;
+        if (i >= M) break;
+        float v = red[i * FR_ROWS + (tid & 63)];
+        if (accumulate) v += dst[i * ld_i];
+        if (bias_n) v += bn;
+        if (bias_i) v += bias_i[i];
+        dst[i * ld_i] = v;
+    }
+}
+
+// K slices so that about `per_cu` workgroups of 4 waves land on every CU
+static int slices_for(int blocks, int K, int cus, int per_cu)
+{
+    int want = (per_cu * cus + blocks - 1) / blocks;
+    const int max_slices = (K + FR_K_UNIT - 1) / FR_K_UNIT;
     if (want > max_slices) want = max_slices;
     return want < 1 ? 1 : want;
 }
 
-bool fewrows_applies(int M, int N, int K)
+static int slice_length(int K, int slices, int* used)
 {
-    // byte offsets inside a chunk (3 rows of B plus 256 columns) must stay below 2^31
-    return M >= 1 && M <= 16 && N >= 512 && K >= 64 && (double)N * 4 * 4 < 2147483648.0;
+    int k_per = (K + slices - 1) / slices;
+    k_per = (k_per + FR_K_UNIT - 1) / FR_K_UNIT * FR_K_UNIT;
+    *used = (K + k_per - 1) / k_per;
+    return k_per;
+}
+
+// workgroups per CU: what the registers of the nn kernel and the LDS of the nt kernel allow
+int fewrows_slices(int N, int K, int cus) { return slices_for((N + FR_COLS - 1) / FR_COLS, K, cus, 2); }
+int fewrows_nt_slices(int N, int K, int cus) { return slices_for((N + FR_ROWS - 1) / FR_ROWS, K, cus, 3); }
+
+bool fewrows_applies(int M, int N, int K, int lda, int ldb)
+{
+    // byte offsets inside a group (15 rows of B plus 256 columns, 15 rows of A) must stay below 2^31
+    return M >= 1 && M <= 16 && N >= 512 && K >= 64 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
+           (double)lda * 16 * 4 < 2147483648.0;
+}
+
+bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
+{
+    // 64 rows of W, and 16 rows (or 16 k) of X, within 2^31 bytes of the block's origin
+    return M >= 1 && M <= 16 && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
+           (double)ldx * 16 * 4 + (x_kmajor ? 64 : 0) < 2147483648.0;
 }
 
 // partial: [slices][M][N] floats when fewrows_slices(N, K, cus) > 1, else unused
@@ -152,19 +397,44 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
                                 int K, int lda, int ldb, int ldc, int accumulate, const float* col_bias,
                                 int cus, hipStream_t stream)
 {
-    const int slices = fewrows_slices(N, K, cus);
-    int k_per = (K + slices - 1) / slices;
-    k_per = (k_per + FR_KC - 1) / FR_KC * FR_KC;
-    const int used = (K + k_per - 1) / k_per;
+    int used;
+    const int k_per = slice_length(K, fewrows_slices(N, K, cus), &used);
     const dim3 grid((N + FR_COLS - 1) / FR_COLS, used), block(256);
     float* out = used > 1 ? partial : C;
     const int out_ld = used > 1 ? N : ldc;
     const size_t stride = used > 1 ? (size_t)M * N : 0;
-    hipLaunchKernelGGL(sgemm_fewrows_kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per, out_ld,
-                       stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
+    hipLaunchKernelGGL(sgemm_fewrows_nn_kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
+                       out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || used == 1) return e;
     return launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, 0, col_bias);
+}
+
+// C'(i, n) = sum_k X(i, k) W[n][k] for i < M <= 16, n < N.
+// c_is_n_by_m = false: C is M x N (C[i * ldc + n], bias per n);  true: C is N x M (C[n * ldc + i],
+// bias per i): in both cases `bias` runs along the columns of C.
+// partial: [slices] copies of C without padding when fewrows_nt_slices(N, K, cus) > 1
+hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, float* partial, int M, int N,
+                                   int K, int ldx, int ldw, int ldc, bool x_kmajor, bool c_is_n_by_m,
+                                   int accumulate, const float* bias, int cus, hipStream_t stream)
+{
+    int used;
+    const int k_per = slice_length(K, fewrows_nt_slices(N, K, cus), &used);
+    const dim3 grid((N + FR_ROWS - 1) / FR_ROWS, used), block(256);
+    const bool split = used > 1;
+    float* out = split ? partial : C;
+    const long long ld_i = c_is_n_by_m ? 1 : (split ? N : ldc);
+    const long long ld_n = c_is_n_by_m ? (split ? M : ldc) : 1;
+    const size_t stride = split ? (size_t)M * N : 0;
+    const float* bias_n = split || c_is_n_by_m ? nullptr : bias;
+    const float* bias_i = split || !c_is_n_by_m ? nullptr : bias;
+    auto kernel = x_kmajor ? sgemm_fewrows_nt_kernel<true> : sgemm_fewrows_nt_kernel<false>;
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, X, W, out, M, N, K, ldx, ldw, k_per, ld_i, ld_n, stride,
+                       split ? 0 : accumulate, bias_n, bias_i);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !split) return e;
+    return c_is_n_by_m ? launch_splitk_reduce(partial, C, N, M, ldc, used, accumulate, stream, 0, bias)
+                       : launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, 0, bias);
 }
 
 }  // namespace cake

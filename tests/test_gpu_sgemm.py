@@ -165,6 +165,23 @@ def test_few_rows_times_wide_matrix(shape):
     assert np.array_equal(_run(M, K, N)[2], Cm)
 
 
+@pytest.mark.parametrize("shape", [(512, 64, 2), (1000, 300, 3), (4096, 1000, 5), (4097, 4096, 8), (2050, 777, 13),
+                                   (16384, 2111, 16), (1024, 16384, 16), (600, 100, 1), (515, 65, 9),
+                                   (1000, 300, 17), (5000, 4099, 4)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_tall_matrix_times_few_columns(shape):
+    """N <= 16 columns of B against a tall A: A streamed once along its rows (17 columns take the tile
+    kernel), ragged M and K, K slices summed in order, accumulation, run-to-run identical sums."""
+    M, K, N = shape
+    print(f"sgemm few columns M={M} K={K} N={N}", flush=True)
+    A, B, Cm = _run(M, K, N)
+    _check(A, B, Cm, oracle.cake_sgemm(A, B, 4, oracle.make_cntx()).astype(np.float64), shape)
+    C0 = oracle.uniform((M, N), 3)
+    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    assert np.allclose(acc - Cm, C0, atol=2e-4)
+    assert np.array_equal(_run(M, K, N)[2], Cm)
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
