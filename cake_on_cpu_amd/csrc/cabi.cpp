@@ -240,7 +240,10 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
              const TunedChoice* choice = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
-    if (vec && !conv && !choice && !tile_override && fewrows_applies(M, N, K, lda, ldb)) {
+    // Products with a few rows or columns have streaming kernels of their own; a macro-tile is
+    // only used for them on request or when the tuner measured one to be faster.
+    const bool streaming_ok = vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, true, nullptr);
+    if (streaming_ok && fewrows_applies(M, N, K, lda, ldb)) {
         // a few rows of A against a wide B: bound by reading B, served by the streaming kernel
         const int slices = fewrows_slices(N, K, g_ctx.model.cus);
         float* partial = nullptr;
@@ -254,7 +257,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
                                         g_ctx.model.cus, stream);
         });
     }
-    if (vec && !conv && !choice && !tile_override && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
+    if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
         // a tall A against a few columns of B: the same with A streamed along its rows
         const int slices = fewrows_nt_slices(M, K, g_ctx.model.cus);
         float* partial = nullptr;
@@ -1078,14 +1081,14 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
 
     // time one explicit choice: a warm-up launch, then the fastest of three batches of
     // back-to-back launches (clock ramps and other tenants only ever make a batch slower)
-    auto measure = [&](const TunedChoice& c, double* secs) -> int {
+    auto measure = [&](const TunedChoice* c, double* secs) -> int {
         Timer untimed(stream, nullptr);
         double est = 0, best_batch = 1e30;
         for (int pass = 0; pass < 4; ++pass) {
             const int reps = pass == 0 ? 1 : (est < 2e-4 ? 20 : est < 5e-3 ? 5 : 2);
             HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
             for (int r = 0; r < reps; ++r) {
-                int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, stream, untimed, nullptr, nullptr, &c);
+                int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, stream, untimed, nullptr, nullptr, c);
                 if (e) return e;
             }
             HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));
@@ -1106,8 +1109,16 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
         if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, any, vec, g_ctx.model, &model_plan))) return st;
     }
     TunedChoice best{model_plan.tile_id, model_plan.pub.split_k, 1, 0.0};
-    if ((st = measure(best, &best.seconds))) return st;
-    if (default_seconds) *default_seconds = best.seconds;
+    if ((st = measure(&best, &best.seconds))) return st;
+    // a product with a few rows or columns runs on a streaming kernel unless a tile is measured
+    // to beat it: that kernel is the default here, and the table keeps no entry when it wins
+    const bool streaming = vec && (fewrows_applies(M, N, K, K, N) || fewrows_nt_applies(N, M, K, N, K, true));
+    double streaming_seconds = 0;
+    if (streaming) {
+        tune_erase(M, N, K, true);
+        if ((st = measure(nullptr, &streaming_seconds))) return st;
+    }
+    if (default_seconds) *default_seconds = streaming ? streaming_seconds : best.seconds;
 
     const auto t0 = std::chrono::steady_clock::now();
     auto spent = [&] { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count(); };
@@ -1130,12 +1141,21 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
                 // skip candidates the model already puts far behind: a split whose slices alone outweigh the product
                 if ((double)split * M * N * 4.0 > 64.0 * ((double)M * K + (double)K * N) * 4.0 && split > 1) continue;
                 double secs = 0;
-                if ((st = measure(c, &secs))) return st;
+                if ((st = measure(&c, &secs))) return st;
                 c.seconds = secs;
                 if (secs < best.seconds) best = c;
             }
             if (out_of_time) break;
         }
+    }
+    if (streaming && streaming_seconds <= best.seconds) {
+        if (best_seconds) *best_seconds = streaming_seconds;
+        if (best_plan) {
+            GemmPlan plan;
+            if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
+            *best_plan = plan.pub;
+        }
+        return CAKE_HIP_OK;
     }
     tune_store(M, N, K, vec, best);
     if (vec) {

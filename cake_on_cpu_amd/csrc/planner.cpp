@@ -114,6 +114,12 @@ void tune_store(int M, int N, int K, bool vector_ok, const TunedChoice& c)
     g_tuned[TuneKey{M, N, K, vector_ok ? 1 : 0}] = c;
 }
 
+void tune_erase(int M, int N, int K, bool vector_ok)
+{
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    g_tuned.erase(TuneKey{M, N, K, vector_ok ? 1 : 0});
+}
+
 void tune_clear()
 {
     std::lock_guard<std::mutex> lock(g_tuned_mutex);

@@ -53,6 +53,7 @@ int plan_gemm_choice(int M, int N, int K, int sched, const TunedChoice& c, bool 
 // when the caller gives no override.  Thread-safe.
 bool tune_lookup(int M, int N, int K, bool vector_ok, TunedChoice* out);
 void tune_store(int M, int N, int K, bool vector_ok, const TunedChoice& c);
+void tune_erase(int M, int N, int K, bool vector_ok);
 void tune_clear();
 int tune_count();
 int tune_save(const char* path);  // CAKE_HIP_* status

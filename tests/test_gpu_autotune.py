@@ -41,3 +41,20 @@ def test_autotune_picks_a_measured_plan_and_results_stay_right(shape, tmp_path):
     assert cake.plan(M, N, K).as_dict() == before
     assert cake.tune_load(path) >= 1
     assert cake.plan(M, N, K).as_dict() == now
+
+
+@pytest.mark.parametrize("shape", [(16, 2048, 4096), (4096, 2048, 8)], ids=lambda s: "x".join(map(str, s)))
+def test_autotune_of_a_streaming_shape(shape):
+    """Few rows or columns: the streaming kernel is the measured default, a tile only enters the
+    table when it is faster, and the product stays right either way."""
+    M, K, N = shape
+    plan, best, base = cake.autotune(M, N, K, budget_seconds=2.0)
+    print(f"autotune streaming M={M} K={K} N={N} best={best * 1e6:.1f} us default={base * 1e6:.1f} us "
+          f"entries={cake.tune_count()}", flush=True)
+    assert best > 0 and base > 0 and best <= base
+    assert (cake.tune_count() >= 1) == (best < base)       # no entry when the streaming kernel wins
+    A, B = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+    Cm = np.zeros((M, N), np.float32)
+    cake.cake_sgemm(A, B, Cm, M, N, K, 4)
+    C64, S = oracle.gemm_f64(A, B)
+    assert oracle.max_rel_err(Cm, C64, S) <= 5e-6
