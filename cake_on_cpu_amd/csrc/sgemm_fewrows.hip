@@ -48,6 +48,7 @@ __device__ __forceinline__ float load_f32(const float* base, int byte_offset, un
 
 static constexpr int FR_COLS = 256;     // nn: columns of B per workgroup
 static constexpr int FR_ROWS = 64;      // nt: rows of W per workgroup
+static constexpr int FR_STAGES = 2;     // nn: half groups of 16 k (8 loads of B each) in flight per wave
 static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave and loop step
 
 // The part of [kbeg, kend) that wave `wave` of 4 walks: quarters rounded up to 16 k
@@ -90,22 +91,30 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
 #pragma unroll
     for (int c = 0; c < 16; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // Groups of 16 k that lie wholly below kw1 <= K: every row asked for exists, so the record
-    // counts are exact (records_left must not be asked about a start past the end of an operand:
-    // its difference would wrap to "everything in range").  Half a group (8 loads of B) is in
-    // flight while the other half is multiplied.
-    auto load_a = [&](int k) { return buffer_load_f32x4(A + k, a_off, records_left(a_elems, (unsigned)k)); };
-    auto load_half = [&](int k, int h, f32x4 (&b)[2][4]) {
+    // Groups of 16 k that lie wholly below kw1 <= K, in units of half a group (8 loads of B, 32
+    // MFMAs).  FR_STAGES units are in flight: each is multiplied and its registers refilled with
+    // the unit FR_STAGES further on.  A unit past the end gets a record count of 0, which turns
+    // its loads into zeros without a memory access, so the loop body needs no branch and the
+    // wait counts in front of the MFMAs are exact.  Every row asked for below the end exists, so
+    // those record counts are exact too (records_left must not be asked about a start past the
+    // end of an operand: its difference would wrap to "everything in range").
+    const int units = 2 * ((kw1 - kw0) >> 4);
+    auto load_a = [&](int q) {
+        const int kq = kw0 + 16 * (q >> 1);
+        return buffer_load_f32x4(A + kq, a_off, q < units ? records_left(a_elems, (unsigned)kq) : 0u);
+    };
+    auto load_unit = [&](int q, int h, f32x4 (&b)[2][4]) {
+        const int kq = kw0 + 16 * (q >> 1) + 2 * h;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const unsigned skip = (unsigned)(k + 2 * h + e) * (unsigned)ldb;
-            const unsigned rec = records_left(b_elems, skip);
+            const unsigned skip = (unsigned)(kq + e) * (unsigned)ldb;
+            const unsigned rec = q < units ? records_left(b_elems, skip) : 0u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) b[e][j] = stream_load_f32x4(B + n0 + (size_t)skip, b_off[j], rec);
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
     };
-    auto mma_half = [&](const f32x4& a, int h, const f32x4 (&b)[2][4]) {
+    auto mma_unit = [&](const f32x4& a, int h, const f32x4 (&b)[2][4]) {
 #pragma unroll
         for (int e = 0; e < 2; ++e)
 #pragma unroll
@@ -116,28 +125,24 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
                         __builtin_amdgcn_mfma_f32_16x16x4f32(a[2 * h + e], b[e][j][c], acc[4 * j + c], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
-    int k = kw0;
-    {
-        f32x4 a_cur = {0.f, 0.f, 0.f, 0.f}, a_nxt = a_cur;
-        f32x4 b0[2][4], b1[2][4];
-        if (k + 16 <= kw1) {
-            a_cur = load_a(k);
-            load_half(k, 0, b0);
-            // no branch inside the loop body: the wait counts in front of the MFMAs are exact
-            for (; k + 32 <= kw1; k += 16) {
-                load_half(k, 1, b1);
-                mma_half(a_cur, 0, b0);
-                a_nxt = load_a(k + 16);
-                load_half(k + 16, 0, b0);
-                mma_half(a_cur, 1, b1);
-                a_cur = a_nxt;
+    if (units > 0) {
+        f32x4 a[FR_STAGES / 2];
+        f32x4 b[FR_STAGES][2][4];
+#pragma unroll
+        for (int i = 0; i < FR_STAGES; ++i) {
+            if (i % 2 == 0) a[i / 2] = load_a(i);
+            load_unit(i, i % 2, b[i]);
+        }
+        for (int q = 0; q < units; q += FR_STAGES) {
+#pragma unroll
+            for (int i = 0; i < FR_STAGES; ++i) {
+                mma_unit(a[i / 2], i % 2, b[i]);
+                if (i % 2 == 1) a[i / 2] = load_a(q + i + FR_STAGES);  // both halves of the group are done
+                load_unit(q + i + FR_STAGES, i % 2, b[i]);
             }
-            load_half(k, 1, b1);
-            mma_half(a_cur, 0, b0);
-            mma_half(a_cur, 1, b1);
-            k += 16;
         }
     }
+    const int k = kw0 + 8 * units;
     if (k < kw1) {
         // the last 1..15 k of the wave's part, element by element: k at or past kw1 reads as zero
         // on both sides (rows of B between kw1 and K belong to another wave or slice)
@@ -199,6 +204,7 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
 // of a workgroup take the steps of 32 k in turn, so together they read 512 contiguous bytes of
 // every row at a time.
 static constexpr int NT_STEP = 32;                               // k per step of a wave
+static constexpr int NT_STAGES = 1;                             // steps in flight per wave
 static constexpr int NT_PITCH = 36;                              // floats per staged row: 16-byte reads of 16 rows spread over all banks
 static constexpr int NT_WAVE_FLOATS = (FR_ROWS + 16) * NT_PITCH; // 64 rows of W and 16 of X
 
@@ -249,13 +255,15 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     // a group of 8 rows that starts past the end gets a count of 0 (records_left must not be asked
     // about a start past the end: its difference would wrap to "everything in range").
     // TAIL: the last, partial step of the slice; k at and past kend reads as zero on both sides.
-    auto load_step = [&](int k, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2], float (&gk)[8]) {
+    // live = false: a step past the end of the wave's share, loaded as zeros without a memory
+    // access (record count 0), so that the loop below needs no branch
+    auto load_step = [&](int k, bool live, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2], float (&gk)[8]) {
         constexpr bool TAIL = decltype(tail)::value;
         const int below = kend - (k + 4 * lc);   // of this lane's 4 k, how many lie below kend
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const unsigned used = (unsigned)(8 * t) * (unsigned)ldw + (unsigned)k;
-            const unsigned rec = 8 * t < rows_left ? records_left(w_elems, used) : 0u;
+            const unsigned rec = live && 8 * t < rows_left ? records_left(w_elems, used) : 0u;
             gw[t] = stream_load_f32x4(Wb + (size_t)(8 * t) * ldw + k, TAIL && below <= 0 ? BUF_OOB : w_off, rec);
             if (TAIL) gw[t] = keep_below(gw[t], below);
         }
@@ -263,7 +271,7 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const unsigned used = (unsigned)(8 * t) * (unsigned)ldx + (unsigned)k;
-                const unsigned rec = 8 * t < M ? records_left(x_elems, used) : 0u;
+                const unsigned rec = live && 8 * t < M ? records_left(x_elems, used) : 0u;
                 gx[t] = buffer_load_f32x4(X + (size_t)(8 * t) * ldx + k, TAIL && below <= 0 ? BUF_OOB : x_off, rec);
                 if (TAIL) gx[t] = keep_below(gx[t], below);
             }
@@ -271,7 +279,7 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
 #pragma unroll
             for (int t = 0; t < 8; ++t) {   // k = 4 t + lq of the step, i = li
                 const unsigned used = (unsigned)(k + 4 * t) * (unsigned)ldx;
-                const unsigned rec = (!TAIL || k + 4 * t < kend) ? records_left(x_elems, used) : 0u;
+                const unsigned rec = live && (!TAIL || k + 4 * t < kend) ? records_left(x_elems, used) : 0u;
                 gk[t] = load_f32(X + (size_t)(k + 4 * t) * ldx, TAIL && k + 4 * t + lq >= kend ? BUF_OOB : x_off, rec);
             }
         }
@@ -304,24 +312,27 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     };
 
     {
-        f32x4 gw[8], gx[2];
-        float gk[8];
+        // The wave's steps are wave, wave + 4, ... below `full`; NT_STAGES of them are in flight.
+        f32x4 gw[NT_STAGES][8], gx[NT_STAGES][2];
+        float gk[NT_STAGES][8];
         const int full = (kend - kbeg) / NT_STEP;
-        int s = wave;
-        if (s < full) {
-            load_step(kbeg + NT_STEP * s, std::false_type{}, gw, gx, gk);
-            // no branch inside the loop body: the wait counts in front of the stores are exact
-            for (; s + 4 < full; s += 4) {
-                store_step(gw, gx, gk);
-                load_step(kbeg + NT_STEP * (s + 4), std::false_type{}, gw, gx, gk);
-                compute_step();
+        const int mine = full > wave ? (full - wave + 3) >> 2 : 0;
+        auto step_k = [&](int j) { return kbeg + NT_STEP * (wave + 4 * j); };
+        if (mine > 0) {
+#pragma unroll
+            for (int i = 0; i < NT_STAGES; ++i) load_step(step_k(i), i < mine, std::false_type{}, gw[i], gx[i], gk[i]);
+            for (int j = 0; j < mine; j += NT_STAGES) {
+#pragma unroll
+                for (int i = 0; i < NT_STAGES; ++i) {
+                    store_step(gw[i], gx[i], gk[i]);
+                    load_step(step_k(j + i + NT_STAGES), j + i + NT_STAGES < mine, std::false_type{}, gw[i], gx[i], gk[i]);
+                    compute_step();
+                }
             }
-            store_step(gw, gx, gk);
-            compute_step();
         }
         if (((kend - kbeg) & (NT_STEP - 1)) && wave == (full & 3)) {
-            load_step(kbeg + NT_STEP * full, std::true_type{}, gw, gx, gk);
-            store_step(gw, gx, gk);
+            load_step(kbeg + NT_STEP * full, true, std::true_type{}, gw[0], gx[0], gk[0]);
+            store_step(gw[0], gx[0], gk[0]);
             compute_step();
         }
     }
