@@ -590,8 +590,9 @@ static int pack_common(int which, int dir, const float* src, float* dst, int M, 
     IndexTables tab;
     if ((st = build_tables(which, g, &at, &tab, stream))) return st;
     st = timer.family(4, [&] {
-        return dir == 0 ? launch_pack(in.dev, out.dev, rows, cols, cols, rows_p, cols_p, tab, stream)
-                        : launch_unpack(in.dev, out.dev, rows, cols, cols, tab, stream);
+        const int fast = which == 0 ? g.mr : g.nr;
+        return dir == 0 ? launch_pack(in.dev, out.dev, rows, cols, cols, rows_p, cols_p, tab, fast, which == 0, stream)
+                        : launch_unpack(in.dev, out.dev, rows, cols, cols, tab, fast, which == 0, stream);
     });
     if (st) return st;
     if ((st = timer.stop())) return st;
@@ -663,11 +664,11 @@ int cake_hip_sgemm_packed(const float* A, const float* B, float* C, int M, int N
     IndexTables ta{}, tb{};
     if (packedA) {
         if ((st = build_tables(0, g, &at, &ta, stream))) return st;
-        if ((st = timer.family(4, [&] { return launch_unpack(a.dev, ua, M, K, K, ta, stream); }))) return st;
+        if ((st = timer.family(4, [&] { return launch_unpack(a.dev, ua, M, K, K, ta, g.mr, true, stream); }))) return st;
     }
     if (packedB) {
         if ((st = build_tables(1, g, &at, &tb, stream))) return st;
-        if ((st = timer.family(4, [&] { return launch_unpack(b.dev, ub, K, N, N, tb, stream); }))) return st;
+        if ((st = timer.family(4, [&] { return launch_unpack(b.dev, ub, K, N, N, tb, g.nr, false, stream); }))) return st;
     }
     const float* ga = packedA ? ua : a.dev;
     const float* gb = packedB ? ub : b.dev;

@@ -129,11 +129,14 @@ hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hi
 // Packed layouts.  which: 0 = A, 1 = B, 2 = C.
 hipError_t launch_build_index_tables(int which, const PackGeom& g, int4* row_tab, int4* col_tab,
                                      hipStream_t stream);
-// dst_packed[offset(r,c)] = (r,c) inside the matrix ? src[r*ld + c] : 0   over the padded extent
+// dst_packed[offset(r,c)] = (r,c) inside the matrix ? src[r*ld + c] : 0   over the padded extent.
+// fast / rows_fast: the short axis of a micro-panel (A: mr rows, rows_fast; B and C: nr columns),
+// which the packed layout stores fastest; 0 selects the element-wise kernel.
 hipError_t launch_pack(const float* src, float* dst_packed, int rows, int cols, int ld,
-                       int rows_padded, int cols_padded, IndexTables tab, hipStream_t stream);
+                       int rows_padded, int cols_padded, IndexTables tab, int fast, bool rows_fast,
+                       hipStream_t stream);
 // dst[r*ld + c] = src_packed[offset(r,c)] over the real extent
 hipError_t launch_unpack(const float* src_packed, float* dst, int rows, int cols, int ld,
-                         IndexTables tab, hipStream_t stream);
+                         IndexTables tab, int fast, bool rows_fast, hipStream_t stream);
 
 }  // namespace cake

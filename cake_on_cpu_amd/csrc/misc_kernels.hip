@@ -421,10 +421,126 @@ static dim3 rowwise_grid(int rows, int cols)
     return dim3(bx, rows);
 }
 
+// The same two copies through an LDS tile, so that BOTH sides move in contiguous runs.  In the
+// packed layouts a micro-panel is stored with its short axis fastest: A as [k][mr rows], B and C
+// as [k or row][nr columns].  A thread per row-major element therefore scatters 4-byte stores
+// `fast` floats apart (A) or writes 64-byte pieces (B, C).  Here a workgroup takes a tile of up
+// to 64 x 64 elements whose short-axis extent is a whole number of panels, moves it between the
+// row-major side and LDS with rows of 256 bytes, and walks the packed side in packed order
+// (short axis fastest, then the long axis, then the next panel), which is ascending addresses
+// wherever the tile lies inside one block of the schedule.  Offsets still come from the index
+// tables, so a tile that straddles blocks or starts off a panel boundary is only slower.
+static constexpr int PT = 64;
+
+template <bool UNPACK>
+__global__ void __launch_bounds__(256) pack_tile_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                        int rows, int cols, int ld, int rows_p, int cols_p,
+                                                        IndexTables tab, int fast, int rows_fast, int tr, int tc)
+{
+    // Row pitch 64 + ceil(64 / fast): a wave walking the packed order touches `fast` short-axis
+    // positions times 64 / fast long-axis positions, which this pitch spreads over all banks
+    __shared__ float tile[PT * 2 * PT];
+    __shared__ int4 Rt[PT], Ct[PT];
+    const int pitch = PT + (PT + fast - 1) / fast;
+    const int tid = threadIdx.x;
+    const int r0 = blockIdx.y * tr, c0 = blockIdx.x * tc;
+    if (tid < PT) {
+        if (tid < tr && r0 + tid < rows_p) Rt[tid] = tab.row[r0 + tid];
+    } else if (tid < 2 * PT) {
+        const int i = tid - PT;
+        if (i < tc && c0 + i < cols_p) Ct[i] = tab.col[c0 + i];
+    }
+    const int lim_r = UNPACK ? rows : rows_p, lim_c = UNPACK ? cols : cols_p;  // extent of the packed-side walk
+    const int dc_rm = tid & 63;   // row-major side: a wave per row of the tile
+    const float inv_fast = 1.0f / (float)fast;
+    const int count = tr * tc;
+
+    // Fixed trip counts and full unrolling: all 16 loads of a thread are in flight together
+    // (with a run-time bound the compiler keeps one load per thread in flight, and the kernel
+    // runs at the speed of 16 memory latencies per tile).
+    if (!UNPACK) {
+        float v[PT / 4];
+#pragma unroll
+        for (int i = 0; i < PT / 4; ++i) {
+            const int dr = (tid >> 6) + 4 * i;
+            const int r = r0 + dr, c = c0 + dc_rm;
+            v[i] = (dr < tr && dc_rm < tc && r < rows && c < cols) ? src[(size_t)r * ld + c] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < PT / 4; ++i) tile[((tid >> 6) + 4 * i) * pitch + dc_rm] = v[i];
+    }
+    __syncthreads();
+    {
+        float v[PT * PT / 256];
+        size_t off[PT * PT / 256];
+        int at[PT * PT / 256];
+        bool live[PT * PT / 256];
+#pragma unroll
+        for (int i = 0; i < PT * PT / 256; ++i) {
+            const int e = tid + 256 * i;
+            // e = (panel * long + l) * fast + j; exact for e < 2^22: (e + 0.5) / fast is at least
+            // 0.5 / fast away from an integer
+            const int q = (int)(((float)e + 0.5f) * inv_fast);
+            const int j = e - q * fast;
+            const int panel = q >> 6, l = q & 63;      // the long axis of a tile is 64
+            const int dr = rows_fast ? panel * fast + j : l;
+            const int dc = rows_fast ? l : panel * fast + j;
+            const int r = r0 + dr, c = c0 + dc;
+            live[i] = e < count && dr < tr && dc < tc && r < lim_r && c < lim_c;
+            off[i] = live[i] ? table_offset(Rt[dr], Ct[dc]) : 0;
+            at[i] = dr * pitch + dc;
+            if (UNPACK) v[i] = live[i] ? src[off[i]] : 0.f;
+            else v[i] = live[i] ? tile[at[i]] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < PT * PT / 256; ++i) {
+            if (!live[i]) continue;
+            if (UNPACK) tile[at[i]] = v[i];
+            else dst[off[i]] = v[i];
+        }
+    }
+    if (UNPACK) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PT / 4; ++i) {
+            const int dr = (tid >> 6) + 4 * i;
+            const int r = r0 + dr, c = c0 + dc_rm;
+            if (dr < tr && dc_rm < tc && r < rows && c < cols) dst[(size_t)r * ld + c] = tile[dr * pitch + dc_rm];
+        }
+    }
+}
+
+// fast = rows (rows_fast) or columns of a micro-panel; 0 or more than 64: the element-wise kernels
+template <bool UNPACK>
+static hipError_t launch_pack_tiles(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
+                                    int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
+{
+    const int whole = fast * (PT / fast);   // a whole number of panels, at most 64
+    const int tr = rows_fast ? whole : PT, tc = rows_fast ? PT : whole;
+    const int ext_r = UNPACK ? rows : rows_p, ext_c = UNPACK ? cols : cols_p;
+    const int tiles_c = (ext_c + tc - 1) / tc;
+    const int tiles_r = (ext_r + tr - 1) / tr;
+    for (int t0 = 0; t0 < tiles_r; t0 += 65535) {   // grid.y is limited to 65535
+        const int nt = tiles_r - t0 < 65535 ? tiles_r - t0 : 65535;
+        const int r0 = t0 * tr;
+        IndexTables t = {tab.row + r0, tab.col};
+        const float* s = UNPACK ? src : src + (size_t)r0 * ld;
+        float* d = UNPACK ? dst + (size_t)r0 * ld : dst;
+        const int live = rows - r0 < 0 ? 0 : rows - r0;
+        hipLaunchKernelGGL(pack_tile_kernel<UNPACK>, dim3(tiles_c, nt), dim3(256), 0, stream, s, d, live, cols, ld,
+                           rows_p - r0, cols_p, t, fast, rows_fast ? 1 : 0, tr, tc);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 hipError_t launch_pack(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
-                       int cols_p, IndexTables tab, hipStream_t stream)
+                       int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
 {
     if (rows_p <= 0 || cols_p <= 0) return hipSuccess;
+    if (fast >= 1 && fast <= PT)
+        return launch_pack_tiles<false>(src, dst, rows, cols, ld, rows_p, cols_p, tab, fast, rows_fast, stream);
     // grid.y is limited to 65535 rows per launch
     for (int r0 = 0; r0 < rows_p; r0 += 65535) {
         const int nr = rows_p - r0 < 65535 ? rows_p - r0 : 65535;
@@ -439,9 +555,11 @@ hipError_t launch_pack(const float* src, float* dst, int rows, int cols, int ld,
 }
 
 hipError_t launch_unpack(const float* src, float* dst, int rows, int cols, int ld, IndexTables tab,
-                         hipStream_t stream)
+                         int fast, bool rows_fast, hipStream_t stream)
 {
     if (rows <= 0 || cols <= 0) return hipSuccess;
+    if (fast >= 1 && fast <= PT)
+        return launch_pack_tiles<true>(src, dst, rows, cols, ld, rows, cols, tab, fast, rows_fast, stream);
     for (int r0 = 0; r0 < rows; r0 += 65535) {
         const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
         IndexTables t = {tab.row + r0, tab.col};
