@@ -758,6 +758,33 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
     return stage_out(o, stream);
 }
 
+// How the input of a convolution is staged for the on-the-fly gather (conv_stage_input_kernel):
+// zero padding written out, of every `stride` rows the RH reachable ones kept, every row split
+// into its PW reachable column phases of Wq floats.
+struct ConvStage {
+    bool copy;      // false: stride 1 without padding reads the input as it lies
+    int RH, PW, Hs, Wq, pitch;
+    double elems;   // floats of the staged input
+};
+
+static ConvStage conv_stage(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad)
+{
+    ConvStage s{};
+    s.copy = pad > 0 || stride > 1;
+    if (!s.copy) {
+        s.RH = s.PW = 1; s.Hs = Hin; s.Wq = s.pitch = Win;
+    } else {
+        const int Hp = Hin + 2 * pad, Wp = Win + 2 * pad;
+        s.RH = Hf < stride ? Hf : stride;
+        s.PW = Wf < stride ? Wf : stride;
+        s.Hs = (Hp + stride - 1) / stride * s.RH;
+        s.Wq = ((Wp + stride - 1) / stride + 3) & ~3;
+        s.pitch = s.PW * s.Wq;
+    }
+    s.elems = (double)batch * Cin * s.Hs * s.pitch;
+    return s;
+}
+
 size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout, int Hf, int Wf,
                                  int stride, int pad)
 {
@@ -765,13 +792,11 @@ size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
     if (batch <= 0 || Cin <= 0 || Cout <= 0 || conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout)) return 0;
     const size_t ncols = (size_t)batch * Hout * Wout;
     // two-step path: column matrix + a [Cout][ncols] product when the caller wants NCHW;
-    // gather path: a zero-padded copy of the input
+    // gather path: the staged copy of the input
     const size_t two_step = ((size_t)Cin * Hf * Wf * ncols + (size_t)Cout * ncols) * sizeof(float);
-    const size_t padded = (size_t)batch * Cin * (Hin + 2 * pad) * ((Win + 2 * pad + 3) & ~3) * sizeof(float);
-    return (two_step > padded ? two_step : padded) + 512;
+    const size_t staged = (size_t)conv_stage(batch, Cin, Hin, Win, Hf, Wf, stride, pad).elems * sizeof(float);
+    return (two_step > staged ? two_step : staged) + 512;
 }
-
-// ceil(2^32 / d), or 0 for d == 1 (the loaders then skip the division)
 
 // explicit == 0: gather the column matrix inside the GEMM when the geometry allows it
 static int conv2d_common(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
@@ -801,20 +826,18 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
 
     // The on-the-fly gather needs: 4 consecutive columns inside one output row and
-    // byte offsets into the (padded) input below 2^31
-    // (rows of the padded copy are a multiple of 4 floats apart, so it is written in 16-byte pieces)
-    const int Hp = Hin + 2 * pad, Wp = pad > 0 ? (Win + 2 * pad + 3) & ~3 : Win;
-    const double padded_elems = (double)batch * Cin * Hp * Wp;
+    // byte offsets into the staged input below 2^31
+    const ConvStage sg = conv_stage(batch, Cin, Hin, Win, Hf, Wf, stride, pad);
     const bool implicit = !explicit_cols && (Wout % 4 == 0) &&
-                          padded_elems * 4 < 2147483648.0 &&
+                          sg.elems * 4 < 2147483648.0 &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
     if (implicit) {
         const float* image = i.dev;
-        if (pad > 0) {  // a zero-padded copy, so that the gather has no edge cases
+        if (sg.copy) {
             char* ws = static_cast<char*>(workspace);
             if (!ws) {
-                if ((st = g_ctx.conv.reserve((size_t)padded_elems * 4 + 256))) return st;
+                if ((st = g_ctx.conv.reserve((size_t)sg.elems * 4 + 256))) return st;
                 ws = static_cast<char*>(g_ctx.conv.ptr);
             } else if (!is_device_pointer(ws)) {
                 return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
@@ -823,25 +846,30 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         }
         ConvGeom cv{};
         cv.in = image;
-        cv.Cin = Cin; cv.Hin = Hp; cv.Win = Wp; cv.Hf = Hf; cv.Wf = Wf;
-        cv.Hout = Hout; cv.Wout = Wout; cv.stride = stride;
+        cv.in_bytes = (unsigned)(sg.elems * 4);
+        cv.Cin = Cin; cv.plane_rows = sg.Hs; cv.pitch = sg.pitch; cv.row_step = sg.RH;
+        cv.Hout = Hout; cv.Wout = Wout; cv.row_n = Wout;
         if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
         int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
         cv.tap_table = taps;
         cv.out_nchw = out_nchw ? 1 : 0;
         if ((st = timer.start())) return st;
-        st = timer.family(3, [&] { return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, Hp, Wp, Hf, Wf, stream); });
+        st = timer.family(3, [&] {
+            return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, sg.Hs, sg.pitch, sg.Wq, Hf, Wf, stride, sg.RH, stream);
+        });
         if (st) return st;
-        if (pad > 0) {
+        if (sg.copy) {
             st = timer.family(3, [&] {
-                return launch_pad_planes(i.dev, const_cast<float*>(image), (size_t)batch * Cin, Hin, Win, pad, Wp, stream);
+                float* dst = const_cast<float*>(image);
+                // stride 1: the plain zero-padded copy has a kernel of its own (a workgroup per plane)
+                return stride == 1 ? launch_pad_planes(i.dev, dst, (size_t)batch * Cin, Hin, Win, pad, sg.pitch, stream)
+                                   : launch_conv_stage_input(i.dev, dst, (size_t)batch * Cin, Hin, Win, pad, stride,
+                                                             sg.RH, sg.PW, sg.Hs, sg.Wq, stream);
             });
             if (st) return st;
         }
-        // stride 1: 4 consecutive columns are one 16-byte load from an image row
-        const int b_mode = stride == 1 ? LOAD_IM2COL_ROW : LOAD_IM2COL;
         st = run_gemm(w.dev, nullptr, o.dev, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
-                      b_mode, stream, timer, &cv);
+                      LOAD_IM2COL_ROW, stream, timer, &cv);
         if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);

@@ -20,13 +20,20 @@ struct IndexTables {
     const int4* col;
 };
 
-// Geometry of a convolution whose column matrix B[k][n] is gathered on the fly:
-// k = c*Hf*Wf + h*Wf + w, n = b*Hout*Wout + ho*Wout + wo,
-// B[k][n] = in[b][c][ho*stride + h][wo*stride + w].  `in` carries its padding
-// already (Hin, Win include it), so every window position is inside the image.
+// Geometry of a convolution whose column matrix B[k][n] is gathered on the fly from a staged
+// copy of the input (conv_stage_input_kernel in misc_kernels.hip: padding written out, rows split
+// into column phases when the stride is above 1):
+// k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
+// B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
 struct ConvGeom {
-    const float* in;
-    int Cin, Hin, Win, Hf, Wf, Hout, Wout, stride;
+    const float* in;        // the staged input (the input itself for stride 1 without padding)
+    unsigned in_bytes;      // its size: loads past it read as zero
+    int Cin;
+    int plane_rows;         // stored rows per (image, channel) plane
+    int pitch;              // floats per stored row
+    int row_step;           // stored rows per output row
+    int Hout, Wout;
+    int row_n;              // columns of the product per output row (a multiple of 4)
     const int* tap_table;   // byte offset of tap k = (c, h, w) inside one image, K + CONV_TAP_TABLE_EXTRA entries
     int out_nchw;           // epilogue writes C as [batch][M][Hout*Wout] instead of [M][N]
 };
@@ -72,8 +79,8 @@ const TileInfo& tile_info(int tile_id);
 enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
-    LOAD_IM2COL = 3, // B only: column matrix of a convolution gathered from the NCHW input
-    LOAD_IM2COL_ROW = 4  // the same for stride 1: one 16-byte load per 4 columns
+    LOAD_IM2COL_ROW = 4  // B only: column matrix of a convolution gathered from the staged NCHW input,
+                         // one 16-byte load per 4 columns
 };
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
@@ -113,10 +120,14 @@ hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int H
 // are (Hin+2pad) rows of `pitch` floats (pitch % 4 == 0, pitch >= Win+2pad, out 16-byte aligned)
 hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
                              int pitch, hipStream_t stream);
-// table[k] = byte offset of filter tap k inside one image; `extra` zero entries follow
+// The input of a convolution staged for the gather: see conv_stage_input_kernel.  `out` holds
+// planes * Hs * PW * Wq floats (Wq % 4 == 0, 16-byte aligned).
+hipError_t launch_conv_stage_input(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
+                                   int stride, int RH, int PW, int Hs, int Wq, hipStream_t stream);
+// table[k] = byte offset of filter tap k inside one staged image; `extra` zero entries follow
 enum { CONV_TAP_TABLE_EXTRA = 256 };
-hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win, int Hf, int Wf,
-                                 hipStream_t stream);
+hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch, int Wq, int Hf, int Wf,
+                                 int stride, int RH, hipStream_t stream);
 // [Cout][batch*HW] -> [batch][Cout][HW]
 hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
                              hipStream_t stream);

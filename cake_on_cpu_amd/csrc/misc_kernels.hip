@@ -9,6 +9,28 @@
 namespace cake {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));  // 16 bytes at any 4-byte address
+
+// n / d for n < 2^31 as one 32 x 32 -> 64 bit multiply and a shift (division by an invariant
+// integer): with s = ceil(log2 d) and m = floor(2^(31+s) / d) + 1 the error m d - 2^(31+s) is at
+// most d <= 2^s, so n (m d - 2^(31+s)) < 2^(31+s) for every n < 2^31 and the quotient is exact.
+// A hardware division costs tens of vector instructions (a 64-bit one well over a hundred), enough
+// to make a write-bound copy compute-bound.
+struct FastDiv {
+    unsigned d, m, sh;
+    __host__ static FastDiv make(unsigned d)
+    {
+        unsigned s = 0;
+        while ((1ull << s) < d) ++s;
+        FastDiv f;
+        f.d = d;
+        f.m = (unsigned)((1ull << (31 + s)) / d + 1);
+        f.sh = 31 + s;
+        return f;
+    }
+    __device__ __forceinline__ unsigned div(unsigned n) const { return (unsigned)(((unsigned long long)n * m) >> sh); }
+};
+
 
 // ---------------------------------------------------------------------------
 // transpose: dst[c][r] = src[r][c] for a rows x cols row-major matrix
@@ -100,24 +122,77 @@ hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin
     return hipGetLastError();
 }
 
-// Byte offset of filter tap k = (c, h, w) inside one image of a convolution's
-// input: table[k] = ((c*Hin + h)*Win + w) * 4 for k < K, 0 for the `extra`
-// entries after it (the gather prefetches a few stages past the end).
+// The input of a strided convolution, staged so that the gather reads consecutive floats: a row
+// of the zero-padded image is split into its `stride` column phases (wi = wq * stride + phase), of
+// which only the PW = min(Wf, stride) phases that a filter tap can reach are kept, each Wq floats
+// long (Wq a multiple of 4); of every `stride` rows only the RH = min(Hf, stride) reachable ones
+// are kept.  Stored row of padded row hi: (hi / stride) * RH + hi % stride.  Output pixel (ho, wo)
+// under tap (h, w) then reads
+//     plane[(ho + h / s) * RH + h % s][w % s][wo + w / s]
+// whose address splits into a pixel part (ho * RH * pitch + wo, pitch = PW * Wq) and a tap part,
+// and 4 consecutive wo are 4 consecutive floats.  stride 1 is the plain zero-padded copy.
+// One thread per float4 of the staged image.
+__global__ void __launch_bounds__(256) conv_stage_input_kernel(const float* __restrict__ in,
+                                                               float* __restrict__ out, unsigned total4,
+                                                               int Hin, int Win, int pad, int stride, int RH,
+                                                               int PW, int Hs, int Wq, FastDiv by_wq4,
+                                                               FastDiv by_pw, FastDiv by_hs, FastDiv by_rh)
+{
+    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < total4; i += gridDim.x * 256) {
+        unsigned t = by_wq4.div(i);
+        const int wq = (int)(i - t * by_wq4.d) * 4;
+        unsigned u = by_pw.div(t);
+        const int ph = (int)(t - u * PW);
+        const unsigned plane = by_hs.div(u);
+        const int sr = (int)(u - plane * Hs);
+        const int grp = (int)by_rh.div((unsigned)sr);
+        const int yi = grp * stride + (sr - grp * RH) - pad;
+        const float* src = in + ((size_t)plane * Hin + yi) * Win;
+        const bool row_in = (unsigned)yi < (unsigned)Hin;
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int xi = (wq + e) * stride + ph - pad;
+            v[e] = (row_in && (unsigned)xi < (unsigned)Win) ? src[xi] : 0.f;
+        }
+        *reinterpret_cast<f32x4*>(out + (size_t)i * 4) = v;
+    }
+}
+
+hipError_t launch_conv_stage_input(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
+                                   int stride, int RH, int PW, int Hs, int Wq, hipStream_t stream)
+{
+    const size_t total4 = planes * Hs * PW * (Wq / 4);
+    if (total4 == 0) return hipSuccess;
+    if (Wq % 4 != 0 || total4 >= (1ull << 31)) return hipErrorInvalidValue;
+    size_t blocks = (total4 + 255) / 256;
+    if (blocks > (1u << 20)) blocks = 1u << 20;
+    hipLaunchKernelGGL(conv_stage_input_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, in, out,
+                       (unsigned)total4, Hin, Win, pad, stride, RH, PW, Hs, Wq, FastDiv::make((unsigned)(Wq / 4)),
+                       FastDiv::make((unsigned)PW), FastDiv::make((unsigned)Hs), FastDiv::make((unsigned)RH));
+    return hipGetLastError();
+}
+
+// Byte offset of filter tap k = (c, h, w) inside one staged image (see above):
+// table[k] = (c * Hs * pitch + ((h / s) * RH + h % s) * pitch + (w % s) * Wq + w / s) * 4 for
+// k < K, 0 for the `extra` entries after it (the gather prefetches a few stages past the end).
 __global__ void __launch_bounds__(256) conv_tap_table_kernel(int* __restrict__ table, int K, int extra,
-                                                             int Hin, int Win, int Hf, int Wf)
+                                                             int Hs, int pitch, int Wq, int Hf, int Wf,
+                                                             int stride, int RH)
 {
     const int k = blockIdx.x * 256 + threadIdx.x;
     if (k >= K + extra) return;
     const int c = k / (Hf * Wf), tap = k - c * (Hf * Wf);
     const int h = tap / Wf, w = tap - h * Wf;
-    table[k] = k < K ? ((c * Hin + h) * Win + w) * 4 : 0;
+    const int row = (h / stride) * RH + h % stride;
+    table[k] = k < K ? ((c * Hs + row) * pitch + (w % stride) * Wq + w / stride) * 4 : 0;
 }
 
-hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win, int Hf, int Wf,
-                                 hipStream_t stream)
+hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch, int Wq, int Hf, int Wf,
+                                 int stride, int RH, hipStream_t stream)
 {
     hipLaunchKernelGGL(conv_tap_table_kernel, dim3((K + extra + 255) / 256), dim3(256), 0, stream, table, K,
-                       extra, Hin, Win, Hf, Wf);
+                       extra, Hs, pitch, Wq, Hf, Wf, stride, RH);
     return hipGetLastError();
 }
 
@@ -126,39 +201,41 @@ hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hin, int Win,
 // stride.  grid.y = row k of the column matrix (one (c, h, w) filter tap),
 // threads run along n = (b, ho, wo).
 // ---------------------------------------------------------------------------
-template <int VEC>
+// Each thread writes 4 consecutive n (16 bytes at any 4-byte alignment); they may run over the end
+// of an output row or image, so the position is carried from element to element.  ncols < 2^31.
 __global__ void __launch_bounds__(256) im2col_kernel(const float* __restrict__ in,
-                                                     float* __restrict__ cols, int batch, int Cin,
+                                                     float* __restrict__ cols, unsigned ncols, int Cin,
                                                      int Hin, int Win, int Hf, int Wf, int Hout,
-                                                     int Wout, int stride, int pad)
+                                                     int Wout, int stride, int pad, FastDiv by_hw,
+                                                     FastDiv by_wout, FastDiv by_taps, FastDiv by_wf)
 {
-    const int k = blockIdx.y;
-    const int c = k / (Hf * Wf);
-    const int hw = k - c * (Hf * Wf);
-    const int h = hw / Wf, w = hw - h * Wf;
-    const int HW = Hout * Wout;
-    const size_t ncols = (size_t)batch * HW;
+    const unsigned k = blockIdx.y;
+    const unsigned c = by_taps.div(k);
+    const unsigned hw = k - c * (Hf * Wf);
+    const int h = (int)by_wf.div(hw), w = (int)(hw - h * Wf);
     float* row = cols + (size_t)k * ncols;
 
-    for (size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC; n < ncols;
-         n += (size_t)gridDim.x * 256 * VEC) {
-        const int b = (int)(n / HW);
-        const int r = (int)(n - (size_t)b * HW);
-        const int ho = r / Wout, wo = r - ho * Wout;
-        const int hi = ho * stride + h - pad;
-        const float* src = in + (((size_t)b * Cin + c) * Hin + hi) * Win;
-        const bool hrow = hi >= 0 && hi < Hin;
-        float v[VEC];
+    for (unsigned n = (blockIdx.x * 256 + threadIdx.x) * 4; n < ncols; n += gridDim.x * 1024) {
+        unsigned b = by_hw.div(n);
+        const unsigned r = n - b * by_hw.d;
+        int ho = (int)by_wout.div(r);
+        int wo = (int)(r - ho * Wout);
+        float v[4];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const int wi = (wo + e) * stride + w - pad;  // VEC > 1 only when Wout % VEC == 0
-            v[e] = (hrow && wi >= 0 && wi < Win) ? src[wi] : 0.f;
+        for (int e = 0; e < 4; ++e) {
+            const int hi = ho * stride + h - pad, wi = wo * stride + w - pad;
+            const bool ok = n + e < ncols && hi >= 0 && hi < Hin && wi >= 0 && wi < Win;
+            v[e] = ok ? in[(((size_t)b * Cin + c) * Hin + hi) * Win + wi] : 0.f;
+            if (++wo == Wout) {
+                wo = 0;
+                if (++ho == Hout) { ho = 0; ++b; }
+            }
         }
-        if (VEC == 4) {
-            f32x4 o = {v[0], v[1], v[2], v[3]};
-            __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(row + n));
+        if (n + 4 <= ncols) {
+            const f32x4_u o = {v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(o, reinterpret_cast<f32x4_u*>(row + n));
         } else {
-            row[n] = v[0];
+            for (unsigned e = 0; n + e < ncols; ++e) row[n + e] = v[e];
         }
     }
 }
@@ -169,16 +246,13 @@ hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int H
     const int krows = Cin * Hf * Wf;
     const size_t ncols = (size_t)batch * Hout * Wout;
     if (krows <= 0 || ncols == 0) return hipSuccess;
-    if (krows > 65535) return hipErrorInvalidValue;
-    const bool vec = (Wout % 4 == 0) && (reinterpret_cast<uintptr_t>(cols) % 16 == 0);
-    const size_t per_block = 256 * (vec ? 4 : 1);
-    size_t bx = (ncols + per_block - 1) / per_block;
+    if (krows > 65535 || ncols >= (1ull << 31)) return hipErrorInvalidValue;
+    size_t bx = (ncols + 1023) / 1024;
     if (bx > 4096) bx = 4096;
     const dim3 grid((unsigned)bx, krows);
-    if (vec)
-        hipLaunchKernelGGL(im2col_kernel<4>, grid, dim3(256), 0, stream, in, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad);
-    else
-        hipLaunchKernelGGL(im2col_kernel<1>, grid, dim3(256), 0, stream, in, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad);
+    hipLaunchKernelGGL(im2col_kernel, grid, dim3(256), 0, stream, in, cols, (unsigned)ncols, Cin, Hin, Win, Hf, Wf,
+                       Hout, Wout, stride, pad, FastDiv::make((unsigned)(Hout * Wout)), FastDiv::make((unsigned)Wout),
+                       FastDiv::make((unsigned)(Hf * Wf)), FastDiv::make((unsigned)Wf));
     return hipGetLastError();
 }
 

@@ -1,5 +1,7 @@
-// Macro-tile GEMM instantiations for stride-1 convolution: as sgemm_inst_conv.hip,
-// with the column matrix gathered 4 consecutive pixels per load.
+// Macro-tile GEMM instantiations for convolution: A (the OIHW weights as a
+// Cout x Cin*Hf*Wf matrix) through 16-byte loads, B gathered from the staged NCHW
+// input on the fly, 4 consecutive pixels per load, so the K x N column matrix never
+// exists in memory.
 #include "sgemm_tile.hpp"
 
 namespace cake {

@@ -5,7 +5,6 @@ namespace cake {
 
 hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
-hipError_t launch_sgemm_conv(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_convrow(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 
 template <class T>
@@ -28,10 +27,9 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
                         hipStream_t stream)
 {
     if (grid <= 0) return hipSuccess;
-    if (b_mode == LOAD_IM2COL || b_mode == LOAD_IM2COL_ROW) {
+    if (b_mode == LOAD_IM2COL_ROW) {
         if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
-        return b_mode == LOAD_IM2COL ? launch_sgemm_conv(tile_id, args, grid, stream)
-                                     : launch_sgemm_convrow(tile_id, args, grid, stream);
+        return launch_sgemm_convrow(tile_id, args, grid, stream);
     }
     if (a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4) return launch_sgemm_vec(tile_id, args, grid, stream);
     return launch_sgemm_scalar(tile_id, args, grid, stream);

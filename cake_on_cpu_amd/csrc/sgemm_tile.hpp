@@ -438,18 +438,19 @@ __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_off
 }
 
 // A through 16-byte buffer loads as in VecLoader; B = the column matrix of a
-// convolution, gathered element by element from the NCHW input ("implicit
-// im2col": examples/cake_conv.cpp:1178-1213 without the K x N intermediate).
-// The input the kernel sees has no padding left (the host hands over a
-// zero-padded copy when the convolution has one), so every window position is
-// inside the image and the gather needs no masks beyond the tile edges.
-// A thread's B chunk is 4 consecutive n at one k; with Wout % 4 == 0 those are
-// 4 consecutive output pixels of one image row, so one (image, row, column)
-// triple per thread serves the whole K walk, and only the filter tap (c, h, w)
-// of each k has to be decoded per stage.
+// convolution, gathered from a staged copy of the NCHW input ("implicit im2col":
+// examples/cake_conv.cpp:1178-1213 without the K x N intermediate).
+// The staged input (conv_stage_input_kernel) has its zero padding written out and,
+// for a strided convolution, its rows split into column phases, so that every
+// window position is inside the copy and the 4 consecutive output pixels of a
+// chunk read 4 consecutive floats: a chunk is ONE 16-byte load (4-byte aligned,
+// which buffer loads allow).  A thread's chunk is 4 consecutive n at one k; they
+// lie in one output row (rows of n are a multiple of 4 long), so one (image, row,
+// column) triple per thread serves the whole K walk and only the filter tap
+// (c, h, w) of each k changes from stage to stage.
 template <class T>
-struct ConvLoader {
-    static constexpr int NUM_LOADS = T::A_ITERS + 4 * T::B_ITERS;
+struct ConvRowLoader {
+    static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
     static constexpr bool MASK_A_STORES = true;   // K need not be a multiple of 4 (see VecLoader)
     int a_off[T::A_ITERS];
     int a_k[T::A_ITERS];
@@ -458,7 +459,7 @@ struct ConvLoader {
     const float* a_base;
     unsigned a_elems;     // from a_base to the end of A
     ConvGeom cv;
-    int pix4;             // byte offset of in[b][0][ho*s][wo*s] for the chunk's first n; BUF_OOB for n >= N
+    int pix4;             // byte offset of the chunk's first pixel under tap (0, 0, 0); BUF_OOB for n >= N
                           // (adding a tap offset, which is below 2^31, keeps it out of range)
     // Byte offset of the filter tap of the chunk's k inside an image, for the
     // stage the NEXT load call fetches.  It comes from a small table in memory,
@@ -484,10 +485,10 @@ struct ConvLoader {
         }
         static_assert(T::THREADS % (T::BN / 4) == 0, "a thread keeps the same 4 columns in every chunk");
         const int n = n0 + (tid % (T::BN / 4)) * 4;
-        const int HW = cv.Hout * cv.Wout;
-        const int b = n / HW, r = n - b * HW;
-        const int ho = r / cv.Wout, wo = r - ho * cv.Wout;
-        pix4 = n < g.N ? (((b * cv.Cin) * cv.Hin + ho * cv.stride) * cv.Win + wo * cv.stride) * 4 : BUF_OOB;
+        const int per_image = cv.Hout * cv.row_n;
+        const int b = n / per_image, r = n - b * per_image;
+        const int ho = r / cv.row_n, wo = r - ho * cv.row_n;
+        pix4 = n < g.N ? (((b * cv.Cin) * cv.plane_rows + ho * cv.row_step) * cv.pitch + wo) * 4 : BUF_OOB;
     }
 
     __device__ __forceinline__ f32x4 load_a(int k0, int off) const
@@ -519,76 +520,23 @@ struct ConvLoader {
         return off;
     }
 
-    // The chunk's offset is computed by its first load and kept for the other
-    // three (the loads of a chunk are issued in order).
-    mutable int tap_off[T::B_ITERS];
-
     template <int OP>
     __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
                                              f32x4 (&rb)[T::B_ITERS]) const
     {
-        if constexpr (OP < T::A_ITERS) {
+        if constexpr (OP < T::A_ITERS)
             ra[OP] = load_a(k0, a_k[OP] < kend - k0 ? a_off[OP] : BUF_OOB);
-        } else {
-            constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
-            if constexpr (e == 0) tap_off[it] = tap_offset(it, k0, kend);
-            // BUF_OOB plus a few strides stays out of range
-            rb[it][e] = buffer_load_f32(cv.in, tap_off[it] + e * cv.stride * 4);
-        }
+        else
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(cv.in, tap_offset(OP - T::A_ITERS, k0, kend), cv.in_bytes);
     }
 
     template <int OP>
     __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
-        if constexpr (OP < T::A_ITERS) {
+        if constexpr (OP < T::A_ITERS)
             ra[OP] = load_a(k0, a_off[OP]);
-        } else {
-            constexpr int it = (OP - T::A_ITERS) / 4, e = (OP - T::A_ITERS) % 4;
-            if constexpr (e == 0) tap_off[it] = tap_offset_inside(it, k0);
-            rb[it][e] = buffer_load_f32(cv.in, tap_off[it] + e * cv.stride * 4);
-        }
-    }
-
-    __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
-    {
-        load_all<0>(k0, kend, ra, rb);
-    }
-
-    template <int OP>
-    __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
-    {
-        if constexpr (OP < NUM_LOADS) {
-            load_one<OP>(k0, kend, ra, rb);
-            load_all<OP + 1>(k0, kend, ra, rb);
-        }
-    }
-};
-
-// ConvLoader for stride 1: the 4 consecutive n of a chunk are 4 consecutive
-// input pixels of one image row, so the chunk is ONE 16-byte load (4-byte
-// aligned, which buffer loads allow) instead of four 4-byte loads.
-template <class T>
-struct ConvRowLoader : ConvLoader<T> {
-    using Base = ConvLoader<T>;
-    static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
-
-    template <int OP>
-    __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
-                                             f32x4 (&rb)[T::B_ITERS]) const
-    {
-        if constexpr (OP < T::A_ITERS)
-            ra[OP] = Base::load_a(k0, Base::a_k[OP] < kend - k0 ? Base::a_off[OP] : BUF_OOB);
         else
-            rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset(OP - T::A_ITERS, k0, kend));
-    }
-
-    template <int OP>
-    __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
-    {
-        if constexpr (OP < T::A_ITERS)
-            ra[OP] = Base::load_a(k0, Base::a_off[OP]);
-        else
-            rb[OP - T::A_ITERS] = buffer_load_f32x4(Base::cv.in, Base::tap_offset_inside(OP - T::A_ITERS, k0));
+            rb[OP - T::A_ITERS] = buffer_load_f32x4(cv.in, tap_offset_inside(OP - T::A_ITERS, k0), cv.in_bytes);
     }
 
     __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
@@ -902,8 +850,6 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
 
     if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4)
         k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
-    else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL)
-        k_walk_vec<T, ConvLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
         k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else
@@ -953,7 +899,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const bool add = (g.partial == nullptr) && g.accumulate;
     const float* bias = g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
-    const bool nchw = (B_MODE == LOAD_IM2COL || B_MODE == LOAD_IM2COL_ROW) && g.conv.out_nchw && g.partial == nullptr;
+    const bool nchw = B_MODE == LOAD_IM2COL_ROW && g.conv.out_nchw && g.partial == nullptr;
     const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
     // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
     // register group).  Each wave turns its block around through LDS, 32 rows at a time, so

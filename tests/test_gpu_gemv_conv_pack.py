@@ -148,7 +148,14 @@ CONV_GEOMS = [
     (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
     (3, 5, 8, 8, 7, 1, 1, 1, 0),         # 1x1, K = 5
     (2, 3, 17, 17, 33, 3, 3, 2, 1),      # stride 2, K = 27, Wout = 9 (two-step) ...
-    (2, 3, 15, 16, 33, 3, 3, 2, 1),      # ... and Wout = 8 (gathered, element loads)
+    (2, 3, 15, 16, 33, 3, 3, 2, 1),      # ... and Wout = 8 (gathered from the phase-split copy)
+    (2, 8, 16, 16, 12, 1, 1, 2, 0),      # 1x1 stride 2: one row in two and one column phase are staged
+    (2, 3, 32, 32, 16, 7, 7, 2, 3),      # 7x7 stride 2 pad 3 (a first layer), Wout = 16
+    (1, 4, 33, 29, 6, 3, 3, 4, 1),       # stride 4 over a 3x3 filter: rows and phases skipped, Wout = 8
+    (2, 2, 21, 27, 5, 2, 5, 3, 0),       # 2x5 filter, stride 3: Hf below and Wf above the stride, Wout = 8
+    (2, 5, 19, 35, 9, 4, 4, 2, 1),       # even filter, stride 2, Wout = 17 -> two-step
+    (1, 6, 18, 34, 9, 4, 4, 2, 1),       # even filter, stride 2, Wout = 17 ... and
+    (1, 6, 18, 32, 9, 4, 4, 2, 1),       # ... Wout = 16: gathered
 ]
 
 
