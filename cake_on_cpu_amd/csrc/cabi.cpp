@@ -285,7 +285,6 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.accumulate = accumulate;
     g.col_bias = col_bias;
     if (conv) g.conv = *conv;
-    const int nchw_hw = (conv && conv->out_nchw) ? conv->Hout * conv->Wout : 0;
     g.partial = nullptr;
     g.tail_tiles = plan.pub.tail_tiles;
     g.tail_split = plan.pub.tail_split;
@@ -306,7 +305,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     if (st) return st;
     if (plan.pub.split_k > 1)
         st = timer.family(1, [&] {
-            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream, nchw_hw,
+            return launch_splitk_reduce(g.partial, C, M, N, ldc, plan.pub.split_k, accumulate, stream, conv,
                                         col_bias);
         });
     else if (plan.pub.tail_tiles > 0)
@@ -825,11 +824,17 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if ((st = stage_in(weights, (size_t)Cout * K * 4, 1, true, &w))) return st;
     if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
 
-    // The on-the-fly gather needs: 4 consecutive columns inside one output row and
-    // byte offsets into the staged input below 2^31
+    // The on-the-fly gather needs byte offsets into the staged input below 2^31
+    // (a chunk of 4 columns must lie in one output row: the product is computed with rows of
+    // row_n = Wout rounded up to 4 columns, and the columns past Wout are dropped when C is written.
+    // That costs row_n / Wout - 1 of extra arithmetic, where the column matrix costs a write and a
+    // read of K x N floats, a share of the product's time that falls with Cout: measured on 7x7 to
+    // 30x30 maps the padded rows win while (row_n / Wout - 1) * Cout stays below about 60.)
     const ConvStage sg = conv_stage(batch, Cin, Hin, Win, Hf, Wf, stride, pad);
-    const bool implicit = !explicit_cols && (Wout % 4 == 0) &&
-                          sg.elems * 4 < 2147483648.0 &&
+    const int row_n = (Wout + 3) & ~3;
+    const double ncols_p = (double)batch * Hout * row_n;
+    const bool implicit = !explicit_cols && (double)(row_n - Wout) / Wout * Cout < 60.0 &&
+                          sg.elems * 4 + 4096 < 2147483648.0 && fits_int(Cout * ncols_p) &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
     if (implicit) {
@@ -848,7 +853,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.in = image;
         cv.in_bytes = (unsigned)(sg.elems * 4);
         cv.Cin = Cin; cv.plane_rows = sg.Hs; cv.pitch = sg.pitch; cv.row_step = sg.RH;
-        cv.Hout = Hout; cv.Wout = Wout; cv.row_n = Wout;
+        cv.Hout = Hout; cv.Wout = Wout; cv.row_n = row_n;
         if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
         int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
         cv.tap_table = taps;
@@ -868,7 +873,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             });
             if (st) return st;
         }
-        st = run_gemm(w.dev, nullptr, o.dev, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
+        const int Np = (int)ncols_p;
+        st = run_gemm(w.dev, nullptr, o.dev, Cout, Np, K, K, Np, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
                       LOAD_IM2COL_ROW, stream, timer, &cv);
         if (st) return st;
         if ((st = timer.stop())) return st;
@@ -961,7 +967,7 @@ static int linear_gemm(const float* A, const float* B, float* C, int M, int N, i
 {
     if (M == 0 || N == 0) return CAKE_HIP_OK;
     if (K == 0) {
-        hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream, 0, col_bias);
+        hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream, nullptr, col_bias);
         return e == hipSuccess ? CAKE_HIP_OK : fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
     }
     const int mode = vec4_loadable(A, B, K, N) ? LOAD_VEC4 : LOAD_SCALAR;

@@ -86,9 +86,9 @@ enum LoadMode {
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
                         hipStream_t stream);
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
-// nchw_hw != 0: C is a convolution output written as [N / nchw_hw][M][nchw_hw]
+// conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream, int nchw_hw = 0,
+                                int accumulate, hipStream_t stream, const ConvGeom* conv = nullptr,
                                 const float* col_bias = nullptr);
 
 // scratch: at least sgemv_rowmajor_scratch_floats(M, K, cus) floats (0 for most shapes), or nullptr

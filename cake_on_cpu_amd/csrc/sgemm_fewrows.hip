@@ -418,7 +418,7 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
                        out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || used == 1) return e;
-    return launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, 0, col_bias);
+    return launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, nullptr, col_bias);
 }
 
 // C'(i, n) = sum_k X(i, k) W[n][k] for i < M <= 16, n < N.
@@ -444,8 +444,8 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
                        split ? 0 : accumulate, bias_n, bias_i);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !split) return e;
-    return c_is_n_by_m ? launch_splitk_reduce(partial, C, N, M, ldc, used, accumulate, stream, 0, bias)
-                       : launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, 0, bias);
+    return c_is_n_by_m ? launch_splitk_reduce(partial, C, N, M, ldc, used, accumulate, stream, nullptr, bias)
+                       : launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, nullptr, bias);
 }
 
 }  // namespace cake

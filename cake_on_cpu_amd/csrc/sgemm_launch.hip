@@ -58,7 +58,7 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial,
                                                             float* __restrict__ C, int M, int N,
                                                             int ldc, int splits, int accumulate,
-                                                            int nchw_hw,
+                                                            ConvGeom conv,
                                                             const float* __restrict__ col_bias)
 {
     const size_t total = (size_t)M * N;
@@ -66,9 +66,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
          i += (size_t)gridDim.x * blockDim.x) {
         const int row = (int)(i / N), col = (int)(i - (size_t)row * N);
         float* dst = C + (size_t)row * ldc + col;
-        if (nchw_hw) {  // column (image b, pixel) of a convolution written as NCHW
-            const int b = col / nchw_hw;
-            dst = C + ((size_t)b * M + row) * nchw_hw + (col - b * nchw_hw);
+        if (conv.in) {  // a convolution's column: see conv_out_map
+            size_t off, row_stride;
+            if (conv_out_map(conv, M, ldc, col, 1, off, row_stride) < 1) continue;
+            dst = C + (size_t)row * row_stride + off;
         }
         float acc = accumulate ? *dst : 0.f;
         for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * total + i];
@@ -78,14 +79,14 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
 }
 
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
-                                int accumulate, hipStream_t stream, int nchw_hw, const float* col_bias)
+                                int accumulate, hipStream_t stream, const ConvGeom* conv, const float* col_bias)
 {
     const size_t total = (size_t)M * N;
     if (total == 0) return hipSuccess;
     size_t blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
-                       M, N, ldc, splits, accumulate, nchw_hw, col_bias);
+                       M, N, ldc, splits, accumulate, conv ? *conv : ConvGeom{}, col_bias);
     return hipGetLastError();
 }
 

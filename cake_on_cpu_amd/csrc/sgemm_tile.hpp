@@ -554,6 +554,25 @@ struct ConvRowLoader {
     }
 };
 
+// Where `count` (<= 4) consecutive columns of a convolution's product go, starting at GEMM
+// column col (they lie in one output row: rows of n are a multiple of 4 long, and columns at and
+// past Wout inside a row are computed but dropped).  Returns how many of them exist; the
+// destination of row m is C + m * row_stride + off.
+__device__ __forceinline__ int conv_out_map(const ConvGeom& cv, int M, int ldc, int col, int count,
+                                            size_t& off, size_t& row_stride)
+{
+    const int row_id = col / cv.row_n, wo = col - row_id * cv.row_n;
+    if (cv.out_nchw) {
+        const int b = row_id / cv.Hout, ho = row_id - b * cv.Hout, HW = cv.Hout * cv.Wout;
+        off = (size_t)b * M * HW + ho * cv.Wout + wo;
+        row_stride = HW;
+    } else {
+        off = (size_t)row_id * cv.Wout + wo;
+        row_stride = ldc;
+    }
+    return min(count, cv.Wout - wo);
+}
+
 // K walk for 16-byte-loadable operands.
 //
 // Per K step a wave issues 4*TM*TN*NKG MFMAs and a few dozen memory
@@ -898,9 +917,9 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const int ldo = g.partial ? g.N : g.ldc;
     const bool add = (g.partial == nullptr) && g.accumulate;
     const float* bias = g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
-    // convolution written as NCHW: column n = (image b, pixel) goes to out[b][row][pixel]
-    const bool nchw = B_MODE == LOAD_IM2COL_ROW && g.conv.out_nchw && g.partial == nullptr;
-    const int HW = nchw ? g.conv.Hout * g.conv.Wout : 1;
+    // a convolution's columns n = (image, output row, column of a row padded to 4) go to
+    // [M][batch*Hout*Wout] or NCHW: see conv_out_map
+    const bool conv_out = B_MODE == LOAD_IM2COL_ROW && g.partial == nullptr;
     // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
     // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
     // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
@@ -915,18 +934,15 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const int col = n0 + wn0 + rd_col;          // first of the lane's 4 columns
     size_t col_off = col;
     size_t row_stride = ldo;
-    if (nchw) {  // 4 consecutive n stay inside one image (Hout*Wout % 4 == 0 on this path)
-        const int b = col / HW;
-        col_off = (size_t)b * g.M * HW + (col - b * HW);
-        row_stride = HW;
-    }
+    int valid = min(4, g.N - col);              // how many of the 4 columns exist (<= 0: none)
+    if (conv_out && valid > 0) valid = conv_out_map(g.conv, g.M, g.ldc, col, valid, col_off, row_stride);
     f32x4 bias_v = {0.f, 0.f, 0.f, 0.f};
     if (bias) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            if (col + e < g.N) bias_v[e] = bias[col + e];
+            if (e < valid) bias_v[e] = bias[col + e];
     }
-    const bool whole = col + 3 < g.N;
+    const bool whole = valid == 4;
 #pragma unroll
     for (int tm = 0; tm < T::TM; ++tm) {
 #pragma unroll
@@ -940,7 +956,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
             const int lr = pass * ROWS + rd_row;
             const int row = m0 + wm0 + tm * 32 + lr;
             f32x4 v = *reinterpret_cast<const f32x4*>(wbuf + lr * PITCH + rd_col);
-            if (row < g.M && col < g.N) {
+            if (row < g.M && valid > 0) {
                 float* dst = out + (size_t)row * row_stride + col_off;
                 if (whole) {
                     f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst);
@@ -950,7 +966,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (col + e < g.N) {
+                        if (e < valid) {
                             float x = add ? dst[e] + v[e] : v[e];
                             if (bias) x += bias_v[e];
                             dst[e] = x;
@@ -979,20 +995,22 @@ __global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmArgs g)
     const float* src = g.tail_partial + (size_t)j * (T::BM * T::BN) + e;
     const size_t slice_stride = (size_t)g.tail_tiles * (T::BM * T::BN);
     float* dst = g.C + (size_t)row * g.ldc + col;
-    if (g.conv.in && g.conv.out_nchw) {  // 4 consecutive n stay inside one image row (Wout % 4 == 0)
-        const int HW = g.conv.Hout * g.conv.Wout, b = col / HW;
-        dst = g.C + ((size_t)b * g.M + row) * HW + (col - b * HW);
+    int valid = min(4, g.N - col);
+    if (g.conv.in) {
+        size_t off, row_stride;
+        valid = conv_out_map(g.conv, g.M, g.ldc, col, valid, off, row_stride);
+        dst = g.C + (size_t)row * row_stride + off;
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-        if (g.accumulate && col + q < g.N) acc[q] = dst[q];
+        if (g.accumulate && q < valid) acc[q] = dst[q];
     for (int s = 0; s < g.tail_split; ++s) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(src + s * slice_stride);
         acc += v;
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-        if (col + q < g.N) dst[q] = g.col_bias ? acc[q] + g.col_bias[col + q] : acc[q];
+        if (q < valid) dst[q] = g.col_bias ? acc[q] + g.col_bias[col + q] : acc[q];
 }
 
 template <class T, int A_MODE, int B_MODE>
