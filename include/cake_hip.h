@@ -199,15 +199,19 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * out_nchw == 0: out is [Cout][batch*Hout*Wout] (the GEMM's own layout, which
  * is what the reference produces for its single image); != 0: NCHW.
  *
- * cake_hip_conv2d gathers the column matrix inside the GEMM's B loader when the
- * geometry allows it (Wout % 4 == 0, padded input below
- * 2 GiB), so the K x N intermediate is never written (with pad > 0 the input is
- * first copied once into a zero-padded image, so that the gather has no edge
- * cases); otherwise it runs the two-step path.
+ * cake_hip_conv2d gathers the column matrix inside the GEMM's B loader, so the
+ * K x N intermediate is never written.  With padding or a stride above 1 the
+ * input is first copied once into a staged image (zero padding written out,
+ * rows split into their column phases, so that 4 neighbouring output pixels
+ * read 4 neighbouring floats); an output width that is not a multiple of 4 is
+ * computed with rows padded to one and the extra columns dropped.  It runs the
+ * two-step path instead when that padding would cost more than the column
+ * matrix (narrow maps with many output channels) or the staged input reaches
+ * 2 GiB.
  * cake_hip_conv2d_im2col always runs the two steps the reference runs: im2col
  * into a column matrix, then the GEMM.  Both give the same result.
  * workspace (device, cake_hip_conv2d_workspace bytes: the column matrix of the
- * two-step path or the padded image of the gather path) may be NULL: the
+ * two-step path or the staged image of the gather path) may be NULL: the
  * library then uses a buffer of its own. */
 size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
                                  int Hf, int Wf, int stride, int pad);
