@@ -159,6 +159,34 @@ CONV_GEOMS = [
 ]
 
 
+def test_conv2d_random_geometries():
+    """Seeded random geometries (filters 1..7 square or not, stride 1..4, padding up to the filter,
+    widths around multiples of 4) through the gather path, NCHW and matrix output, against the
+    naive fp64 convolution."""
+    rng = np.random.default_rng(77)
+    done = 0
+    while done < 60:
+        Hf, Wf = int(rng.integers(1, 8)), int(rng.integers(1, 8))
+        stride, pad = int(rng.integers(1, 5)), int(rng.integers(0, 4))
+        Hin, Win = int(rng.integers(Hf, 40)), int(rng.integers(Wf, 40))
+        Bn, Cin, Cout = int(rng.integers(1, 4)), int(rng.integers(1, 20)), int(rng.integers(1, 70))
+        if Hin + 2 * pad < Hf or Win + 2 * pad < Wf:
+            continue
+        nchw = bool(done % 2)
+        print(f"conv2d random {done}: b={Bn} Cin={Cin} {Hin}x{Win} Cout={Cout} {Hf}x{Wf} s={stride} p={pad} nchw={nchw}",
+              flush=True)
+        inp = oracle.uniform((Bn, Cin, Hin, Win), 700 + done)
+        wt = oracle.uniform((Cout, Cin, Hf, Wf), 900 + done)
+        ref64, S = oracle.conv_naive_f64(inp, wt, stride, pad)
+        _, _, Hout, Wout = ref64.shape
+        out = np.full((Bn, Cout, Hout, Wout) if nchw else (Cout, Bn * Hout * Wout), np.nan, np.float32)
+        cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=nchw)
+        got = out if nchw else out.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
+        err = float(np.max(np.abs(got.astype(np.float64) - ref64) / np.maximum(S, 1e-300)))
+        assert err <= TIGHT, (done, err)
+        done += 1
+
+
 @pytest.mark.parametrize("geom", CONV_GEOMS, ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
 @pytest.mark.parametrize("explicit", [False, True])

@@ -182,6 +182,33 @@ def test_tall_matrix_times_few_columns(shape):
     assert np.array_equal(_run(M, K, N)[2], Cm)
 
 
+def test_random_shapes_against_fp64():
+    """Seeded random shapes drawn around every dispatch boundary (a single row or column, up to 16
+    and just past 16 rows or columns, below and above the 512 columns and 64 k where the streaming
+    kernels start, ragged everything), each against the fp64 product with C prefilled."""
+    rng = np.random.default_rng(2024)
+    small = lambda: int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 31, 33]))
+    mid = lambda: int(rng.integers(1, 700))
+    wide = lambda: int(rng.choice([511, 512, 513, 600, 1023, 1030, 2049, 3001]))
+    deep = lambda: int(rng.choice([1, 3, 63, 64, 65, 100, 255, 257, 1000, 2050, 4099]))
+    for case in range(120):
+        kind = case % 4
+        if kind == 0: M, N, K = small(), wide(), deep()
+        elif kind == 1: M, N, K = wide(), small(), deep()
+        elif kind == 2: M, N, K = mid(), mid(), deep()
+        else: M, N, K = small(), small(), int(rng.integers(1, 20000))
+        print(f"sgemm random case {case}: M={M} K={K} N={N}", flush=True)
+        A, B = oracle.uniform((M, K), 100 + case), oracle.uniform((K, N), 300 + case)
+        C0 = oracle.uniform((M, N), 500 + case)
+        beta = float(case % 3 == 0)
+        Cm = C0.copy()
+        # beta only counts under the M- and N-first schedules, as in the reference (K-first overwrites C)
+        cake.cake_sgemm(A, B, Cm, M, N, K, 4, None, None, False, False, 1.0, beta, cake.MKN if beta else cake.NA)
+        C64, S = oracle.gemm_f64(A, B)
+        err = float(np.max(np.abs(Cm.astype(np.float64) - beta * C0 - C64) / (S + beta * np.abs(C0) + 1e-300)))
+        assert err <= TIGHT, (case, M, N, K, err)
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
