@@ -40,7 +40,10 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # this script, each scaled by what the same counter reads for a plain 256 MiB
 # copy (FETCH_SIZE reads half the true size, WRITE_SIZE the true size).  The
 # summaries are kept under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": (1049023 + 256) * 1024}
+MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": (1049023 + 256) * 1024,
+                          # streaming kernel + its slice reduction, 16 x 16384 x 16384 and transposes of it
+                          "fewrows_nn": (1056762 + 8192 + 4775 + 1024) * 1024,
+                          "fewrows_nt": (1056793 + 3091 + 4775 + 1024) * 1024}
 
 
 def main() -> int:
@@ -174,7 +177,7 @@ def main() -> int:
     if not args.no_extras:
         extras = []
 
-        def gemm_extra(name, M, N, K, streaming_kernel=None):
+        def gemm_extra(name, M, N, K, streaming_kernel=None, traffic=None):
             a, b = dev_uniform((M, K), 1), dev_uniform((K, N), 2)
             c = torch.zeros((M, N), dtype=torch.float32, device=dev)
             p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
@@ -188,7 +191,7 @@ def main() -> int:
                                "kernel": streaming_kernel,
                                "roofline": {"bound": "hbm", "achieved": round(by / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
                                             "unit": "GB/s", "frac": round(by / avg / 1e9 / HBM_PEAK_GBPS, 4),
-                                            "traffic": None, "algorithmic_bytes_per_launch": by}})
+                                            "traffic": traffic, "algorithmic_bytes_per_launch": by}})
                 return
             extras.append({"workload": name, "ms": round(avg * 1e3, 4), "tflops": round(fl / avg / 1e12, 2),
                            "frac_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4),
@@ -199,9 +202,9 @@ def main() -> int:
         gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024)
         gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024)
         gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384,
-                   "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
+                   "sgemm_fewrows_nn_kernel + splitk_reduce_kernel", MEASURED_TRAFFIC_BYTES["fewrows_nn"])
         gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384,
-                   "sgemm_fewrows_nt_kernel + splitk_reduce_kernel")
+                   "sgemm_fewrows_nt_kernel + splitk_reduce_kernel", MEASURED_TRAFFIC_BYTES["fewrows_nt"])
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
@@ -268,7 +271,7 @@ def main() -> int:
                        "kernel": "sgemm_fewrows_nt_kernel + splitk_reduce_kernel",
                        "roofline": {"bound": "hbm", "achieved": round(sby / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
                                     "unit": "GB/s", "frac": round(sby / avg / 1e9 / HBM_PEAK_GBPS, 4),
-                                    "traffic": None, "algorithmic_bytes_per_launch": sby}})
+                                    "traffic": MEASURED_TRAFFIC_BYTES["fewrows_nt"], "algorithmic_bytes_per_launch": sby}})
         out["extras"] = extras
 
     # -------------------------------------------------------------- CPU baseline
