@@ -227,10 +227,11 @@ def main() -> int:
         ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
         ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
         cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
-        for fn, label in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM"),
-                          (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps)")):
+        # output written as NCHW: inside the GEMM's epilogue on the gather path, a layout pass on the other
+        for fn, label in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM, NCHW output"),
+                          (lib.cake_hip_conv2d_im2col, "im2col kernel, GEMM (the reference's two steps), NCHW layout pass")):
             _, avg, _ = time_steps(lambda: _lib.check(
-                fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 0,
+                fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 1,
                    ws.data_ptr(), stream, None), "conv2d"), 20, 3, 40.0)
             extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
                            "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
