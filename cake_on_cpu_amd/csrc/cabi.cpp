@@ -245,7 +245,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     const bool streaming_ok = vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, true, nullptr);
     if (streaming_ok && fewrows_applies(M, N, K, lda, ldb)) {
         // a few rows of A against a wide B: bound by reading B, served by the streaming kernel
-        const int slices = fewrows_slices(N, K, g_ctx.model.cus);
+        const int slices = fewrows_slices(M, N, K, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
             int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
@@ -259,7 +259,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     }
     if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
         // a tall A against a few columns of B: the same with A streamed along its rows
-        const int slices = fewrows_nt_slices(M, K, g_ctx.model.cus);
+        const int slices = fewrows_nt_slices(N, M, K, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
             int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
@@ -1001,7 +1001,7 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
     if ((st = timer.start())) return st;
     if (small_batch) {
         // a small batch: y = x w^T with w streamed once as it lies, no transposed copy
-        const int slices = fewrows_nt_slices(N, K, g_ctx.model.cus);
+        const int slices = fewrows_nt_slices(M, N, K, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
             if ((st = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float)))) return st;

@@ -16,7 +16,7 @@
 //                             the linear layer y = x w^T for a small batch without
 //                             transposing w, and C[M][N<=16] = A.B with W = A, X = B^T
 //
-// A workgroup owns 256 columns of B (64 rows of W) and a slice of k; its four
+// A workgroup owns 64 or 128 columns of B (64 rows of W) and a slice of k; its four
 // waves take a quarter of the slice each and add their sums in LDS in wave
 // order; K slices are summed by splitk_reduce_kernel in slice order, so results
 // are run-to-run identical.
@@ -46,9 +46,7 @@ __device__ __forceinline__ float load_f32(const float* base, int byte_offset, un
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
 }
 
-static constexpr int FR_COLS = 256;     // nn: columns of B per workgroup
 static constexpr int FR_ROWS = 64;      // nt: rows of W per workgroup
-static constexpr int FR_STAGES = 2;     // nn: half groups of 16 k (8 loads of B each) in flight per wave
 static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave and loop step
 
 // The part of [kbeg, kend) that wave `wave` of 4 walks: quarters rounded up to 16 k
@@ -59,18 +57,25 @@ __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0
     kw1 = min(kend, kw0 + part);
 }
 
-__global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
+// MG groups of 16 rows of A (M <= 16 MG) against NJ pieces of 64 columns per workgroup: every
+// B value loaded feeds MG MFMAs, so the arithmetic per byte grows with MG.  One and two groups
+// (up to 32 rows) stay bound by memory; four groups (up to 64 rows) are bound by the matrix pipe
+// and were measured no faster than the 64 x 64 macro-tile, so they are not instantiated.
+template <int MG, int NJ>
+__global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
                                                                const float* __restrict__ B,
                                                                float* __restrict__ out, int M, int N, int K,
                                                                int lda, int ldb, int k_per_slice,
                                                                int out_ld, size_t out_slice_stride,
                                                                int accumulate, const float* __restrict__ col_bias)
 {
-    __shared__ __align__(16) float red[16 * FR_COLS];
+    constexpr int COLS = 64 * NJ;                     // columns of B per workgroup
+    constexpr int STAGES = 8 / NJ;                    // units in flight per wave: 16 loads of B
+    __shared__ __align__(16) float red[16 * MG * COLS];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    const int n0 = blockIdx.x * FR_COLS;
+    const int n0 = blockIdx.x * COLS;
     const int kbeg = blockIdx.y * k_per_slice;
     const int kend = min(K, kbeg + k_per_slice);
     int kw0, kw1;
@@ -78,67 +83,75 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
 
     const unsigned a_elems = clamp_elems((long long)(M - 1) * lda + K);
     const unsigned b_elems = clamp_elems((long long)(K - 1) * ldb + N - n0);
-    // A: row li, k = 4 lq .. 4 lq + 3 of the group.  B: rows 4 lq + e of the group (e = 0..3 by
-    // moving the base), and of each row four 16-byte pieces: piece j is columns 64 j + 4 li .. + 3,
+    // A: rows 16 g + li, k = 4 lq .. 4 lq + 3 of the group.  B: rows 4 lq + e of the group (e = 0..3
+    // by moving the base), and of each row NJ 16-byte pieces: piece j is columns 64 j + 4 li .. + 3,
     // so that the 16 lanes of a row read 256 contiguous bytes per load instruction.
-    const int a_off = li < M ? (li * lda + 4 * lq) * 4 : BUF_OOB;
-    int b_off[4];
+    int a_off[MG];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int g = 0; g < MG; ++g) a_off[g] = 16 * g + li < M ? ((16 * g + li) * lda + 4 * lq) * 4 : BUF_OOB;
+    int b_off[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
         b_off[j] = n0 + 64 * j + 4 * li < N ? (4 * lq * ldb + 64 * j + 4 * li) * 4 : BUF_OOB;
 
-    f32x4 acc[16];
+    f32x4 acc[MG][4 * NJ];
 #pragma unroll
-    for (int c = 0; c < 16; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < MG; ++g)
+#pragma unroll
+        for (int c = 0; c < 4 * NJ; ++c) acc[g][c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // Groups of 16 k that lie wholly below kw1 <= K, in units of half a group (8 loads of B, 32
-    // MFMAs).  FR_STAGES units are in flight: each is multiplied and its registers refilled with
-    // the unit FR_STAGES further on.  A unit past the end gets a record count of 0, which turns
+    // Groups of 16 k that lie wholly below kw1 <= K, in units of half a group (2 NJ loads of B,
+    // 8 MG NJ MFMAs).  STAGES units are in flight: each is multiplied and its registers refilled
+    // with the unit STAGES further on.  A unit past the end gets a record count of 0, which turns
     // its loads into zeros without a memory access, so the loop body needs no branch and the
     // wait counts in front of the MFMAs are exact.  Every row asked for below the end exists, so
     // those record counts are exact too (records_left must not be asked about a start past the
     // end of an operand: its difference would wrap to "everything in range").
     const int units = 2 * ((kw1 - kw0) >> 4);
-    auto load_a = [&](int q) {
+    auto load_a = [&](int q, f32x4 (&a)[MG]) {
         const int kq = kw0 + 16 * (q >> 1);
-        return buffer_load_f32x4(A + kq, a_off, q < units ? records_left(a_elems, (unsigned)kq) : 0u);
+        const unsigned rec = q < units ? records_left(a_elems, (unsigned)kq) : 0u;
+#pragma unroll
+        for (int g = 0; g < MG; ++g) a[g] = buffer_load_f32x4(A + kq, a_off[g], rec);
     };
-    auto load_unit = [&](int q, int h, f32x4 (&b)[2][4]) {
+    auto load_unit = [&](int q, int h, f32x4 (&b)[2][NJ]) {
         const int kq = kw0 + 16 * (q >> 1) + 2 * h;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const unsigned skip = (unsigned)(kq + e) * (unsigned)ldb;
             const unsigned rec = q < units ? records_left(b_elems, skip) : 0u;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[e][j] = stream_load_f32x4(B + n0 + (size_t)skip, b_off[j], rec);
+            for (int j = 0; j < NJ; ++j) b[e][j] = stream_load_f32x4(B + n0 + (size_t)skip, b_off[j], rec);
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
     };
-    auto mma_unit = [&](const f32x4& a, int h, const f32x4 (&b)[2][4]) {
+    auto mma_unit = [&](const f32x4 (&a)[MG], int h, const f32x4 (&b)[2][NJ]) {
 #pragma unroll
         for (int e = 0; e < 2; ++e)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    acc[4 * j + c] =
-                        __builtin_amdgcn_mfma_f32_16x16x4f32(a[2 * h + e], b[e][j][c], acc[4 * j + c], 0, 0, 0);
+#pragma unroll
+                    for (int g = 0; g < MG; ++g)
+                        acc[g][4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g][2 * h + e], b[e][j][c],
+                                                                                 acc[g][4 * j + c], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     if (units > 0) {
-        f32x4 a[FR_STAGES / 2];
-        f32x4 b[FR_STAGES][2][4];
+        f32x4 a[STAGES / 2][MG];
+        f32x4 b[STAGES][2][NJ];
 #pragma unroll
-        for (int i = 0; i < FR_STAGES; ++i) {
-            if (i % 2 == 0) a[i / 2] = load_a(i);
+        for (int i = 0; i < STAGES; ++i) {
+            if (i % 2 == 0) load_a(i, a[i / 2]);
             load_unit(i, i % 2, b[i]);
         }
-        for (int q = 0; q < units; q += FR_STAGES) {
+        for (int q = 0; q < units; q += STAGES) {
 #pragma unroll
-            for (int i = 0; i < FR_STAGES; ++i) {
+            for (int i = 0; i < STAGES; ++i) {
                 mma_unit(a[i / 2], i % 2, b[i]);
-                if (i % 2 == 1) a[i / 2] = load_a(q + i + FR_STAGES);  // both halves of the group are done
-                load_unit(q + i + FR_STAGES, i % 2, b[i]);
+                if (i % 2 == 1) load_a(q + i + STAGES, a[i / 2]);  // both halves of the group are done
+                load_unit(q + i + STAGES, i % 2, b[i]);
             }
         }
     }
@@ -149,44 +162,52 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
 #pragma nounroll
         for (int e = 0; e < 4; ++e) {
             const bool below = k + 4 * lq + e < kw1;
-            const float a = buffer_load_f32(A + k, below && li < M ? (li * lda + 4 * lq + e) * 4 : BUF_OOB);
+            float a[MG];
+#pragma unroll
+            for (int g = 0; g < MG; ++g)
+                a[g] = buffer_load_f32(A + k, below && 16 * g + li < M ? ((16 * g + li) * lda + 4 * lq + e) * 4 : BUF_OOB);
             const float* row = B + n0 + (size_t)(k + e) * ldb;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NJ; ++j) {
                 const bool col = n0 + 64 * j + 4 * li < N;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     // element loads: a 16-byte load of the last row could hang over the end of B
                     const bool ok = below && col && n0 + 64 * j + 4 * li + c < N;
                     const float b = buffer_load_f32(row, ok ? b_off[j] + 4 * c : BUF_OOB);
-                    acc[4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[4 * j + c], 0, 0, 0);
+#pragma unroll
+                    for (int g = 0; g < MG; ++g)
+                        acc[g][4 * j + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g], b, acc[g][4 * j + c], 0, 0, 0);
                 }
             }
         }
     }
 
-    // register r of MFMA 4j+c holds C[4*lq + r][n0 + 64 j + 4 li + c].  Wave sums meet in LDS in
-    // wave order: red[row][column].
+    // register r of MFMA (g, 4j+c) holds C[16 g + 4 lq + r][n0 + 64 j + 4 li + c].  Wave sums meet in
+    // LDS in wave order: red[row][column].
     for (int w = 0; w < 4; ++w) {
         if (w) __syncthreads();
         if (wave == w) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+            for (int g = 0; g < MG; ++g)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    f32x4* p = reinterpret_cast<f32x4*>(red + (4 * lq + r) * FR_COLS + 64 * j + 4 * li);
-                    const f32x4 v = {acc[4 * j][r], acc[4 * j + 1][r], acc[4 * j + 2][r], acc[4 * j + 3][r]};
-                    *p = w == 0 ? v : *p + v;
-                }
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        f32x4* p = reinterpret_cast<f32x4*>(red + (16 * g + 4 * lq + r) * COLS + 64 * j + 4 * li);
+                        const f32x4 v = {acc[g][4 * j][r], acc[g][4 * j + 1][r], acc[g][4 * j + 2][r], acc[g][4 * j + 3][r]};
+                        *p = w == 0 ? v : *p + v;
+                    }
         }
     }
     __syncthreads();
-    const int n = n0 + tid;
+    // a thread per column, the rows dealt over the 256 / COLS threads that share it
+    const int cl = tid % COLS, n = n0 + cl;
     if (n >= N) return;
     float* dst = out + (size_t)blockIdx.y * out_slice_stride + n;
     const float bias = col_bias ? col_bias[n] : 0.f;
-    for (int m = 0; m < M; ++m) {
-        float v = red[m * FR_COLS + tid];
+    for (int m = tid / COLS; m < M; m += 256 / COLS) {
+        float v = red[m * COLS + cl];
         if (accumulate) v += dst[(size_t)m * out_ld];
         if (col_bias) v += bias;
         dst[(size_t)m * out_ld] = v;
@@ -206,8 +227,6 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nn_kernel(const float* __re
 static constexpr int NT_STEP = 32;                               // k per step of a wave
 static constexpr int NT_STAGES = 1;                             // steps in flight per wave
 static constexpr int NT_PITCH = 36;                              // floats per staged row: 16-byte reads of 16 rows spread over all banks
-static constexpr int NT_WAVE_FLOATS = (FR_ROWS + 16) * NT_PITCH; // 64 rows of W and 16 of X
-
 __device__ __forceinline__ f32x4 keep_below(f32x4 v, int valid)  // zero the elements at and past `valid`
 {
     if (valid < 4) v[3] = 0.f;
@@ -217,7 +236,8 @@ __device__ __forceinline__ f32x4 keep_below(f32x4 v, int valid)  // zero the ele
     return v;
 }
 
-template <bool X_KMAJOR>
+// XG groups of 16 rows of X (M <= 16 XG): every W value staged feeds XG MFMAs.
+template <bool X_KMAJOR, int XG>
 __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __restrict__ X,
                                                                const float* __restrict__ W,
                                                                float* __restrict__ out, int M, int N, int K,
@@ -227,8 +247,10 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
                                                                const float* __restrict__ bias_n,
                                                                const float* __restrict__ bias_i)
 {
-    __shared__ __align__(16) float smem[4 * NT_WAVE_FLOATS];
-    static_assert(4 * NT_WAVE_FLOATS >= 16 * FR_ROWS, "the reduction buffer fits the staging memory");
+    constexpr int XROWS = 16 * XG;
+    constexpr int WAVE_FLOATS = (FR_ROWS + XROWS) * NT_PITCH;   // 64 rows of W and 16 XG of X
+    __shared__ __align__(16) float smem[4 * WAVE_FLOATS];
+    static_assert(4 * WAVE_FLOATS >= XROWS * FR_ROWS, "the reduction buffer fits the staging memory");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;   // MFMA order: row li, k = 4 lq .. + 3 of a group of 16
@@ -236,8 +258,8 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     const int n0 = blockIdx.x * FR_ROWS;
     const int kbeg = blockIdx.y * k_per_slice;
     const int kend = min(K, kbeg + k_per_slice);
-    float* Ws = smem + wave * NT_WAVE_FLOATS;   // [64][NT_PITCH]
-    float* Xs = Ws + FR_ROWS * NT_PITCH;        // [16][NT_PITCH]
+    float* Ws = smem + wave * WAVE_FLOATS;      // [64][NT_PITCH]
+    float* Xs = Ws + FR_ROWS * NT_PITCH;        // [16 XG][NT_PITCH]
 
     const float* Wb = W + (size_t)n0 * ldw;
     const int rows_left = N - n0;
@@ -246,9 +268,11 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     const int w_off = (lr * ldw + 4 * lc) * 4;
     const int x_off = X_KMAJOR ? (lq * ldx + li) * 4 : (lr * ldx + 4 * lc) * 4;
 
-    f32x4 acc[4];
+    f32x4 acc[XG][4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int xg = 0; xg < XG; ++xg)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[xg][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Rows at and past N (or M) are not masked: what they bring only reaches results that are
     // never written.  Their addresses are kept inside the operands by exact record counts, and
@@ -257,7 +281,7 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     // TAIL: the last, partial step of the slice; k at and past kend reads as zero on both sides.
     // live = false: a step past the end of the wave's share, loaded as zeros without a memory
     // access (record count 0), so that the loop below needs no branch
-    auto load_step = [&](int k, bool live, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2], float (&gk)[8]) {
+    auto load_step = [&](int k, bool live, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2 * XG], float (&gk)[8 * XG]) {
         constexpr bool TAIL = decltype(tail)::value;
         const int below = kend - (k + 4 * lc);   // of this lane's 4 k, how many lie below kend
 #pragma unroll
@@ -269,7 +293,7 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
         }
         if constexpr (!X_KMAJOR) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < 2 * XG; ++t) {
                 const unsigned used = (unsigned)(8 * t) * (unsigned)ldx + (unsigned)k;
                 const unsigned rec = live && 8 * t < M ? records_left(x_elems, used) : 0u;
                 gx[t] = buffer_load_f32x4(X + (size_t)(8 * t) * ldx + k, TAIL && below <= 0 ? BUF_OOB : x_off, rec);
@@ -277,35 +301,46 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {   // k = 4 t + lq of the step, i = li
+            for (int t = 0; t < 8; ++t) {   // k = 4 t + lq of the step, i = 16 xg + li
                 const unsigned used = (unsigned)(k + 4 * t) * (unsigned)ldx;
                 const unsigned rec = live && (!TAIL || k + 4 * t < kend) ? records_left(x_elems, used) : 0u;
-                gk[t] = load_f32(X + (size_t)(k + 4 * t) * ldx, TAIL && k + 4 * t + lq >= kend ? BUF_OOB : x_off, rec);
+                const int off = TAIL && k + 4 * t + lq >= kend ? BUF_OOB : x_off;
+#pragma unroll
+                for (int xg = 0; xg < XG; ++xg)  // BUF_OOB plus 64 bytes stays out of range
+                    gk[XG * t + xg] = load_f32(X + (size_t)(k + 4 * t) * ldx, off + 64 * xg, rec);
             }
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
     };
-    auto store_step = [&](const f32x4 (&gw)[8], const f32x4 (&gx)[2], const float (&gk)[8]) {
+    auto store_step = [&](const f32x4 (&gw)[8], const f32x4 (&gx)[2 * XG], const float (&gk)[8 * XG]) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(Ws + (8 * t + lr) * NT_PITCH + 4 * lc) = gw[t];
         if constexpr (!X_KMAJOR) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) *reinterpret_cast<f32x4*>(Xs + (8 * t + lr) * NT_PITCH + 4 * lc) = gx[t];
+            for (int t = 0; t < 2 * XG; ++t) *reinterpret_cast<f32x4*>(Xs + (8 * t + lr) * NT_PITCH + 4 * lc) = gx[t];
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) Xs[li * NT_PITCH + 4 * t + lq] = gk[t];
+            for (int t = 0; t < 8; ++t)
+#pragma unroll
+                for (int xg = 0; xg < XG; ++xg) Xs[(16 * xg + li) * NT_PITCH + 4 * t + lq] = gk[XG * t + xg];
         }
         __builtin_amdgcn_sched_barrier(0);
     };
     auto compute_step = [&]() {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const f32x4 x = *reinterpret_cast<const f32x4*>(Xs + li * NT_PITCH + 16 * u + 4 * lq);
+            f32x4 x[XG];
+#pragma unroll
+            for (int xg = 0; xg < XG; ++xg)
+                x[xg] = *reinterpret_cast<const f32x4*>(Xs + (16 * xg + li) * NT_PITCH + 16 * u + 4 * lq);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const f32x4 w = *reinterpret_cast<const f32x4*>(Ws + (16 * g + li) * NT_PITCH + 16 * u + 4 * lq);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], w[e], acc[g], 0, 0, 0);
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int xg = 0; xg < XG; ++xg)
+                        acc[xg][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[xg][e], w[e], acc[xg][g], 0, 0, 0);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -313,8 +348,8 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
 
     {
         // The wave's steps are wave, wave + 4, ... below `full`; NT_STAGES of them are in flight.
-        f32x4 gw[NT_STAGES][8], gx[NT_STAGES][2];
-        float gk[NT_STAGES][8];
+        f32x4 gw[NT_STAGES][8], gx[NT_STAGES][2 * XG];
+        float gk[NT_STAGES][8 * XG];
         const int full = (kend - kbeg) / NT_STEP;
         const int mine = full > wave ? (full - wave + 3) >> 2 : 0;
         auto step_k = [&](int j) { return kbeg + NT_STEP * (wave + 4 * j); };
@@ -337,18 +372,21 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
         }
     }
 
-    // register r of acc[g] holds C'[4 lq + r][n0 + 16 g + li]; wave sums meet in LDS in wave order
+    // register r of acc[xg][g] holds C'[16 xg + 4 lq + r][n0 + 16 g + li]; wave sums meet in LDS in
+    // wave order
     float* red = smem;
     for (int w = 0; w < 4; ++w) {
         __syncthreads();  // the first: every wave is done with its staging area
         if (wave == w) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
+            for (int xg = 0; xg < XG; ++xg)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float* p = red + (4 * lq + r) * FR_ROWS + 16 * g + li;
-                    *p = w == 0 ? acc[g][r] : *p + acc[g][r];
-                }
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float* p = red + (16 * xg + 4 * lq + r) * FR_ROWS + 16 * g + li;
+                        *p = w == 0 ? acc[xg][g][r] : *p + acc[xg][g][r];
+                    }
         }
     }
     __syncthreads();
@@ -357,8 +395,8 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     float* dst = out + (size_t)blockIdx.y * out_slice_stride + (long long)n * ld_n;
     const float bn = bias_n ? bias_n[n] : 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int i = 4 * (tid >> 6) + r;
+    for (int r = 0; r < 4 * XG; ++r) {
+        const int i = 4 * XG * (tid >> 6) + r;
         if (i >= M) break;
         float v = red[i * FR_ROWS + (tid & 63)];
         if (accumulate) v += dst[i * ld_i];
@@ -368,10 +406,12 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     }
 }
 
-// K slices so that about `per_cu` workgroups of 4 waves land on every CU
+// K slices so that at most `per_cu` workgroups of 4 waves land on every CU: one round of
+// workgroups that all run from start to end (a few more than fit would leave a second, nearly
+// empty round: 16 x 12288 x 12288 took 112 us with 576 workgroups, 99 us with 480)
 static int slices_for(int blocks, int K, int cus, int per_cu)
 {
-    int want = (per_cu * cus + blocks - 1) / blocks;
+    int want = per_cu * cus / blocks;
     const int max_slices = (K + FR_K_UNIT - 1) / FR_K_UNIT;
     if (want > max_slices) want = max_slices;
     return want < 1 ? 1 : want;
@@ -385,52 +425,64 @@ static int slice_length(int K, int slices, int* used)
     return k_per;
 }
 
+// Columns of B per workgroup of the nn kernel: 128, or 64 for small products, which then spread
+// over more workgroups with fewer K slices (measured: 16 x 4096 x 4096 17 us against 21 us;
+// 256 columns were slower throughout, 16 x 8192 x 8192: 63 us against 49 us).
+static int nn_cols(int N, int K) { return (double)N * K <= 24.0e6 ? 64 : 128; }
+
 // workgroups per CU: what the registers of the nn kernel and the LDS of the nt kernel allow
-int fewrows_slices(int N, int K, int cus) { return slices_for((N + FR_COLS - 1) / FR_COLS, K, cus, 2); }
-int fewrows_nt_slices(int N, int K, int cus) { return slices_for((N + FR_ROWS - 1) / FR_ROWS, K, cus, 3); }
+int fewrows_slices(int M, int N, int K, int cus)
+{
+    (void)M;
+    return slices_for((N + nn_cols(N, K) - 1) / nn_cols(N, K), K, cus, 2);
+}
+int fewrows_nt_slices(int M, int N, int K, int cus) { return slices_for((N + FR_ROWS - 1) / FR_ROWS, K, cus, M <= 16 ? 3 : 2); }
 
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
-    // byte offsets inside a group (15 rows of B plus 256 columns, 15 rows of A) must stay below 2^31
-    return M >= 1 && M <= 16 && N >= 512 && K >= 64 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
-           (double)lda * 16 * 4 < 2147483648.0;
+    // byte offsets inside a group (15 rows of B plus 256 columns, 31 rows of A) must stay below 2^31
+    return M >= 1 && M <= 32 && N >= 512 && K >= 64 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
+           (double)lda * 32 * 4 < 2147483648.0;
 }
 
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
 {
-    // 64 rows of W, and 16 rows (or 16 k) of X, within 2^31 bytes of the block's origin
-    return M >= 1 && M <= 16 && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
-           (double)ldx * 16 * 4 + (x_kmajor ? 64 : 0) < 2147483648.0;
+    // 64 rows of W, and 32 rows (or 32 k) of X, within 2^31 bytes of the block's origin
+    return M >= 1 && M <= 32 && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
+           (double)ldx * 32 * 4 + (x_kmajor ? 128 : 0) < 2147483648.0;
 }
 
-// partial: [slices][M][N] floats when fewrows_slices(N, K, cus) > 1, else unused
+// partial: [slices][M][N] floats when fewrows_slices(M, N, K, cus) > 1, else unused
 hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float* partial, int M, int N,
                                 int K, int lda, int ldb, int ldc, int accumulate, const float* col_bias,
                                 int cus, hipStream_t stream)
 {
     int used;
-    const int k_per = slice_length(K, fewrows_slices(N, K, cus), &used);
-    const dim3 grid((N + FR_COLS - 1) / FR_COLS, used), block(256);
+    const int k_per = slice_length(K, fewrows_slices(M, N, K, cus), &used);
+    const int cols = nn_cols(N, K);
+    const dim3 grid((N + cols - 1) / cols, used), block(256);
     float* out = used > 1 ? partial : C;
     const int out_ld = used > 1 ? N : ldc;
     const size_t stride = used > 1 ? (size_t)M * N : 0;
-    hipLaunchKernelGGL(sgemm_fewrows_nn_kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
+    auto kernel = M <= 16 ? (cols == 128 ? sgemm_fewrows_nn_kernel<1, 2> : sgemm_fewrows_nn_kernel<1, 1>)
+                          : (cols == 128 ? sgemm_fewrows_nn_kernel<2, 2> : sgemm_fewrows_nn_kernel<2, 1>);
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
                        out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || used == 1) return e;
     return launch_splitk_reduce(partial, C, M, N, ldc, used, accumulate, stream, nullptr, col_bias);
 }
 
-// C'(i, n) = sum_k X(i, k) W[n][k] for i < M <= 16, n < N.
+// C'(i, n) = sum_k X(i, k) W[n][k] for i < M <= 32, n < N.
 // c_is_n_by_m = false: C is M x N (C[i * ldc + n], bias per n);  true: C is N x M (C[n * ldc + i],
 // bias per i): in both cases `bias` runs along the columns of C.
-// partial: [slices] copies of C without padding when fewrows_nt_slices(N, K, cus) > 1
+// partial: [slices] copies of C without padding when fewrows_nt_slices(M, N, K, cus) > 1
 hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, float* partial, int M, int N,
                                    int K, int ldx, int ldw, int ldc, bool x_kmajor, bool c_is_n_by_m,
                                    int accumulate, const float* bias, int cus, hipStream_t stream)
 {
     int used;
-    const int k_per = slice_length(K, fewrows_nt_slices(N, K, cus), &used);
+    const int k_per = slice_length(K, fewrows_nt_slices(M, N, K, cus), &used);
     const dim3 grid((N + FR_ROWS - 1) / FR_ROWS, used), block(256);
     const bool split = used > 1;
     float* out = split ? partial : C;
@@ -439,7 +491,8 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
     const size_t stride = split ? (size_t)M * N : 0;
     const float* bias_n = split || c_is_n_by_m ? nullptr : bias;
     const float* bias_i = split || !c_is_n_by_m ? nullptr : bias;
-    auto kernel = x_kmajor ? sgemm_fewrows_nt_kernel<true> : sgemm_fewrows_nt_kernel<false>;
+    auto kernel = M <= 16 ? (x_kmajor ? sgemm_fewrows_nt_kernel<true, 1> : sgemm_fewrows_nt_kernel<false, 1>)
+                          : (x_kmajor ? sgemm_fewrows_nt_kernel<true, 2> : sgemm_fewrows_nt_kernel<false, 2>);
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, X, W, out, M, N, K, ldx, ldw, k_per, ld_i, ld_n, stride,
                        split ? 0 : accumulate, bias_n, bias_i);
     hipError_t e = hipGetLastError();

@@ -216,7 +216,7 @@ static constexpr int COL_BLOCK_M = 256;  // columns of y per workgroup
 static int colmajor_slices(int M, int K, int cus)
 {
     const int mblocks = (M + COL_BLOCK_M - 1) / COL_BLOCK_M;
-    int want = (2 * cus + mblocks / 2) / mblocks;  // ~2 workgroups (8 waves) per CU: more concurrent
+    int want = 2 * cus / mblocks;                  // at most 2 workgroups (8 waves) per CU in one round: more concurrent
                                                     // strided streams than that lose HBM page locality
     int max_slices = (K + 63) / 64;                // at least 64 k per slice
     if (want > max_slices) want = max_slices;

@@ -150,11 +150,13 @@ def test_very_long_k_takes_the_element_loader():
 
 @pytest.mark.parametrize("shape", [(2, 64, 512), (3, 300, 1000), (5, 1000, 4096), (8, 4096, 4097), (13, 777, 2050),
                                    (16, 2111, 16384), (16, 16384, 1024), (1, 100, 600), (9, 65, 515),
-                                   (17, 300, 1000), (32, 1000, 2048)],
+                                   (17, 300, 1000), (32, 1000, 2048), (33, 777, 2050), (48, 2111, 1030),
+                                   (64, 4096, 1024), (50, 65, 513), (65, 300, 1000)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_few_rows_times_wide_matrix(shape):
-    """M <= 16 against a wide B: the streaming kernel (B read once, 16-row MFMAs; 17 and 32 rows take the tile kernel),
-    with K slices summed in order, ragged N and K, accumulation, and run-to-run identical sums."""
+    """Up to 32 rows of A against a wide B: the streaming kernels (B read once, one or two groups
+    of 16-row MFMAs; more rows take the tile kernel), with K slices summed in order, ragged N and K,
+    accumulation, and run-to-run identical sums."""
     M, K, N = shape
     print(f"sgemm few rows M={M} K={K} N={N}", flush=True)
     A, B, Cm = _run(M, K, N)
@@ -167,11 +169,12 @@ def test_few_rows_times_wide_matrix(shape):
 
 @pytest.mark.parametrize("shape", [(512, 64, 2), (1000, 300, 3), (4096, 1000, 5), (4097, 4096, 8), (2050, 777, 13),
                                    (16384, 2111, 16), (1024, 16384, 16), (600, 100, 1), (515, 65, 9),
-                                   (1000, 300, 17), (5000, 4099, 4)],
+                                   (1000, 300, 17), (5000, 4099, 4), (4096, 1000, 24), (2050, 777, 32),
+                                   (513, 65, 31), (1000, 300, 33)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_tall_matrix_times_few_columns(shape):
-    """N <= 16 columns of B against a tall A: A streamed once along its rows (17 columns take the tile
-    kernel), ragged M and K, K slices summed in order, accumulation, run-to-run identical sums."""
+    """Up to 32 columns of B against a tall A: A streamed once along its rows (33 columns take the
+    tile kernel), ragged M and K, K slices summed in order, accumulation, run-to-run identical sums."""
     M, K, N = shape
     print(f"sgemm few columns M={M} K={K} N={N}", flush=True)
     A, B, Cm = _run(M, K, N)
