@@ -255,7 +255,7 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
  * table keyed by (M, N, K).  From then on cake_hip_plan / cake_hip_sgemm and the
  * other products use that choice whenever the caller gives no tile override.
  * The planner's own choice is always measured first, so the result is never
- * slower than the default by more than timing noise.  A product with at most 16
+ * slower than the default by more than timing noise.  A product with at most 32
  * rows of A or columns of B runs on a streaming kernel instead of a macro-tile:
  * that kernel is then the default that is measured, and the table only gets an
  * entry (which from then on replaces the streaming kernel) when a tile beats it.
