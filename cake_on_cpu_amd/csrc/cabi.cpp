@@ -10,6 +10,8 @@
 #include <chrono>
 #include <mutex>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "blockdims.hpp"
 #include "cake_hip.h"
@@ -79,6 +81,10 @@ struct Context {
     DeviceBuffer splitk, gemv, conv, conv_taps, tables, unpacked, linear;
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
+    // host <-> device transfers of large host operands: two pinned buffers, a stream, an event each
+    void* pinned[2] = {nullptr, nullptr};
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t copy_done[2] = {nullptr, nullptr};
 };
 
 Context g_ctx;
@@ -107,6 +113,82 @@ struct Operand {
     size_t bytes = 0;
 };
 
+// Transfers between a caller's (pageable) host memory and the device.  hipMemcpy on pageable
+// memory moves 17 (to the host) to 29 GB/s (to the device) on this platform, pinned memory 53 GB/s
+// either way.  Large operands therefore travel in chunks through two pinned buffers: worker
+// threads copy between the caller's memory and one buffer while the DMA engine moves the other.
+constexpr size_t PIN_CHUNK = 32u << 20;
+constexpr size_t PIN_THRESHOLD = 8u << 20;   // below this a plain hipMemcpy is as fast
+constexpr int PIN_THREADS = 8;
+
+static int pinned_ready()
+{
+    for (int i = 0; i < 2; ++i) {
+        if (!g_ctx.pinned[i]) HIP_TRY(hipHostMalloc(&g_ctx.pinned[i], PIN_CHUNK, hipHostMallocDefault));
+        if (!g_ctx.copy_done[i]) HIP_TRY(hipEventCreateWithFlags(&g_ctx.copy_done[i], hipEventDisableTiming));
+    }
+    if (!g_ctx.copy_stream) HIP_TRY(hipStreamCreateWithFlags(&g_ctx.copy_stream, hipStreamNonBlocking));
+    return CAKE_HIP_OK;
+}
+
+static void parallel_memcpy(void* dst, const void* src, size_t bytes)
+{
+    const size_t piece = ((bytes + PIN_THREADS - 1) / PIN_THREADS + 4095) & ~(size_t)4095;
+    std::vector<std::thread> workers;
+    for (size_t off = piece; off < bytes; off += piece)
+        workers.emplace_back([=] { memcpy(static_cast<char*>(dst) + off, static_cast<const char*>(src) + off,
+                                          bytes - off < piece ? bytes - off : piece); });
+    memcpy(dst, src, bytes < piece ? bytes : piece);
+    for (std::thread& t : workers) t.join();
+}
+
+static int host_to_device(void* dev, const void* host, size_t bytes)
+{
+    if (bytes < PIN_THRESHOLD) {
+        HIP_TRY(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice));
+        return CAKE_HIP_OK;
+    }
+    int st = pinned_ready();
+    if (st) return st;
+    int i = 0;
+    for (size_t off = 0; off < bytes; off += PIN_CHUNK, ++i) {
+        const size_t n = bytes - off < PIN_CHUNK ? bytes - off : PIN_CHUNK;
+        const int b = i & 1;
+        if (i >= 2) HIP_TRY(hipEventSynchronize(g_ctx.copy_done[b]));   // the buffer's last transfer is over
+        parallel_memcpy(g_ctx.pinned[b], static_cast<const char*>(host) + off, n);
+        HIP_TRY(hipMemcpyAsync(static_cast<char*>(dev) + off, g_ctx.pinned[b], n, hipMemcpyHostToDevice, g_ctx.copy_stream));
+        HIP_TRY(hipEventRecord(g_ctx.copy_done[b], g_ctx.copy_stream));
+    }
+    HIP_TRY(hipStreamSynchronize(g_ctx.copy_stream));
+    return CAKE_HIP_OK;
+}
+
+static int device_to_host(void* host, const void* dev, size_t bytes)
+{
+    if (bytes < PIN_THRESHOLD) {
+        HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost));
+        return CAKE_HIP_OK;
+    }
+    int st = pinned_ready();
+    if (st) return st;
+    const size_t chunks = (bytes + PIN_CHUNK - 1) / PIN_CHUNK;
+    auto chunk_bytes = [&](size_t c) { return bytes - c * PIN_CHUNK < PIN_CHUNK ? bytes - c * PIN_CHUNK : PIN_CHUNK; };
+    auto issue = [&](size_t c) -> hipError_t {
+        const int b = (int)(c & 1);
+        hipError_t e = hipMemcpyAsync(g_ctx.pinned[b], static_cast<const char*>(dev) + c * PIN_CHUNK, chunk_bytes(c),
+                                      hipMemcpyDeviceToHost, g_ctx.copy_stream);
+        return e != hipSuccess ? e : hipEventRecord(g_ctx.copy_done[b], g_ctx.copy_stream);
+    };
+    HIP_TRY(issue(0));
+    for (size_t c = 0; c < chunks; ++c) {
+        // the other buffer was emptied in the previous round: fill it while this one is copied out
+        if (c + 1 < chunks) HIP_TRY(issue(c + 1));
+        HIP_TRY(hipEventSynchronize(g_ctx.copy_done[c & 1]));
+        parallel_memcpy(static_cast<char*>(host) + c * PIN_CHUNK, g_ctx.pinned[c & 1], chunk_bytes(c));
+    }
+    return CAKE_HIP_OK;
+}
+
 int stage_in(const float* p, size_t bytes, int slot, bool copy, Operand* op)
 {
     op->bytes = bytes;
@@ -123,7 +205,7 @@ int stage_in(const float* p, size_t bytes, int slot, bool copy, Operand* op)
         // an earlier call may have left kernels in flight that still read this slot (device
         // outputs make a call asynchronous); hipMemcpy alone does not wait for non-blocking streams
         HIP_TRY(hipDeviceSynchronize());
-        HIP_TRY(hipMemcpy(op->dev, p, bytes, hipMemcpyHostToDevice));
+        if ((st = host_to_device(op->dev, p, bytes))) return st;
     }
     return CAKE_HIP_OK;
 }
@@ -132,8 +214,7 @@ int stage_out(const Operand& op, hipStream_t stream)
 {
     if (!op.host) return CAKE_HIP_OK;
     HIP_TRY(hipStreamSynchronize(stream));
-    HIP_TRY(hipMemcpy(op.host, op.dev, op.bytes, hipMemcpyDeviceToHost));
-    return CAKE_HIP_OK;
+    return device_to_host(op.host, op.dev, op.bytes);
 }
 
 // Event bracket for `seconds`.
@@ -378,10 +459,16 @@ int cake_hip_shutdown(void)
     for (DeviceBuffer& b : g_ctx.stage) b.release();
     g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
     g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.conv_taps.release();
-    for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1]}) {
+    for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1], &g_ctx.copy_done[0], &g_ctx.copy_done[1]}) {
         if (*e) (void)hipEventDestroy(*e);
         *e = nullptr;
     }
+    for (void*& p : g_ctx.pinned) {
+        if (p) (void)hipHostFree(p);
+        p = nullptr;
+    }
+    if (g_ctx.copy_stream) (void)hipStreamDestroy(g_ctx.copy_stream);
+    g_ctx.copy_stream = nullptr;
     g_ctx.ready = false;
     return CAKE_HIP_OK;
 }

@@ -148,3 +148,20 @@ def test_reference_run_tests_sweep():
     print(tail, res.stderr[-2000:])
     assert res.returncode == 0 and "ALL TESTS PASSED!" in res.stdout and "TESTS FAILED" not in res.stdout
     assert res.stdout.count("CORRECT!") >= 216 * 5
+
+
+@pytest.mark.parametrize("rows,cols", [(4100, 4099), (2048, 1024), (1449, 1448), (8193, 1025)],
+                         ids=lambda v: str(v))
+def test_large_host_operands_survive_the_staging_pipeline(rows, cols):
+    """Host arrays of 8 MB and more travel through pinned buffers in 32 MB chunks (below that a
+    plain copy): a transpose moves every byte both ways, so the result must be bit-exact, also when
+    the last chunk is ragged and when the size sits just under and over the threshold."""
+    src = oracle.uniform((rows, cols), 21)
+    dst = np.full((cols, rows), np.nan, np.float32)
+    print(f"host staging {rows}x{cols}: {src.nbytes / 2**20:.1f} MiB", flush=True)
+    cake.transpose_mat(src, dst, rows, cols)
+    assert np.array_equal(dst, src.T)
+    # twice in a row: the buffers and events are reused
+    dst2 = np.full((cols, rows), np.nan, np.float32)
+    cake.transpose_mat(src, dst2, rows, cols)
+    assert np.array_equal(dst2, src.T)
