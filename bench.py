@@ -188,7 +188,7 @@ def main() -> int:
             by = 4.0 * (M * K + K * N + M * N)
             if streaming_kernel:   # few rows or columns: bound by reading the large operand once
                 extras.append({"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
-                               "kernel": streaming_kernel,
+                               "kernel": streaming_kernel, "kernel_family": cake.KERNEL_NAMES[pl.kernel],
                                "roofline": {"bound": "hbm", "achieved": round(by / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
                                             "unit": "GB/s", "frac": round(by / avg / 1e9 / HBM_PEAK_GBPS, 4),
                                             "traffic": traffic, "algorithmic_bytes_per_launch": by}})
@@ -196,6 +196,7 @@ def main() -> int:
             extras.append({"workload": name, "ms": round(avg * 1e3, 4), "tflops": round(fl / avg / 1e12, 2),
                            "frac_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4),
                            "compulsory_GBps": round(by / avg / 1e9, 1),
+                           "kernel_family": cake.KERNEL_NAMES[pl.kernel],
                            "tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
                            "schedule": cake.SCHED_NAMES[pl.sched]})
 

@@ -4,7 +4,7 @@ Host-side mirror of the reference's interface for this path (cake_sgemm,
 cake_sgemv, init_block_dims, pack_A/pack_B/unpack_C, im_2_col, the linear layer) over the
 C-ABI of libcake_hip.so.  PyTorch is not required; torch ROCm tensors and numpy
 arrays are both accepted wherever a matrix is."""
-from ._lib import (KMN, MKN, NKM, NA, SCHED_NAMES, BlkDims, CakeHipError, CpuCntx, DeviceInfo,
+from ._lib import (KMN, MKN, NKM, NA, SCHED_NAMES, KERNEL_NAMES, BlkDims, CakeHipError, CpuCntx, DeviceInfo,
                    Plan, load)
 from .api import (autotune, cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_size, cake_sgemm_packed_B_size,
                   cake_sgemm_packed_C_size, cake_sgemv, conv2d, device_info, fill_uniform, im2col,
@@ -13,7 +13,7 @@ from .api import (autotune, cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_siz
                   update_mr_nr)
 
 __all__ = [
-    "KMN", "MKN", "NKM", "NA", "SCHED_NAMES", "BlkDims", "CpuCntx", "Plan", "DeviceInfo",
+    "KMN", "MKN", "NKM", "NA", "SCHED_NAMES", "KERNEL_NAMES", "BlkDims", "CpuCntx", "Plan", "DeviceInfo",
     "CakeHipError", "load", "cake_query_cntx", "update_mr_nr", "init_block_dims", "plan",
     "cake_sgemm", "cake_sgemv", "pack_A", "pack_B", "pack_C", "unpack_C",
     "cake_sgemm_packed_A_size", "cake_sgemm_packed_B_size", "cake_sgemm_packed_C_size",

@@ -15,6 +15,8 @@ CXX_LIB_PATH = LIB_DIR / "libcake.so"
 
 KMN, MKN, NKM, NA = 0, 1, 2, 3
 SCHED_NAMES = {KMN: "KMN", MKN: "MKN", NKM: "NKM", NA: "NA"}
+# Plan.kernel: which kernel family cake_hip_sgemm runs for a shape
+KERNEL_NAMES = {0: "macro-tile", 1: "matrix-vector", 2: "streaming, few rows", 3: "streaming, few columns"}
 
 OK, ERR_ARG, ERR_NO_DEVICE, ERR_HIP, ERR_ALLOC, ERR_RANGE, ERR_ARCH = range(7)
 
@@ -43,7 +45,8 @@ class CpuCntx(C.Structure):
 class Plan(C.Structure):
     _fields_ = [(n, C.c_int) for n in
                 ("sched", "tile_m", "tile_n", "tile_k", "wave_m", "wave_n", "threads", "split_k",
-                 "tail_tiles", "tail_split", "tiles_m", "tiles_n", "group", "grid", "lds_bytes", "vector_loads", "cus")] + \
+                 "tail_tiles", "tail_split", "tiles_m", "tiles_n", "group", "grid", "lds_bytes", "vector_loads", "cus",
+                 "kernel")] + \
                [("flops", C.c_double), ("min_bytes", C.c_double), ("model_bytes", C.c_double)]
 
     def as_dict(self):

@@ -530,6 +530,18 @@ int cake_hip_synchronize(void)
     return CAKE_HIP_OK;
 }
 
+// Which kernel cake_hip_sgemm runs for dense row-major operands of this shape (CAKE_HIP_KERNEL_*)
+static int kernel_family(int M, int N, int K, bool tile_forced, bool vec)
+{
+    if (tile_forced || M <= 0 || N <= 0 || K <= 0) return CAKE_HIP_KERNEL_TILE;
+    if (M == 1 || N == 1) return CAKE_HIP_KERNEL_GEMV;
+    if (vec && !tune_lookup(M, N, K, true, nullptr)) {
+        if (fewrows_applies(M, N, K, K, N)) return CAKE_HIP_KERNEL_STREAM_ROWS;
+        if (fewrows_nt_applies(N, M, K, N, K, true)) return CAKE_HIP_KERNEL_STREAM_COLS;
+    }
+    return CAKE_HIP_KERNEL_TILE;
+}
+
 int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake_hip_plan_t* out)
 {
     if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
@@ -539,6 +551,7 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     int st = plan_gemm(M, N, K, sched, tile_override, vec, model, &plan);
     if (st) return fail(st, "cake_hip_plan: bad shape, schedule or tile override");
     *out = plan.pub;
+    out->kernel = kernel_family(M, N, K, tile_override != nullptr, vec);
     return CAKE_HIP_OK;
 }
 
@@ -1276,6 +1289,8 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
             GemmPlan plan;
             if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
             *best_plan = plan.pub;
+        best_plan->kernel = kernel_family(M, N, K, false, vec);
+            best_plan->kernel = kernel_family(M, N, K, false, vec);
         }
         return CAKE_HIP_OK;
     }
@@ -1290,6 +1305,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
         GemmPlan plan;
         if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
         *best_plan = plan.pub;
+        best_plan->kernel = kernel_family(M, N, K, false, vec);
     }
     return CAKE_HIP_OK;
 }

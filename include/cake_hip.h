@@ -66,6 +66,17 @@ typedef struct cake_hip_cpu_cntx_t {
     int ncores;
 } cake_hip_cpu_cntx_t;
 
+/* Kernel families of cake_hip_plan_t.kernel.  Dense row-major operands without a tile override:
+ * a product with a single row or column runs on the matrix-vector kernels, one with at most 32
+ * rows of A or columns of B (and at least 512 of the other, K >= 64) on the streaming kernels,
+ * everything else on the macro-tile kernel the other fields describe. */
+enum {
+    CAKE_HIP_KERNEL_TILE = 0,
+    CAKE_HIP_KERNEL_GEMV = 1,
+    CAKE_HIP_KERNEL_STREAM_ROWS = 2, /* few rows of A: B streamed once    */
+    CAKE_HIP_KERNEL_STREAM_COLS = 3  /* few columns of B: A streamed once */
+};
+
 /* What the GPU planner decided for one GEMM: the successor of
  * get_cache_dims / derive_schedule (src/block_sizing.cpp:304-462). */
 typedef struct cake_hip_plan_t {
@@ -82,6 +93,7 @@ typedef struct cake_hip_plan_t {
     int lds_bytes;    /* LDS per workgroup (double buffered)                      */
     int vector_loads; /* 1: 16-byte global loads usable (K below 2M and N below 8M floats) */
     int cus;          /* compute units the plan was made for                      */
+    int kernel;       /* CAKE_HIP_KERNEL_*: which kernel family cake_hip_sgemm runs for this shape */
     double flops;     /* 2*M*N*K                                                  */
     double min_bytes; /* compulsory traffic 4*(MK+KN+MN)                          */
     double model_bytes; /* modelled HBM traffic of the chosen order and CB block  */

@@ -275,3 +275,18 @@ def test_tune_table_load_lookup_save_clear(tmp_path):
             cake.tune_load(tmp_path / "missing.txt")
     finally:
         cake.tune_clear()
+
+
+def test_plan_names_the_kernel_family():
+    """Single rows or columns go to the matrix-vector kernels, up to 32 rows or columns against a
+    wide operand to the streaming kernels, the rest (and anything with a tile override) to the
+    macro-tile kernel."""
+    fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
+    assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
+    assert fam(16, 16384, 16384) == 2 and fam(32, 600, 64) == 2 and fam(2, 512, 100) == 2
+    assert fam(16384, 16, 16384) == 3 and fam(512, 32, 64) == 3
+    assert fam(33, 16384, 16384) == 0 and fam(16384, 33, 16384) == 0
+    assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0
+    assert fam(1024, 1024, 1024) == 0
+    assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
+    assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
