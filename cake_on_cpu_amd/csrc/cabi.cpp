@@ -82,8 +82,10 @@ struct Context {
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
     // host <-> device transfers of large host operands: two pinned buffers, a stream, an event each
-    void* pinned[2] = {nullptr, nullptr};
-    hipStream_t copy_stream = nullptr;
+    // (buffers 0, 1 and copy_stream: towards the device; 2, 3 and copy_back_stream: back, used
+    // only when both directions run at once)
+    void* pinned[4] = {nullptr, nullptr, nullptr, nullptr};
+    hipStream_t copy_stream = nullptr, copy_back_stream = nullptr;
     hipEvent_t copy_done[2] = {nullptr, nullptr};
 };
 
@@ -128,6 +130,16 @@ static int pinned_ready()
         if (!g_ctx.copy_done[i]) HIP_TRY(hipEventCreateWithFlags(&g_ctx.copy_done[i], hipEventDisableTiming));
     }
     if (!g_ctx.copy_stream) HIP_TRY(hipStreamCreateWithFlags(&g_ctx.copy_stream, hipStreamNonBlocking));
+    return CAKE_HIP_OK;
+}
+
+static int pinned_both_ways_ready()
+{
+    int st = pinned_ready();
+    if (st) return st;
+    for (int i = 2; i < 4; ++i)
+        if (!g_ctx.pinned[i]) HIP_TRY(hipHostMalloc(&g_ctx.pinned[i], PIN_CHUNK, hipHostMallocDefault));
+    if (!g_ctx.copy_back_stream) HIP_TRY(hipStreamCreateWithFlags(&g_ctx.copy_back_stream, hipStreamNonBlocking));
     return CAKE_HIP_OK;
 }
 
@@ -467,8 +479,10 @@ int cake_hip_shutdown(void)
         if (p) (void)hipHostFree(p);
         p = nullptr;
     }
-    if (g_ctx.copy_stream) (void)hipStreamDestroy(g_ctx.copy_stream);
-    g_ctx.copy_stream = nullptr;
+    for (hipStream_t* cs : {&g_ctx.copy_stream, &g_ctx.copy_back_stream}) {
+        if (*cs) (void)hipStreamDestroy(*cs);
+        *cs = nullptr;
+    }
     g_ctx.ready = false;
     return CAKE_HIP_OK;
 }
@@ -569,6 +583,82 @@ int cake_hip_derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_
     return derive_schedule(M, N, K, p, mc, cntx);
 }
 
+// Rows of A (and of C) per block of the pipelined host path: about a quarter of the rows, whole
+// macro-tile rows, and a block of either matrix fits a pinned buffer.  0: rows too long for this path.
+static int host_row_block(int M, int K, int N)
+{
+    const size_t widest = (size_t)(K > N ? K : N) * sizeof(float);
+    const int fit = (int)(PIN_CHUNK / widest / 256 * 256);
+    const int quarter = (M / 4 + 255) / 256 * 256;
+    return fit < quarter ? fit : quarter;
+}
+
+// C = A . B with A and C in host memory and large: instead of "upload all, multiply, download
+// all", the rows of A travel in blocks through a three-stage pipeline.  While block i is
+// multiplied, block i + 1 is copied into a pinned buffer and sent to the device, block i - 1 comes
+// back into another pinned buffer and block i - 2 is copied out to the caller's C.  B (device
+// memory by now) is needed by every block and goes first.  The products of the blocks are
+// ordinary calls of the row-major kernel on device memory.
+static int sgemm_host_pipelined(const float* A, const float* b_dev, float* C, int M, int N, int K, int sched,
+                                const int* tile_override, hipStream_t stream, double* seconds)
+{
+    const int RB = host_row_block(M, K, N);
+    const int nblk = (M + RB - 1) / RB;
+    int st = pinned_both_ways_ready();
+    if (st) return st;
+    if ((st = g_ctx.stage[0].reserve((size_t)M * K * 4))) return st;
+    if ((st = g_ctx.stage[2].reserve((size_t)M * N * 4))) return st;
+    float* a_dev = static_cast<float*>(g_ctx.stage[0].ptr);
+    float* c_dev = static_cast<float*>(g_ctx.stage[2].ptr);
+    HIP_TRY(hipDeviceSynchronize());   // nothing of an earlier call still uses the staging slots
+
+    struct Events {
+        std::vector<hipEvent_t> ev;
+        ~Events() { for (hipEvent_t e : ev) if (e) (void)hipEventDestroy(e); }
+    } events;
+    events.ev.assign((size_t)3 * nblk, nullptr);
+    for (hipEvent_t& e : events.ev) HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    hipEvent_t* up = events.ev.data();            // block i has arrived on the device
+    hipEvent_t* done = up + nblk;                 // block i has been multiplied
+    hipEvent_t* back = done + nblk;               // block i of C sits in its pinned buffer
+
+    auto rows_of = [&](int i) { return M - i * RB < RB ? M - i * RB : RB; };
+    // `seconds`: from the first product's start to the last one's end on the stream (the waits for
+    // arriving blocks included); no per-kernel timing, which would stop the host after every launch
+    Timer timer(stream, seconds), untimed(stream, nullptr);
+    if ((st = timer.start())) return st;
+    for (int i = 0; i < nblk + 2; ++i) {
+        if (i < nblk) {
+            const size_t off = (size_t)i * RB * K, bytes = (size_t)rows_of(i) * K * 4;
+            void* pin = g_ctx.pinned[i & 1];
+            if (i >= 2) HIP_TRY(hipEventSynchronize(up[i - 2]));   // the buffer's last transfer is over
+            parallel_memcpy(pin, A + off, bytes);
+            HIP_TRY(hipMemcpyAsync(a_dev + off, pin, bytes, hipMemcpyHostToDevice, g_ctx.copy_stream));
+            HIP_TRY(hipEventRecord(up[i], g_ctx.copy_stream));
+            HIP_TRY(hipStreamWaitEvent(stream, up[i], 0));
+            const float* ai = a_dev + off;
+            float* ci = c_dev + (size_t)i * RB * N;
+            const int mode = vec4_loadable(ai, b_dev, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
+            if ((st = run_gemm(ai, b_dev, ci, rows_of(i), N, K, K, N, N, sched, 0, tile_override, mode, mode, stream, untimed)))
+                return st;
+            HIP_TRY(hipEventRecord(done[i], stream));
+        }
+        if (i >= 1 && i - 1 < nblk) {   // block i - 1 starts its way back (its buffer was emptied one round ago)
+            const int j = i - 1;
+            HIP_TRY(hipStreamWaitEvent(g_ctx.copy_back_stream, done[j], 0));
+            HIP_TRY(hipMemcpyAsync(g_ctx.pinned[2 + (j & 1)], c_dev + (size_t)j * RB * N, (size_t)rows_of(j) * N * 4,
+                                   hipMemcpyDeviceToHost, g_ctx.copy_back_stream));
+            HIP_TRY(hipEventRecord(back[j], g_ctx.copy_back_stream));
+        }
+        if (i >= 2) {                   // block i - 2 has arrived: out to the caller's C
+            const int j = i - 2;
+            HIP_TRY(hipEventSynchronize(back[j]));
+            parallel_memcpy(C + (size_t)j * RB * N, g_ctx.pinned[2 + (j & 1)], (size_t)rows_of(j) * N * 4);
+        }
+    }
+    return timer.stop();
+}
+
 int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K, int sched,
                    int accumulate, const int* tile_override, void* stream_, double* seconds)
 {
@@ -585,6 +675,13 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     Operand a, b, c;
+    // large host operands: transfers and arithmetic overlap block by block
+    const int RB = K > 0 ? host_row_block(M, K, N) : 0;
+    if (RB > 0 && M >= 3 * RB && N > 32 && ((double)M * K + (double)M * N) * 4 >= 32.0 * (1 << 20) && !accumulate &&
+        !is_device_pointer(A) && !is_device_pointer(C)) {
+        if ((st = stage_in(B, (size_t)K * N * 4, 1, true, &b))) return st;
+        return sgemm_host_pipelined(A, b.dev, C, M, N, K, sched, tile_override, stream, seconds);
+    }
     if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
     if ((st = stage_in(B, (size_t)K * N * 4, 1, true, &b))) return st;
     if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;

@@ -212,6 +212,30 @@ def test_random_shapes_against_fp64():
         assert err <= TIGHT, (case, M, N, K, err)
 
 
+@pytest.mark.parametrize("shape", [(3000, 1500, 2000), (4096, 1024, 4096), (1100, 9000, 520), (2500, 300, 9000)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_large_host_operands_take_the_block_pipeline(shape):
+    """A and C in host memory and 32 MB or more between them: blocks of rows are uploaded,
+    multiplied and downloaded in a pipeline (ragged last block, K-first overwrite of a prefilled C);
+    against fp64 on sampled rows, and twice in a row since buffers and events are reused."""
+    M, K, N = shape
+    print(f"sgemm host pipeline M={M} K={K} N={N}", flush=True)
+    A, B = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+    rows = sorted({0, 1, 255, 256, M // 4, M // 2, (3 * M) // 4, M - 257, M - 2, M - 1})
+    ref = A[rows].astype(np.float64) @ B.astype(np.float64)
+    S = np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64)
+    first = None
+    for _ in range(2):
+        Cm = np.full((M, N), np.nan, np.float32)
+        cake.cake_sgemm(A, B, Cm, M, N, K, 1)
+        assert not np.isnan(Cm).any()
+        assert float(np.max(np.abs(Cm[rows] - ref) / S)) <= TIGHT
+        if first is None:
+            first = Cm
+        else:
+            assert np.array_equal(first, Cm)
+
+
 def test_identity_all_ones_single_nonzero():
     n = 300
     B = oracle.uniform((n, 260), 5)
