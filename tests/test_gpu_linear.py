@@ -165,3 +165,22 @@ def test_large_host_operands_survive_the_staging_pipeline(rows, cols):
     dst2 = np.full((cols, rows), np.nan, np.float32)
     cake.transpose_mat(src, dst2, rows, cols)
     assert np.array_equal(dst2, src.T)
+
+
+def test_zz_shutdown_releases_and_the_next_call_starts_over():
+    """cake_hip_shutdown frees the workspaces, pinned buffers, streams and events; the next
+    call initialises again and computes the same product (host operands large enough to use the
+    pinned staging on both sides of the shutdown)."""
+    import ctypes as C
+    lib = cake.load()
+    M, K, N = 1536, 1500, 1400
+    A, B = oracle.uniform((M, K), 31), oracle.uniform((K, N), 32)
+    before = np.zeros((M, N), np.float32)
+    cake.cake_sgemm(A, B, before, M, N, K, 1)
+    assert lib.cake_hip_shutdown() == 0
+    assert lib.cake_hip_shutdown() == 0          # idempotent
+    after = np.zeros((M, N), np.float32)
+    cake.cake_sgemm(A, B, after, M, N, K, 1)
+    assert np.array_equal(before, after)
+    C64, S = oracle.gemm_f64(A, B)
+    assert oracle.max_rel_err(after, C64, S) <= 5e-6
