@@ -222,21 +222,26 @@ def test_conv2d_paths_agree_bitwise_layouts():
     assert np.array_equal(a, b)
 
 
-def test_conv2d_with_a_caller_workspace_on_device_tensors():
+@pytest.mark.parametrize("geom", [(3, 12, 18, 20, 40, 3, 3, 1, 1), (2, 8, 17, 22, 24, 3, 3, 2, 1),
+                                  (2, 8, 16, 16, 12, 1, 1, 2, 0), (1, 6, 20, 13, 9, 5, 5, 1, 0)], ids=str)
+def test_conv2d_with_a_caller_workspace_on_device_tensors(geom):
     """Device operands and a caller-owned workspace of cake_hip_conv2d_workspace bytes, offset so it
-    is not 256-byte aligned: both paths must give what they give with the library's own buffer."""
+    is not 256-byte aligned: both paths must give what they give with the library's own buffer
+    (stride 1 with padding, stride 2 with the phase-split staged input and an output width of 11,
+    a 1x1 stride-2 layer, and an unpadded layer that reads the input as it lies)."""
     import torch
     dev = torch.device("cuda:0")
-    Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad = 3, 12, 18, 20, 40, 3, 3, 1, 1
+    Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad = geom
+    Hout, Wout = (Hin + 2 * pad - Hf) // stride + 1, (Win + 2 * pad - Wf) // stride + 1
     inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 58), oracle.uniform((Cout, Cin, Hf, Wf), 59)
-    want = np.empty((Bn, Cout, Hin, Win), np.float32)
+    want = np.empty((Bn, Cout, Hout, Wout), np.float32)
     cake.conv2d(inp, wt, want, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=True)
     need = cake.load().cake_hip_conv2d_workspace(Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)
-    assert need >= 4 * Cin * 9 * Bn * Hin * Win
+    assert need >= 4 * Cin * Hf * Wf * Bn * Hout * Wout
     ws = torch.empty((need + 3) // 4 + 1, dtype=torch.float32, device=dev)[1:]
     ti, tw = torch.from_numpy(inp).to(dev), torch.from_numpy(wt).to(dev)
     for explicit in (False, True):
-        out = torch.full((Bn, Cout, Hin, Win), float("nan"), dtype=torch.float32, device=dev)
+        out = torch.full((Bn, Cout, Hout, Wout), float("nan"), dtype=torch.float32, device=dev)
         cake.conv2d(ti, tw, out, Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw=True,
                     workspace=ws, explicit_im2col=explicit)
         torch.cuda.synchronize()
