@@ -42,8 +42,8 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": (1049023 + 256) * 1024,
                           # streaming kernel + its slice reduction, 16 x 16384 x 16384 and transposes of it
-                          "fewrows_nn": (1056762 + 8192 + 4775 + 1024) * 1024,
-                          "fewrows_nt": (1056793 + 3091 + 4775 + 1024) * 1024}
+                          "fewrows_nn": (1056751 + 4096 + 3490 + 1024) * 1024,
+                          "fewrows_nt": (1056793 + 3095 + 3490 + 1024) * 1024}
 
 
 def main() -> int:
