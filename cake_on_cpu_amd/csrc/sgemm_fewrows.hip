@@ -1,25 +1,26 @@
-// sgemm_fewrows.hip -- products in which one operand has at most 16 rows or
+// sgemm_fewrows.hip -- products in which one operand has at most 32 rows or
 // columns ("a few vectors times a matrix": small-batch linear layers, blocks of
 // matrix-vector products).
 //
 // Such a product is bound by reading the large operand once from HBM, not by
 // arithmetic, and a 64-row macro-tile would spend most of the matrix pipe on
 // zero rows while reading the large operand in short pieces.  The kernels here
-// stream the large operand straight from global memory into the operand
-// registers of v_mfma_f32_16x16x4_f32, whose 16 rows fit the problem: no LDS
-// and no barrier inside the k loop, so every wave keeps its loads in flight on
-// its own.  The small operand comes from L2 with one load per 4 to 16 loads of
-// the large one.
+// stream the large operand once, 16 bytes per lane, into the operand registers
+// of v_mfma_f32_16x16x4_f32, whose 16 rows fit the problem (17 to 32 rows or
+// columns run two MFMA groups per value loaded): no barrier inside the k loop,
+// so every wave keeps its loads in flight on its own.  The small operand comes
+// from L2 with one load per 4 to 16 loads of the large one.
 //
-//   sgemm_fewrows_nn_kernel   C[M<=16][N] = A[M][K] . B[K][N]      streams B (n contiguous)
-//   sgemm_fewrows_nt_kernel   C'[i<=16][n] = sum_k X[i][k] W[n][k]  streams W (k contiguous):
-//                             the linear layer y = x w^T for a small batch without
-//                             transposing w, and C[M][N<=16] = A.B with W = A, X = B^T
+//   sgemm_fewrows_nn_kernel   C[M<=32][N] = A[M][K] . B[K][N]      streams B (n contiguous),
+//                             straight from global memory into MFMA operands
+//   sgemm_fewrows_nt_kernel   C'[i<=32][n] = sum_k X[i][k] W[n][k]  streams W (k contiguous)
+//                             through a wave-private LDS area that turns rows into MFMA
+//                             operands: the linear layer y = x w^T for a small batch without
+//                             transposing w, and C[M][N<=32] = A.B with W = A, X = B^T
 //
 // A workgroup owns 64 or 128 columns of B (64 rows of W) and a slice of k; its four
-// waves take a quarter of the slice each and add their sums in LDS in wave
-// order; K slices are summed by splitk_reduce_kernel in slice order, so results
-// are run-to-run identical.
+// waves share the slice and add their sums in LDS in wave order; K slices are summed
+// by splitk_reduce_kernel in slice order, so results are run-to-run identical.
 //
 // Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l % 16][l / 16]
 // and B[l / 16][l % 16]; result register r of lane l is C[4 * (l / 16) + r][l % 16].
@@ -47,7 +48,7 @@ __device__ __forceinline__ float load_f32(const float* base, int byte_offset, un
 }
 
 static constexpr int FR_ROWS = 64;      // nt: rows of W per workgroup
-static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave and loop step
+static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave
 
 // The part of [kbeg, kend) that wave `wave` of 4 walks: quarters rounded up to 16 k
 __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0, int& kw1)
