@@ -313,9 +313,10 @@ def _opt_ptr(a, what):
     return None if a is None else _ptr(a, what)
 
 
-def linear_forward(x, w, bias, y, M, N, K) -> float:
+def linear_forward(x, w, bias, y, M, N, K, timed=True) -> float:
     """y[M][N] = x[M][K] . w[N][K]^T + bias[N] (bias may be None): linear_forward of
-    src/linear.cpp:12-50.  Returns seconds."""
+    src/linear.cpp:12-50.  Returns seconds; timed=False skips the event timing, which makes
+    the call asynchronous on device operands (it then returns 0)."""
     _need(x, M * K, "x")
     _need(w, N * K, "w")
     _need(y, M * N, "y")
@@ -323,13 +324,27 @@ def linear_forward(x, w, bias, y, M, N, K) -> float:
         _need(bias, N, "bias")
     secs = C.c_double(0.0)
     check(load().cake_hip_linear_forward(_ptr(x, "x"), _ptr(w, "w"), _opt_ptr(bias, "bias"), _ptr(y, "y"),
-                                         M, N, K, _stream(x, w, y), C.byref(secs)), "linear_forward")
+                                         M, N, K, _stream(x, w, y), C.byref(secs) if timed else None), "linear_forward")
     return secs.value
 
 
-def linear_backward(grad_y, x, w, grad_x, grad_w, grad_bias, M, N, K) -> float:
+def linear_forward_wt(x, wt, bias, y, M, N, K, timed=True) -> float:
+    """The same with the weights already transposed: wt is [K][N] (transpose_mat of w), for callers
+    that keep the transposed copy while the weights stay the same."""
+    _need(x, M * K, "x")
+    _need(wt, N * K, "wt")
+    _need(y, M * N, "y")
+    if bias is not None:
+        _need(bias, N, "bias")
+    secs = C.c_double(0.0)
+    check(load().cake_hip_linear_forward_wt(_ptr(x, "x"), _ptr(wt, "wt"), _opt_ptr(bias, "bias"), _ptr(y, "y"),
+                                            M, N, K, _stream(x, wt, y), C.byref(secs) if timed else None), "linear_forward_wt")
+    return secs.value
+
+
+def linear_backward(grad_y, x, w, grad_x, grad_w, grad_bias, M, N, K, timed=True) -> float:
     """grad_x = grad_y . w, grad_w = grad_y^T . x, grad_bias = column sums of grad_y
-    (src/linear.cpp:53-102).  Outputs passed as None are skipped.  Returns seconds."""
+    (src/linear.cpp:53-102).  Outputs passed as None are skipped.  Returns seconds (0 with timed=False)."""
     _need(grad_y, M * N, "grad_y")
     for a, n, what in ((x, M * K, "x"), (w, N * K, "w"), (grad_x, M * K, "grad_x"),
                        (grad_w, N * K, "grad_w"), (grad_bias, N, "grad_bias")):
@@ -339,7 +354,7 @@ def linear_backward(grad_y, x, w, grad_x, grad_w, grad_bias, M, N, K) -> float:
     check(load().cake_hip_linear_backward(_ptr(grad_y, "grad_y"), _opt_ptr(x, "x"), _opt_ptr(w, "w"),
                                           _opt_ptr(grad_x, "grad_x"), _opt_ptr(grad_w, "grad_w"),
                                           _opt_ptr(grad_bias, "grad_bias"), M, N, K,
-                                          _stream(grad_y, x, w), C.byref(secs)), "linear_backward")
+                                          _stream(grad_y, x, w), C.byref(secs) if timed else None), "linear_backward")
     return secs.value
 
 

@@ -1221,6 +1221,30 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
     return stage_out(yo, stream);
 }
 
+int cake_hip_linear_forward_wt(const float* x, const float* wt, const float* bias, float* y, int M, int N,
+                               int K, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int st = linear_dims_ok(M, N, K);
+    if (st) return st;
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (!y || (K > 0 && (!x || !wt))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    Operand xo, wo, bo, yo;
+    if ((st = stage_in(x, (size_t)M * K * 4, 0, true, &xo))) return st;
+    if ((st = stage_in(wt, (size_t)N * K * 4, 1, true, &wo))) return st;
+    if (bias && (st = stage_in(bias, (size_t)N * 4, 2, true, &bo))) return st;
+    if ((st = stage_in(y, (size_t)M * N * 4, 3, false, &yo))) return st;
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if ((st = linear_gemm(xo.dev, wo.dev, yo.dev, M, N, K, bias ? bo.dev : nullptr, stream, timer))) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(yo, stream);
+}
+
 int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w, float* grad_x,
                              float* grad_w, float* grad_bias, int M, int N, int K, void* stream_,
                              double* seconds)

@@ -20,20 +20,31 @@ def _f32c(t: torch.Tensor, what: str) -> torch.Tensor:
     return t.detach().contiguous()
 
 
-def forward(cache_sz, input, weight, bias=None):
+SMALL_BATCH = 32   # up to here the library streams the weights as they lie: no transposed copy is needed
+
+
+def forward(cache_sz, input, weight, bias=None, weight_t=None):
     """output[M][N] = input[M][K] . weight[N][K]^T (+ bias).  `cache_sz` (the
     reference passes the host's L2/L3 sizes, src/linear.cpp:37) is accepted and
-    unused: block sizes come from the device."""
+    unused: block sizes come from the device.  weight_t: the weights already
+    transposed ([K][N]), from a caller that keeps that copy (see cake_linear)."""
     if input.dim() != 2 or weight.dim() != 2 or input.size(1) != weight.size(1):
         raise ValueError(f"linear forward: input {tuple(input.shape)} does not match weight {tuple(weight.shape)}")
     M, K = input.shape
     N = weight.size(0)
     if bias is not None and tuple(bias.shape) != (N,):
         raise ValueError(f"linear forward: bias {tuple(bias.shape)} does not match {N} outputs")
-    x, w = _f32c(input, "input"), _f32c(weight, "weight")
+    x = _f32c(input, "input")
     b = None if bias is None else _f32c(bias, "bias")
     out = torch.empty((M, N), dtype=torch.float32, device=input.device)
-    api.linear_forward(x, w, b, out, M, N, K)
+    # device tensors: no event timing, so the call only enqueues work on torch's current stream
+    timed = not input.is_cuda
+    if weight_t is not None and M > SMALL_BATCH:
+        if tuple(weight_t.shape) != (K, N):
+            raise ValueError(f"linear forward: weight_t {tuple(weight_t.shape)} is not {(K, N)}")
+        api.linear_forward_wt(x, _f32c(weight_t, "weight_t"), b, out, M, N, K, timed=timed)
+    else:
+        api.linear_forward(x, _f32c(weight, "weight"), b, out, M, N, K, timed=timed)
     return out
 
 
@@ -50,20 +61,21 @@ def backward(cache_sz, grad_output, input, weight, bias=None, needs=(True, True,
     gx = torch.empty((M, K), dtype=torch.float32, device=dev) if needs[0] else None
     gw = torch.empty((N, K), dtype=torch.float32, device=dev) if needs[1] else None
     gb = torch.empty((N,), dtype=torch.float32, device=dev) if (needs[2] and bias is not None) else None
-    api.linear_backward(g, x if gw is not None else None, w if gx is not None else None, gx, gw, gb, M, N, K)
+    api.linear_backward(g, x if gw is not None else None, w if gx is not None else None, gx, gw, gb, M, N, K,
+                        timed=not grad_output.is_cuda)
     return gx, gw, gb
 
 
 class cake_linear_function(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, data, weight, bias=None):
+    def forward(ctx, data, weight, bias=None, weight_t=None):
         ctx.save_for_backward(data, weight, bias)
-        return forward(None, data, weight, bias)
+        return forward(None, data, weight, bias, weight_t)
 
     @staticmethod
     def backward(ctx, grad_output):
         data, weight, bias = ctx.saved_tensors
-        return backward(None, grad_output, data, weight, bias, ctx.needs_input_grad)
+        return (*backward(None, grad_output, data, weight, bias, ctx.needs_input_grad[:3]), None)
 
 
 class cake_linear(nn.Module):
@@ -80,9 +92,23 @@ class cake_linear(nn.Module):
         else:
             self.register_parameter("bias", None)
 
+    def _transposed_weight(self):
+        """[input_features][output_features] copy of the weights, made again only when they have
+        changed (torch counts in-place updates of a tensor in `_version`) or moved: a layer that is
+        only evaluated transposes its weights once instead of on every call."""
+        w = self.weight
+        key = (w.data_ptr(), w._version, w.device)
+        if getattr(self, "_wt_key", None) != key:
+            wt = torch.empty((self.input_features, self.output_features), dtype=torch.float32, device=w.device)
+            api.transpose_mat(_f32c(w, "weight"), wt, self.output_features, self.input_features)
+            self._wt, self._wt_key = wt, key
+        return self._wt
+
     def forward(self, data):
         lead = data.shape[:-1]
-        out = cake_linear_function.apply(data.reshape(-1, self.input_features), self.weight, self.bias)
+        flat = data.reshape(-1, self.input_features)
+        wt = self._transposed_weight() if flat.size(0) > SMALL_BATCH else None
+        out = cake_linear_function.apply(flat, self.weight, self.bias, wt)
         return out.reshape(*lead, self.output_features)
 
     def extra_repr(self):

@@ -251,6 +251,15 @@ int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* s
 int cake_hip_linear_forward(const float* x, const float* w, const float* bias, float* y, int M,
                             int N, int K, void* stream, double* seconds);
 
+/* The same with the weights already transposed: wt is [K][N] (input x output
+ * features), y = x . wt (+ bias).  This is the product of linear_forward alone
+ * (the cake_sgemm call of src/linear.cpp:38 with its bias loop), for callers
+ * whose weights stay the same over many calls and who keep the transposed copy
+ * (cake_hip_transpose) instead of paying for it every time; batches of at most
+ * 32 do not need it, cake_hip_linear_forward streams w as it lies for them. */
+int cake_hip_linear_forward_wt(const float* x, const float* wt, const float* bias, float* y, int M,
+                               int N, int K, void* stream, double* seconds);
+
 /* Gradients of the layer above for grad_y[M][N] (src/linear.cpp:53-102):
  *   grad_x[M][K] = grad_y . w,   grad_w[N][K] = grad_y^T . x,
  *   grad_bias[N] = column sums of grad_y (summed in a fixed order).

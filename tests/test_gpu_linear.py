@@ -139,6 +139,41 @@ def test_torch_module_matches_nn_linear():
     assert torch.allclose(yc, torch.nn.functional.linear(xc, layer_cpu.weight, layer_cpu.bias), atol=1e-5)
 
 
+def test_torch_module_keeps_its_transposed_weights_until_they_change():
+    """The module transposes its weights once per version of the tensor: evaluating twice reuses
+    the copy, an optimizer step (an in-place update) makes a new one, batches of at most 32 never
+    need it, and every output matches torch's layer."""
+    import torch
+    from cake_on_cpu_amd.torch_linear import cake_linear
+    torch.manual_seed(1)
+    dev = torch.device("cuda:0")
+    layer = cake_linear(300, 520).to(dev)
+    x = torch.rand(200, 300, device=dev) * 2 - 1
+    want = lambda t: torch.nn.functional.linear(t.double(), layer.weight.double(), layer.bias.double())
+    with torch.no_grad():
+        y1 = layer(x)
+        first = layer._wt
+        y2 = layer(x)
+        assert layer._wt is first                       # same weights: same transposed copy
+        assert torch.equal(y1, y2)
+        assert (y1.double() - want(x)).abs().max().item() <= TIGHT * 300
+        layer.weight.mul_(0.5)                          # what an optimizer step does: in place
+        y3 = layer(x)
+        assert layer._wt is not first
+        assert (y3.double() - want(x)).abs().max().item() <= TIGHT * 300
+        small = layer(x[:8])                            # streamed from the weights as they lie
+        assert (small.double() - want(x[:8])).abs().max().item() <= TIGHT * 300
+    # training steps through autograd and an optimizer keep working with the cache in place
+    opt = torch.optim.SGD(layer.parameters(), lr=0.01)
+    for _ in range(2):
+        opt.zero_grad()
+        out = layer(x)
+        assert (out.double() - want(x)).abs().max().item() <= TIGHT * 300
+        out.sum().backward()
+        opt.step()
+    torch.cuda.synchronize()
+
+
 def test_reference_run_tests_sweep():
     """run_tests of src/util.cpp:3-136 through libcake.so: 216 shapes x five entry points."""
     exe = _lib.LIB_DIR / "dropin_test"
