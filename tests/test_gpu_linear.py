@@ -139,6 +139,30 @@ def test_torch_module_matches_nn_linear():
     assert torch.allclose(yc, torch.nn.functional.linear(xc, layer_cpu.weight, layer_cpu.bias), atol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(64, 96, 48), (33, 130, 257), (300, 2111, 96), (7, 5, 3)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_forward_with_pretransposed_weights(shape):
+    """cake_hip_linear_forward_wt on a transposed copy of the weights gives what
+    cake_hip_linear_forward gives on the weights themselves (same product, same bias rounding)."""
+    M, K, N = shape
+    x, w, b = oracle.uniform((M, K), 11), oracle.uniform((N, K), 12), oracle.uniform((N,), 13)
+    wt = np.empty((K, N), np.float32)
+    cake.transpose_mat(w, wt, N, K)
+    assert np.array_equal(wt, w.T)
+    y1 = np.full((M, N), np.nan, np.float32)
+    y2 = np.full((M, N), np.nan, np.float32)
+    cake.linear_forward(x, w, b, y1, M, N, K)
+    cake.linear_forward_wt(x, wt, b, y2, M, N, K)
+    y64 = x.astype(np.float64) @ w.astype(np.float64).T + b.astype(np.float64)[None, :]
+    S = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T + np.abs(b)[None, :]
+    assert _rel(y2, y64, S) <= TIGHT
+    if M > 32:   # above the streaming kernels' range both run the same product on the same operands
+        assert np.array_equal(y1, y2)
+    y3 = np.full((M, N), np.nan, np.float32)
+    cake.linear_forward_wt(x, wt, None, y3, M, N, K, timed=False)
+    assert _rel(y3, x.astype(np.float64) @ w.astype(np.float64).T, S) <= TIGHT
+
+
 def test_torch_module_keeps_its_transposed_weights_until_they_change():
     """The module transposes its weights once per version of the tensor: evaluating twice reuses
     the copy, an optimizer step (an in-place update) makes a new one, batches of at most 32 never
