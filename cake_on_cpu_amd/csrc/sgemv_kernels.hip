@@ -279,9 +279,11 @@ __global__ void sgemv_slice_reduce_kernel(const float* __restrict__ part, float*
 {
     const int m = blockIdx.x * 256 + threadIdx.x;
     if (m >= M) return;
-    float acc = accumulate ? y[m] : 0.f;
+    // the slices first, then one addition to what y held: y += A.x rounds the same way whether
+    // or not K was cut into slices
+    float acc = 0.f;
     for (int s = 0; s < slices; ++s) acc += part[(size_t)s * M + m];
-    y[m] = acc;
+    y[m] = accumulate ? y[m] + acc : acc;
 }
 
 hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,
