@@ -1211,6 +1211,15 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
         if ((st = timer.stop())) return st;
         return stage_out(yo, stream);
     }
+    if (small_batch && sgemv_rowmajor_multi_applies(N, K, M, K, wo.dev, xo.dev, g_ctx.model.cus)) {
+        // two samples on a mid-size layer: one pass of the matrix-vector sweep over w serves both
+        st = timer.family(2, [&] {
+            return launch_sgemv_rowmajor_multi(wo.dev, xo.dev, yo.dev, bias ? bo.dev : nullptr, N, K, M, K, N, stream);
+        });
+        if (st) return st;
+        if ((st = timer.stop())) return st;
+        return stage_out(yo, stream);
+    }
     if (small_batch) {
         // a small batch: y = x w^T with w streamed once as it lies, no transposed copy
         const int slices = fewrows_nt_slices(M, N, K, g_ctx.model.cus);

@@ -108,6 +108,11 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
 
 hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M, int K,
                                  int accumulate, float* scratch, int cus, hipStream_t stream);
+// Y[v][m] = bias[m] + sum_k A[m][k] * X[v][k] for 2 vectors (rows of X, ldx apart; rows of Y,
+// ldy apart) in one pass over the row-major A; bias may be nullptr
+bool sgemv_rowmajor_multi_applies(int M, int K, int vectors, int ldx, const float* A, const float* X, int cus);
+hipError_t launch_sgemv_rowmajor_multi(const float* A, const float* X, float* Y, const float* bias, int M,
+                                       int K, int vectors, int ldx, int ldy, hipStream_t stream);
 // scratch: at least sgemv_colmajor_scratch_floats(M, K) floats
 size_t sgemv_colmajor_scratch_floats(int M, int K, int cus);
 hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,

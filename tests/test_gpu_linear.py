@@ -41,6 +41,8 @@ LINEAR_SHAPES = [(1, 1, 1), (7, 5, 3), (64, 96, 48), (33, 130, 257), (128, 10, 9
                  # small batches: w streamed once as it lies (forward), grad_y . w by the few-rows kernel
                  (8, 1024, 4096), (3, 333, 1030), (16, 4099, 2048), (1, 64, 512), (13, 16390, 600), (16, 70, 5000),
                  (32, 1024, 2048), (20, 333, 1030), (17, 4099, 513), (33, 1024, 2048),
+                 # 2 samples on long rows: one matrix-vector sweep over w for both
+                 (2, 2048, 1024), (2, 4096, 2050), (2, 2052, 4097), (2, 16384, 2051), (2, 2048, 1023),
                  # a single sample: the row-major matrix-vector kernels (long rows, K slices, short rows, odd K)
                  (1, 8192, 300), (1, 20000, 8), (1, 24, 5000), (1, 2111, 777)]
 
