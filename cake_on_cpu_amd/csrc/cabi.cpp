@@ -1008,7 +1008,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const double K_d = (double)Cin * Hf * Wf;
     const double ncols_d = (double)batch * Hout * Wout;
     const double in_elems = (double)batch * Cin * Hin * Win;
-    if (!fits_int(K_d) || !fits_int(Cout * K_d) || !fits_int(Cout * ncols_d) || !fits_int(in_elems))
+    if (!fits_int(K_d) || !fits_int(Cout * K_d) || !fits_int(ncols_d) || in_elems * 4 >= 1e15 || Cout * ncols_d * 4 >= 1e15)
         return fail(CAKE_HIP_ERR_RANGE, "convolution lowers to a %dx%gx%g product that is out of range", Cout, K_d, ncols_d);
     const int K = (int)K_d, N = (int)ncols_d;
     int st = ensure_init();
@@ -1027,15 +1027,23 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // That costs row_n / Wout - 1 of extra arithmetic, where the column matrix costs a write and a
     // read of K x N floats, a share of the product's time that falls with Cout: measured on 7x7 to
     // 30x30 maps the padded rows win while (row_n / Wout - 1) * Cout stays below about 60.)
-    const ConvStage sg = conv_stage(batch, Cin, Hin, Win, Hf, Wf, stride, pad);
+    // The batch is cut into chunks of images when the whole of it does not meet those bounds:
+    // images are independent, the chunks run one after the other through the same staged copy.
     const int row_n = (Wout + 3) & ~3;
-    const double ncols_p = (double)batch * Hout * row_n;
-    const bool implicit = !explicit_cols && (double)(row_n - Wout) / Wout * Cout < 60.0 &&
-                          sg.elems * 4 + 4096 < 2147483648.0 && fits_int(Cout * ncols_p) &&
+    auto chunk_fits = [&](int nb) {
+        return conv_stage(nb, Cin, Hin, Win, Hf, Wf, stride, pad).elems * 4 + 4096 < 2147483648.0 &&
+               fits_int((double)Cout * nb * Hout * row_n) && fits_int((double)Cout * nb * Hout * Wout);
+    };
+    int chunk = batch;
+    while (chunk > 1 && !chunk_fits(chunk)) chunk = (chunk + 1) / 2;
+    const int chunks = (batch + chunk - 1) / chunk;
+    chunk = (batch + chunks - 1) / chunks;
+    const ConvStage sg = conv_stage(chunk, Cin, Hin, Win, Hf, Wf, stride, pad);
+    const bool implicit = !explicit_cols && (double)(row_n - Wout) / Wout * Cout < 60.0 && chunk_fits(chunk) &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
     if (implicit) {
-        const float* image = i.dev;
+        float* staged = nullptr;
         if (sg.copy) {
             char* ws = static_cast<char*>(workspace);
             if (!ws) {
@@ -1044,41 +1052,47 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             } else if (!is_device_pointer(ws)) {
                 return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
             }
-            image = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+            staged = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
         }
-        ConvGeom cv{};
-        cv.in = image;
-        cv.in_bytes = (unsigned)(sg.elems * 4);
-        cv.Cin = Cin; cv.plane_rows = sg.Hs; cv.pitch = sg.pitch; cv.row_step = sg.RH;
-        cv.Hout = Hout; cv.Wout = Wout; cv.row_n = row_n;
         if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
         int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
-        cv.tap_table = taps;
-        cv.out_nchw = out_nchw ? 1 : 0;
         if ((st = timer.start())) return st;
         st = timer.family(3, [&] {
             return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, sg.Hs, sg.pitch, sg.Wq, Hf, Wf, stride, sg.RH, stream);
         });
         if (st) return st;
-        if (sg.copy) {
-            st = timer.family(3, [&] {
-                float* dst = const_cast<float*>(image);
-                // stride 1: the plain zero-padded copy has a kernel of its own (a workgroup per plane)
-                return stride == 1 ? launch_pad_planes(i.dev, dst, (size_t)batch * Cin, Hin, Win, pad, sg.pitch, stream)
-                                   : launch_conv_stage_input(i.dev, dst, (size_t)batch * Cin, Hin, Win, pad, stride,
-                                                             sg.RH, sg.PW, sg.Hs, sg.Wq, stream);
-            });
+        const size_t HW = (size_t)Hout * Wout;
+        for (int b0 = 0; b0 < batch; b0 += chunk) {
+            const int nb = batch - b0 < chunk ? batch - b0 : chunk;
+            const float* src = i.dev + (size_t)b0 * Cin * Hin * Win;
+            if (sg.copy) {
+                st = timer.family(3, [&] {
+                    // stride 1: the plain zero-padded copy has a kernel of its own (a workgroup per plane)
+                    return stride == 1 ? launch_pad_planes(src, staged, (size_t)nb * Cin, Hin, Win, pad, sg.pitch, stream)
+                                       : launch_conv_stage_input(src, staged, (size_t)nb * Cin, Hin, Win, pad, stride,
+                                                                 sg.RH, sg.PW, sg.Hs, sg.Wq, stream);
+                });
+                if (st) return st;
+            }
+            ConvGeom cv{};
+            cv.in = sg.copy ? staged : src;
+            cv.in_bytes = (unsigned)((double)nb * Cin * sg.Hs * sg.pitch * 4);
+            cv.Cin = Cin; cv.plane_rows = sg.Hs; cv.pitch = sg.pitch; cv.row_step = sg.RH;
+            cv.Hout = Hout; cv.Wout = Wout; cv.row_n = row_n;
+            cv.tap_table = taps;
+            cv.out_nchw = out_nchw ? 1 : 0;
+            // [batch][Cout][HW]: the chunk's images are contiguous; [Cout][batch*HW]: its columns are
+            float* dst = o.dev + (out_nchw ? (size_t)b0 * Cout * HW : (size_t)b0 * HW);
+            const int Np = nb * Hout * row_n;
+            st = run_gemm(w.dev, nullptr, dst, Cout, Np, K, K, Np, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
+                          LOAD_IM2COL_ROW, stream, timer, &cv);
             if (st) return st;
         }
-        const int Np = (int)ncols_p;
-        st = run_gemm(w.dev, nullptr, o.dev, Cout, Np, K, K, Np, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
-                      LOAD_IM2COL_ROW, stream, timer, &cv);
-        if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);
     }
 
-    if (!fits_int(K_d * ncols_d) || K > 65535)
+    if (!fits_int(K_d * ncols_d) || !fits_int(Cout * ncols_d) || !fits_int(in_elems) || K > 65535)
         return fail(CAKE_HIP_ERR_RANGE, "column matrix %gx%g out of range", K_d, ncols_d);
     char* ws = static_cast<char*>(workspace);
     if (!ws) {

@@ -218,8 +218,11 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * read 4 neighbouring floats); an output width that is not a multiple of 4 is
  * computed with rows padded to one and the extra columns dropped.  It runs the
  * two-step path instead when that padding would cost more than the column
- * matrix (narrow maps with many output channels) or the staged input reaches
- * 2 GiB.
+ * matrix (narrow maps with many output channels).  A batch whose staged input
+ * would reach 2 GiB, or whose product 2^31 elements, is run in chunks of whole
+ * images through the same staged buffer, so input and output may be as large
+ * as memory holds; only a single image of 2 GiB takes the two-step path, whose
+ * column matrix is limited to 2^31 elements (CAKE_HIP_ERR_RANGE beyond).
  * cake_hip_conv2d_im2col always runs the two steps the reference runs: im2col
  * into a column matrix, then the GEMM.  Both give the same result.
  * workspace (device, cake_hip_conv2d_workspace bytes: the column matrix of the
