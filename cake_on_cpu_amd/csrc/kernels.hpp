@@ -67,6 +67,7 @@ enum TileId {
     TILE_128x128x32_W64x64,       // 4 waves: mid-size shapes, 2 workgroups per CU
     TILE_64x64x32_W32x32,         // 4 waves: small shapes with several workgroups per CU
     TILE_64x64x64_W32x32,         // 8 waves, two per 32x32 block of C (one per K half): small shapes, one workgroup per CU
+    TILE_96x128x32_W96x32,        // 4 waves side by side, each 96 rows tall: products with 65..96 (or 129..192) rows
     TILE_COUNT
 };
 

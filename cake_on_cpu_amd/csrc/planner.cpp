@@ -27,6 +27,7 @@ double tile_efficiency(int tile_id)
         case TILE_256x128x32_W64x64: return 0.94;
         case TILE_128x256x32_W64x64: return 0.94;
         case TILE_128x128x32_W64x64: return 0.93;
+        case TILE_96x128x32_W96x32: return 0.90;  // 12 MFMAs per 7 operand reads, where the 64x64 wave tile has 16 per 10
         case TILE_64x64x32_W32x32: return 0.85;  // one wave per SIMD per workgroup, 16 MFMAs between barriers
         default: return 0.80;  // 64x64x64 with two waves per block of C: see model_seconds
     }

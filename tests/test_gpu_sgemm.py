@@ -67,7 +67,7 @@ def test_edge_shapes_with_2111(shape):
         _check(A, B, Cm, ref, (shape, sch))
 
 
-TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64)]
+TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64), (96, 128, 32)]
 
 
 @pytest.mark.parametrize("tile", TILES, ids=lambda t: "x".join(map(str, t)))
@@ -86,7 +86,7 @@ def test_every_tile_shape(tile, shape):
 TAIL_CASES = [  # (shape M,K,N; tile) -- tile count = a whole number of rounds plus a thin last one
     ((1100, 520, 1100), (64, 64, 64)), ((1100, 517, 1101), (64, 64, 64)),
     ((2111, 2111, 2111), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
-    ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)),
+    ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)), ((1632, 1024, 2048), (96, 128, 32)),
 ]
 
 
