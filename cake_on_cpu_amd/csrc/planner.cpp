@@ -27,7 +27,8 @@ double tile_efficiency(int tile_id)
         case TILE_256x128x32_W64x64: return 0.94;
         case TILE_128x256x32_W64x64: return 0.94;
         case TILE_128x128x32_W64x64: return 0.93;
-        case TILE_96x128x32_W96x32: return 0.90;  // 12 MFMAs per 7 operand reads, where the 64x64 wave tile has 16 per 10
+        case TILE_96x128x32_W96x32: return 0.86;  // 0.90 on a long K walk (192 x 16384^2); rated lower so that it is taken where it
+                                                  // saves a quarter of padded rows, not for 512 rows as 6 x 96 (measured 68 against 60 us)
         case TILE_64x64x32_W32x32: return 0.85;  // one wave per SIMD per workgroup, 16 MFMAs between barriers
         default: return 0.80;  // 64x64x64 with two waves per block of C: see model_seconds
     }
