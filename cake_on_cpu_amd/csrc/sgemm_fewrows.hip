@@ -60,8 +60,10 @@ __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0
 
 // MG groups of 16 rows of A (M <= 16 MG) against NJ pieces of 64 columns per workgroup: every
 // B value loaded feeds MG MFMAs, so the arithmetic per byte grows with MG.  One and two groups
-// (up to 32 rows) stay bound by memory; four groups (up to 64 rows) are bound by the matrix pipe
-// and were measured no faster than the 64 x 64 macro-tile, so they are not instantiated.
+// (up to 32 rows) stay bound by memory; three (up to 48 rows) need about as long for the matrix
+// work as for the memory and still beat the 64-row macro-tile on large operands (48 x 16384 x
+// 16384: 220 us against 289 us); four groups (up to 64 rows) are bound by the matrix pipe and
+// were measured no faster than the macro-tile, so they are not instantiated.
 template <int MG, int NJ>
 __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
                                                                const float* __restrict__ B,
@@ -89,7 +91,10 @@ __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* _
     // so that the 16 lanes of a row read 256 contiguous bytes per load instruction.
     int a_off[MG];
 #pragma unroll
-    for (int g = 0; g < MG; ++g) a_off[g] = 16 * g + li < M ? ((16 * g + li) * lda + 4 * lq) * 4 : BUF_OOB;
+    // rows at and past M repeat the last row (their results are never written): lanes that ask for
+    // an out-of-range offset instead make every load of A slower (33 x 16384 x 16384: 258 us
+    // against 224 us)
+    for (int g = 0; g < MG; ++g) a_off[g] = (min(16 * g + li, M - 1) * lda + 4 * lq) * 4;
     int b_off[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
@@ -441,9 +446,11 @@ int fewrows_nt_slices(int M, int N, int K, int cus) { return slices_for((N + FR_
 
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
-    // byte offsets inside a group (15 rows of B plus 256 columns, 31 rows of A) must stay below 2^31
-    return M >= 1 && M <= 32 && N >= 512 && K >= 64 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
-           (double)lda * 32 * 4 < 2147483648.0;
+    // byte offsets inside a group (15 rows of B plus 256 columns, 47 rows of A) must stay below 2^31
+    // 33 to 48 rows only against a large B: at 4096 x 4096 the macro-tile is the faster one (23 against 26 us)
+    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && (double)N * K >= 48.0e6));
+    return rows_ok && N >= 512 && K >= 64 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
+           (double)lda * 48 * 4 < 2147483648.0;
 }
 
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
@@ -466,7 +473,8 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
     const int out_ld = used > 1 ? N : ldc;
     const size_t stride = used > 1 ? (size_t)M * N : 0;
     auto kernel = M <= 16 ? (cols == 128 ? sgemm_fewrows_nn_kernel<1, 2> : sgemm_fewrows_nn_kernel<1, 1>)
-                          : (cols == 128 ? sgemm_fewrows_nn_kernel<2, 2> : sgemm_fewrows_nn_kernel<2, 1>);
+                : M <= 32 ? (cols == 128 ? sgemm_fewrows_nn_kernel<2, 2> : sgemm_fewrows_nn_kernel<2, 1>)
+                          : (cols == 128 ? sgemm_fewrows_nn_kernel<3, 2> : sgemm_fewrows_nn_kernel<3, 1>);
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
                        out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();

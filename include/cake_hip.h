@@ -69,6 +69,7 @@ typedef struct cake_hip_cpu_cntx_t {
 /* Kernel families of cake_hip_plan_t.kernel.  Dense row-major operands without a tile override:
  * a product with a single row or column runs on the matrix-vector kernels, one with at most 32
  * rows of A or columns of B (and at least 512 of the other, K >= 64) on the streaming kernels,
+ * as does one with 33 to 48 rows of A against a B of 48 million elements or more,
  * everything else on the macro-tile kernel the other fields describe. */
 enum {
     CAKE_HIP_KERNEL_TILE = 0,
@@ -279,8 +280,8 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
  * table keyed by (M, N, K).  From then on cake_hip_plan / cake_hip_sgemm and the
  * other products use that choice whenever the caller gives no tile override.
  * The planner's own choice is always measured first, so the result is never
- * slower than the default by more than timing noise.  A product with at most 32
- * rows of A or columns of B runs on a streaming kernel instead of a macro-tile:
+ * slower than the default by more than timing noise.  A product with few rows of A
+ * or columns of B (CAKE_HIP_KERNEL_STREAM_*) runs on a streaming kernel instead of a macro-tile:
  * that kernel is then the default that is measured, and the table only gets an
  * entry (which from then on replaces the streaming kernel) when a tile beats it.
  * best_plan, best_seconds, default_seconds may be NULL.

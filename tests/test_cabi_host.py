@@ -279,13 +279,14 @@ def test_tune_table_load_lookup_save_clear(tmp_path):
 
 def test_plan_names_the_kernel_family():
     """Single rows or columns go to the matrix-vector kernels, up to 32 rows or columns against a
-    wide operand to the streaming kernels, the rest (and anything with a tile override) to the
+    wide operand (up to 48 rows against a large one) to the streaming kernels, the rest (and anything with a tile override) to the
     macro-tile kernel."""
     fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
     assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
     assert fam(16, 16384, 16384) == 2 and fam(32, 600, 64) == 2 and fam(2, 512, 100) == 2
     assert fam(16384, 16, 16384) == 3 and fam(512, 32, 64) == 3
-    assert fam(33, 16384, 16384) == 0 and fam(16384, 33, 16384) == 0
+    assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 16384, 16384) == 0
+    assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
