@@ -105,6 +105,7 @@ SIGNATURES = {
     "cake_hip_transpose": (_i, [_fp, _fp, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_forward": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_forward_wt": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),
+    "cake_hip_sgemm_nt": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, C.POINTER(_i), C.c_void_p, _dp]),
     "cake_hip_linear_backward": (_i, [_fp] * 6 + [_i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_autotune": (_i, [_i, _i, _i, C.c_double, C.POINTER(Plan), _dp, _dp]),
     "cake_hip_tune_save": (_i, [C.c_char_p]),

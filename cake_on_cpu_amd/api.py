@@ -328,6 +328,20 @@ def linear_forward(x, w, bias, y, M, N, K, timed=True) -> float:
     return secs.value
 
 
+def sgemm_nt(A, Bt, Cm, M, N, K, accumulate=False, tile=None, timed=True) -> float:
+    """C[M][N] = (C if accumulate else 0) + A[M][K] . Bt[N][K]^T with Bt read as it lies (the
+    product of linear_forward, src/linear.cpp:38, without its transposed copy and bias).
+    tile = (tile_m, tile_n, tile_k, split_k) forces the macro-tile kernel.  Returns seconds."""
+    _need(A, M * K, "A")
+    _need(Bt, N * K, "Bt")
+    _need(Cm, M * N, "C")
+    secs = C.c_double(0.0)
+    ov = (C.c_int * 4)(*tile) if tile is not None else None
+    check(load().cake_hip_sgemm_nt(_ptr(A, "A"), _ptr(Bt, "Bt"), _ptr(Cm, "C"), M, N, K, int(accumulate), ov,
+                                   _stream(A, Bt, Cm), C.byref(secs) if timed else None), "sgemm_nt")
+    return secs.value
+
+
 def linear_forward_wt(x, wt, bias, y, M, N, K, timed=True) -> float:
     """The same with the weights already transposed: wt is [K][N] (transpose_mat of w), for callers
     that keep the transposed copy while the weights stay the same."""

@@ -333,6 +333,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
              const TunedChoice* choice = nullptr)
 {
     const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
+    const bool vec_plan = vec || (a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4_T);  // planned (and tuned) alike
     // Products with a few rows or columns have streaming kernels of their own; a macro-tile is
     // only used for them on request or when the tuner measured one to be faster.
     const bool streaming_ok = vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, true, nullptr);
@@ -365,8 +366,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         });
     }
     GemmPlan plan;
-    int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec, g_ctx.model, &plan)
-                    : plan_gemm(M, N, K, sched, tile_override, vec, g_ctx.model, &plan);
+    int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec_plan, g_ctx.model, &plan)
+                    : plan_gemm(M, N, K, sched, tile_override, vec_plan, g_ctx.model, &plan);
     if (st) return fail(st, "no tile matches the requested override");
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C;
@@ -1186,6 +1187,96 @@ static int linear_gemm(const float* A, const float* B, float* C, int M, int N, i
                     stream, timer, nullptr, col_bias);
 }
 
+// C[M][N] = (accumulate ? C : 0) + X[M][K] . W[N][K]^T (+ bias[N] on every row) on device operands,
+// W read as it lies: a single row of X (or of W) is a row-major matrix-vector product, two rows
+// against a mid-size W the two-vector sweep, up to 32 rows of either the streaming kernel, the
+// rest the macro-tile kernel with 16-byte loads along k on both sides.  Only rows of 2^21 floats
+// and more, beyond that kernel's 32-bit offsets, go through a transposed copy of W.
+// tile_override != nullptr forces the macro-tile kernel.
+static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K, int accumulate,
+                   const int* tile_override, const float* bias, hipStream_t stream, Timer& timer)
+{
+    int st;
+    if (K == 0) {
+        if (accumulate && !bias) return CAKE_HIP_OK;
+        hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, accumulate, stream, nullptr, bias);
+        return e == hipSuccess ? CAKE_HIP_OK : fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
+    }
+    const int cus = g_ctx.model.cus;
+    if ((M == 1 || N == 1) && !tile_override && !(bias && accumulate)) {
+        // y = W . x (one row of X), or C[:, 0] = X . w (one row of W): the matrix is read row-major at
+        // 7.2 TB/s where the streaming kernel reaches 6.4.  A bias goes first and the product is
+        // added to it, which rounds as fl(sum + bias) does.
+        const float* mat = M == 1 ? W : X;
+        const float* vec = M == 1 ? X : W;
+        const int rows = M == 1 ? N : M;
+        const size_t floats = sgemv_rowmajor_scratch_floats(rows, K, cus);
+        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
+        float* scratch = static_cast<float*>(g_ctx.gemv.ptr);
+        if (bias) {   // C[m][n] = bias[n], by a kernel (no copy or memset node for a captured graph)
+            hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream, nullptr, bias);
+            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
+        }
+        return timer.family(2, [&] {
+            return launch_sgemv_rowmajor(mat, vec, C, rows, K, bias ? 1 : accumulate, scratch, cus, stream);
+        });
+    }
+    if (!tile_override && !accumulate && fewrows_nt_applies(M, N, K, K, K, false) &&
+        sgemv_rowmajor_multi_applies(N, K, M, K, W, X, cus)) {
+        // two rows against a mid-size W: one pass of the matrix-vector sweep over W serves both
+        return timer.family(2, [&] { return launch_sgemv_rowmajor_multi(W, X, C, bias, N, K, M, K, N, stream); });
+    }
+    const bool few_x = !tile_override && fewrows_nt_applies(M, N, K, K, K, false);
+    const bool few_w = !tile_override && !few_x && fewrows_nt_applies(N, M, K, K, K, false);
+    if (few_x || few_w) {
+        // a few rows on one side: the other operand is streamed once as it lies
+        const int slices = few_x ? fewrows_nt_slices(M, N, K, cus) : fewrows_nt_slices(N, M, K, cus);
+        float* partial = nullptr;
+        if (slices > 1) {
+            if ((st = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float)))) return st;
+            partial = static_cast<float*>(g_ctx.splitk.ptr);
+        }
+        return timer.family(0, [&] {
+            return few_x ? launch_sgemm_fewrows_nt(X, W, C, partial, M, N, K, K, K, N, false, false, accumulate, bias, cus, stream)
+                         : launch_sgemm_fewrows_nt(W, X, C, partial, N, M, K, K, K, N, false, true, accumulate, bias, cus, stream);
+        });
+    }
+    if ((double)K * 256 * 4 < 2147483648.0)
+        return run_gemm(X, W, C, M, N, K, K, K, N, CAKE_HIP_NA, accumulate, tile_override, LOAD_VEC4, LOAD_VEC4_T,
+                        stream, timer, nullptr, bias);
+    if ((st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
+    float* wt = static_cast<float*>(g_ctx.linear.ptr);
+    st = timer.family(4, [&] { return launch_transpose(W, wt, N, K, stream); });
+    if (st) return st;
+    const int mode = vec4_loadable(X, wt, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
+    return run_gemm(X, wt, C, M, N, K, K, N, N, CAKE_HIP_NA, accumulate, tile_override, mode, mode, stream, timer,
+                    nullptr, bias);
+}
+
+int cake_hip_sgemm_nt(const float* A, const float* Bt, float* C, int M, int N, int K, int accumulate,
+                      const int* tile_override, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    if (M < 0 || N < 0 || K < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (!C || (K > 0 && (!A || !Bt))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
+    int st = ensure_init();
+    if (st) return st;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Operand a, b, c;
+    if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
+    if ((st = stage_in(Bt, (size_t)N * K * 4, 1, true, &b))) return st;
+    if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if ((st = gemm_nt(a.dev, b.dev, c.dev, M, N, K, accumulate, tile_override, nullptr, stream, timer))) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(c, stream);
+}
+
 int cake_hip_linear_forward(const float* x, const float* w, const float* bias, float* y, int M, int N,
                             int K, void* stream_, double* seconds)
 {
@@ -1203,58 +1294,9 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
     if ((st = stage_in(w, (size_t)N * K * 4, 1, true, &wo))) return st;
     if (bias && (st = stage_in(bias, (size_t)N * 4, 2, true, &bo))) return st;
     if ((st = stage_in(y, (size_t)M * N * 4, 3, false, &yo))) return st;
-    // workspace: the weights as a K x N matrix (256-byte aligned so the 16-byte loader applies)
-    const bool small_batch = fewrows_nt_applies(M, N, K, K, K, false);
-    if (!small_batch && M != 1 && (st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
-    float* wt = static_cast<float*>(g_ctx.linear.ptr);
-
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
-    if (M == 1 && K > 0) {
-        // a single sample: y = w . x is a row-major matrix-vector product (7.2 TB/s where the
-        // streaming kernel reaches 6.4); the bias goes first and the product is added to it,
-        // which rounds as fl(sum + bias) does
-        const size_t floats = sgemv_rowmajor_scratch_floats(N, K, g_ctx.model.cus);
-        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
-        float* scratch = static_cast<float*>(g_ctx.gemv.ptr);
-        if (bias) HIP_TRY(hipMemcpyAsync(yo.dev, bo.dev, (size_t)N * 4, hipMemcpyDeviceToDevice, stream));
-        st = timer.family(2, [&] {
-            return launch_sgemv_rowmajor(wo.dev, xo.dev, yo.dev, N, K, bias ? 1 : 0, scratch, g_ctx.model.cus, stream);
-        });
-        if (st) return st;
-        if ((st = timer.stop())) return st;
-        return stage_out(yo, stream);
-    }
-    if (small_batch && sgemv_rowmajor_multi_applies(N, K, M, K, wo.dev, xo.dev, g_ctx.model.cus)) {
-        // two samples on a mid-size layer: one pass of the matrix-vector sweep over w serves both
-        st = timer.family(2, [&] {
-            return launch_sgemv_rowmajor_multi(wo.dev, xo.dev, yo.dev, bias ? bo.dev : nullptr, N, K, M, K, N, stream);
-        });
-        if (st) return st;
-        if ((st = timer.stop())) return st;
-        return stage_out(yo, stream);
-    }
-    if (small_batch) {
-        // a small batch: y = x w^T with w streamed once as it lies, no transposed copy
-        const int slices = fewrows_nt_slices(M, N, K, g_ctx.model.cus);
-        float* partial = nullptr;
-        if (slices > 1) {
-            if ((st = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float)))) return st;
-            partial = static_cast<float*>(g_ctx.splitk.ptr);
-        }
-        st = timer.family(0, [&] {
-            return launch_sgemm_fewrows_nt(xo.dev, wo.dev, yo.dev, partial, M, N, K, K, K, N, false, false, 0,
-                                           bias ? bo.dev : nullptr, g_ctx.model.cus, stream);
-        });
-        if (st) return st;
-        if ((st = timer.stop())) return st;
-        return stage_out(yo, stream);
-    }
-    if (K > 0) {
-        st = timer.family(4, [&] { return launch_transpose(wo.dev, wt, N, K, stream); });
-        if (st) return st;
-    }
-    if ((st = linear_gemm(xo.dev, wt, yo.dev, M, N, K, bias ? bo.dev : nullptr, stream, timer))) return st;
+    if ((st = gemm_nt(xo.dev, wo.dev, yo.dev, M, N, K, 0, nullptr, bias ? bo.dev : nullptr, stream, timer))) return st;
     if ((st = timer.stop())) return st;
     return stage_out(yo, stream);
 }

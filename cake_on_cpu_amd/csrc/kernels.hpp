@@ -80,6 +80,7 @@ const TileInfo& tile_info(int tile_id);
 enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
+    LOAD_VEC4_T = 2, // B only: B handed over as its transpose Bt[N][K] (rows ldb apart), 16-byte loads along k
     LOAD_IM2COL_ROW = 4  // B only: column matrix of a convolution gathered from the staged NCHW input,
                          // one 16-byte load per 4 columns
 };

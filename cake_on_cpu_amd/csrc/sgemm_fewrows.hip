@@ -456,7 +456,13 @@ bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
 {
     // 64 rows of W, and 32 rows (or 32 k) of X, within 2^31 bytes of the block's origin
-    return M >= 1 && M <= 32 && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
+    // X as the few columns of a product (k-major): up to 16 columns win against the 64 x 64
+    // macro-tile at every size, 17 to 32 only from about 50 million elements of W on (8192 x 8192:
+    // 74-78 us against 69 us; 16384 x 16384: 205 against 270 us).  X as the rows of a small batch
+    // (a linear layer, W as it lies): up to 32 rows; a third group of 16 was measured and lost to
+    // the macro-tile kernel that reads W along k (48 x 8192 x 8192: 82 against 72 us).
+    const bool rows_ok = M <= 16 || (M <= 32 && (!x_kmajor || (double)N * K >= 50.0e6));
+    return M >= 1 && rows_ok && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
            (double)ldx * 32 * 4 + (x_kmajor ? 128 : 0) < 2147483648.0;
 }
 

@@ -61,7 +61,9 @@ struct Tile {
     static constexpr int LDA = BK + 4;                 // floats; 16-byte reads of 8 consecutive rows hit 8 distinct bank quads
     static constexpr int LDB = BN + 8;                 // floats; rows k and k+4 land 32 banks apart
     static constexpr int A_STAGE = BM * LDA;
-    static constexpr int B_STAGE = BK * LDB;
+    // B as [k][n] rows of LDB floats, or (B handed over as its transpose, VecLoaderNT) as [n][k]
+    // rows of LDA floats like A: room for either
+    static constexpr int B_STAGE = BK * LDB > BN * LDA ? BK * LDB : BN * LDA;
     static constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE) * 4;
     static constexpr int A_CHUNKS = BM * BK / 4;       // 16-byte chunks per stage
     static constexpr int B_CHUNKS = BK * BN / 4;
@@ -206,6 +208,9 @@ __device__ __forceinline__ void load_b_stage(const GemmArgs& g, int n0, int k0, 
 
 // registers -> LDS stage
 template <class T>
+__device__ __forceinline__ void store_b_chunk_along_k(float* Bs, int W, int tid, const f32x4& v);
+
+template <class T, bool B_ALONG_K = false>
 __device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
                                             const f32x4 (&ra)[T::A_ITERS],
                                             const f32x4 (&rb)[T::B_ITERS])
@@ -217,8 +222,12 @@ __device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
     }
 #pragma unroll
     for (int it = 0; it < T::B_ITERS; ++it) {
-        const int c = tid + it * T::THREADS;
-        *reinterpret_cast<f32x4*>(Bs + (c / (T::BN / 4)) * T::LDB + (c % (T::BN / 4)) * 4) = rb[it];
+        if constexpr (B_ALONG_K) {
+            store_b_chunk_along_k<T>(Bs, it, tid, rb[it]);
+        } else {
+            const int c = tid + it * T::THREADS;
+            *reinterpret_cast<f32x4*>(Bs + (c / (T::BN / 4)) * T::LDB + (c % (T::BN / 4)) * 4) = rb[it];
+        }
     }
 }
 
@@ -235,10 +244,12 @@ struct Frag {
     float b[T::TN][4];
 };
 
-template <class T>
+template <class T, bool B_ALONG_K = false>
 // a_lane / b_lane: where the lane's operands start inside a stage (floats):
 // its row of A (times LDA) and its column of B, plus the wave's K slice of the
 // stage when several waves share a block of C.
+// B_ALONG_K: the B stage is laid out like A ([n][k], rows of LDA floats) and b_lane is the lane's
+// row of it times LDA.
 __device__ __forceinline__ void load_frag(const float* As, const float* Bs, int a_lane, int b_lane,
                                           int lh, int kg, Frag<T>& f)
 {
@@ -247,9 +258,16 @@ __device__ __forceinline__ void load_frag(const float* As, const float* Bs, int 
     for (int tm = 0; tm < T::TM; ++tm)
         f.a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + kk);
 #pragma unroll
-    for (int tn = 0; tn < T::TN; ++tn)
+    for (int tn = 0; tn < T::TN; ++tn) {
+        if constexpr (B_ALONG_K) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(Bs + b_lane + tn * 32 * T::LDA + kk);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) f.b[tn][i] = Bs[(kk + i) * T::LDB + b_lane + tn * 32];
+            for (int i = 0; i < 4; ++i) f.b[tn][i] = v[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) f.b[tn][i] = Bs[(kk + i) * T::LDB + b_lane + tn * 32];
+        }
+    }
 }
 
 template <class T>
@@ -333,6 +351,7 @@ template <class T>
 struct VecLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;  // load instructions per stage
     static constexpr bool MASK_A_STORES = true;
+    static constexpr bool B_ALONG_K = false;     // a chunk of B is 4 consecutive n of one k
     int a_off[T::A_ITERS];  // byte offset from the A tile origin, or BUF_OOB for rows >= M
     int a_k[T::A_ITERS];    // first k of the chunk inside a stage
     int b_off[T::B_ITERS];  // byte offset from the B tile origin per stage, or BUF_OOB for cols >= N
@@ -430,6 +449,104 @@ __device__ __forceinline__ f32x4 a_chunk_below(const f32x4& v, int W, int tid, i
     return r;
 }
 
+// B handed over as its transpose: Bt[n][k], rows ldb apart (the weights of a linear layer as
+// they lie, y = x . w^T).  Both operands are then read like A: a chunk of B is 4 consecutive k
+// of one row n (chunk c: n = c / (BK/4), k = 4 (c % (BK/4))), loaded with one 16-byte load and
+// stored to an [n][k] stage of LDS laid out like A's, from which a lane fetches its four B values
+// of a group with one 16-byte read.  (Stored as scalars into the [k][n] stage the 8 lanes of a row
+// hit 2 banks: measured 5 % slower than the plain kernel at 8192^3 and 40 % at 64 x 16384^2.)
+// Rows at and past N read as zero; a chunk that straddles kend is masked when stored.
+template <class T>
+struct VecLoaderNT {
+    static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
+    static constexpr bool MASK_A_STORES = true;
+    static constexpr bool B_ALONG_K = true;
+    int a_off[T::A_ITERS];
+    int a_k[T::A_ITERS];
+    int b_off[T::B_ITERS];  // byte offset from the B tile origin, or BUF_OOB for rows >= N
+    int b_k[T::B_ITERS];    // first k of the chunk inside a stage
+    const float* a_base;    // A + m0*lda
+    const float* b_base;    // Bt + n0*ldb
+    unsigned a_elems;
+    unsigned b_elems;
+
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int n0, int tid)
+    {
+        a_base = g.A + (size_t)m0 * g.lda;
+        b_base = g.B + (size_t)n0 * g.ldb;
+        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
+        b_elems = clamp_elems((long long)(g.N - 1 - n0) * g.ldb + g.K);
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            a_k[it] = (c % (T::BK / 4)) * 4;
+            a_off[it] = (m0 + r < g.M) ? (r * g.lda + a_k[it]) * 4 : BUF_OOB;
+        }
+#pragma unroll
+        for (int it = 0; it < T::B_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            b_k[it] = (c % (T::BK / 4)) * 4;
+            b_off[it] = (n0 + r < g.N) ? (r * g.ldb + b_k[it]) * 4 : BUF_OOB;
+        }
+    }
+
+    __device__ __forceinline__ void prime(int) {}
+
+    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
+    {
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
+    }
+    __device__ __forceinline__ f32x4 load_b(int k0, int off) const
+    {
+        return buffer_load_f32x4(b_base + k0, off, records_left(b_elems, (unsigned)k0));
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_one_inside(int k0, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = load_a(k0, a_off[OP]);
+        else
+            rb[OP - T::A_ITERS] = load_b(k0, b_off[OP - T::A_ITERS]);
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_one(int k0, int kend, f32x4 (&ra)[T::A_ITERS],
+                                             f32x4 (&rb)[T::B_ITERS]) const
+    {
+        const int left = kend - k0;
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = load_a(k0, a_k[OP] < left ? a_off[OP] : BUF_OOB);
+        else
+            rb[OP - T::A_ITERS] = load_b(k0, b_k[OP - T::A_ITERS] < left ? b_off[OP - T::A_ITERS] : BUF_OOB);
+    }
+
+    __device__ __forceinline__ void load(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        load_all<0>(k0, kend, ra, rb);
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        if constexpr (OP < NUM_LOADS) {
+            load_one<OP>(k0, kend, ra, rb);
+            load_all<OP + 1>(k0, kend, ra, rb);
+        }
+    }
+};
+
+// chunk number W of a B stage whose chunks run along k (VecLoaderNT): the stage is [n][k], rows of
+// LDA floats, exactly like A's
+template <class T>
+__device__ __forceinline__ void store_b_chunk_along_k(float* Bs, int W, int tid, const f32x4& v)
+{
+    const int c = tid + W * T::THREADS;
+    *reinterpret_cast<f32x4*>(Bs + (c / (T::BK / 4)) * T::LDA + (c % (T::BK / 4)) * 4) = v;
+}
+
 __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_offset)
 {
     __amdgpu_buffer_rsrc_t rsrc =
@@ -452,6 +569,7 @@ template <class T>
 struct ConvRowLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
     static constexpr bool MASK_A_STORES = true;   // K need not be a multiple of 4 (see VecLoader)
+    static constexpr bool B_ALONG_K = false;
     int a_off[T::A_ITERS];
     int a_k[T::A_ITERS];
     int b_k[T::B_ITERS];  // k row of the chunk inside a stage
@@ -597,7 +715,7 @@ template <class T, class L>
 struct Slots {
     static constexpr int NKG = T::WAVE_BK / 8;      // operand groups of 8 k a wave walks per stage
     static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
-    static constexpr int FRAG_OPS = T::TM + 4 * T::TN;          // LDS reads that fill one Frag
+    static constexpr int FRAG_OPS = T::TM + (L::B_ALONG_K ? 1 : 4) * T::TN;   // LDS reads that fill one Frag
     static constexpr int LOAD_OPS = L::NUM_LOADS;               // global load instructions per stage
     static constexpr int STORE_OPS = T::A_ITERS + T::B_ITERS;   // 16-byte LDS stores per stage
     static constexpr int STORE_KG = NKG - 1 - T::STORE_LEAD;
@@ -625,6 +743,7 @@ template <class L>
 struct InsideStages {
     static constexpr int NUM_LOADS = L::NUM_LOADS;
     static constexpr bool MASK_A_STORES = false;
+    static constexpr bool B_ALONG_K = L::B_ALONG_K;
     const L& ld;
     template <int OP, class RA, class RB>
     __device__ __forceinline__ void load_one(int k0, int /*kend*/, RA& ra, RB& rb) const
@@ -665,6 +784,11 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
         const int kk = (wrap ? 0 : KG + 1) * 8 + c.lh * 4;
         if constexpr (OP < T::TM) {
             next.a[OP] = *reinterpret_cast<const f32x4*>(A + c.a_lane + OP * 32 * T::LDA + kk);
+        } else if constexpr (L::B_ALONG_K) {
+            constexpr int tn = OP - T::TM;
+            const f32x4 v = *reinterpret_cast<const f32x4*>(B + c.b_lane + tn * 32 * T::LDA + kk);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) next.b[tn][i] = v[i];
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
@@ -680,8 +804,15 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
             if constexpr (L::MASK_A_STORES) v = a_chunk_below<T>(v, W, c.tid, c.k_next - T::BK, c.kend);
             *reinterpret_cast<f32x4*>(c.An + (ch / (T::BK / 4)) * T::LDA + (ch % (T::BK / 4)) * 4) = v;
         } else {
-            const int ch = c.tid + (W - T::A_ITERS) * T::THREADS;
-            *reinterpret_cast<f32x4*>(c.Bn + (ch / (T::BN / 4)) * T::LDB + (ch % (T::BN / 4)) * 4) = c.rb[W - T::A_ITERS];
+            if constexpr (L::B_ALONG_K) {
+                f32x4 v = c.rb[W - T::A_ITERS];
+                // same chunk geometry as A: the k tail is zeroed here
+                if constexpr (L::MASK_A_STORES) v = a_chunk_below<T>(v, W - T::A_ITERS, c.tid, c.k_next - T::BK, c.kend);
+                store_b_chunk_along_k<T>(c.Bn, W - T::A_ITERS, c.tid, v);
+            } else {
+                const int ch = c.tid + (W - T::A_ITERS) * T::THREADS;
+                *reinterpret_cast<f32x4*>(c.Bn + (ch / (T::BN / 4)) * T::LDB + (ch % (T::BN / 4)) * 4) = c.rb[W - T::A_ITERS];
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -750,11 +881,15 @@ __device__ __forceinline__ void k_walk_vec(const GemmArgs& g, float* As, float* 
     if constexpr (L::MASK_A_STORES) {
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) ra[0][it] = a_chunk_below<T>(ra[0][it], it, tid, kbeg, kend);
+        if constexpr (L::B_ALONG_K) {
+#pragma unroll
+            for (int it = 0; it < T::B_ITERS; ++it) rb[0][it] = a_chunk_below<T>(rb[0][it], it, tid, kbeg, kend);
+        }
     }
-    store_stage<T>(As, Bs, tid, ra[0], rb[0]);
+    store_stage<T, L::B_ALONG_K>(As, Bs, tid, ra[0], rb[0]);
     ld.load(kbeg + T::BK, kend, ra[1 % RS], rb[1 % RS]);
     __syncthreads();
-    load_frag<T>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
+    load_frag<T, L::B_ALONG_K>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
 
     // One K step s: stage s is in LDS, stage s+1 waits in registers.  The step
     // stores stage s+1 to the other LDS buffer and fetches stage s+2 -- with two
@@ -852,7 +987,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
     const int wm0 = (wblk / T::WAVES_N) * T::WM;
     const int wn0 = (wblk % T::WAVES_N) * T::WN;
     const int a_lane = (wm0 + l32) * T::LDA + ks * T::WAVE_BK;
-    const int b_lane = wn0 + l32 + ks * T::WAVE_BK * T::LDB;
+    const int b_lane = B_MODE == LOAD_VEC4_T ? (wn0 + l32) * T::LDA + ks * T::WAVE_BK
+                                             : wn0 + l32 + ks * T::WAVE_BK * T::LDB;
 
     const WorkItem w = decode_tile(g, blockIdx.x);
     const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
@@ -871,6 +1007,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
         k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
         k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
+    else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4_T)
+        k_walk_vec<T, VecLoaderNT<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else
         k_walk_generic<T, A_MODE, B_MODE>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
 

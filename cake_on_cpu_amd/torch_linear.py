@@ -20,14 +20,12 @@ def _f32c(t: torch.Tensor, what: str) -> torch.Tensor:
     return t.detach().contiguous()
 
 
-SMALL_BATCH = 32   # up to here the library streams the weights as they lie: no transposed copy is needed
-
-
 def forward(cache_sz, input, weight, bias=None, weight_t=None):
     """output[M][N] = input[M][K] . weight[N][K]^T (+ bias).  `cache_sz` (the
     reference passes the host's L2/L3 sizes, src/linear.cpp:37) is accepted and
     unused: block sizes come from the device.  weight_t: the weights already
-    transposed ([K][N]), from a caller that keeps that copy (see cake_linear)."""
+    transposed ([K][N]), from a caller that holds them that way; the library itself reads
+    `weight` as it lies and needs no such copy."""
     if input.dim() != 2 or weight.dim() != 2 or input.size(1) != weight.size(1):
         raise ValueError(f"linear forward: input {tuple(input.shape)} does not match weight {tuple(weight.shape)}")
     M, K = input.shape
@@ -39,7 +37,7 @@ def forward(cache_sz, input, weight, bias=None, weight_t=None):
     out = torch.empty((M, N), dtype=torch.float32, device=input.device)
     # device tensors: no event timing, so the call only enqueues work on torch's current stream
     timed = not input.is_cuda
-    if weight_t is not None and M > SMALL_BATCH:
+    if weight_t is not None:
         if tuple(weight_t.shape) != (K, N):
             raise ValueError(f"linear forward: weight_t {tuple(weight_t.shape)} is not {(K, N)}")
         api.linear_forward_wt(x, _f32c(weight_t, "weight_t"), b, out, M, N, K, timed=timed)
@@ -92,23 +90,10 @@ class cake_linear(nn.Module):
         else:
             self.register_parameter("bias", None)
 
-    def _transposed_weight(self):
-        """[input_features][output_features] copy of the weights, made again only when they have
-        changed (torch counts in-place updates of a tensor in `_version`) or moved: a layer that is
-        only evaluated transposes its weights once instead of on every call."""
-        w = self.weight
-        key = (w.data_ptr(), w._version, w.device)
-        if getattr(self, "_wt_key", None) != key:
-            wt = torch.empty((self.input_features, self.output_features), dtype=torch.float32, device=w.device)
-            api.transpose_mat(_f32c(w, "weight"), wt, self.output_features, self.input_features)
-            self._wt, self._wt_key = wt, key
-        return self._wt
-
     def forward(self, data):
         lead = data.shape[:-1]
         flat = data.reshape(-1, self.input_features)
-        wt = self._transposed_weight() if flat.size(0) > SMALL_BATCH else None
-        out = cake_linear_function.apply(flat, self.weight, self.bias, wt)
+        out = cake_linear_function.apply(flat, self.weight, self.bias)
         return out.reshape(*lead, self.output_features)
 
     def extra_repr(self):

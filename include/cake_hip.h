@@ -249,18 +249,28 @@ int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* s
 
 /* y[M][N] = x[M][K] . w[N][K]^T (+ bias[N] on every row when bias != NULL).
  * Replaces linear_forward (src/linear.cpp:12-50), which transposes the weights
- * into a K x N matrix, calls cake_sgemm and adds the bias afterwards; here the
- * transpose is a device kernel into a library workspace and the bias is added
- * by the product's epilogue (same rounding: fl(fl(sum) + bias)). */
+ * into a K x N matrix, calls cake_sgemm and adds the bias afterwards.  Here w is
+ * read as it lies: a single sample is a matrix-vector product, up to 32 samples
+ * stream w once, larger batches run on the macro-tile kernel with 16-byte loads
+ * along k for both operands.  (Only rows of 2^21 floats and more still go
+ * through a transposed copy in a library workspace.)  The bias is added to the
+ * finished fp32 product in every case (same rounding: fl(fl(sum) + bias)). */
 int cake_hip_linear_forward(const float* x, const float* w, const float* bias, float* y, int M,
                             int N, int K, void* stream, double* seconds);
+
+/* C[M][N] = (accumulate ? C : 0) + A[M][K] . Bt[N][K]^T: the product above without the bias, for
+ * any caller whose second operand lies transposed (rows of length K).  It has no counterpart in
+ * the reference's API, which can only transpose such an operand first (transpose_mat,
+ * src/linear.cpp:26-36); here Bt is read as it lies by the same kernels as the linear layer.
+ * tile_override as for cake_hip_sgemm (it forces the macro-tile kernel). */
+int cake_hip_sgemm_nt(const float* A, const float* Bt, float* C, int M, int N, int K, int accumulate,
+                      const int* tile_override, void* stream, double* seconds);
 
 /* The same with the weights already transposed: wt is [K][N] (input x output
  * features), y = x . wt (+ bias).  This is the product of linear_forward alone
  * (the cake_sgemm call of src/linear.cpp:38 with its bias loop), for callers
  * whose weights stay the same over many calls and who keep the transposed copy
- * (cake_hip_transpose) instead of paying for it every time; batches of at most
- * 32 do not need it, cake_hip_linear_forward streams w as it lies for them. */
+ * (cake_hip_transpose).  cake_hip_linear_forward needs no such copy. */
 int cake_hip_linear_forward_wt(const float* x, const float* wt, const float* bias, float* y, int M,
                                int N, int K, void* stream, double* seconds);
 

@@ -284,7 +284,8 @@ def test_plan_names_the_kernel_family():
     fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
     assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
     assert fam(16, 16384, 16384) == 2 and fam(32, 600, 64) == 2 and fam(2, 512, 100) == 2
-    assert fam(16384, 16, 16384) == 3 and fam(512, 32, 64) == 3
+    assert fam(16384, 16, 16384) == 3 and fam(512, 16, 64) == 3 and fam(16384, 32, 16384) == 3
+    assert fam(512, 32, 64) == 0 and fam(4096, 17, 4096) == 0   # 17 to 32 columns: only against a large A
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 16384, 16384) == 0
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0

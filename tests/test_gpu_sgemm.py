@@ -171,10 +171,11 @@ def test_few_rows_times_wide_matrix(shape):
 @pytest.mark.parametrize("shape", [(512, 64, 2), (1000, 300, 3), (4096, 1000, 5), (4097, 4096, 8), (2050, 777, 13),
                                    (16384, 2111, 16), (1024, 16384, 16), (600, 100, 1), (515, 65, 9),
                                    (1000, 300, 17), (5000, 4099, 4), (4096, 1000, 24), (2050, 777, 32),
-                                   (513, 65, 31), (1000, 300, 33)],
+                                   (513, 65, 31), (1000, 300, 33), (4096, 1000, 40), (2050, 777, 48), (513, 65, 47),
+                                   (1000, 300, 49)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_tall_matrix_times_few_columns(shape):
-    """Up to 32 columns of B against a tall A: A streamed once along its rows (33 columns take the
+    """Up to 48 columns of B against a tall A: A streamed once along its rows (49 columns take the
     tile kernel), ragged M and K, K slices summed in order, accumulation, run-to-run identical sums."""
     M, K, N = shape
     print(f"sgemm few columns M={M} K={K} N={N}", flush=True)
