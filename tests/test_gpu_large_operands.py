@@ -129,7 +129,7 @@ def test_transpose(big):
 @pytest.mark.parametrize("batch", [1, 2, 16, 40], ids=lambda b: f"batch{b}")
 def test_linear_forward(big, batch):
     """y = x . big^T + b: matrix-vector sweep, its two-vector form, the streaming kernel, and the
-    transposed copy of the weights followed by the macro-tiles."""
+    macro-tiles that read the weights along k."""
     x, b = _filled((batch, R), 907), _filled((R,), 908)
     y = torch.full((batch, R), float("nan"), dtype=torch.float32, device=_dev())
     print(f"linear forward batch={batch} {R}->{R}", flush=True)
