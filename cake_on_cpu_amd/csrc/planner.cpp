@@ -62,8 +62,14 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     // The K-split 64x64 tile pays off when the grid leaves a CU with a single workgroup: its two
     // waves per SIMD hide each other's latencies.  With more workgroups than that the plain
     // 64x64 tile does the same with half the LDS, so four of them share a CU.
-    // (measured, 512 x 25088 x 256, 3136 workgroups: 70 us against 59 us), so there it is kept out of the way.
-    if (tile_id == TILE_64x64x64_W32x32) eff = wgs <= dev.cus ? 0.88 : 0.75;
+    // (measured, 512 x 25088 x 256, 3136 workgroups: 70 us against 59 us), so there it is kept out of the way --
+    // unless the K walk is long enough to carry the final sum of the K halves through LDS (32 steps
+    // and more; measured 512 x 11008 x 4096: 336 us against 364 us, 512 x 14336 x 4096: 432 against 443).
+    if (tile_id == TILE_64x64x64_W32x32) eff = wgs <= dev.cus ? 0.88 : (ksteps >= 32 ? 0.87 : 0.75);
+    // The 96 x 128 tile with two workgroups on every CU and a long K walk does as well as the
+    // 128 x 128 tile (3000^3: 386 us, where 256 x 128 with its thin last round takes 417 us;
+    // 4352 x 4096 x 1024: 270 against 290 us).
+    if (tile_id == TILE_96x128x32_W96x32 && wgs >= 2 * dev.cus && ksteps >= 32) eff = 0.93;
     const double cu_rate = dev.mfma_flops / dev.cus * eff;
     double rounds = (double)((wgs + dev.cus - 1) / dev.cus);
     bool tail = false;
