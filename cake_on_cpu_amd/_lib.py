@@ -16,7 +16,8 @@ CXX_LIB_PATH = LIB_DIR / "libcake.so"
 KMN, MKN, NKM, NA = 0, 1, 2, 3
 SCHED_NAMES = {KMN: "KMN", MKN: "MKN", NKM: "NKM", NA: "NA"}
 # Plan.kernel: which kernel family cake_hip_sgemm runs for a shape
-KERNEL_NAMES = {0: "macro-tile", 1: "matrix-vector", 2: "streaming, few rows", 3: "streaming, few columns"}
+KERNEL_NAMES = {0: "macro-tile", 1: "matrix-vector", 2: "streaming, few rows", 3: "streaming, few columns",
+                4: "short K, tiles walked by resident workgroups"}
 
 OK, ERR_ARG, ERR_NO_DEVICE, ERR_HIP, ERR_ALLOC, ERR_RANGE, ERR_ARCH = range(7)
 

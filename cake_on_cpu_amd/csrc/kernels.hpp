@@ -88,6 +88,10 @@ enum LoadMode {
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
                         hipStream_t stream);
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
+// Products with K <= 64 and many 64 x 64 tiles: workgroups that walk over tiles with the next
+// tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
+bool shortk_applies(int M, int N, int K, int cus);
+hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
                                 int accumulate, hipStream_t stream, const ConvGeom* conv = nullptr,

@@ -1,0 +1,138 @@
+// Products with a short K (at most 64) and many tiles of C: the macro-tile kernel spends a
+// workgroup per tile, and with two k steps per tile the load latency of every tile sits in front
+// of its few MFMAs (measured 256 x 100352 x 64: 37 us for loads and arithmetic where the matrix
+// work alone takes 21 us, plus 6 us of stores).  Here a workgroup stays and walks over tiles: the
+// whole K of a tile is one stage of LDS, and the operands of the NEXT tile are already on their
+// way into registers while the current tile is multiplied and written out (256 x 100352 x 64:
+// 48 -> 40 us; 16384 x 16384 x 16: 308 -> 263 us).  Loaders, LDS layout, operand reads and the
+// epilogue are the macro-tile kernel's.
+// Measured and left out: the same with K up to 128 in one stage (71 KB of LDS, two workgroups per
+// CU: 85 us against 73 us at 256 x 100352 x 128), and an epilogue that stores 4 bytes per lane
+// straight from the accumulators instead of 16 through LDS (43 against 40 us).
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+// 64 x 64 tiles of C, 4 waves of 32 x 32; BK is the longest K it takes
+using TileShortK64 = Tile<64, 64, 64, 32, 32>;
+
+template <class T>
+static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE) * 4; }  // one stage
+
+// PLAIN: C is overwritten and there is no bias, so the epilogue loads nothing and the next
+// tile's operands stay in flight across it
+template <class T, int B_MODE, bool PLAIN>
+__global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs g)
+{
+    static_assert(B_MODE == LOAD_VEC4, "row-major operands");
+    using L = VecLoader<T>;
+    static_assert(T::KSPLIT == 1, "one wave per block of C");
+    extern __shared__ __align__(16) float smem[];
+    float* As = smem;
+    float* Bs = smem + T::A_STAGE;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm0 = (wave / T::WAVES_N) * T::WM;
+    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    const int a_lane = (wm0 + l32) * T::LDA;
+    const int b_lane = wn0 + l32;
+
+    const int tiles = g.tiles_m * g.tiles_n;
+    const int groups = (g.K + 7) >> 3;        // operand groups of 8 k that hold anything
+    int t = blockIdx.x;                       // the grid is at most `tiles` workgroups
+    int tile_m, tile_n;
+    raster_tile(g, t, tile_m, tile_n);
+    int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+
+    L ld;
+    f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
+    ld.init(g, m0, n0, tid);
+    ld.prime(0);
+    ld.load(0, g.K, ra, rb);
+    for (;;) {
+        // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = a_chunk_below<T>(ra[it], it, tid, 0, g.K);
+        __syncthreads();   // every wave is done with the staging reads of the previous tile's epilogue
+        store_stage<T>(As, Bs, tid, ra, rb);
+        __syncthreads();
+
+        // the next tile's operands start their way into the registers just emptied
+        const int t_next = t + gridDim.x;
+        const bool more = t_next < tiles;   // the same for every thread of the workgroup
+        int m0_next = 0, n0_next = 0;
+        if (more) {
+            raster_tile(g, t_next, tile_m, tile_n);
+            m0_next = tile_m * T::BM;
+            n0_next = tile_n * T::BN;
+            ld.init(g, m0_next, n0_next, tid);
+            ld.prime(0);
+            ld.load(0, g.K, ra, rb);
+        }
+
+        f32x16 acc[T::TM][T::TN];
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
+        Frag<T> frag[2];
+        load_frag<T>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
+#pragma unroll
+        for (int kg = 0; kg < T::BK / 8; ++kg) {
+            if (kg < groups) {   // uniform: K is the same for everyone
+                if (kg + 1 < T::BK / 8) load_frag<T>(As, Bs, a_lane, b_lane, lh, kg + 1, frag[(kg + 1) & 1]);
+                mma_frag<T>(frag[kg & 1], acc);
+            }
+        }
+        store_c_tile<T, B_MODE, PLAIN>(g, smem, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
+        if (!more) break;
+        t = t_next;
+        m0 = m0_next;
+        n0 = n0_next;
+    }
+}
+
+template <class T, int B_MODE, bool PLAIN>
+static hipError_t launch_shortk_as(const GemmArgs& args, int grid, hipStream_t stream)
+{
+    auto kern = sgemm_shortk_kernel<T, B_MODE, PLAIN>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       shortk_lds_bytes<T>());
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::THREADS), shortk_lds_bytes<T>(), stream, args);
+    return hipGetLastError();
+}
+
+template <class T, int B_MODE>
+static hipError_t launch_shortk(const GemmArgs& args, int grid, hipStream_t stream)
+{
+    return !args.accumulate && !args.col_bias ? launch_shortk_as<T, B_MODE, true>(args, grid, stream)
+                                              : launch_shortk_as<T, B_MODE, false>(args, grid, stream);
+}
+
+// K at most 64, 16-byte-loadable row-major operands, no K slices, and
+// enough 64 x 64 tiles that every workgroup of a full grid walks over several of them
+bool shortk_applies(int M, int N, int K, int cus)
+{
+    if (K < 1 || K > 64) return false;
+    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    return tiles >= 12L * cus;
+}
+
+// args: tiles_m, tiles_n, group, group_along_n set for 64 x 64 tiles; split_k = 1, no tail tiles
+hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream)
+{
+    const long tiles = (long)args.tiles_m * args.tiles_n;
+    if (tiles <= 0) return hipSuccess;
+    if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
+    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 36 KB per workgroup
+    const int grid = (int)(tiles < slots ? tiles : slots);
+    return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
+}
+
+}  // namespace cake

@@ -971,6 +971,80 @@ __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, flo
     }
 }
 
+// Epilogue of one macro-tile: the accumulators of every wave go to C (or to the tile's split-K
+// slice), through the stage memory, which nobody may be reading any more after the barrier at
+// the start.  PLAIN: the caller knows that C is overwritten and no bias is added, so the epilogue
+// holds no load at all (a load here would make a kernel that has other loads in flight wait for
+// all of them: the counter of outstanding loads is served in order).
+template <class T, int B_MODE, bool PLAIN = false>
+__device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, const f32x16 (&acc)[T::TM][T::TN],
+                                             int m0, int n0, int slice, int wblk, int wm0, int wn0, int lane,
+                                             int l32, int lh)
+{
+    float* out = g.partial ? g.partial + (size_t)slice * g.M * g.N : g.C;
+    const int ldo = g.partial ? g.N : g.ldc;
+    const bool add = !PLAIN && (g.partial == nullptr) && g.accumulate;
+    const float* bias = !PLAIN && g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
+    // a convolution's columns n = (image, output row, column of a row padded to 4) go to
+    // [M][batch*Hout*Wout] or NCHW: see conv_out_map
+    const bool conv_out = B_MODE == LOAD_IM2COL_ROW && g.partial == nullptr;
+    // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
+    // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
+    // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
+    // quarter of the store instructions, and rows written in runs of WN floats.
+    constexpr int PITCH = T::WN + 4;            // floats between rows of the wave's staging block
+    constexpr int CH = T::WN / 4;               // 16-byte pieces per row
+    constexpr int ROWS = 64 / CH;               // rows one wave-wide 16-byte read covers
+    static_assert(T::WAVES_M * T::WAVES_N * 32 * PITCH * 4 <= T::LDS_BYTES, "staging blocks fit the stage memory");
+    __syncthreads();  // nobody reads operand stages any more
+    float* wbuf = smem + wblk * (32 * PITCH);
+    const int rd_row = lane / CH, rd_col = (lane % CH) * 4;
+    const int col = n0 + wn0 + rd_col;          // first of the lane's 4 columns
+    size_t col_off = col;
+    size_t row_stride = ldo;
+    int valid = min(4, g.N - col);              // how many of the 4 columns exist (<= 0: none)
+    if (conv_out && valid > 0) valid = conv_out_map(g.conv, g.M, g.ldc, col, valid, col_off, row_stride);
+    f32x4 bias_v = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e < valid) bias_v[e] = bias[col + e];
+    }
+    const bool whole = valid == 4;
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm) {
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                wbuf[(8 * (r >> 2) + 4 * lh + (r & 3)) * PITCH + tn * 32 + l32] = acc[tm][tn][r];
+        // LDS serves a wave's requests in order, so the reads below see the writes above
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS; ++pass) {
+            const int lr = pass * ROWS + rd_row;
+            const int row = m0 + wm0 + tm * 32 + lr;
+            f32x4 v = *reinterpret_cast<const f32x4*>(wbuf + lr * PITCH + rd_col);
+            if (row < g.M && valid > 0) {
+                float* dst = out + (size_t)row * row_stride + col_off;
+                if (whole) {
+                    f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst);
+                    if (add) v += *d4;
+                    if (bias) v += bias_v;
+                    *d4 = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (e < valid) {
+                            float x = add ? dst[e] + v[e] : v[e];
+                            if (bias) x += bias_v[e];
+                            dst[e] = x;
+                        }
+                }
+            }
+        }
+    }
+}
+
 template <class T, int A_MODE, int B_MODE>
 __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g)
 {
@@ -1051,68 +1125,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
                     out[(wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3)) * T::BN + wn0 + tn * 32 + l32] = acc[tm][tn][r];
         return;
     }
-    float* out = g.partial ? g.partial + (size_t)w.slice * g.M * g.N : g.C;
-    const int ldo = g.partial ? g.N : g.ldc;
-    const bool add = (g.partial == nullptr) && g.accumulate;
-    const float* bias = g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
-    // a convolution's columns n = (image, output row, column of a row padded to 4) go to
-    // [M][batch*Hout*Wout] or NCHW: see conv_out_map
-    const bool conv_out = B_MODE == LOAD_IM2COL_ROW && g.partial == nullptr;
-    // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
-    // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
-    // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
-    // quarter of the store instructions, and rows written in runs of WN floats.
-    constexpr int PITCH = T::WN + 4;            // floats between rows of the wave's staging block
-    constexpr int CH = T::WN / 4;               // 16-byte pieces per row
-    constexpr int ROWS = 64 / CH;               // rows one wave-wide 16-byte read covers
-    static_assert(T::WAVES_M * T::WAVES_N * 32 * PITCH * 4 <= T::LDS_BYTES, "staging blocks fit the stage memory");
-    __syncthreads();  // nobody reads operand stages any more
-    float* wbuf = smem + wblk * (32 * PITCH);
-    const int rd_row = lane / CH, rd_col = (lane % CH) * 4;
-    const int col = n0 + wn0 + rd_col;          // first of the lane's 4 columns
-    size_t col_off = col;
-    size_t row_stride = ldo;
-    int valid = min(4, g.N - col);              // how many of the 4 columns exist (<= 0: none)
-    if (conv_out && valid > 0) valid = conv_out_map(g.conv, g.M, g.ldc, col, valid, col_off, row_stride);
-    f32x4 bias_v = {0.f, 0.f, 0.f, 0.f};
-    if (bias) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (e < valid) bias_v[e] = bias[col + e];
-    }
-    const bool whole = valid == 4;
-#pragma unroll
-    for (int tm = 0; tm < T::TM; ++tm) {
-#pragma unroll
-        for (int tn = 0; tn < T::TN; ++tn)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                wbuf[(8 * (r >> 2) + 4 * lh + (r & 3)) * PITCH + tn * 32 + l32] = acc[tm][tn][r];
-        // LDS serves a wave's requests in order, so the reads below see the writes above
-#pragma unroll
-        for (int pass = 0; pass < 32 / ROWS; ++pass) {
-            const int lr = pass * ROWS + rd_row;
-            const int row = m0 + wm0 + tm * 32 + lr;
-            f32x4 v = *reinterpret_cast<const f32x4*>(wbuf + lr * PITCH + rd_col);
-            if (row < g.M && valid > 0) {
-                float* dst = out + (size_t)row * row_stride + col_off;
-                if (whole) {
-                    f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst);
-                    if (add) v += *d4;
-                    if (bias) v += bias_v;
-                    *d4 = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (e < valid) {
-                            float x = add ? dst[e] + v[e] : v[e];
-                            if (bias) x += bias_v[e];
-                            dst[e] = x;
-                        }
-                }
-            }
-        }
-    }
+    store_c_tile<T, B_MODE>(g, smem, acc, m0, n0, w.slice, wblk, wm0, wn0, lane, l32, lh);
 }
 
 // C tile = (accumulate ? C : 0) + sum over the K slices of a tail tile, in

@@ -70,12 +70,14 @@ typedef struct cake_hip_cpu_cntx_t {
  * a product with a single row or column runs on the matrix-vector kernels, one with at most 32
  * rows of A or columns of B (and at least 512 of the other, K >= 64) on the streaming kernels,
  * as does one with 33 to 48 rows of A against a B of 48 million elements or more,
+ * one with K <= 64 and at least 12 tiles of 64 x 64 per CU on workgroups that walk over tiles,
  * everything else on the macro-tile kernel the other fields describe. */
 enum {
     CAKE_HIP_KERNEL_TILE = 0,
     CAKE_HIP_KERNEL_GEMV = 1,
     CAKE_HIP_KERNEL_STREAM_ROWS = 2, /* few rows of A: B streamed once    */
-    CAKE_HIP_KERNEL_STREAM_COLS = 3  /* few columns of B: A streamed once */
+    CAKE_HIP_KERNEL_STREAM_COLS = 3, /* few columns of B: A streamed once */
+    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K, many tiles: 64 x 64 tiles, next tile's operands in flight */
 };
 
 /* What the GPU planner decided for one GEMM: the successor of

@@ -290,5 +290,6 @@ def test_plan_names_the_kernel_family():
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
+    assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(2048, 2048, 64) == 0   # short K, 12 tiles per CU
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"

@@ -187,6 +187,25 @@ def test_tall_matrix_times_few_columns(shape):
     assert np.array_equal(_run(M, K, N)[2], Cm)
 
 
+@pytest.mark.parametrize("shape", [(4096, 64, 4096), (3000, 33, 5000), (4100, 63, 3300), (5000, 1, 4000), (2000, 7, 9000),
+                                   (256, 64, 100352), (9000, 4, 2111), (3584, 64, 3520), (3584, 65, 3520)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_short_k_many_tiles(shape):
+    """K of at most 64 under 12 or more 64 x 64 tiles per CU: workgroups that walk over tiles with
+    the next tile's operands in flight (K = 65 and fewer tiles stay on the macro-tile kernel),
+    ragged M, N and K, overwriting and accumulating, run-to-run identical."""
+    M, K, N = shape
+    want = 4 if K <= 64 and ((M + 63) // 64) * ((N + 63) // 64) >= 12 * cake.device_info().cus else 0
+    assert cake.plan(M, N, K).kernel == want
+    print(f"sgemm short K M={M} K={K} N={N}", flush=True)
+    A, B, Cm = _run(M, K, N)
+    _check(A, B, Cm, None, shape)
+    C0 = oracle.uniform((M, N), 3)
+    _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
+    assert np.allclose(acc - Cm, C0, atol=2e-4)
+    assert np.array_equal(_run(M, K, N)[2], Cm)
+
+
 def test_random_shapes_against_fp64():
     """Seeded random shapes drawn around every dispatch boundary (a single row or column, up to 16
     and just past 16 rows or columns, below and above the 512 columns and 64 k where the streaming
