@@ -366,9 +366,9 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         });
     }
     // A short K under many tiles of C: workgroups that walk over tiles, the next tile's operands in flight
-    // (plain operands only: a convolution's gather needs its tap offsets before it can issue the
-    // next tile's loads, and waiting for those in front of every tile cost more than it saved --
-    // 1 x 1, 64 -> 256 channels on 56 x 56: 57 us against 50 us)
+    // (plain operands only: with a convolution's gathered B the integer divisions that place a
+    // tile's columns in the image, paid per tile instead of once per workgroup, cost more than
+    // the overlap gives -- 1 x 1, 64 -> 256 channels on 56 x 56: 56 us against 50 us)
     if (vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, vec_plan, nullptr) &&
         shortk_applies(M, N, K, g_ctx.model.cus)) {
         GemmArgs g{};

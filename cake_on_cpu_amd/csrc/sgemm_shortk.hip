@@ -39,9 +39,16 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     const int a_lane = (wm0 + l32) * T::LDA;
     const int b_lane = wn0 + l32;
 
-    const int tiles = g.tiles_m * g.tiles_n;
     const int groups = (g.K + 7) >> 3;        // operand groups of 8 k that hold anything
-    int t = blockIdx.x;                       // the grid is at most `tiles` workgroups
+    // Hardware deals workgroup ids round-robin to the 8 XCDs.  Each XCD takes one contiguous
+    // eighth of the tile sequence, and its workgroups walk through it side by side, so that the
+    // tiles in flight on an XCD at any moment are neighbours and share their panels in its L2.
+    const int tiles_all = g.tiles_m * g.tiles_n;
+    const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;   // the grid is a multiple of 8
+    const int first = xcd * (tiles_all >> 3) + min(xcd, tiles_all & 7);
+    const int tiles = first + (tiles_all >> 3) + (xcd < (tiles_all & 7) ? 1 : 0);   // end of this XCD's run
+    int t = first + (blockIdx.x >> 3);
+    if (t >= tiles) return;                   // before any barrier: the whole workgroup leaves
     int tile_m, tile_n;
     raster_tile(g, t, tile_m, tile_n);
     int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
@@ -49,8 +56,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     L ld;
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
     ld.init(g, m0, n0, tid);
-    ld.prime(0);
-    ld.load(0, g.K, ra, rb);
+    ld.load_first_stage(g.K, ra, rb);
     for (;;) {
         // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
 #pragma unroll
@@ -60,7 +66,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
         __syncthreads();
 
         // the next tile's operands start their way into the registers just emptied
-        const int t_next = t + gridDim.x;
+        const int t_next = t + stride;
         const bool more = t_next < tiles;   // the same for every thread of the workgroup
         int m0_next = 0, n0_next = 0;
         if (more) {
@@ -68,8 +74,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
             m0_next = tile_m * T::BM;
             n0_next = tile_n * T::BN;
             ld.init(g, m0_next, n0_next, tid);
-            ld.prime(0);
-            ld.load(0, g.K, ra, rb);
+            ld.load_first_stage(g.K, ra, rb);
         }
 
         f32x16 acc[T::TM][T::TN];
@@ -131,7 +136,7 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream
     if (tiles <= 0) return hipSuccess;
     if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     const long slots = (long)cus * 4;   // what the LDS of a CU holds: 36 KB per workgroup
-    const int grid = (int)(tiles < slots ? tiles : slots);
+    const int grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
     return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
 }
 

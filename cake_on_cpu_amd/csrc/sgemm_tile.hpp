@@ -425,6 +425,11 @@ struct VecLoader {
     {
         load_all<0>(k0, kend, ra, rb);
     }
+    // the stage that starts at k = 0, for a kernel whose every stage does (sgemm_shortk.hip)
+    __device__ __forceinline__ void load_first_stage(int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        load_all<0>(0, kend, ra, rb);
+    }
 
     template <int OP>
     __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
@@ -661,7 +666,6 @@ struct ConvRowLoader {
     {
         load_all<0>(k0, kend, ra, rb);
     }
-
     template <int OP>
     __device__ __forceinline__ void load_all(int k0, int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
