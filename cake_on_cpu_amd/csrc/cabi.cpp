@@ -1061,6 +1061,31 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const bool implicit = !explicit_cols && (double)(row_n - Wout) / Wout * Cout < 60.0 && chunk_fits(chunk) &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
+    // A 1 x 1 convolution at stride 1 without padding is one plain product per image on the input
+    // as it lies, out[b] (Cout x HW) = weights (Cout x Cin) . in[b] (Cin x HW): with few input
+    // channels and many tiles the images are walked as a batch by the short-K kernel
+    // (64 -> 256 channels on 32 x 56 x 56: 50 -> 43 us).
+    const int HW = Hout * Wout;
+    if (!explicit_cols && Hf == 1 && Wf == 1 && stride == 1 && pad == 0 &&
+        shortk_applies(Cout, HW, K, g_ctx.model.cus, batch) && vec4_loadable(w.dev, i.dev, K, HW)) {
+        GemmArgs g{};
+        g.A = w.dev; g.B = i.dev; g.C = o.dev;
+        g.M = Cout; g.N = HW; g.K = K;
+        g.lda = K; g.ldb = HW;
+        g.ldc = out_nchw ? HW : N;                             // [batch][Cout][HW] or [Cout][batch*HW]
+        g.b_batch_stride = (size_t)Cin * HW;
+        g.c_batch_stride = out_nchw ? (size_t)Cout * HW : (size_t)HW;
+        g.tiles_m = (Cout + 63) / 64;
+        g.tiles_n_per_image = (HW + 63) / 64;
+        g.tiles_n = g.tiles_n_per_image * batch;
+        g.split_k = 1; g.k_per_split = K;
+        g.group = g.tiles_m; g.group_along_n = 0;
+        if ((st = timer.start())) return st;
+        st = timer.family(0, [&] { return launch_sgemm_shortk(g, g_ctx.model.cus, stream); });
+        if (st) return st;
+        if ((st = timer.stop())) return st;
+        return stage_out(o, stream);
+    }
     if (implicit) {
         float* staged = nullptr;
         if (sg.copy) {

@@ -57,6 +57,11 @@ struct GemmArgs {
     int tail_tiles, tail_split, tail_k_per_split;
     float* tail_partial;
     ConvGeom conv;             // used by the implicit-im2col loader only
+    // A batch of products with one A (sgemm_shortk.hip only): image b reads B + b * b_batch_stride
+    // as a K x N matrix and writes C + b * c_batch_stride; tiles_n then counts the column tiles of
+    // all images, tiles_n_per_image of them per image.  0 = a single product.
+    int tiles_n_per_image;
+    size_t b_batch_stride, c_batch_stride;
 };
 
 // Macro-tile shapes the planner can choose from.
@@ -90,7 +95,7 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
 // Products with K <= 64 and many 64 x 64 tiles: workgroups that walk over tiles with the next
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
-bool shortk_applies(int M, int N, int K, int cus);
+bool shortk_applies(int M, int N, int K, int cus, int batch = 1);
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,

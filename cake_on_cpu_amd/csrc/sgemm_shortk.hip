@@ -49,13 +49,26 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     const int tiles = first + (tiles_all >> 3) + (xcd < (tiles_all & 7) ? 1 : 0);   // end of this XCD's run
     int t = first + (blockIdx.x >> 3);
     if (t >= tiles) return;                   // before any barrier: the whole workgroup leaves
-    int tile_m, tile_n;
-    raster_tile(g, t, tile_m, tile_n);
-    int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+    // tile number -> origin of the tile and, for a batch of products, the image's B and C
+    GemmArgs gt = g, gt_next = g;
+    auto place = [&](int tile, GemmArgs& ga, int& m0_, int& n0_) {
+        int tile_m, tile_n;
+        raster_tile(g, tile, tile_m, tile_n);
+        if (g.tiles_n_per_image) {
+            const int b = tile_n / g.tiles_n_per_image;
+            tile_n -= b * g.tiles_n_per_image;
+            ga.B = g.B + (size_t)b * g.b_batch_stride;
+            ga.C = g.C + (size_t)b * g.c_batch_stride;
+        }
+        m0_ = tile_m * T::BM;
+        n0_ = tile_n * T::BN;
+    };
+    int m0, n0;
+    place(t, gt, m0, n0);
 
     L ld;
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
-    ld.init(g, m0, n0, tid);
+    ld.init(gt, m0, n0, tid);
     ld.load_first_stage(g.K, ra, rb);
     for (;;) {
         // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
@@ -70,10 +83,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
         const bool more = t_next < tiles;   // the same for every thread of the workgroup
         int m0_next = 0, n0_next = 0;
         if (more) {
-            raster_tile(g, t_next, tile_m, tile_n);
-            m0_next = tile_m * T::BM;
-            n0_next = tile_n * T::BN;
-            ld.init(g, m0_next, n0_next, tid);
+            place(t_next, gt_next, m0_next, n0_next);
+            ld.init(gt_next, m0_next, n0_next, tid);
             ld.load_first_stage(g.K, ra, rb);
         }
 
@@ -93,11 +104,13 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
                 mma_frag<T>(frag[kg & 1], acc);
             }
         }
-        store_c_tile<T, B_MODE, PLAIN>(g, smem, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
+        store_c_tile<T, B_MODE, PLAIN>(gt, smem, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
         if (!more) break;
         t = t_next;
         m0 = m0_next;
         n0 = n0_next;
+        gt.B = gt_next.B;
+        gt.C = gt_next.C;
     }
 }
 
@@ -122,10 +135,10 @@ static hipError_t launch_shortk(const GemmArgs& args, int grid, hipStream_t stre
 
 // K at most 64, 16-byte-loadable row-major operands, no K slices, and
 // enough 64 x 64 tiles that every workgroup of a full grid walks over several of them
-bool shortk_applies(int M, int N, int K, int cus)
+bool shortk_applies(int M, int N, int K, int cus, int batch)
 {
     if (K < 1 || K > 64) return false;
-    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64) * batch;
     return tiles >= 12L * cus;
 }
 

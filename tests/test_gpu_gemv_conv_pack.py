@@ -211,6 +211,31 @@ def test_conv2d_matches_oracle(geom, nchw, explicit):
     assert np.max(np.abs(got - cpu) / np.maximum(S, 1e-30)) <= TOL
 
 
+@pytest.mark.parametrize("geom", [(16, 16, 56, 56, 256, 1, 1), (70, 7, 30, 30, 130, 1, 1), (256, 5, 21, 21, 100, 1, 1),
+                                  (16, 64, 56, 56, 256, 1, 1), (16, 65, 56, 56, 256, 1, 1)], ids=str)
+@pytest.mark.parametrize("nchw", [False, True])
+def test_conv2d_1x1_many_images(geom, nchw):
+    """1 x 1 filters at stride 1 without padding, few input channels and many tiles: every image is
+    a plain product on the input as it lies, and the images are walked as a batch by the short-K
+    kernel (65 channels stay on the gather path) -- HW a multiple of 64, of 4 only, and odd."""
+    Bn, Cin, Hin, Win, Cout, Hf, Wf = geom
+    print(f"conv2d 1x1 geom={geom} nchw={nchw}", flush=True)
+    inp = oracle.uniform((Bn, Cin, Hin, Win), 58)
+    wt = oracle.uniform((Cout, Cin, 1, 1), 59)
+    HW = Hin * Win
+    w64 = wt.reshape(Cout, Cin).astype(np.float64)
+    x64 = inp.reshape(Bn, Cin, HW).astype(np.float64)
+    ref64 = np.einsum("ok,bkp->bop", w64, x64)
+    S = np.einsum("ok,bkp->bop", np.abs(w64), np.abs(x64))
+    out = np.full((Bn, Cout, HW) if nchw else (Cout, Bn * HW), np.nan, np.float32)
+    cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, 1, 1, 1, 0, out_nchw=nchw)
+    got = out if nchw else out.reshape(Cout, Bn, HW).transpose(1, 0, 2)
+    assert np.max(np.abs(got - ref64) / np.maximum(S, 1e-30)) <= TIGHT
+    two_step = np.full_like(out, np.nan)
+    cake.conv2d(inp, wt, two_step, Bn, Cin, Hin, Win, Cout, 1, 1, 1, 0, out_nchw=nchw, explicit_im2col=True)
+    assert np.max(np.abs(two_step - out) / np.maximum(S.max(), 1e-30)) <= TIGHT
+
+
 def test_conv2d_paths_agree_bitwise_layouts():
     """Same sums in the same order whichever way the columns reach the GEMM."""
     Bn, Cin, Hin, Win, Cout = 2, 32, 20, 20, 48
