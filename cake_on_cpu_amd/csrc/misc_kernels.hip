@@ -198,44 +198,78 @@ hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch
 
 // ---------------------------------------------------------------------------
 // im2col: im_2_col of examples/cake_conv.cpp:1178-1213 with batch, padding and
-// stride.  grid.y = row k of the column matrix (one (c, h, w) filter tap),
-// threads run along n = (b, ho, wo).
+// stride.  grid.y = input channel c; threads run along n = (b, ho, wo), and every
+// thread writes its 4 consecutive n (16 bytes at any 4-byte alignment) into all
+// Hf * Wf rows k = (c, h, w) of that channel: the position arithmetic is done once
+// for them, and a thread has a filter row's worth of loads and stores in flight.
+// (With a thread per 16 bytes of output, one store each, the kernel wrote 2.9 TB/s
+// where this memory takes 5.5 to 6.5 TB/s from threads that write several pieces.)
+// The 4 elements may run over the end of an output row or image, so their positions
+// are carried from element to element.  ncols < 2^31.
+// WF: the filter width when it is one of the instantiated ones (the loop over a
+// filter row is then unrolled), 0 = any.
 // ---------------------------------------------------------------------------
-// Each thread writes 4 consecutive n (16 bytes at any 4-byte alignment); they may run over the end
-// of an output row or image, so the position is carried from element to element.  ncols < 2^31.
+template <int WF>
 __global__ void __launch_bounds__(256) im2col_kernel(const float* __restrict__ in,
                                                      float* __restrict__ cols, unsigned ncols, int Cin,
-                                                     int Hin, int Win, int Hf, int Wf, int Hout,
+                                                     int Hin, int Win, int Hf, int Wf_, int Hout,
                                                      int Wout, int stride, int pad, FastDiv by_hw,
-                                                     FastDiv by_wout, FastDiv by_taps, FastDiv by_wf)
+                                                     FastDiv by_wout)
 {
-    const unsigned k = blockIdx.y;
-    const unsigned c = by_taps.div(k);
-    const unsigned hw = k - c * (Hf * Wf);
-    const int h = (int)by_wf.div(hw), w = (int)(hw - h * Wf);
-    float* row = cols + (size_t)k * ncols;
+    const int Wf = WF ? WF : Wf_;
+    const unsigned c = blockIdx.y;
+    float* rows = cols + (size_t)c * (Hf * Wf) * ncols;   // row (c, 0, 0)
 
     for (unsigned n = (blockIdx.x * 256 + threadIdx.x) * 4; n < ncols; n += gridDim.x * 1024) {
         unsigned b = by_hw.div(n);
         const unsigned r = n - b * by_hw.d;
         int ho = (int)by_wout.div(r);
         int wo = (int)(r - ho * Wout);
-        float v[4];
+        // top-left input position of each element's window, and its (image, channel) plane
+        int hi0[4], wi0[4];
+        const float* plane[4];
+        // at stride 1 the 4 elements of a thread that lie in one output row read 4 neighbouring
+        // input values: one 16-byte load where the window is inside the image
+        const bool one_row = stride == 1 && wo + 3 < Wout && n + 4 <= ncols;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int hi = ho * stride + h - pad, wi = wo * stride + w - pad;
-            const bool ok = n + e < ncols && hi >= 0 && hi < Hin && wi >= 0 && wi < Win;
-            v[e] = ok ? in[(((size_t)b * Cin + c) * Hin + hi) * Win + wi] : 0.f;
+            hi0[e] = ho * stride - pad;
+            wi0[e] = wo * stride - pad;
+            plane[e] = in + ((size_t)b * Cin + c) * Hin * Win;
             if (++wo == Wout) {
                 wo = 0;
                 if (++ho == Hout) { ho = 0; ++b; }
             }
         }
-        if (n + 4 <= ncols) {
-            const f32x4_u o = {v[0], v[1], v[2], v[3]};
-            __builtin_nontemporal_store(o, reinterpret_cast<f32x4_u*>(row + n));
-        } else {
-            for (unsigned e = 0; n + e < ncols; ++e) row[n + e] = v[e];
+        const int valid = (int)min(4u, ncols - n);   // elements that exist
+        float* dst = rows + n;
+        for (int h = 0; h < Hf; ++h) {
+#pragma unroll
+            for (int w = 0; w < (WF ? WF : 1); ++w) {
+                // WF == 0: this loop runs once per pass of the `wr` loop below
+                for (int wr = WF ? w : 0; wr < Wf; wr += WF ? Wf : 1) {
+                    float v[4];
+                    const int hi_a = hi0[0] + h, wi_a = wi0[0] + wr;
+                    if (one_row && hi_a >= 0 && hi_a < Hin && wi_a >= 0 && wi_a + 3 < Win) {
+                        const f32x4_u q = *reinterpret_cast<const f32x4_u*>(plane[0] + hi_a * Win + wi_a);
+                        v[0] = q[0]; v[1] = q[1]; v[2] = q[2]; v[3] = q[3];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int hi = hi0[e] + h, wi = wi0[e] + wr;
+                            const bool ok = e < valid && hi >= 0 && hi < Hin && wi >= 0 && wi < Win;
+                            v[e] = ok ? plane[e][hi * Win + wi] : 0.f;
+                        }
+                    }
+                    float* out = dst + (size_t)(h * Wf + wr) * ncols;
+                    if (valid == 4) {
+                        const f32x4_u o = {v[0], v[1], v[2], v[3]};
+                        __builtin_nontemporal_store(o, reinterpret_cast<f32x4_u*>(out));
+                    } else {
+                        for (int e = 0; e < valid; ++e) out[e] = v[e];
+                    }
+                }
+            }
         }
     }
 }
@@ -246,13 +280,22 @@ hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int H
     const int krows = Cin * Hf * Wf;
     const size_t ncols = (size_t)batch * Hout * Wout;
     if (krows <= 0 || ncols == 0) return hipSuccess;
-    if (krows > 65535 || ncols >= (1ull << 31)) return hipErrorInvalidValue;
+    if (Cin > 65535 || ncols >= (1ull << 31)) return hipErrorInvalidValue;
     size_t bx = (ncols + 1023) / 1024;
     if (bx > 4096) bx = 4096;
-    const dim3 grid((unsigned)bx, krows);
-    hipLaunchKernelGGL(im2col_kernel, grid, dim3(256), 0, stream, in, cols, (unsigned)ncols, Cin, Hin, Win, Hf, Wf,
-                       Hout, Wout, stride, pad, FastDiv::make((unsigned)(Hout * Wout)), FastDiv::make((unsigned)Wout),
-                       FastDiv::make((unsigned)(Hf * Wf)), FastDiv::make((unsigned)Wf));
+    const dim3 grid((unsigned)bx, Cin);
+    const FastDiv by_hw = FastDiv::make((unsigned)(Hout * Wout)), by_wout = FastDiv::make((unsigned)Wout);
+#define CAKE_IM2COL(W)                                                                                             \
+    hipLaunchKernelGGL(im2col_kernel<W>, grid, dim3(256), 0, stream, in, cols, (unsigned)ncols, Cin, Hin, Win, Hf, \
+                       Wf, Hout, Wout, stride, pad, by_hw, by_wout)
+    switch (Wf) {
+        case 1: CAKE_IM2COL(1); break;
+        case 3: CAKE_IM2COL(3); break;
+        case 5: CAKE_IM2COL(5); break;
+        case 7: CAKE_IM2COL(7); break;
+        default: CAKE_IM2COL(0); break;
+    }
+#undef CAKE_IM2COL
     return hipGetLastError();
 }
 
@@ -271,11 +314,35 @@ __global__ void __launch_bounds__(256) cn_to_nchw_kernel(const float* __restrict
     }
 }
 
+// the same in 16-byte pieces (HW a multiple of 4, both pointers 16-byte aligned); hw4 = HW / 4
+__global__ void __launch_bounds__(256) cn_to_nchw_vec_kernel(const f32x4* __restrict__ src,
+                                                             f32x4* __restrict__ dst, int batch,
+                                                             int Cout, FastDiv by_hw4, FastDiv by_cout)
+{
+    const unsigned hw4 = by_hw4.d;
+    const size_t total = (size_t)batch * Cout * hw4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        // total < 2^31 elements / 4
+        const unsigned t = by_hw4.div((unsigned)i), q = (unsigned)i - t * hw4;
+        const unsigned b = by_cout.div(t), co = t - b * (unsigned)Cout;
+        dst[i] = __builtin_nontemporal_load(src + ((size_t)co * batch + b) * hw4 + q);
+    }
+}
+
 hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
                              hipStream_t stream)
 {
     const size_t total = (size_t)batch * Cout * HW;
     if (total == 0) return hipSuccess;
+    if (HW % 4 == 0 && total < (1ull << 31) &&
+        (reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16 == 0) {
+        size_t blocks = (total / 4 + 255) / 256;
+        if (blocks > 16384) blocks = 16384;
+        hipLaunchKernelGGL(cn_to_nchw_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           reinterpret_cast<const f32x4*>(src), reinterpret_cast<f32x4*>(dst), batch, Cout,
+                           FastDiv::make((unsigned)(HW / 4)), FastDiv::make((unsigned)Cout));
+        return hipGetLastError();
+    }
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     hipLaunchKernelGGL(cn_to_nchw_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, batch, Cout, HW);
