@@ -1023,6 +1023,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if (batch <= 0 || Cin <= 0 || Cout <= 0 || Hin <= 0 || Win <= 0 ||
         conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout))
         return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
+    // A 1 x 1 filter at stride 1 without padding sees every plane as one row of Hin * Win pixels:
+    // rows of the product are then padded to a multiple of 4 once per plane instead of once per
+    // image row (7 x 7 maps: 52 columns for 49 instead of 56, 14 x 14 maps: none at all).
+    if (Hf == 1 && Wf == 1 && stride == 1 && pad == 0 && (double)Hin * Win < 2147483647.0) {
+        Win *= Hin;
+        Hin = 1;
+        Wout = Win;
+        Hout = 1;
+    }
     if (!in || !weights || !out) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
     const double K_d = (double)Cin * Hf * Wf;
     const double ncols_d = (double)batch * Hout * Wout;
@@ -1058,7 +1067,10 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const int chunks = (batch + chunk - 1) / chunk;
     chunk = (batch + chunks - 1) / chunks;
     const ConvStage sg = conv_stage(chunk, Cin, Hin, Win, Hf, Wf, stride, pad);
-    const bool implicit = !explicit_cols && (double)(row_n - Wout) / Wout * Cout < 60.0 && chunk_fits(chunk) &&
+    // (a flattened 1 x 1 filter pads at most 3 columns per plane, which always costs less than a
+    // column matrix that is a copy of the input)
+    const bool flat_1x1 = Hf == 1 && Wf == 1 && stride == 1 && pad == 0;
+    const bool implicit = !explicit_cols && (flat_1x1 || (double)(row_n - Wout) / Wout * Cout < 60.0) && chunk_fits(chunk) &&
                           (double)K * 256 * 4 < 2147483648.0;
     Timer timer(stream, seconds);
     // A 1 x 1 convolution at stride 1 without padding is one plain product per image on the input
@@ -1101,10 +1113,13 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
         int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
         if ((st = timer.start())) return st;
-        st = timer.family(3, [&] {
-            return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, sg.Hs, sg.pitch, sg.Wq, Hf, Wf, stride, sg.RH, stream);
-        });
-        if (st) return st;
+        const bool one_by_one = Hf == 1 && Wf == 1;   // row k is channel k: no table of tap offsets
+        if (!one_by_one) {
+            st = timer.family(3, [&] {
+                return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, sg.Hs, sg.pitch, sg.Wq, Hf, Wf, stride, sg.RH, stream);
+            });
+            if (st) return st;
+        }
         const size_t HW = (size_t)Hout * Wout;
         for (int b0 = 0; b0 < batch; b0 += chunk) {
             const int nb = batch - b0 < chunk ? batch - b0 : chunk;
@@ -1124,12 +1139,13 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             cv.Cin = Cin; cv.plane_rows = sg.Hs; cv.pitch = sg.pitch; cv.row_step = sg.RH;
             cv.Hout = Hout; cv.Wout = Wout; cv.row_n = row_n;
             cv.tap_table = taps;
+            cv.tap_stride = sg.Hs * sg.pitch * 4;   // 1 x 1 filters: channel k starts k planes into the image
             cv.out_nchw = out_nchw ? 1 : 0;
             // [batch][Cout][HW]: the chunk's images are contiguous; [Cout][batch*HW]: its columns are
             float* dst = o.dev + (out_nchw ? (size_t)b0 * Cout * HW : (size_t)b0 * HW);
             const int Np = nb * Hout * row_n;
             st = run_gemm(w.dev, nullptr, dst, Cout, Np, K, K, Np, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
-                          LOAD_IM2COL_ROW, stream, timer, &cv);
+                          one_by_one ? LOAD_IM2COL_1X1 : LOAD_IM2COL_ROW, stream, timer, &cv);
             if (st) return st;
         }
         if ((st = timer.stop())) return st;

@@ -35,6 +35,7 @@ struct ConvGeom {
     int Hout, Wout;
     int row_n;              // columns of the product per output row (a multiple of 4)
     const int* tap_table;   // byte offset of tap k = (c, h, w) inside one image, K + CONV_TAP_TABLE_EXTRA entries
+    int tap_stride;         // 1 x 1 filters (LOAD_IM2COL_1X1): bytes from channel to channel, instead of the table
     int out_nchw;           // epilogue writes C as [batch][M][Hout*Wout] instead of [M][N]
 };
 
@@ -86,8 +87,10 @@ enum LoadMode {
     LOAD_VEC4 = 0,   // row-major, 16-byte loads (ld % 4 == 0, 16-byte aligned bases)
     LOAD_SCALAR = 1, // row-major, any size/alignment
     LOAD_VEC4_T = 2, // B only: B handed over as its transpose Bt[N][K] (rows ldb apart), 16-byte loads along k
-    LOAD_IM2COL_ROW = 4  // B only: column matrix of a convolution gathered from the staged NCHW input,
+    LOAD_IM2COL_ROW = 4, // B only: column matrix of a convolution gathered from the staged NCHW input,
                          // one 16-byte load per 4 columns
+    LOAD_IM2COL_1X1 = 5  // the same for a 1 x 1 filter: row k is channel k, tap_stride bytes after row k - 1,
+                         // so no tap table is read
 };
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,

@@ -1,0 +1,21 @@
+// Macro-tile GEMM instantiations: B = the column matrix of a 1 x 1 convolution gathered from the
+// staged NCHW input, row k a fixed number of bytes after row k - 1 (no tap table).
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+hipError_t launch_sgemm_conv1x1(int tile_id, const GemmArgs& a, int grid, hipStream_t s)
+{
+    switch (tile_id) {
+        case TILE_256x256x32_W128x64: return launch_tile<Tile256x256x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_256x128x32_W64x64: return launch_tile<Tile256x128x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_128x256x32_W64x64: return launch_tile<Tile128x256x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_128x128x32_W64x64: return launch_tile<Tile128x128x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_64x64x32_W32x32: return launch_tile<Tile64x64x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_64x64x64_W32x32: return launch_tile<Tile64x64x64, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_96x128x32_W96x32: return launch_tile<Tile96x128x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace cake

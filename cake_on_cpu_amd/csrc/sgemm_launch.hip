@@ -7,6 +7,7 @@ hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_
 hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_convrow(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_vec_nt(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
+hipError_t launch_sgemm_conv1x1(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 
 template <class T>
 static constexpr TileInfo info_of()
@@ -28,6 +29,10 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
                         hipStream_t stream)
 {
     if (grid <= 0) return hipSuccess;
+    if (b_mode == LOAD_IM2COL_1X1) {
+        if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
+        return launch_sgemm_conv1x1(tile_id, args, grid, stream);
+    }
     if (b_mode == LOAD_IM2COL_ROW) {
         if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
         return launch_sgemm_convrow(tile_id, args, grid, stream);

@@ -570,7 +570,7 @@ __device__ __forceinline__ float buffer_load_f32(const float* base, int byte_off
 // lie in one output row (rows of n are a multiple of 4 long), so one (image, row,
 // column) triple per thread serves the whole K walk and only the filter tap
 // (c, h, w) of each k changes from stage to stage.
-template <class T>
+template <class T, bool LINEAR_TAPS = false>
 struct ConvRowLoader {
     static constexpr int NUM_LOADS = T::A_ITERS + T::B_ITERS;
     static constexpr bool MASK_A_STORES = true;   // K need not be a multiple of 4 (see VecLoader)
@@ -622,6 +622,7 @@ struct ConvRowLoader {
     // before the first load: the stages are then fetched at k0, k0 + BK, k0 + 2 BK, ...
     __device__ __forceinline__ void prime(int k0)
     {
+        if constexpr (LINEAR_TAPS) return;   // a 1 x 1 filter: the offset of row k is k * tap_stride
 #pragma unroll
         for (int it = 0; it < T::B_ITERS; ++it) tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], k0 * 4);
     }
@@ -630,6 +631,7 @@ struct ConvRowLoader {
     __device__ __forceinline__ int tap_offset(int it, int k0, int kend) const
     {
         const int k = k0 + b_k[it];
+        if constexpr (LINEAR_TAPS) return k < kend ? pix4 + k * cv.tap_stride : BUF_OOB;
         const int off = k < kend ? pix4 + tap_next[it] : BUF_OOB;
         tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], (k0 + T::BK) * 4);  // the table has spare entries past K
         return off;
@@ -638,6 +640,7 @@ struct ConvRowLoader {
     // the same for a stage that lies wholly below kend
     __device__ __forceinline__ int tap_offset_inside(int it, int k0) const
     {
+        if constexpr (LINEAR_TAPS) return pix4 + (k0 + b_k[it]) * cv.tap_stride;
         const int off = pix4 + tap_next[it];
         tap_next[it] = buffer_load_i32(cv.tap_table, b_k4[it], (k0 + T::BK) * 4);
         return off;
@@ -991,7 +994,7 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, con
     const float* bias = !PLAIN && g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // a convolution's columns n = (image, output row, column of a row padded to 4) go to
     // [M][batch*Hout*Wout] or NCHW: see conv_out_map
-    const bool conv_out = B_MODE == LOAD_IM2COL_ROW && g.partial == nullptr;
+    const bool conv_out = (B_MODE == LOAD_IM2COL_ROW || B_MODE == LOAD_IM2COL_1X1) && g.partial == nullptr;
     // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
     // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
     // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
@@ -1085,6 +1088,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
         k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
         k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
+    else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_1X1)
+        k_walk_vec<T, ConvRowLoader<T, true>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4_T)
         k_walk_vec<T, VecLoaderNT<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else

@@ -222,9 +222,10 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * computed with rows padded to one and the extra columns dropped.  It runs the
  * two-step path instead when that padding would cost more than the column
  * matrix (narrow maps with many output channels).  A 1 x 1 filter at stride 1
- * without padding needs neither: every image is then a plain product on the
- * input as it lies, and with at most 64 input channels and enough tiles those
- * products run as one batch on the short-K kernel.  A batch whose staged input
+ * without padding needs neither: a plane is then one row of Hin * Win pixels,
+ * gathered from the input as it lies, and with at most 64 input channels and
+ * enough tiles the images run as one batch of plain products on the short-K
+ * kernel.  A batch whose staged input
  * would reach 2 GiB, or whose product 2^31 elements, is run in chunks of whole
  * images through the same staged buffer, so input and output may be as large
  * as memory holds; only a single image of 2 GiB takes the two-step path, whose
