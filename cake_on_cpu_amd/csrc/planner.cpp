@@ -86,7 +86,7 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
     // the slices are written, read back and summed by a second kernel
     if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 8e-6;
-    if (tail) s += 8e-6;
+    if (tail) s += 6e-6;  // the second kernel: about 5 us and the gap in front of it
     return s + 3e-6;  // launch
 }
 
