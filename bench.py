@@ -202,6 +202,7 @@ def main() -> int:
 
         gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024)
         gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024)
+        gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64)
         gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384,
                    "sgemm_fewrows_nn_kernel + splitk_reduce_kernel", MEASURED_TRAFFIC_BYTES["fewrows_nn"])
         gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384,
@@ -238,6 +239,20 @@ def main() -> int:
                            "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
                            "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
         del inp, oc, ws
+        # a 1 x 1 layer: planes read in place (no staged copy, no tap table), NCHW output
+        Pb, Pc, Ph, Po = 32, 256, 14, 1024
+        pin, pw = dev_uniform((Pb, Pc, Ph, Ph), 6), dev_uniform((Po, Pc), 7)
+        po = torch.empty((Pb, Po, Ph, Ph), dtype=torch.float32, device=dev)
+        pws_bytes = lib.cake_hip_conv2d_workspace(Pb, Pc, Ph, Ph, Po, 1, 1, 1, 0)
+        pws = torch.empty((max(1, (pws_bytes + 3) // 4),), dtype=torch.float32, device=dev)
+        pfl = 2.0 * Po * Pc * (Pb * Ph * Ph)
+        _, avg, _ = time_steps(lambda: _lib.check(
+            lib.cake_hip_conv2d(pin.data_ptr(), pw.data_ptr(), po.data_ptr(), Pb, Pc, Ph, Ph, Po, 1, 1, 1, 0, 1,
+                                pws.data_ptr(), stream, None), "conv2d"), 50, 5, 40.0)
+        extras.append({"workload": "conv 1x1, batch 32, 256->1024 ch, 14x14, NCHW output",
+                       "us": round(avg * 1e6, 2), "tflops": round(pfl / avg / 1e12, 2),
+                       "frac_mfma_peak": round(pfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        del pin, po, pws
 
         # the linear layer (src/linear.cpp): batch 8192, 4096 -> 4096 features, with bias
         Lm, Lk, Ln = 8192, 4096, 4096
