@@ -585,6 +585,17 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     if (st) return fail(st, "cake_hip_plan: bad shape, schedule or tile override");
     *out = plan.pub;
     out->kernel = kernel_family(M, N, K, tile_override != nullptr, vec);
+    if (out->kernel == CAKE_HIP_KERNEL_SHORT_K) {
+        // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
+        // column blocks of B by at most four resident workgroups per CU
+        out->tile_m = 64; out->tile_n = 64; out->tile_k = 64;
+        out->wave_m = 32; out->wave_n = 32;
+        out->threads = 256;
+        out->split_k = 1; out->tail_tiles = 0; out->tail_split = 1;
+        out->tiles_m = (M + 63) / 64; out->tiles_n = (N + 63) / 64;
+        out->group = out->tiles_m;
+        shortk_launch_shape((long)out->tiles_m * out->tiles_n, model.cus, &out->grid, &out->lds_bytes);
+    }
     return CAKE_HIP_OK;
 }
 

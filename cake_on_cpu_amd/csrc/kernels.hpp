@@ -100,6 +100,7 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t str
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
 bool shortk_applies(int M, int N, int K, int cus, int batch = 1);
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream);
+void shortk_launch_shape(long tiles, int cus, int* grid, int* lds_bytes);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
                                 int accumulate, hipStream_t stream, const ConvGeom* conv = nullptr,

@@ -150,9 +150,17 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream
     const long tiles = (long)args.tiles_m * args.tiles_n;
     if (tiles <= 0) return hipSuccess;
     if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
-    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 36 KB per workgroup
-    const int grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
+    int grid, lds;
+    shortk_launch_shape(tiles, cus, &grid, &lds);
     return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
+}
+
+// Workgroups launched for `tiles` tiles of 64 x 64, and the LDS each of them takes
+void shortk_launch_shape(long tiles, int cus, int* grid, int* lds_bytes)
+{
+    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 36 KB per workgroup
+    *grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
+    *lds_bytes = shortk_lds_bytes<TileShortK64>();
 }
 
 }  // namespace cake

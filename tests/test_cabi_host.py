@@ -293,3 +293,9 @@ def test_plan_names_the_kernel_family():
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(2048, 2048, 64) == 0   # short K, 12 tiles per CU
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
+    # the plan of a short-K product describes that launch: 64 x 64 tiles holding the whole K, at most
+    # four resident workgroups per CU in whole rows of 8 XCDs, no K slices
+    p = cake.plan(250, 100352, 64)
+    assert (p.kernel, p.tile_m, p.tile_n, p.tile_k, p.threads, p.split_k, p.tail_tiles) == (4, 64, 64, 64, 256, 1, 0)
+    assert (p.tiles_m, p.tiles_n) == (4, 1568) and p.grid == 4 * p.cus and p.grid % 8 == 0
+    assert 4 * p.lds_bytes <= 160 * 1024
