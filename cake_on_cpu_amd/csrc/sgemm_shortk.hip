@@ -4,7 +4,7 @@
 // work alone takes 21 us, plus 6 us of stores).  Here a workgroup stays and walks over tiles: the
 // whole K of a tile is one stage of LDS, and the operands of the NEXT tile are already on their
 // way into registers while the current tile is multiplied and written out (256 x 100352 x 64:
-// 48 -> 40 us; 16384 x 16384 x 16: 308 -> 263 us).  Loaders, LDS layout, operand reads and the
+// 48 -> 40 us, 38 us with A's stage kept across tiles; 16384 x 16384 x 16: 308 -> 263 us).  Loaders, LDS layout, operand reads and the
 // epilogue are the macro-tile kernel's.
 // Measured and left out: the same with K up to 128 in one stage (71 KB of LDS, two workgroups per
 // CU: 85 us against 73 us at 256 x 100352 x 128), K up to 128 as two unrolled stages of 64 with
@@ -29,6 +29,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     static_assert(B_MODE == LOAD_VEC4, "row-major operands");
     using L = VecLoader<T>;
     static_assert(T::KSPLIT == 1, "one wave per block of C");
+    static_assert(T::WAVES_M * T::WAVES_N * 32 * (T::WN + 4) <= T::B_STAGE, "the epilogue's staging blocks fit B's stage");
     extern __shared__ __align__(16) float smem[];
     float* As = smem;
     float* Bs = smem + T::A_STAGE;
@@ -72,12 +73,19 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
     ld.init(gt, m0, n0, tid);
     ld.load_first_stage(g.K, ra, rb);
+    // A's stage outlives a tile (the epilogue turns C around inside B's stage): a workgroup whose
+    // next tile has the same rows of A -- every time when the walk's stride is a multiple of
+    // tiles_m -- neither loads nor stores them again
+    bool a_fresh = true;
     for (;;) {
-        // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
-#pragma unroll
-        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = a_chunk_below<T>(ra[it], it, tid, 0, g.K);
         __syncthreads();   // every wave is done with the staging reads of the previous tile's epilogue
-        store_stage<T>(As, Bs, tid, ra, rb);
+        if (a_fresh) {     // the same for every thread of the workgroup
+            // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
+#pragma unroll
+            for (int it = 0; it < T::A_ITERS; ++it) ra[it] = a_chunk_below<T>(ra[it], it, tid, 0, g.K);
+            store_stage_a<T>(As, tid, ra);
+        }
+        store_stage_b<T>(Bs, tid, rb);
         __syncthreads();
 
         // the next tile's operands start their way into the registers just emptied
@@ -87,7 +95,9 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
         if (more) {
             place(t_next, gt_next, m0_next, n0_next);
             ld.init(gt_next, m0_next, n0_next, tid);
-            ld.load_first_stage(g.K, ra, rb);
+            a_fresh = m0_next != m0;
+            if (a_fresh) ld.load_first_stage(g.K, ra, rb);
+            else ld.load_first_stage_b(g.K, ra, rb);
         }
 
         f32x16 acc[T::TM][T::TN];
@@ -106,7 +116,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
                 mma_frag<T>(frag[kg & 1], acc);
             }
         }
-        store_c_tile<T, B_MODE, PLAIN>(gt, smem, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
+        store_c_tile<T, B_MODE, PLAIN>(gt, Bs, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
         if (!more) break;
         t = t_next;
         m0 = m0_next;

@@ -210,16 +210,19 @@ __device__ __forceinline__ void load_b_stage(const GemmArgs& g, int n0, int k0, 
 template <class T>
 __device__ __forceinline__ void store_b_chunk_along_k(float* Bs, int W, int tid, const f32x4& v);
 
-template <class T, bool B_ALONG_K = false>
-__device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
-                                            const f32x4 (&ra)[T::A_ITERS],
-                                            const f32x4 (&rb)[T::B_ITERS])
+template <class T>
+__device__ __forceinline__ void store_stage_a(float* As, int tid, const f32x4 (&ra)[T::A_ITERS])
 {
 #pragma unroll
     for (int it = 0; it < T::A_ITERS; ++it) {
         const int c = tid + it * T::THREADS;
         *reinterpret_cast<f32x4*>(As + (c / (T::BK / 4)) * T::LDA + (c % (T::BK / 4)) * 4) = ra[it];
     }
+}
+
+template <class T, bool B_ALONG_K = false>
+__device__ __forceinline__ void store_stage_b(float* Bs, int tid, const f32x4 (&rb)[T::B_ITERS])
+{
 #pragma unroll
     for (int it = 0; it < T::B_ITERS; ++it) {
         if constexpr (B_ALONG_K) {
@@ -229,6 +232,15 @@ __device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
             *reinterpret_cast<f32x4*>(Bs + (c / (T::BN / 4)) * T::LDB + (c % (T::BN / 4)) * 4) = rb[it];
         }
     }
+}
+
+template <class T, bool B_ALONG_K = false>
+__device__ __forceinline__ void store_stage(float* As, float* Bs, int tid,
+                                            const f32x4 (&ra)[T::A_ITERS],
+                                            const f32x4 (&rb)[T::B_ITERS])
+{
+    store_stage_a<T>(As, tid, ra);
+    store_stage_b<T, B_ALONG_K>(Bs, tid, rb);
 }
 
 // MFMA operands of one wave for a group of 8 consecutive k.
@@ -429,6 +441,11 @@ struct VecLoader {
     __device__ __forceinline__ void load_first_stage(int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
     {
         load_all<0>(0, kend, ra, rb);
+    }
+    // only its B chunks: the A chunks are the previous tile's and already lie in LDS
+    __device__ __forceinline__ void load_first_stage_b(int kend, f32x4 (&ra)[T::A_ITERS], f32x4 (&rb)[T::B_ITERS]) const
+    {
+        load_all<T::A_ITERS>(0, kend, ra, rb);
     }
 
     template <int OP>
