@@ -1090,7 +1090,9 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // (64 -> 256 channels on 32 x 56 x 56: 50 -> 43 us).
     const int HW = Hout * Wout;
     if (!explicit_cols && Hf == 1 && Wf == 1 && stride == 1 && pad == 0 &&
-        shortk_applies(Cout, HW, K, g_ctx.model.cus, batch) && vec4_loadable(w.dev, i.dev, K, HW)) {
+        shortk_applies(Cout, HW, K, g_ctx.model.cus, batch) &&
+        (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch >= 12L * g_ctx.model.cus &&   // measured from there on
+        vec4_loadable(w.dev, i.dev, K, HW)) {
         GemmArgs g{};
         g.A = w.dev; g.B = i.dev; g.C = o.dev;
         g.M = Cout; g.N = HW; g.K = K;

@@ -153,7 +153,10 @@ def test_plan_covers_any_shape(M, N, K):
         tiles = pl.tiles_m * pl.tiles_n
         assert pl.split_k >= 1 and pl.tail_split >= 1 and 0 <= pl.tail_tiles < tiles
         assert not (pl.split_k > 1 and pl.tail_tiles > 0)
-        assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
+        if pl.kernel == 4:   # short K: resident workgroups, at most four per CU, in whole rows of 8 XCDs
+            assert pl.grid == (min(tiles, 4 * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
+        else:
+            assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
         assert 1 <= pl.group <= max(pl.tiles_m, pl.tiles_n)
         assert pl.sched in (cake.KMN, cake.MKN, cake.NKM)
         if sch != cake.NA:
@@ -290,7 +293,7 @@ def test_plan_names_the_kernel_family():
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
-    assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(2048, 2048, 64) == 0   # short K, 12 tiles per CU
+    assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
     # the plan of a short-K product describes that launch: 64 x 64 tiles holding the whole K, at most
