@@ -106,6 +106,20 @@ def cake_query_cntx() -> CpuCntx:
     return cx
 
 
+_DEFAULT_CNTX = None
+
+
+def _default_cntx() -> CpuCntx:
+    """What a NULL cake_cntx stands for (src/cake_sgemm.cpp:14-16): the host's own description,
+    queried once per process here instead of on every call."""
+    global _DEFAULT_CNTX
+    if _DEFAULT_CNTX is None:
+        _DEFAULT_CNTX = cake_query_cntx()
+    cx = CpuCntx()
+    C.memmove(C.byref(cx), C.byref(_DEFAULT_CNTX), C.sizeof(CpuCntx))
+    return cx
+
+
 def update_mr_nr(cake_cntx: CpuCntx, m_r: int, n_r: int) -> None:
     """update_mr_nr (src/block_sizing.cpp:78-83)."""
     cake_cntx.mr, cake_cntx.nr = m_r, n_r
@@ -155,7 +169,7 @@ def cake_sgemm(A, B, Cm, M, N, K, p, cake_cntx: CpuCntx | None = None, argv=None
     secs = C.c_double(0.0)
     stream = _stream(A, B, Cm)
     if packedA or packedB:
-        cx = cake_cntx if cake_cntx is not None else cake_query_cntx()
+        cx = cake_cntx if cake_cntx is not None else _default_cntx()
         x = init_block_dims(M, N, K, p, cx, sch, argv, 4, mcu, kcu, ncu)
         accumulate = int(x.sch != KMN and beta != 0)
         check(lib.cake_hip_sgemm_packed(_ptr(A, "A"), _ptr(B, "B"), _ptr(Cm, "C"), M, N, K, p,
@@ -164,9 +178,14 @@ def cake_sgemm(A, B, Cm, M, N, K, p, cake_cntx: CpuCntx | None = None, argv=None
         return secs.value
     _need(A, M * K, "A")
     _need(B, K * N, "B")
+    # beta != 0 means "start from C" only under the schedule the reference resolves from the
+    # caller's cntx and p (src/cake_sgemm.cpp:34-35,114); the GPU's tile order stays the planner's.
     resolved = sch
-    if sch == NA:
-        resolved = plan(M, N, K, NA).sched if M > 0 and N > 0 and K > 0 else KMN
+    if M > 0 and N > 0 and K > 0:
+        cx = cake_cntx if cake_cntx is not None else _default_cntx()
+        resolved = init_block_dims(M, N, K, p, cx, sch, argv, 4, mcu, kcu, ncu).sch
+    elif sch == NA:
+        resolved = KMN
     accumulate = int(resolved != KMN and beta != 0)
     ov = _tile_override(M, N, K, sch, mcu, kcu, ncu)
     check(lib.cake_hip_sgemm(_ptr(A, "A"), _ptr(B, "B"), _ptr(Cm, "C"), M, N, K, sch, accumulate, ov,

@@ -86,11 +86,14 @@ double sgemm_common(float* A, float* B, float* C, int M, int N, int K, int p, ca
         die_on(cake_hip_sgemm_packed(A, B, C, M, N, K, p, &d, &cx, packedA, packedB, accumulate, NULL, &dev_s),
                "cake_sgemm");
     } else {
+        // beta != 0 means "start from C" only under the schedule the reference itself resolves
+        // from the caller's cntx and p (src/cake_sgemm.cpp:34-35,114); the order in which the
+        // GPU walks its tiles stays the planner's choice and does not change the result.
         int resolved = sch;
-        if (sch == NA && M > 0 && N > 0 && K > 0) {
-            cake_hip_plan_t plan;
-            die_on(cake_hip_plan(M, N, K, NA, NULL, &plan), "cake_sgemm");
-            resolved = plan.sched;
+        if (M > 0 && N > 0 && K > 0) {
+            blk_dims_t x;
+            init_block_dims(M, N, K, p, &x, cntx, sch, argv, 4, mcu, kcu, ncu);
+            resolved = x.sch;
         }
         const int accumulate = (resolved != KMN) && (beta != 0);
         int ov[4];
@@ -207,28 +210,31 @@ double cake_sgemm(float* A, float* B, float* C, int M, int N, int K, int p, cake
     return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
 }
 
+// The pack-on-the-fly and 2-D entry points always run K-first on row-major operands: they set
+// sch = KMN before sizing their blocks and never look at packedA / packedB or beta
+// (src/cake_sgemm.cpp:200,273,418), so C is assigned whatever the caller passed.
 double cake_sgemm_online(float* A, float* B, float* C, int M, int N, int K, int p,
                          cake_cntx_t* cake_cntx, char* argv[], bool packedA, bool packedB, float alpha,
                          float beta, enum sched sch, int mcu, int kcu, int ncu)
 {
-    (void)alpha;
-    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
+    (void)alpha; (void)beta; (void)sch; (void)packedA; (void)packedB;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, 0, 0, 0.f, KMN, mcu, kcu, ncu);
 }
 
 double cake_sgemm_2d(float* A, float* B, float* C, int M, int N, int K, int p, cake_cntx_t* cake_cntx,
                      char* argv[], bool packedA, bool packedB, float alpha, float beta, enum sched sch,
                      int mcu, int kcu, int ncu)
 {
-    (void)alpha;
-    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, mcu, kcu, ncu);
+    (void)alpha; (void)beta; (void)sch; (void)packedA; (void)packedB;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, 0, 0, 0.f, KMN, mcu, kcu, ncu);
 }
 
 double cake_sgemm_2d_small(float* A, float* B, float* C, int M, int N, int K, int p,
                            cake_cntx_t* cake_cntx, char* argv[], bool packedA, bool packedB,
                            float alpha, float beta, enum sched sch)
 {
-    (void)alpha;
-    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, sch, 0, 0, 0);
+    (void)alpha; (void)beta; (void)sch; (void)packedA; (void)packedB;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, 0, 0, 0.f, KMN, 0, 0, 0);
 }
 
 // ---- packing ----------------------------------------------------------------------

@@ -119,6 +119,38 @@ static void conv_case(cake_cntx_t* cntx)
     free(F); free(In); free(Bm); free(x); free(A_p); free(B_p); free(C); free(C_p); free(C2);
 }
 
+// beta with the default schedule: whether C is added to follows the schedule init_block_dims
+// resolves from the caller's cntx and p (src/cake_sgemm.cpp:34-35,114), not the device's tiling.
+static void beta_case(int M, int K, int N, int p, cake_cntx_t* cntx)
+{
+    float* A = (float*)malloc(sizeof(float) * M * K);
+    float* B = (float*)malloc(sizeof(float) * K * N);
+    float* C0 = (float*)malloc(sizeof(float) * M * N);
+    float* C = (float*)malloc(sizeof(float) * M * N);
+    float* P = (float*)calloc((size_t)M * N, sizeof(float));
+    rand_init(A, M, K);
+    rand_init(B, K, N);
+    rand_init(C0, M, N);
+    memcpy(C, C0, sizeof(float) * M * N);
+    blk_dims_t x;
+    init_block_dims(M, N, K, p, &x, cntx, NA, NULL);
+    cake_sgemm(A, B, P, M, N, K, p, cntx, NULL, 0, 0, 1, 0, KMN);    // the plain product
+    cake_sgemm(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 1);         // sch = NA, beta = 1
+    const bool adds = x.sch != KMN;
+    bool ok = true;
+    for (size_t i = 0; i < (size_t)M * N && ok; ++i)
+        if (fabs((double)C[i] - ((double)P[i] + (adds ? C0[i] : 0.f))) > 1e-4 * (fabs(P[i]) + 1)) ok = false;
+    char what[128];
+    snprintf(what, sizeof what, "cake_sgemm beta=1 sch=NA M=%d K=%d N=%d p=%d: %s C", M, K, N, p,
+             adds ? "adds to" : "assigns");
+    report(what, ok);
+    // the pack-on-the-fly entry point is K-first whatever it is asked for: it assigns
+    memcpy(C, C0, sizeof(float) * M * N);
+    cake_sgemm_online(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 1, MKN);
+    report("cake_sgemm_online beta=1 sch=MKN assigns C", memcmp(C, P, sizeof(float) * M * N) == 0);
+    free(A); free(B); free(C0); free(C); free(P);
+}
+
 // examples/cake_gemv.cpp main: column-major A, mr = 8, y accumulates
 static void gemv_case(cake_cntx_t* cntx, int M, int K)
 {
@@ -177,6 +209,15 @@ int main(int argc, char** argv)
             }
     sgemm_case(960, 2111, 333, 8, NA, cntx);
     variants_case(cntx);
+    {
+        // a fixed host description, so the resolved schedules do not depend on the test machine:
+        // 1024^3 with p = 8 is M-first and 200 x 300 x 3000 N-first for it, 300 x 3000 x 300 K-first
+        cake_cntx_t fixed = *cntx;
+        fixed.L2 = 2 << 20; fixed.L3 = 105 << 20; fixed.ncores = 8;
+        beta_case(1024, 1024, 1024, 8, &fixed);
+        beta_case(200, 300, 3000, 4, &fixed);
+        beta_case(300, 3000, 300, 4, &fixed);
+    }
     conv_case(cntx);
     gemv_case(cntx, 1024, 777);
     gemv_case(cntx, 37, 5);

@@ -302,3 +302,38 @@ def test_plan_names_the_kernel_family():
     assert (p.kernel, p.tile_m, p.tile_n, p.tile_k, p.threads, p.split_k, p.tail_tiles) == (4, 64, 64, 64, 256, 1, 0)
     assert (p.tiles_m, p.tiles_n) == (4, 1568) and p.grid == 4 * p.cus and p.grid % 8 == 0
     assert 4 * p.lds_bytes <= 160 * 1024
+
+
+def test_default_schedule_resolves_accumulate_by_the_reference_rule(monkeypatch):
+    """cake_sgemm(sch=NA, beta=1): the accumulate flag handed to the C-ABI follows
+    init_block_dims on the caller's cntx and p (src/cake_sgemm.cpp:34-35,114), on the unpacked
+    path exactly as on the packed one, not the GPU planner's tile order."""
+    from cake_on_cpu_amd import api
+    real = cake.load()
+    seen = {}
+
+    class Recorder:
+        def __getattr__(self, name):
+            return getattr(real, name)
+
+        def cake_hip_sgemm(self, A, B, Cm, M, N, K, sch, accumulate, ov, stream, secs):
+            seen["unpacked"] = (sch, accumulate)
+            return 0
+
+        def cake_hip_sgemm_packed(self, A, B, Cm, M, N, K, p, x, cx, pa, pb, accumulate, stream, secs):
+            seen["packed"] = accumulate
+            return 0
+
+    monkeypatch.setattr(api, "load", lambda: Recorder())
+    ocx = oracle.make_cntx()
+    for (M, N, K, p) in [(1024, 1024, 1024, 8), (512, 3000, 256, 4), (300, 300, 3000, 4), (64, 4096, 512, 4),
+                         (960, 960, 111, 4), (96, 2111, 111, 8)]:
+        cx = cake.CpuCntx()
+        cx.alpha_n, cx.mr, cx.nr, cx.L1, cx.L2, cx.L3, cx.ncores = 1.0, ocx.mr, ocx.nr, ocx.L1, ocx.L2, ocx.L3, ocx.ncores
+        want = oracle.init_block_dims(M, N, K, p, ocx, oracle.NA).sch != oracle.KMN
+        big = np.zeros(max(M * K, K * N, M * N) + 4096 * 64, np.float32)
+        for beta in (0.0, 1.0):
+            api.cake_sgemm(big, big, big, M, N, K, p, cx, None, False, False, 1.0, beta)
+            api.cake_sgemm(big, big, big, M, N, K, p, cx, None, True, True, 1.0, beta)
+            assert seen["unpacked"] == (cake.NA, int(want and beta != 0)), (M, N, K, p, beta)
+            assert seen["packed"] == int(want and beta != 0)

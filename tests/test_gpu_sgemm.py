@@ -295,6 +295,50 @@ def test_overwrite_and_accumulate_semantics():
     assert np.allclose(acc - plain, C0, atol=1e-4)
 
 
+def _cake_cntx(o):
+    """The library's cntx struct with the fields of an oracle cntx."""
+    cx = cake.CpuCntx()
+    cx.alpha_n, cx.mr, cx.nr, cx.L1, cx.L2, cx.L3, cx.ncores = o.alpha_n, o.mr, o.nr, o.L1, o.L2, o.L3, o.ncores
+    return cx
+
+
+@pytest.mark.parametrize("shape,p", [((1024, 1024, 1024), 8), ((960, 111, 960), 4), ((512, 256, 3000), 4),
+                                     ((96, 111, 2111), 8), ((300, 3000, 300), 4), ((64, 512, 4096), 4),
+                                     ((4096, 512, 64), 4)],
+                         ids=lambda s: "x".join(map(str, s)) if isinstance(s, tuple) else f"p{s}")
+def test_default_schedule_decides_accumulation_like_the_reference(shape, p):
+    """sch = NA, beta = 1 on a prefilled C: whether C is added to follows the schedule the
+    reference resolves from cntx and p (src/cake_sgemm.cpp:34-35,114) -- M-/N-first for the
+    first four shapes, K-first (assign) for the next two -- whatever order the GPU planner
+    walks its tiles in (it differs from the reference's on six of the seven)."""
+    M, K, N = shape
+    print(f"sgemm NA beta=1 M={M} K={K} N={N} p={p}", flush=True)
+    A, B = oracle.uniform((M, K), 21), oracle.uniform((K, N), 22)
+    C0 = oracle.uniform((M, N), 23)
+    ocx = oracle.make_cntx()
+    ref, _, dims = oracle.cake_sgemm(A, B, p, ocx, Cinit=C0, beta=1.0, sch=cake.NA, return_time=True)
+    C64, S = oracle.gemm_f64(A, B)
+    for name, dev in (("host", False), ("device", True)):
+        if dev:
+            import torch
+            tA, tB, tC = (torch.from_numpy(x).cuda() for x in (A, B, C0))
+            cake.cake_sgemm(tA, tB, tC, M, N, K, p, _cake_cntx(ocx), None, False, False, 1.0, 1.0)
+            torch.cuda.synchronize()
+            Cm = tC.cpu().numpy()
+        else:
+            Cm = C0.copy()
+            cake.cake_sgemm(A, B, Cm, M, N, K, p, _cake_cntx(ocx), None, False, False, 1.0, 1.0)
+        d = float(np.max(np.abs(Cm.astype(np.float64) - ref) / (S + np.abs(C0))))
+        assert d <= TOL and d <= 1e-5, (name, shape, dims.sch, d)
+        adds = dims.sch != cake.KMN
+        err = float(np.max(np.abs(Cm.astype(np.float64) - adds * C0 - C64) / (S + np.abs(C0))))
+        assert err <= TIGHT, (name, shape, dims.sch, err)
+    # the packed entry decides the same way (it always used the reference's rule)
+    cx = _cake_cntx(ocx)
+    x = cake.init_block_dims(M, N, K, p, cx)
+    assert x.sch == dims.sch
+
+
 def test_schedules_agree_and_are_deterministic():
     M, K, N = 777, 1030, 515
     outs = [_run(M, K, N, sch)[2] for sch in (cake.KMN, cake.MKN, cake.NKM)]
