@@ -43,28 +43,41 @@ int fail(int status, const char* fmt, ...)
             return fail(CAKE_HIP_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));     \
     } while (0)
 
-// Grow-only device buffer.
+// Grow-only device buffer.  A workspace that kernels of device-operand calls use (`keep_old`) is
+// never freed when it grows: a caller may have captured earlier launches in a HIP graph, which
+// holds the old address, so the outgrown allocation is kept until shutdown.  Such a buffer at
+// least doubles, which bounds everything kept to the size of the live one.  Staging copies of
+// host operands are only touched by synchronous calls and are freed at once.
 struct DeviceBuffer {
     void* ptr = nullptr;
     size_t cap = 0;
+    bool keep_old = false;
+    std::vector<void*> outgrown;
     int reserve(size_t bytes)
     {
         if (bytes <= cap) return CAKE_HIP_OK;
-        if (ptr) (void)hipFree(ptr);
-        ptr = nullptr;
-        cap = 0;
         size_t want = bytes + (bytes >> 3) + 256;
-        if (hipMalloc(&ptr, want) != hipSuccess) {
-            (void)hipGetLastError();
+        if (keep_old && want < 2 * cap) want = 2 * cap;
+        void* fresh = nullptr;
+        if (!keep_old && ptr) {
+            (void)hipFree(ptr);
             ptr = nullptr;
+            cap = 0;
+        }
+        if (hipMalloc(&fresh, want) != hipSuccess) {
+            (void)hipGetLastError();
             return fail(CAKE_HIP_ERR_ALLOC, "device allocation of %zu bytes failed", want);
         }
+        if (ptr) outgrown.push_back(ptr);
+        ptr = fresh;
         cap = want;
         return CAKE_HIP_OK;
     }
     void release()
     {
         if (ptr) (void)hipFree(ptr);
+        for (void* q : outgrown) (void)hipFree(q);
+        outgrown.clear();
         ptr = nullptr;
         cap = 0;
     }
@@ -476,6 +489,8 @@ int cake_hip_init(int device)
     if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
     for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
         if (!*e) HIP_TRY(hipEventCreate(e));
+    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.tables, &c.unpacked, &c.linear})
+        b->keep_old = true;
     if (const char* tuned = std::getenv("CAKE_HIP_TUNE_FILE")) (void)tune_load(tuned);  // optional
     c.ready = true;
     return CAKE_HIP_OK;
@@ -1562,7 +1577,6 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
             GemmPlan plan;
             if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
             *best_plan = plan.pub;
-        best_plan->kernel = kernel_family(M, N, K, false, vec);
             best_plan->kernel = kernel_family(M, N, K, false, vec);
         }
         return CAKE_HIP_OK;

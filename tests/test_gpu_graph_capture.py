@@ -5,6 +5,8 @@ import pytest
 
 torch = pytest.importorskip("torch")
 
+import ctypes
+
 import cake_on_cpu_amd as cake
 
 pytestmark = pytest.mark.gpu
@@ -46,7 +48,29 @@ def test_captured_sequence_replays_like_eager_calls():
     with torch.cuda.graph(graph, stream=side):
         run(captured, torch.cuda.current_stream().cuda_stream)
 
-    for replay in range(4):
+    def grow_every_workspace():
+        """Eager calls whose partial sums need several times the memory the captured ones did: the
+        library's workspaces grow, and the graph must keep working on the addresses it recorded
+        (an outgrown workspace is kept, not freed)."""
+        bigA = torch.empty((1500, 8192), dtype=torch.float32, device=dev)
+        bigB = torch.empty((8192, 1300), dtype=torch.float32, device=dev)
+        bigC = torch.empty((1500, 1300), dtype=torch.float32, device=dev)
+        ov = (ctypes.c_int * 4)(128, 128, 32, 8)
+        assert lib.cake_hip_sgemm(bigA.data_ptr(), bigB.data_ptr(), bigC.data_ptr(), 1500, 1300, 8192, cake.NA, 0, ov,
+                                  None, None) == 0
+        bg = 6144
+        bigG = torch.empty((bg * bg,), dtype=torch.float32, device=dev)
+        by = torch.empty((bg,), dtype=torch.float32, device=dev)
+        assert lib.cake_hip_sgemv(bigG.data_ptr(), bigG.data_ptr(), by.data_ptr(), bg, bg, 1, 0, None, None) == 0
+        bx = torch.empty((24, 4096), dtype=torch.float32, device=dev)
+        bw = torch.empty((8192, 4096), dtype=torch.float32, device=dev)
+        bo = torch.empty((24, 8192), dtype=torch.float32, device=dev)
+        assert lib.cake_hip_linear_forward(bx.data_ptr(), bw.data_ptr(), None, bo.data_ptr(), 24, 8192, 4096, None, None) == 0
+        torch.cuda.synchronize()
+
+    for replay in range(5):
+        if replay == 2:
+            grow_every_workspace()
         for i, t in enumerate((A, x, lx)):       # new inputs, written by eager work between the replays
             cake.fill_uniform(t, 100 + 10 * replay + i)
         for t in captured:
