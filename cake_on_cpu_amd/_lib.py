@@ -89,6 +89,7 @@ SIGNATURES = {
     "cake_hip_init_block_dims": (_i, [_i, _i, _i, _i, _cx, _i, _i, _i, _i, _bd]),
     "cake_hip_derive_schedule": (_i, [_i, _i, _i, _i, _i, _cx]),
     "cake_hip_sgemm": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _i, C.POINTER(_i), C.c_void_p, _dp]),
+    "cake_hip_sgemm_noalloc": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _i, C.c_void_p]),
     "cake_hip_sgemm_packed": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _bd, _cx, _i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_packed_a_size": (C.c_size_t, [_i, _i, _i, _bd, _cx, _i]),
     "cake_hip_packed_b_size": (C.c_size_t, [_i, _i, _i, _bd, _cx]),

@@ -105,6 +105,33 @@ struct Context {
 Context g_ctx;
 std::mutex g_mutex;  // one compute call at a time: the workspaces are shared
 
+// Partial sums (K slices of split-K, tail-split and streaming products, slices of the
+// matrix-vector kernels) of cake_hip_sgemm_noalloc: a file-scope array instead of a buffer from
+// hipMalloc.  The name is a host-side handle, not a device address; cake_hip_init asks the runtime
+// for the address on each device it is called for and the kernels only ever get that pointer.
+constexpr size_t NOALLOC_SCRATCH_BYTES = 64u << 20;
+static __device__ __align__(256) unsigned char noalloc_scratch[NOALLOC_SCRATCH_BYTES];
+enum { MAX_DEVICES = 64 };
+float* g_noalloc_ptr[MAX_DEVICES] = {nullptr};
+bool g_noalloc_call = false;   // set (under g_mutex) while cake_hip_sgemm_noalloc runs
+
+// Where the partial sums of the current call go: `buf` (grown when needed), or the file-scope array
+// during cake_hip_sgemm_noalloc, which never grows.
+int partial_space(DeviceBuffer& buf, size_t bytes, float** out)
+{
+    if (g_noalloc_call) {
+        if (bytes > NOALLOC_SCRATCH_BYTES)
+            return fail(CAKE_HIP_ERR_RANGE, "this product needs %zu bytes of partial sums; cake_hip_sgemm_noalloc has %zu",
+                        bytes, (size_t)NOALLOC_SCRATCH_BYTES);
+        *out = g_noalloc_ptr[g_ctx.device];
+        return CAKE_HIP_OK;
+    }
+    int st = buf.reserve(bytes);
+    if (st) return st;
+    *out = static_cast<float*>(buf.ptr);
+    return CAKE_HIP_OK;
+}
+
 int ensure_init()
 {
     if (g_ctx.ready) return CAKE_HIP_OK;
@@ -355,9 +382,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         const int slices = fewrows_slices(M, N, K, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
-            int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
+            int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
             if (st2) return st2;
-            partial = static_cast<float*>(g_ctx.splitk.ptr);
         }
         return timer.family(0, [&] {
             return launch_sgemm_fewrows(A, B, C, partial, M, N, K, lda, ldb, ldc, accumulate, col_bias,
@@ -369,9 +395,8 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         const int slices = fewrows_nt_slices(N, M, K, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
-            int st2 = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float));
+            int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
             if (st2) return st2;
-            partial = static_cast<float*>(g_ctx.splitk.ptr);
         }
         return timer.family(0, [&] {
             return launch_sgemm_fewrows_nt(B, A, C, partial, N, M, K, ldb, lda, ldc, true, true, accumulate,
@@ -415,15 +440,13 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.tail_k_per_split = plan.tail_k_per_split;
     g.tail_partial = nullptr;
     if (plan.pub.tail_tiles > 0) {
-        st = g_ctx.splitk.reserve((size_t)plan.pub.tail_tiles * plan.pub.tail_split * plan.pub.tile_m *
-                                  plan.pub.tile_n * sizeof(float));
+        st = partial_space(g_ctx.splitk, (size_t)plan.pub.tail_tiles * plan.pub.tail_split * plan.pub.tile_m *
+                                             plan.pub.tile_n * sizeof(float), &g.tail_partial);
         if (st) return st;
-        g.tail_partial = static_cast<float*>(g_ctx.splitk.ptr);
     }
     if (plan.pub.split_k > 1) {
-        st = g_ctx.splitk.reserve((size_t)plan.pub.split_k * M * N * sizeof(float));
+        st = partial_space(g_ctx.splitk, (size_t)plan.pub.split_k * M * N * sizeof(float), &g.partial);
         if (st) return st;
-        g.partial = static_cast<float*>(g_ctx.splitk.ptr);
     }
     st = timer.family(0, [&] { return launch_sgemm(plan.tile_id, a_mode, b_mode, g, plan.pub.grid, stream); });
     if (st) return st;
@@ -491,6 +514,12 @@ int cake_hip_init(int device)
         if (!*e) HIP_TRY(hipEventCreate(e));
     for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.tables, &c.unpacked, &c.linear})
         b->keep_old = true;
+    // this device's copy of the file-scope scratch array (every device has its own, at its own address)
+    if (device < MAX_DEVICES && !g_noalloc_ptr[device]) {
+        void* at = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&at, HIP_SYMBOL(noalloc_scratch)));
+        g_noalloc_ptr[device] = static_cast<float*>(at);
+    }
     if (const char* tuned = std::getenv("CAKE_HIP_TUNE_FILE")) (void)tune_load(tuned);  // optional
     c.ready = true;
     return CAKE_HIP_OK;
@@ -704,6 +733,40 @@ static int sgemm_host_pipelined(const float* A, const float* b_dev, float* C, in
     return timer.stop();
 }
 
+// C = A . B on device operands: the matrix-vector kernels for a single row or column, run_gemm
+// for everything else, a fill for an empty sum.
+static int sgemm_on_device(const float* A, const float* B, float* C, int M, int N, int K, int sched, int accumulate,
+                           const int* tile_override, hipStream_t stream, Timer& timer)
+{
+    int st = CAKE_HIP_OK;
+    if (K == 0) {
+        // empty sum: C = 0 (or unchanged when accumulating); a fill kernel, not a memset node
+        if (!accumulate) {
+            hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream);
+            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
+        }
+    } else if ((M == 1 || N == 1) && !tile_override) {
+        // A product with a single row or column is a matrix-vector product: C[M] = A[M][K] . B[K]
+        // reads A row-major; C[N] = A[K] . B[K][N] is B read as a column-major N x K matrix.
+        const size_t floats = N == 1 ? sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus)
+                                     : sgemv_colmajor_scratch_floats(N, K, g_ctx.model.cus);
+        float* scratch = nullptr;
+        if (floats && (st = partial_space(g_ctx.gemv, floats * sizeof(float), &scratch))) return st;
+        st = timer.family(2, [&] {
+            return N == 1 ? launch_sgemv_rowmajor(A, B, C, M, K, accumulate, scratch, g_ctx.model.cus, stream)
+                          : launch_sgemv_colmajor(B, A, C, N, K, accumulate, scratch, g_ctx.model.cus, stream);
+        });
+        if (st) return st;
+    } else {
+        const bool vec = vec4_loadable(A, B, K, N);
+        const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
+        st = run_gemm(A, B, C, M, N, K, K, N, N, sched, accumulate, tile_override, mode,
+                      mode, stream, timer);
+        if (st) return st;
+    }
+    return CAKE_HIP_OK;
+}
+
 int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K, int sched,
                    int accumulate, const int* tile_override, void* stream_, double* seconds)
 {
@@ -733,33 +796,34 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
 
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
-    if (K == 0) {
-        // empty sum: C = 0 (or unchanged when accumulating); a fill kernel, not a memset node
-        if (!accumulate) {
-            hipError_t e = launch_splitk_reduce(nullptr, c.dev, M, N, N, 0, 0, stream);
-            if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "zero fill failed: %s", hipGetErrorString(e));
-        }
-    } else if ((M == 1 || N == 1) && !tile_override) {
-        // A product with a single row or column is a matrix-vector product: C[M] = A[M][K] . B[K]
-        // reads A row-major; C[N] = A[K] . B[K][N] is B read as a column-major N x K matrix.
-        const size_t floats = N == 1 ? sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus)
-                                     : sgemv_colmajor_scratch_floats(N, K, g_ctx.model.cus);
-        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
-        float* scratch = static_cast<float*>(g_ctx.gemv.ptr);
-        st = timer.family(2, [&] {
-            return N == 1 ? launch_sgemv_rowmajor(a.dev, b.dev, c.dev, M, K, accumulate, scratch, g_ctx.model.cus, stream)
-                          : launch_sgemv_colmajor(b.dev, a.dev, c.dev, N, K, accumulate, scratch, g_ctx.model.cus, stream);
-        });
-        if (st) return st;
-    } else {
-        const bool vec = vec4_loadable(a.dev, b.dev, K, N);
-        const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
-        st = run_gemm(a.dev, b.dev, c.dev, M, N, K, K, N, N, sched, accumulate, tile_override, mode,
-                      mode, stream, timer);
-        if (st) return st;
-    }
+    if ((st = sgemm_on_device(a.dev, b.dev, c.dev, M, N, K, sched, accumulate, tile_override, stream, timer))) return st;
     if ((st = timer.stop())) return st;
     return stage_out(c, stream);
+}
+
+int cake_hip_sgemm_noalloc(const float* A, const float* B, float* C, int M, int N, int K, int sched,
+                           int accumulate, void* stream_)
+{
+    if (M < 0 || N < 0 || K < 0) return fail(CAKE_HIP_ERR_ARG, "negative dimension");
+    if (sched < 0 || sched > CAKE_HIP_NA) return fail(CAKE_HIP_ERR_ARG, "unknown schedule %d", sched);
+    if (M == 0 || N == 0) return CAKE_HIP_OK;
+    if (!A || !B || !C) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
+        return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
+    // nothing is set up here: events, device model and the scratch address come from cake_hip_init
+    if (!g_ctx.ready)
+        return fail(CAKE_HIP_ERR_NO_DEVICE, "cake_hip_sgemm_noalloc needs cake_hip_init to have run: it sets nothing up itself");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_ctx.device >= MAX_DEVICES || !g_noalloc_ptr[g_ctx.device])
+        return fail(CAKE_HIP_ERR_NO_DEVICE, "no scratch address for device %d", g_ctx.device);
+    if (!is_device_pointer(A) || !is_device_pointer(B) || !is_device_pointer(C))
+        return fail(CAKE_HIP_ERR_ARG, "cake_hip_sgemm_noalloc takes device memory only (host operands need staging buffers)");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Timer untimed(stream, nullptr);
+    g_noalloc_call = true;
+    const int st = sgemm_on_device(A, B, C, M, N, K, sched, accumulate, nullptr, stream, untimed);
+    g_noalloc_call = false;
+    return st;
 }
 
 size_t cake_hip_packed_a_size(int M, int K, int p, const cake_hip_blk_dims_t* d,
@@ -1320,8 +1384,7 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
         const int slices = few_x ? fewrows_nt_slices(M, N, K, cus) : fewrows_nt_slices(N, M, K, cus);
         float* partial = nullptr;
         if (slices > 1) {
-            if ((st = g_ctx.splitk.reserve((size_t)slices * M * N * sizeof(float)))) return st;
-            partial = static_cast<float*>(g_ctx.splitk.ptr);
+            if ((st = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial))) return st;
         }
         return timer.family(0, [&] {
             return few_x ? launch_sgemm_fewrows_nt(X, W, C, partial, M, N, K, K, K, N, false, false, accumulate, bias, cus, stream)

@@ -159,6 +159,18 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
                    int sched, int accumulate, const int* tile_override,
                    void* stream, double* seconds);
 
+/* cake_hip_sgemm for callers that must not allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The same kernels as cake_hip_sgemm run on the planner's own choice of tile; the partial sums
+ * that split-K, tail-split and streaming products and the matrix-vector kernels need go into a
+ * 64 MiB array that is part of the library's device image instead of a buffer that grows, and the
+ * call makes no hipMalloc or hipFree.  A, B and C must be device memory; cake_hip_init must have run
+ * (it looks up the array's address on its device); a product whose partial sums would not fit
+ * returns CAKE_HIP_ERR_RANGE and touches nothing.  Every call on a device uses that device's one
+ * array: calls that overlap on one device (different streams) race, calls on one stream do not. */
+int cake_hip_sgemm_noalloc(const float* A, const float* B, float* C, int M, int N, int K,
+                           int sched, int accumulate, void* stream);
+
 /* Same product with A and/or B already in the reference's packed layouts
  * (cake_sgemm with packedA / packedB, src/cake_sgemm.cpp:42-44,64-66), as
  * written by cake_hip_pack_a / cake_hip_pack_b for the same (dims, p, cntx). */
