@@ -7,7 +7,7 @@ arrays are both accepted wherever a matrix is."""
 from ._lib import (KMN, MKN, NKM, NA, SCHED_NAMES, KERNEL_NAMES, BlkDims, CakeHipError, CpuCntx, DeviceInfo,
                    Plan, load)
 from .api import (autotune, cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_size, cake_sgemm_packed_B_size,
-                  cake_sgemm_packed_C_size, cake_sgemv, conv2d, device_info, fill_uniform, im2col,
+                  cake_sgemm_packed_C_size, cake_sconv, cake_sgemv, conv2d, device_info, fill_uniform, im2col,
                   im_2_col, init_block_dims, last_kernel_seconds, linear_backward, linear_forward, linear_forward_wt, sgemm_nt, pack_A, pack_B, pack_C,
                   packed_offset, plan, transpose_mat, tune_clear, tune_count, tune_load, tune_save, unpack_C,
                   update_mr_nr)
@@ -15,7 +15,7 @@ from .api import (autotune, cake_query_cntx, cake_sgemm, cake_sgemm_packed_A_siz
 __all__ = [
     "KMN", "MKN", "NKM", "NA", "SCHED_NAMES", "KERNEL_NAMES", "BlkDims", "CpuCntx", "Plan", "DeviceInfo",
     "CakeHipError", "load", "cake_query_cntx", "update_mr_nr", "init_block_dims", "plan",
-    "cake_sgemm", "cake_sgemv", "pack_A", "pack_B", "pack_C", "unpack_C",
+    "cake_sgemm", "cake_sgemv", "cake_sconv", "pack_A", "pack_B", "pack_C", "unpack_C",
     "cake_sgemm_packed_A_size", "cake_sgemm_packed_B_size", "cake_sgemm_packed_C_size",
     "packed_offset", "im2col", "im_2_col", "conv2d", "fill_uniform", "device_info",
     "last_kernel_seconds", "transpose_mat", "linear_forward", "linear_forward_wt", "linear_backward", "sgemm_nt",

@@ -104,6 +104,7 @@ SIGNATURES = {
     "cake_hip_conv2d_workspace": (C.c_size_t, [_i] * 9),
     "cake_hip_conv2d": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
     "cake_hip_conv2d_im2col": (_i, [_fp, _fp, _fp] + [_i] * 10 + [C.c_void_p, C.c_void_p, _dp]),
+    "cake_hip_sconv": (_i, [_fp, _fp, _fp] + [_i] * 9 + [C.c_void_p, _dp]),
     "cake_hip_transpose": (_i, [_fp, _fp, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_forward": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),
     "cake_hip_linear_forward_wt": (_i, [_fp, _fp, _fp, _fp, _i, _i, _i, C.c_void_p, _dp]),

@@ -314,6 +314,22 @@ def conv2d(inp, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride=1, pad=
     return secs.value
 
 
+def cake_sconv(A, B, Cm, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cake_cntx=None, argv=None,
+               packedA=False, sch=NA) -> float:
+    """cake_sconv (examples/cake_conv.cpp:5-8,765-848): C[Cout][Hout][Wout] += A[Cout][Cin][Hf][Wf] * B[Cin][Hin][Win],
+    one CHW image, no padding; p, cake_cntx and sch are accepted and unused (the reference always
+    runs it K-first).  Returns seconds."""
+    if packedA:
+        raise ValueError("cake_sconv: filters packed by the reference's pack_filters are not supported")
+    _need(A, Cout * Cin * Hf * Wf, "filters")
+    _need(B, Cin * Hin * Win, "input")
+    _need(Cm, Cout * Hout * Wout, "output")
+    secs = C.c_double(0.0)
+    check(load().cake_hip_sconv(_ptr(A, "filters"), _ptr(B, "input"), _ptr(Cm, "output"), Wf, Hf, Win, Hin, Wout, Hout,
+                                Cin, Cout, s, _stream(A, B, Cm), C.byref(secs)), "cake_sconv")
+    return secs.value
+
+
 # ----------------------------------------------------------------------------
 # transpose and the linear layer (include/util.h:32, src/linear.cpp:12-107)
 # ----------------------------------------------------------------------------

@@ -1106,7 +1106,7 @@ size_t cake_hip_conv2d_workspace(int batch, int Cin, int Hin, int Win, int Cout,
 // explicit == 0: gather the column matrix inside the GEMM when the geometry allows it
 static int conv2d_common(const float* in, const float* weights, float* out, int batch, int Cin, int Hin,
                          int Win, int Cout, int Hf, int Wf, int stride, int pad, int out_nchw,
-                         void* workspace, void* stream_, double* seconds, int explicit_cols)
+                         void* workspace, void* stream_, double* seconds, int explicit_cols, int accumulate = 0)
 {
     if (seconds) *seconds = 0;
     int Hout, Wout;
@@ -1123,6 +1123,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         Hout = 1;
     }
     if (!in || !weights || !out) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if (accumulate && out_nchw && batch > 1) return fail(CAKE_HIP_ERR_ARG, "accumulation into a batched NCHW output is not offered");
     const double K_d = (double)Cin * Hf * Wf;
     const double ncols_d = (double)batch * Hout * Wout;
     const double in_elems = (double)batch * Cin * Hin * Win;
@@ -1137,7 +1138,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     Operand i, w, o;
     if ((st = stage_in(in, (size_t)in_elems * 4, 0, true, &i))) return st;
     if ((st = stage_in(weights, (size_t)Cout * K * 4, 1, true, &w))) return st;
-    if ((st = stage_in(out, (size_t)Cout * N * 4, 2, false, &o))) return st;
+    if ((st = stage_in(out, (size_t)Cout * N * 4, 2, accumulate != 0, &o))) return st;
 
     // The on-the-fly gather needs byte offsets into the staged input below 2^31
     // (a chunk of 4 columns must lie in one output row: the product is computed with rows of
@@ -1184,6 +1185,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.tiles_n = g.tiles_n_per_image * batch;
         g.split_k = 1; g.k_per_split = K;
         g.group = g.tiles_m; g.group_along_n = 0;
+        g.accumulate = accumulate;
         if ((st = timer.start())) return st;
         st = timer.family(0, [&] { return launch_sgemm_shortk(g, g_ctx.model.cus, stream); });
         if (st) return st;
@@ -1236,7 +1238,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             // [batch][Cout][HW]: the chunk's images are contiguous; [Cout][batch*HW]: its columns are
             float* dst = o.dev + (out_nchw ? (size_t)b0 * Cout * HW : (size_t)b0 * HW);
             const int Np = nb * Hout * row_n;
-            st = run_gemm(w.dev, nullptr, dst, Cout, Np, K, K, Np, N, CAKE_HIP_NA, 0, nullptr, LOAD_VEC4,
+            st = run_gemm(w.dev, nullptr, dst, Cout, Np, K, K, Np, N, CAKE_HIP_NA, accumulate, nullptr, LOAD_VEC4,
                           one_by_one ? LOAD_IM2COL_1X1 : LOAD_IM2COL_ROW, stream, timer, &cv);
             if (st) return st;
         }
@@ -1262,10 +1264,11 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         return launch_im2col(i.dev, cols, batch, Cin, Hin, Win, Hf, Wf, Hout, Wout, stride, pad, stream);
     });
     if (st) return st;
+    if (accumulate) out_nchw = 0;   // a single image: [Cout][HW] is its NCHW layout
     float* prod = out_nchw ? cn : o.dev;
     const bool vec = vec4_loadable(w.dev, cols, K, N);
     const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
-    st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode,
+    st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, accumulate, nullptr, mode, mode,
                   stream, timer);
     if (st) return st;
     if (out_nchw) {
@@ -1290,6 +1293,19 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out, in
 {
     return conv2d_common(in, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad, out_nchw,
                          workspace, stream, seconds, 1);
+}
+
+int cake_hip_sconv(const float* filters, const float* in, float* out, int Wf, int Hf, int Win, int Hin,
+                   int Wout, int Hout, int Cin, int Cout, int stride, void* stream, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    int ho = 0, wo = 0;
+    if (Cin <= 0 || Cout <= 0 || Hin <= 0 || Win <= 0 || conv_out_dims(Hin, Win, Hf, Wf, stride, 0, &ho, &wo))
+        return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
+    if (ho != Hout || wo != Wout)
+        return fail(CAKE_HIP_ERR_ARG, "a %dx%d filter at stride %d maps %dx%d to %dx%d, not %dx%d", Hf, Wf, stride, Hin,
+                    Win, ho, wo, Hout, Wout);
+    return conv2d_common(in, filters, out, 1, Cin, Hin, Win, Cout, Hf, Wf, stride, 0, 0, nullptr, stream, seconds, 0, 1);
 }
 
 int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* stream_, double* seconds)
@@ -1598,7 +1614,9 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     if ((st = measure(&best, &best.seconds))) return st;
     // a product with a few rows or columns runs on a streaming kernel unless a tile is measured
     // to beat it: that kernel is the default here, and the table keeps no entry when it wins
-    const bool streaming = vec && (fewrows_applies(M, N, K, K, N) || fewrows_nt_applies(N, M, K, N, K, true));
+    // (the same holds for the short-K kernel that walks over tiles)
+    const bool streaming = vec && (fewrows_applies(M, N, K, K, N) || fewrows_nt_applies(N, M, K, N, K, true) ||
+                                   shortk_applies(M, N, K, g_ctx.model.cus));
     double streaming_seconds = 0;
     if (streaming) {
         tune_erase(M, N, K, true);

@@ -322,6 +322,33 @@ float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
     return cols;
 }
 
+// ---- direct convolution --------------------------------------------------------------
+
+double cake_sconv(float* A, float* B, float* C, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
+                  int Cin, int Cout, int s, int p, cake_cntx_t* cake_cntx, char* argv[], bool packedA,
+                  enum sched sch)
+{
+    (void)p; (void)cake_cntx; (void)argv; (void)sch;   // always K-first in the reference (cake_conv.cpp:790)
+    if (packedA) {
+        printf("cake_sconv: filters packed by pack_filters are not supported; pass them as [Cout][Cin][Hf][Wf]\n");
+        exit(1);
+    }
+    const double t0 = wall_seconds();
+    die_on(cake_hip_sconv(A, B, C, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, NULL, NULL), "cake_sconv");
+    return wall_seconds() - t0;
+}
+
+void conv_gemm_checker(float* conv, float* gemm, int M, int N)
+{
+    const float eps = 1e-3f;  // cake_conv.cpp:1219
+    long wrong = 0, correct = 0;
+    for (size_t i = 0; i < (size_t)M * N; ++i) (fabsf(gemm[i] - conv[i]) > eps ? wrong : correct)++;
+    if (wrong)
+        printf("WRONG = %ld , CORRECT = %ld\n", wrong, correct);
+    else
+        printf("CORRECT!\n");
+}
+
 // ---- test helpers (host code) -------------------------------------------------------
 
 void rand_init(float* mat, int r, int c)

@@ -118,6 +118,16 @@ double cake_sgemv(float* A, float* B, float* C, int M, int K, int p, cake_cntx_t
 float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
                 int Cin, int Cout, int s);
 
+// Direct convolution of one CHW image (reference: examples/cake_conv.cpp:5-8,765-848):
+// C[Cout][Hout][Wout] += A[Cout][Cin][Hf][Wf] * B[Cin][Hin][Win], no padding,
+// Hout = (Hin - Hf) / s + 1 and Wout = (Win - Wf) / s + 1.  On the GPU the windows are gathered
+// inside the product, so there is no column matrix either.  packedA (filters from the
+// reference's file-local pack_filters) is not offered: the call prints a message and exits.
+double cake_sconv(float* A, float* B, float* C, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
+                  int Cin, int Cout, int s, int p, cake_cntx_t* cake_cntx, char* argv[] = NULL,
+                  bool packedA = 0, enum sched sch = NA);
+void conv_gemm_checker(float* conv, float* gemm, int M, int N);    // cake_conv.cpp:1216
+
 // ---- test helpers (reference: include/util.h) -------------------------------
 
 void rand_init(float* mat, int r, int c);                          // util.cpp:259

@@ -259,6 +259,14 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
                            int stride, int pad, int out_nchw, void* workspace,
                            void* stream, double* seconds);
 
+/* out[Cout][Hout][Wout] += filters[Cout][Cin][Hf][Wf] * in[Cin][Hin][Win]: the direct convolution
+ * of one CHW image without padding, cake_sconv (examples/cake_conv.cpp:5-8,765-848), whose
+ * micro-kernel starts from the values out already holds (:36-47).  Runs as cake_hip_conv2d does
+ * (columns gathered inside the product, no column matrix).  Hout and Wout must be
+ * (Hin - Hf) / stride + 1 and (Win - Wf) / stride + 1. */
+int cake_hip_sconv(const float* filters, const float* in, float* out, int Wf, int Hf, int Win, int Hin,
+                   int Wout, int Hout, int Cin, int Cout, int stride, void* stream, double* seconds);
+
 /* ---- transpose and the linear layer ---------------------------------------- */
 /* dst[c][r] = src[r][c] for a rows x cols row-major matrix; dst is cols x rows.
  * Replaces transpose_mat (include/util.h:32, src/transpose.cpp:5-29; its blocking
@@ -310,9 +318,10 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
  * other products use that choice whenever the caller gives no tile override.
  * The planner's own choice is always measured first, so the result is never
  * slower than the default by more than timing noise.  A product with few rows of A
- * or columns of B (CAKE_HIP_KERNEL_STREAM_*) runs on a streaming kernel instead of a macro-tile:
+ * or columns of B (CAKE_HIP_KERNEL_STREAM_*) or a short K under many tiles
+ * (CAKE_HIP_KERNEL_SHORT_K) runs on a kernel of its own instead of a macro-tile:
  * that kernel is then the default that is measured, and the table only gets an
- * entry (which from then on replaces the streaming kernel) when a tile beats it.
+ * entry (which from then on replaces that kernel) when a tile beats it.
  * best_plan, best_seconds, default_seconds may be NULL.
  * Successor of the reference's user-tile hook and stubbed simulated-annealing
  * tuner (mcu,kcu,ncu of cake_sgemm, src/block_sizing.cpp:363-368;

@@ -119,6 +119,34 @@ static void conv_case(cake_cntx_t* cntx)
     free(F); free(In); free(Bm); free(x); free(A_p); free(B_p); free(C); free(C_p); free(C2);
 }
 
+// examples/cake_conv.cpp main: the direct convolution against the im2col product of the same
+// filters and image (conv_gemm_checker, :1216-1234), on a geometry whose sizes agree
+static void sconv_case(cake_cntx_t* cntx, int Cin, int Cout, int Hin, int Win, int Hf, int Wf)
+{
+    const int Hout = Hin - Hf + 1, Wout = Win - Wf + 1, p = 4, s = 1;
+    const int M = Cout, K = Cin * Hf * Wf, N = Hout * Wout;
+    float* F = (float*)malloc(sizeof(float) * M * K);
+    float* In = (float*)malloc(sizeof(float) * Cin * Hin * Win);
+    rand_init(F, M, K);
+    rand_init(In, Cin, Hin * Win);
+    float* Out = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_sconv(F, In, Out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cntx);
+    float* Bm = im_2_col(In, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s);
+    float* C = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_sgemm(F, Bm, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, KMN);
+    conv_gemm_checker(Out, C, M, N);
+    bool ok = close_to_naive(F, Bm, Out, M, N, K);
+    for (size_t i = 0; i < (size_t)M * N && ok; ++i)
+        if (fabsf(Out[i] - C[i]) > 1e-3f) ok = false;
+    cake_sconv(F, In, Out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cntx);   // adds to Out
+    for (size_t i = 0; i < (size_t)M * N && ok; ++i)
+        if (fabsf(Out[i] - 2 * C[i]) > 2e-3f) ok = false;
+    char what[128];
+    snprintf(what, sizeof what, "cake_sconv %dx%d filters, %d->%d channels on %dx%d", Hf, Wf, Cin, Cout, Hin, Win);
+    report(what, ok);
+    free(F); free(In); free(Out); free(Bm); free(C);
+}
+
 // beta with the default schedule: whether C is added to follows the schedule init_block_dims
 // resolves from the caller's cntx and p (src/cake_sgemm.cpp:34-35,114), not the device's tiling.
 static void beta_case(int M, int K, int N, int p, cake_cntx_t* cntx)
@@ -219,6 +247,8 @@ int main(int argc, char** argv)
         beta_case(300, 3000, 300, 4, &fixed);
     }
     conv_case(cntx);
+    sconv_case(cntx, 16, 24, 34, 34, 3, 3);
+    sconv_case(cntx, 5, 130, 21, 37, 5, 3);
     gemv_case(cntx, 1024, 777);
     gemv_case(cntx, 37, 5);
     transpose_case(130, 77);

@@ -43,10 +43,12 @@ def test_autotune_picks_a_measured_plan_and_results_stay_right(shape, tmp_path):
     assert cake.plan(M, N, K).as_dict() == now
 
 
-@pytest.mark.parametrize("shape", [(16, 2048, 4096), (4096, 2048, 8)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(16, 2048, 4096), (4096, 2048, 8), (4096, 64, 4096), (2000, 48, 3000)],
+                         ids=lambda s: "x".join(map(str, s)))
 def test_autotune_of_a_streaming_shape(shape):
-    """Few rows or columns: the streaming kernel is the measured default, a tile only enters the
-    table when it is faster, and the product stays right either way."""
+    """Few rows or columns, or a short K under many tiles: the kernel those shapes have of their own
+    is the measured default, a tile only enters the table when it is faster, and the product stays
+    right either way."""
     M, K, N = shape
     plan, best, base = cake.autotune(M, N, K, budget_seconds=2.0)
     print(f"autotune streaming M={M} K={K} N={N} best={best * 1e6:.1f} us default={base * 1e6:.1f} us "

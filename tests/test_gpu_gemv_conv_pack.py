@@ -211,6 +211,40 @@ def test_conv2d_matches_oracle(geom, nchw, explicit):
     assert np.max(np.abs(got - cpu) / np.maximum(S, 1e-30)) <= TOL
 
 
+@pytest.mark.parametrize("geom", [(8, 14, 12, 20, 3, 3, 1), (64, 34, 34, 96, 3, 3, 1), (3, 37, 29, 10, 5, 3, 1),
+                                  (16, 33, 33, 24, 3, 3, 2), (40, 19, 23, 33, 1, 1, 1), (5, 30, 31, 7, 7, 7, 3)], ids=str)
+def test_cake_sconv_accumulates_the_direct_convolution(geom):
+    """cake_sconv (examples/cake_conv.cpp:765-848): one CHW image, no padding, the result added
+    to what C holds (its micro-kernel starts from C, :36-47) -- against the naive fp64 convolution,
+    against the oracle's im_2_col -> cake_sgemm sequence (the reference's own cross-check,
+    conv_gemm_checker :1216-1234), on host and on device memory, and twice to see it add."""
+    Cin, Hin, Win, Cout, Hf, Wf, s = geom
+    Hout, Wout = (Hin - Hf) // s + 1, (Win - Wf) // s + 1
+    print(f"cake_sconv geom={geom}", flush=True)
+    inp = oracle.uniform((Cin, Hin, Win), 61)
+    wt = oracle.uniform((Cout, Cin, Hf, Wf), 62)
+    C0 = oracle.uniform((Cout, Hout, Wout), 63)
+    ref64, S = oracle.conv_naive_f64(inp[None], wt, s, 0)
+    ref64, S = ref64[0], S[0]
+    out = C0.copy()
+    cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, 4)
+    assert np.max(np.abs(out.astype(np.float64) - C0 - ref64) / (S + np.abs(C0))) <= TIGHT
+    cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, 4)
+    assert np.max(np.abs(out.astype(np.float64) - C0 - 2 * ref64) / (2 * S + np.abs(C0))) <= TIGHT
+    import torch
+    tw, ti, to = (torch.from_numpy(x).cuda() for x in (wt, inp, C0))
+    cake.cake_sconv(tw, ti, to, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, 4)
+    torch.cuda.synchronize()
+    dev = to.cpu().numpy()
+    assert np.max(np.abs(dev.astype(np.float64) - C0 - ref64) / (S + np.abs(C0))) <= TIGHT
+    if s == 1:
+        cols = oracle.im_2_col(inp, Hf, Wf, Hout, Wout)
+        cpu = oracle.cake_sgemm(wt.reshape(Cout, -1), cols, 4, oracle.make_cntx(), sch=oracle.KMN).reshape(Cout, Hout, Wout)
+        assert np.max(np.abs(dev - C0 - cpu) / (S + np.abs(C0))) <= TOL
+    with pytest.raises(cake.CakeHipError):
+        cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout - 1, Hout, Cin, Cout, s, 4)
+
+
 @pytest.mark.parametrize("geom", [(16, 16, 56, 56, 256, 1, 1), (70, 7, 30, 30, 130, 1, 1), (256, 5, 21, 21, 100, 1, 1),
                                   (16, 64, 56, 56, 256, 1, 1), (16, 65, 56, 56, 256, 1, 1)], ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
