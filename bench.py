@@ -16,8 +16,10 @@ timed steps between two synchronisations.  Prints ONE JSON line:
   cpu_baseline   the CPU restatement of the reference cake_sgemm (oracle/, kind
                  "port") on this host's physical cores, same inputs, full 8192^3
                  product once after a small warm-up
-  extras         the other BASELINE configs (not bench lines: reported for
-                 information, each with its own roofline figure)
+  extras         the other BASELINE configs and a few more workloads (not bench
+                 lines: reported for information), each with a roofline object
+                 of its own and, for the BASELINE configs, the CPU restatement
+                 of the reference's call timed beside it
 """
 from __future__ import annotations
 
@@ -36,14 +38,43 @@ METRIC = "fp32 GEMM TFLOP/s @8192^3 (% MFMA peak); GEMV GB/s (% HBM peak)"
 MFMA_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 
-# HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script, each scaled by what the same counter reads for a plain 256 MiB
-# copy (FETCH_SIZE reads half the true size, WRITE_SIZE the true size).  The
-# summaries are kept under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"sgemm_8192": 4456489 * 1024, "sgemv_16384": (1049023 + 256) * 1024,
-                          # streaming kernel + its slice reduction, 16 x 16384 x 16384 and transposes of it
-                          "fewrows_nn": (1056751 + 4096 + 3490 + 1024) * 1024,
-                          "fewrows_nt": (1056793 + 3095 + 3490 + 1024) * 1024}
+# HBM-side bytes per launch of the kernels behind each workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script (KiB per dispatch, each scaled by what the same counter reads for a
+# plain 256 MiB copy: FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0000; `--copy-calibration`).  Every entry
+# names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
+KIB = 1024
+MEASURED_TRAFFIC = {
+    "sgemm_8192": ((4194306 + 262144) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,0>` grid 1048576 (8192^3)"),
+    "sgemm_1024": ((24688 + 4096) * KIB, "row `sgemm_tile_kernel<Tile<64,64,..>,0,0>` (1024^3)"),
+    "sgemm_tall_skinny": ((266447 + 32768) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,0>` grid 131072 (65536 x 1024 x 128)"),
+    "sgemv_16384_rowmajor": ((1049023 + 256) * KIB, "row `sgemv_rowmajor_wg_kernel<2,8>` (GEMV 16384^2, row-major A)"),
+    "sgemv_16384_colmajor": ((1049552 + 576) * KIB, "row `sgemv_colmajor_kernel<true>` + `sgemv_slice_reduce_kernel` (GEMV 16384^2, column-major A)"),
+    "conv_c5_gather": ((100370 + 111537 + 212453 + 116736) * KIB,
+                       "rows `pad_planes_kernel` + `sgemm_tile_kernel<Tile<128,128,..>,0,4>` + `tail_reduce_kernel`"),
+    "conv_c5_two_step": ((112692 + 903172 + 1025061 + 114688 + 100365 + 100352) * KIB,
+                         "rows `im2col_kernel<3>` + `sgemm_tile_kernel<Tile<128,128,..>,0,0>` grid 458752 + `cn_to_nchw_vec_kernel`"),
+    "shortk_256x64x100352": ((25697 + 100352) * KIB, "row `sgemm_shortk_kernel<Tile<64,64,64,32,32>,0,true>` (256 x 100352 x 64)"),
+    "conv_1x1_14x14": ((15519 + 25312) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,5>` (conv 1x1, 32x256x14x14 -> 1024)"),
+    "fewrows_nn": ((1060242 + 5120) * KIB, "row `sgemm_fewrows_nn_kernel<1,2>` + `splitk_reduce_kernel` (16 x 16384 x 16384)"),
+    "fewrows_nt": ((1060285 + 4119) * KIB, "row `sgemm_fewrows_nt_kernel<true,1>` + `splitk_reduce_kernel` (16384 x 16 x 16384)"),
+    "linear_fwd_8192x4096x4096": (int(1.208e9), "row `sgemm_tile_kernel<Tile<256,128,..>,0,2>` grid 524288 (linear forward)"),
+}
+
+
+def roofline(bound, work, seconds, traffic_key=None, **more):
+    """The roofline object of one workload: `work` algorithmic FLOPs (bound "mfma") or bytes (bound
+    "hbm") per launch over the measured seconds per launch, against the published peak."""
+    if bound == "mfma":
+        achieved, peak, unit, key = work / seconds / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s", "algorithmic_flops_per_launch"
+    else:
+        achieved, peak, unit, key = work / seconds / 1e9, HBM_PEAK_GBPS, "GB/s", "algorithmic_bytes_per_launch"
+    traffic, source = MEASURED_TRAFFIC.get(traffic_key, (None, None))
+    r = {"bound": bound, "achieved": round(achieved, 3 if bound == "mfma" else 1), "peak": peak, "unit": unit,
+         "frac": round(achieved / peak, 4), "traffic": traffic, key: work}
+    if source:
+        r["traffic_source"] = "profiles/all_kernels_hbm_traffic_pmc.md, " + source
+    r.update(more)
+    return r
 
 
 def main() -> int:
@@ -158,26 +189,31 @@ def main() -> int:
             "device": info.arch.decode(),
             "cus": info.cus,
         },
-        "roofline": {
-            "kernel": f"sgemm_tile_kernel<Tile<{plan.tile_m},{plan.tile_n},{plan.tile_k},{plan.wave_m},{plan.wave_n},...>,0,0>",
-            "bound": "mfma",
-            "achieved": round(achieved, 3),
-            "peak": MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["sgemm_8192"],
-            "algorithmic_flops_per_launch": flops,
-            "avg_launch_ms": round(k_avg * 1e3, 4),
-            "min_launch_ms": round(k_min * 1e3, 4),
-        },
+        "roofline": roofline("mfma", flops, k_avg, "sgemm_8192",
+                             kernel=f"sgemm_tile_kernel<Tile<{plan.tile_m},{plan.tile_n},{plan.tile_k},{plan.wave_m},{plan.wave_n},...>,0,0>",
+                             avg_launch_ms=round(k_avg * 1e3, 4), min_launch_ms=round(k_min * 1e3, 4)),
         "check": {"max_rel_err_sampled_rows": check_err, "tolerance": 1e-4},
     }
 
     # ------------------------------------------------------------ other configs
+    p_cores = oracle.physical_cores()
+    cpu_cx = oracle.query_cntx()
+
+    def cpu_leg(run, work, unit, sample, repeats=3):
+        """The CPU restatement of the reference's call on this host's physical cores: one warm-up,
+        then the median of `repeats` runs; `run` returns the seconds the call itself reports."""
+        if args.no_cpu:
+            return None
+        run()
+        secs = float(np.median([run() for _ in range(repeats)]))
+        scale = 1e12 if unit == "TFLOP/s" else 1e9
+        return {"value": round(work / secs / scale, 4), "unit": unit, "cores": p_cores, "kind": "port",
+                "seconds": round(secs, 5), "sample": sample}
+
     if not args.no_extras:
         extras = []
 
-        def gemm_extra(name, M, N, K, streaming_kernel=None, traffic=None):
+        def gemm_extra(name, M, N, K, traffic_key=None, streaming_kernel=None, cpu=False):
             a, b = dev_uniform((M, K), 1), dev_uniform((K, N), 2)
             c = torch.zeros((M, N), dtype=torch.float32, device=dev)
             p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
@@ -186,41 +222,58 @@ def main() -> int:
             pl = cake.plan(M, N, K)
             fl = 2.0 * M * N * K
             by = 4.0 * (M * K + K * N + M * N)
+            e = {"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
+                 "compulsory_GBps": round(by / avg / 1e9, 1), "kernel_family": cake.KERNEL_NAMES[pl.kernel]}
             if streaming_kernel:   # few rows or columns: bound by reading the large operand once
-                extras.append({"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
-                               "kernel": streaming_kernel, "kernel_family": cake.KERNEL_NAMES[pl.kernel],
-                               "roofline": {"bound": "hbm", "achieved": round(by / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
-                                            "unit": "GB/s", "frac": round(by / avg / 1e9 / HBM_PEAK_GBPS, 4),
-                                            "traffic": traffic, "algorithmic_bytes_per_launch": by}})
-                return
-            extras.append({"workload": name, "ms": round(avg * 1e3, 4), "tflops": round(fl / avg / 1e12, 2),
-                           "frac_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4),
-                           "compulsory_GBps": round(by / avg / 1e9, 1),
-                           "kernel_family": cake.KERNEL_NAMES[pl.kernel],
-                           "tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
-                           "schedule": cake.SCHED_NAMES[pl.sched]})
+                e["kernel"] = streaming_kernel
+                e["roofline"] = roofline("hbm", by, avg, traffic_key)
+            else:
+                e.update({"tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
+                          "schedule": cake.SCHED_NAMES[pl.sched]})
+                e["roofline"] = roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by)
+            if cpu:
+                Ah, Bh = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+                dims = {}
 
-        gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024)
-        gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024)
-        gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64)
-        gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384,
-                   "sgemm_fewrows_nn_kernel + splitk_reduce_kernel", MEASURED_TRAFFIC_BYTES["fewrows_nn"])
-        gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384,
-                   "sgemm_fewrows_nt_kernel + splitk_reduce_kernel", MEASURED_TRAFFIC_BYTES["fewrows_nt"])
+                def run():
+                    _, secs, x = oracle.cake_sgemm(Ah, Bh, p_cores, cpu_cx, return_time=True)
+                    dims["x"] = x
+                    return secs
+                e["cpu_baseline"] = cpu_leg(run, fl, "TFLOP/s", "")
+                if e["cpu_baseline"]:
+                    x = dims["x"]
+                    e["cpu_baseline"]["sample"] = (f"the full product, cake_sgemm with the reference's default schedule "
+                                                   f"({oracle.SCHED_NAMES[x.sch]}, m_c=k_c={x.m_c}, n_c={x.n_c}); median of 3 after a warm-up")
+            extras.append(e)
+
+        gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024, "sgemm_1024", cpu=True)
+        gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024, "sgemm_tall_skinny", cpu=True)
+        gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64, "shortk_256x64x100352")
+        gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
+                   "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
+        gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
+                   "sgemm_fewrows_nt_kernel + splitk_reduce_kernel")
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
         yg = torch.zeros((m,), dtype=torch.float32, device=dev)
         gbytes = 4.0 * (m * m + m + m)
-        for col, label in ((0, "row-major A (configs[3])"), (1, "column-major A (cake_sgemv's own layout)")):
+        gemv_cpu = None
+        if not args.no_cpu:
+            # cake_sgemv as examples/cake_gemv.cpp runs it: column-major A, m_r = 8, y accumulates
+            Agh, xgh = oracle.uniform((m, m), 1), oracle.uniform(m, 3)
+            gcx = oracle.query_cntx()
+            gcx.mr = 8
+            gemv_cpu = cpu_leg(lambda: oracle.cake_sgemv(Agh, xgh, p_cores, gcx, M=m, K=m, return_time=True)[1], gbytes, "GB/s",
+                               "the full 16384 x 16384 cake_sgemv (column-major A, the reference's own layout); median of 3 after a warm-up")
+            del Agh
+        for col, label, key in ((0, "row-major A (configs[3])", "sgemv_16384_rowmajor"),
+                                (1, "column-major A (cake_sgemv's own layout)", "sgemv_16384_colmajor")):
             _, avg, _ = time_steps(lambda: _lib.check(
                 lib.cake_hip_sgemv(Ag.data_ptr(), xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None), "sgemv"), 50, 10, 40.0)
             extras.append({"workload": f"sgemv 16384x16384 {label}", "us": round(avg * 1e6, 2),
-                           "GBps": round(gbytes / avg / 1e9, 1),
-                           "roofline": {"bound": "hbm", "achieved": round(gbytes / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
-                                        "unit": "GB/s", "frac": round(gbytes / avg / 1e9 / HBM_PEAK_GBPS, 4),
-                                        "traffic": MEASURED_TRAFFIC_BYTES["sgemv_16384"],
-                                        "algorithmic_bytes_per_launch": gbytes}})
+                           "GBps": round(gbytes / avg / 1e9, 1), "roofline": roofline("hbm", gbytes, avg, key),
+                           "cpu_baseline": gemv_cpu})
         del Ag
 
         Bn, Cc, H = 32, 256, 56
@@ -229,15 +282,38 @@ def main() -> int:
         ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
         ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
         cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
+        cby = 4.0 * (Bn * Cc * H * H + Cc * Cc * 9 + Bn * Cc * H * H)      # input + weights + output
+        conv_cpu = None
+        if not args.no_cpu:
+            # the reference's sequence for one image (examples/cake_conv.cpp:1007-1066): im_2_col of the
+            # zero-padded CHW image, then cake_sgemm (which packs both operands); 2 of the 32 images
+            imgs = oracle.uniform((2, Cc, H, H), 5)
+            wh = oracle.uniform((Cc, Cc * 9), 4)
+            padded = np.zeros((2, Cc, H + 2, H + 2), np.float32)
+            padded[:, :, 1:-1, 1:-1] = imgs
+
+            def conv_cpu_run():
+                total = 0.0
+                for b in range(2):
+                    t0 = time.perf_counter()
+                    cols = oracle.im_2_col(padded[b], 3, 3, H, H)
+                    total += time.perf_counter() - t0
+                    total += oracle.cake_sgemm(wh, cols, p_cores, cpu_cx, sch=oracle.KMN, return_time=True)[1]
+                return total
+            conv_cpu = cpu_leg(conv_cpu_run, cfl * 2 / Bn, "TFLOP/s",
+                               "2 of the 32 images: im_2_col + cake_sgemm(KMN) per image as examples/cake_conv.cpp does "
+                               "(M=256, K=2304, N=3136 each); median of 3 after a warm-up")
         # output written as NCHW: inside the GEMM's epilogue on the gather path, a layout pass on the other
-        for fn, label in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM, NCHW output"),
-                          (lib.cake_hip_conv2d_im2col, "im2col kernel, GEMM (the reference's two steps), NCHW layout pass")):
+        for fn, label, key in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM, NCHW output", "conv_c5_gather"),
+                               (lib.cake_hip_conv2d_im2col, "im2col kernel, GEMM (the reference's two steps), NCHW layout pass",
+                                "conv_c5_two_step")):
             _, avg, _ = time_steps(lambda: _lib.check(
                 fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 1,
                    ws.data_ptr(), stream, None), "conv2d"), 20, 3, 40.0)
             extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
                            "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
-                           "frac_mfma_peak": round(cfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                           "roofline": roofline("mfma", cfl, avg, key, algorithmic_bytes_per_launch=cby),
+                           "cpu_baseline": conv_cpu})
         del inp, oc, ws
         # a 1 x 1 layer: planes read in place (no staged copy, no tap table), NCHW output
         Pb, Pc, Ph, Po = 32, 256, 14, 1024
@@ -246,12 +322,13 @@ def main() -> int:
         pws_bytes = lib.cake_hip_conv2d_workspace(Pb, Pc, Ph, Ph, Po, 1, 1, 1, 0)
         pws = torch.empty((max(1, (pws_bytes + 3) // 4),), dtype=torch.float32, device=dev)
         pfl = 2.0 * Po * Pc * (Pb * Ph * Ph)
+        pby = 4.0 * (Pb * Pc * Ph * Ph + Po * Pc + Pb * Po * Ph * Ph)
         _, avg, _ = time_steps(lambda: _lib.check(
             lib.cake_hip_conv2d(pin.data_ptr(), pw.data_ptr(), po.data_ptr(), Pb, Pc, Ph, Ph, Po, 1, 1, 1, 0, 1,
                                 pws.data_ptr(), stream, None), "conv2d"), 50, 5, 40.0)
         extras.append({"workload": "conv 1x1, batch 32, 256->1024 ch, 14x14, NCHW output",
                        "us": round(avg * 1e6, 2), "tflops": round(pfl / avg / 1e12, 2),
-                       "frac_mfma_peak": round(pfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                       "roofline": roofline("mfma", pfl, avg, "conv_1x1_14x14", algorithmic_bytes_per_launch=pby)})
         del pin, po, pws
 
         # the linear layer (src/linear.cpp): batch 8192, 4096 -> 4096 features, with bias
@@ -267,13 +344,13 @@ def main() -> int:
                                         stream, None), "linear_forward"), 20, 3, 40.0)
         extras.append({"workload": "linear forward, batch 8192, 4096->4096, bias (weights read as they lie, no transposed copy)",
                        "ms": round(avg * 1e3, 4), "tflops": round(lfl / avg / 1e12, 2),
-                       "frac_mfma_peak": round(lfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                       "roofline": roofline("mfma", lfl, avg, "linear_fwd_8192x4096x4096")})
         _, avg, _ = time_steps(lambda: _lib.check(
             lib.cake_hip_linear_backward(lg.data_ptr(), lx.data_ptr(), lw.data_ptr(), lgx.data_ptr(), lgw.data_ptr(),
                                          lgb.data_ptr(), Lm, Ln, Lk, stream, None), "linear_backward"), 20, 3, 40.0)
         extras.append({"workload": "linear backward, same layer (two products, one transpose, bias sums)",
                        "ms": round(avg * 1e3, 4), "tflops": round(2 * lfl / avg / 1e12, 2),
-                       "frac_mfma_peak": round(2 * lfl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                       "roofline": roofline("mfma", 2 * lfl, avg)})
         del lx, lg, ly, lgx
         # a small batch: the weights are streamed once as they lie, no transposed copy
         Sm, Sk, Sn = 16, 16384, 16384
@@ -286,15 +363,12 @@ def main() -> int:
         extras.append({"workload": "linear forward, batch 16, 16384->16384, bias",
                        "us": round(avg * 1e6, 2), "tflops": round(2.0 * Sm * Sn * Sk / avg / 1e12, 2),
                        "kernel": "sgemm_fewrows_nt_kernel + splitk_reduce_kernel",
-                       "roofline": {"bound": "hbm", "achieved": round(sby / avg / 1e9, 1), "peak": HBM_PEAK_GBPS,
-                                    "unit": "GB/s", "frac": round(sby / avg / 1e9 / HBM_PEAK_GBPS, 4),
-                                    "traffic": MEASURED_TRAFFIC_BYTES["fewrows_nt"], "algorithmic_bytes_per_launch": sby}})
+                       "roofline": roofline("hbm", sby, avg, "fewrows_nt")})
         out["extras"] = extras
 
     # -------------------------------------------------------------- CPU baseline
     if not args.no_cpu:
-        p = oracle.physical_cores()
-        cx = oracle.query_cntx()
+        p, cx = p_cores, cpu_cx
         Ah, Bh = oracle.uniform((n, n), 1), oracle.uniform((n, n), 2)
         oracle.cake_sgemm(Ah[:2048, :2048].copy(), Bh[:2048, :2048].copy(), p, cx)   # warm-up
         _, secs, dims = oracle.cake_sgemm(Ah, Bh, p, cx, return_time=True)
