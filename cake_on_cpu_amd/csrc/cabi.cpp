@@ -91,7 +91,7 @@ struct Context {
     cake_hip_device_t info{};
     DeviceModel model;
     DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
-    DeviceBuffer splitk, gemv, conv, conv_taps, tables, unpacked, linear;
+    DeviceBuffer splitk, gemv, conv, conv_taps, conv_filters, tables, unpacked, linear;
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
     // host <-> device transfers of large host operands: two pinned buffers, a stream, an event each
@@ -512,7 +512,7 @@ int cake_hip_init(int device)
     if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
     for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
         if (!*e) HIP_TRY(hipEventCreate(e));
-    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.tables, &c.unpacked, &c.linear})
+    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.conv_filters, &c.tables, &c.unpacked, &c.linear})
         b->keep_old = true;
     // this device's copy of the file-scope scratch array (every device has its own, at its own address)
     if (device < MAX_DEVICES && !g_noalloc_ptr[device]) {
@@ -532,7 +532,7 @@ int cake_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     for (DeviceBuffer& b : g_ctx.stage) b.release();
     g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
-    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.conv_taps.release();
+    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.conv_taps.release(); g_ctx.conv_filters.release();
     for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1], &g_ctx.copy_done[0], &g_ctx.copy_done[1]}) {
         if (*e) (void)hipEventDestroy(*e);
         *e = nullptr;
@@ -1189,6 +1189,55 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         if ((st = timer.start())) return st;
         st = timer.family(0, [&] { return launch_sgemm_shortk(g, g_ctx.model.cus, stream); });
         if (st) return st;
+        if ((st = timer.stop())) return st;
+        return stage_out(o, stream);
+    }
+    // Stride 1 with whole blocks of 32 channels and maps up to about 60 pixels wide: the input is
+    // read where it lies, a patch of it per workgroup and channel block kept in LDS with the zero
+    // padding around it (sgemm_conv_patch.hip) -- no padded copy, no table of tap offsets.
+    int patch_rows = 0, patch_pitch = 0;
+    if (!explicit_cols && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_k(Cin, Hf, Wf)) &&
+        conv_patch_geometry(batch, Cin, Hin, Win, Hf, Wf, stride, pad, Hout, Wout, &patch_rows, &patch_pitch)) {
+        const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n;
+        if ((st = g_ctx.conv_filters.reserve((size_t)Cout * Kp * sizeof(float)))) return st;
+        float* wt = static_cast<float*>(g_ctx.conv_filters.ptr);
+        const int tile[4] = {256, 128, 32, 0};
+        GemmPlan plan;
+        if ((st = plan_gemm(Cout, Np, Kp, CAKE_HIP_NA, tile, true, g_ctx.model, &plan))) return fail(st, "conv2d: no plan");
+        GemmArgs g{};
+        g.A = wt; g.B = nullptr; g.C = o.dev;
+        g.M = Cout; g.N = Np; g.K = Kp;
+        g.lda = Kp; g.ldb = Np; g.ldc = N;
+        g.tiles_m = plan.pub.tiles_m; g.tiles_n = plan.pub.tiles_n;
+        g.split_k = 1; g.k_per_split = Kp;
+        g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
+        g.accumulate = accumulate;
+        // tiles of a thin last round are cut along K in whole channel blocks
+        int grid = g.tiles_m * g.tiles_n;
+        if (plan.pub.tail_tiles > 0) {
+            const int block_k = 32 * taps, blocks = Kp / block_k;
+            const int per = (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
+            const int slices = (blocks + per - 1) / per;
+            if (slices > 1) {
+                g.tail_tiles = plan.pub.tail_tiles;
+                g.tail_split = slices;
+                g.tail_k_per_split = per * block_k;
+                if ((st = partial_space(g_ctx.splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
+                    return st;
+                grid += g.tail_tiles * (slices - 1);
+            }
+        }
+        ConvGeom& cv = g.conv;
+        cv.in = i.dev;
+        cv.in_bytes = (unsigned)(in_elems * 4);
+        cv.Cin = Cin; cv.Hout = Hout; cv.Wout = Wout; cv.row_n = row_n;
+        cv.out_nchw = out_nchw ? 1 : 0;
+        cv.batch = batch; cv.Hin = Hin; cv.Win = Win; cv.pad = pad; cv.Hf = Hf; cv.Wf = Wf;
+        cv.patch_rows = patch_rows; cv.patch_pitch = patch_pitch;
+        if ((st = timer.start())) return st;
+        if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, taps, stream); }))) return st;
+        if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;
+        if (g.tail_tiles > 0 && (st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); }))) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);
     }

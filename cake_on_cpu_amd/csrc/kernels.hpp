@@ -37,6 +37,9 @@ struct ConvGeom {
     const int* tap_table;   // byte offset of tap k = (c, h, w) inside one image, K + CONV_TAP_TABLE_EXTRA entries
     int tap_stride;         // 1 x 1 filters (LOAD_IM2COL_1X1): bytes from channel to channel, instead of the table
     int out_nchw;           // epilogue writes C as [batch][M][Hout*Wout] instead of [M][N]
+    // sgemm_conv_patch.hip only (the input read where it lies, `in` = the NCHW input itself):
+    int batch, Hin, Win, pad, Hf, Wf;
+    int patch_rows, patch_pitch;   // rows and floats per row of the input patch a workgroup keeps in LDS
 };
 
 struct GemmArgs {
@@ -151,6 +154,19 @@ hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch
 // [Cout][batch*HW] -> [batch][Cout][HW]
 hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, int HW,
                              hipStream_t stream);
+
+// Stride-1 convolutions that read the input where it lies (sgemm_conv_patch.hip).  The product is
+// out[Cout][n] = Wt[Cout][K'] . B with K' = conv_patch_k(...) walked as (channel block of 32, tap,
+// channel); Wt is the filters re-laid to that order by launch_conv_filter_relayout.
+// conv_patch_geometry: false when the kernel does not take the geometry, else the patch's shape.
+enum { CONV_PATCH_PLANE = 512 };   // floats per channel of the LDS patch: rows x pitch must fit
+bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout,
+                         int Wout, int* rows, int* pitch);
+int conv_patch_k(int Cin, int Hf, int Wf);
+hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int taps, hipStream_t stream);
+// args as for launch_sgemm with the 256 x 128 x 32 tile; K slices (tail tiles) must be whole channel
+// blocks of 32 * Hf * Wf
+hipError_t launch_sgemm_conv_patch(const GemmArgs& args, int grid, hipStream_t stream);
 
 hipError_t launch_fill_uniform(float* dst, size_t n, uint64_t seed, hipStream_t stream);
 hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stream);

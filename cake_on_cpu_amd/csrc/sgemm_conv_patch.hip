@@ -1,0 +1,354 @@
+// sgemm_conv_patch.hip -- stride-1 convolution as an implicit GEMM that reads the NCHW input
+// where it lies (the direct convolution of examples/cake_conv.cpp:31-258,614-716 on the MFMA
+// macro-tile): no padded copy, no column matrix, no table of tap offsets.
+//
+// out[co][n] = sum_k' Wt[co][k'] * B[k'][n] with the sum walked channel block by channel block:
+//     k' = (cb * taps + tap) * 32 + c,   channel = cb * 32 + c,   tap = h * Wf + w
+// (the order of a sum is free as long as both operands agree; the filters are re-laid to it by
+// conv_filter_relayout_kernel, 2 MB for 256 x 256 x 3 x 3).  A K stage of 32 is then 32 channels
+// under ONE filter tap, so B[k'][n] = patch[c][row(n) + h][col(n) + w] for a patch of the input
+// that stays in LDS for all taps of a channel block:
+//   * the patch holds, for 32 channels, the R input rows the tile's pixels can reach and whole
+//     rows of P floats: 4 + Win + pad columns, the image's own starting at column 4 so that the
+//     16-byte global loads land 16-byte aligned in LDS.  Rows above and below an image and the
+//     margins left and right of a row are zero: the padding exists in LDS only.  Rows come from
+//     the "virtual" sequence image 0 padded, image 1 padded, ...: a tile whose pixels straddle two
+//     images sees the lower margin of one and the upper margin of the next as distinct rows;
+//   * the MFMA's B operand of lane n for stage (tap, group of 8 channels) is a 4-byte LDS read at
+//     pixel(n) + tap offset + channel * PLANE: the pixel part is fixed per lane, the tap part per
+//     stage, the channel part an immediate -- no integer work between the MFMAs;
+//   * A (the filters) walks through the usual double-buffered stages; the patch is loaded once per
+//     channel block (8 x 16 bytes per thread for 9 stages, where the gather from a staged copy
+//     issued 2 per stage), at the start of the block's last stage, and swapped in between that
+//     stage's barrier and its last operand group.
+// Everything else -- tile raster, tail tiles cut along K, epilogue with the NCHW layout -- is the
+// macro-tile kernel's (sgemm_tile.hpp).
+#include "sgemm_tile.hpp"
+
+namespace cake {
+
+namespace {
+
+using TilePatch = Tile<256, 128, 32, 64, 64, 2, 1, 1>;   // 8 waves of 64 x 64, two register stages for A
+
+constexpr int PATCH_PLANE_FLOATS = CONV_PATCH_PLANE;      // floats per channel of the patch (rows x pitch fit in it)
+constexpr int PATCH_CHANNELS = 32;                        // = BK: one tap of 32 channels per K stage
+constexpr int PATCH_FLOATS = PATCH_PLANE_FLOATS * PATCH_CHANNELS;
+
+template <class T>
+constexpr int patch_smem_bytes() { return (2 * T::A_STAGE + PATCH_FLOATS) * 4; }
+
+// Everything about the operands that is fixed per thread for a whole tile.
+template <class T>
+struct PatchLoader {
+    static constexpr int PATCH_ITERS = PATCH_FLOATS / 4 / T::THREADS;   // 16-byte chunks of a patch per thread
+    static_assert(PATCH_FLOATS / 4 % T::THREADS == 0, "patch chunks are dealt evenly");
+    int a_off[T::A_ITERS];      // byte offset from the A tile origin, or BUF_OOB for rows >= M
+    const float* a_base;        // Wt + m0 * lda
+    unsigned a_elems;
+    int p_off[PATCH_ITERS];     // byte offset of the chunk inside channel block 0 of the input, or BUF_OOB
+    int p_lds[PATCH_ITERS];     // where it goes in the patch (floats, a multiple of 4), or -1; the two low bits
+                                // say how many of its 4 floats hang over the end of the row (the last chunk may)
+    f32x4 pr[PATCH_ITERS];      // the next block's patch on its way
+    const float* in;
+    unsigned in_bytes;
+    unsigned block_bytes;       // bytes of the input between channel blocks
+    float* patch;
+
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int tid, float* patch_)
+    {
+        const ConvGeom& cv = g.conv;
+        a_base = g.A + (size_t)m0 * g.lda;
+        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            a_off[it] = (m0 + r < g.M) ? (r * g.lda + (c % (T::BK / 4)) * 4) * 4 : BUF_OOB;
+        }
+        in = cv.in;
+        in_bytes = cv.in_bytes;
+        block_bytes = (unsigned)PATCH_CHANNELS * cv.Hin * cv.Win * 4u;
+        patch = patch_;
+        const int wc = (cv.Win + 3) >> 2;                 // chunks per input row
+        const int per_channel = cv.patch_rows * wc;
+        const int total = PATCH_CHANNELS * per_channel;
+        const int vrows = cv.Hin + 2 * cv.pad;            // rows of a padded image
+#pragma unroll
+        for (int it = 0; it < PATCH_ITERS; ++it) {
+            const int q = tid + it * T::THREADS;
+            const int c = q / per_channel, rem = q - c * per_channel;
+            const int r = rem / wc, j = rem - r * wc;
+            const int v = v0 + r;
+            const int b = v / vrows, hi = v - b * vrows - cv.pad;
+            const bool data = q < total && b < cv.batch && hi >= 0 && hi < cv.Hin;
+            p_off[it] = data ? (((b * cv.Cin + c) * cv.Hin + hi) * cv.Win + 4 * j) * 4 : BUF_OOB;
+            p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : -1;
+        }
+    }
+
+    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
+    {
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
+    }
+
+    // chunk `it` of channel block cb's patch (rows outside an image read as zero).  cb must be a
+    // block of the input: the record count is a plain difference on purpose (a saturating one only
+    // exists as a vector instruction, and a record count in a vector register makes the compiler
+    // loop over the load).
+    template <int IT>
+    __device__ __forceinline__ void load_patch_chunk(int cb)
+    {
+        const unsigned skip = (unsigned)cb * block_bytes;
+        pr[IT] = buffer_load_f32x4(reinterpret_cast<const float*>(reinterpret_cast<const char*>(in) + skip), p_off[IT],
+                                   in_bytes - skip);
+    }
+    template <int IT = 0>
+    __device__ __forceinline__ void load_patch(int cb)
+    {
+        if constexpr (IT < PATCH_ITERS) {
+            load_patch_chunk<IT>(cb);
+            load_patch<IT + 1>(cb);
+        }
+    }
+
+    __device__ __forceinline__ void store_patch()
+    {
+#pragma unroll
+        for (int it = 0; it < PATCH_ITERS; ++it) {
+            f32x4 v = pr[it];
+            const int over = p_lds[it] & 3;
+            if (over > 0) v[3] = 0.f;
+            if (over > 1) v[2] = 0.f;
+            if (over > 2) v[1] = 0.f;
+            if (p_lds[it] >= 0) *reinterpret_cast<f32x4*>(patch + (p_lds[it] & ~3)) = v;
+        }
+    }
+};
+
+// One K step as the slot machinery of sgemm_tile.hpp sees it.
+// PAIRED: one of two consecutive taps inside a channel block, which alternate between the two
+// register stages of A so that their loads are dealt over the whole step.
+// SINGLE: a tap on its own (a block with an even number of taps starts with one): its loads of A
+// follow its stores, into the registers just stored.
+// LAST: the last tap of a channel block, as SINGLE; it also fetches the next block's patch in its
+// first operand group and swaps it in between its barrier and its last group.
+enum PatchStepKind { PATCH_PAIRED, PATCH_SINGLE, PATCH_LAST };
+template <class T, int KIND>
+struct PatchStep {
+    using PL = PatchLoader<T>;
+    static constexpr int NUM_LOADS = T::A_ITERS;
+    static constexpr int EARLY_LOADS = KIND == PATCH_LAST ? PL::PATCH_ITERS : 0;
+    static constexpr bool SINGLE_STAGE = KIND != PATCH_PAIRED;
+    static constexpr bool MASK_A_STORES = false;   // K' is a whole number of stages
+    static constexpr bool B_ALONG_K = false;
+    static constexpr int PATCH_PLANE = PATCH_PLANE_FLOATS;
+    static constexpr bool END_OF_BLOCK = KIND == PATCH_LAST;
+    PL& pl;
+    int next_block;
+    template <int OP, class RA, class RB>
+    __device__ __forceinline__ void load_one(int k0, int /*kend*/, RA& ra, RB& /*rb*/) const
+    {
+        if constexpr (OP < T::A_ITERS)
+            ra[OP] = pl.load_a(k0, pl.a_off[OP]);
+        else
+            pl.template load_patch_chunk<OP - T::A_ITERS>(next_block);
+    }
+    __device__ __forceinline__ void swap_patch() const { pl.store_patch(); }
+};
+
+template <class T>
+__global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const GemmArgs g)
+{
+    static_assert(T::KSPLIT == 1 && T::REG_STAGES == 2 && T::BK == PATCH_CHANNELS && T::TN <= 2, "tile shape");
+    using PL = PatchLoader<T>;
+    extern __shared__ __align__(16) float smem[];
+    float* As = smem;
+    float* patch = smem + 2 * T::A_STAGE;
+    const ConvGeom& cv = g.conv;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm0 = (wave / T::WAVES_N) * T::WM;
+    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    const int a_lane = (wm0 + l32) * T::LDA;
+
+    const WorkItem w = decode_tile(g, blockIdx.x);
+    const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
+    const int taps = cv.Hf * cv.Wf;
+    const int steps = (w.kend - w.kbeg) / T::BK;          // K slices are whole channel blocks
+    const int cb0 = w.kbeg / (T::BK * taps);
+    const int last_block = cv.Cin / PATCH_CHANNELS - 1;
+
+    // the tile's first pixel fixes which virtual row the patch starts at
+    const int vrows = cv.Hin + 2 * cv.pad;
+    const int g0 = n0 / cv.row_n, img0 = g0 / cv.Hout;
+    const int v0 = img0 * vrows + (g0 - img0 * cv.Hout);
+    // where the lane's pixels (one per 32-column block of the wave) sit in the patch under tap (0, 0);
+    // the lane's half of an operand group (channels 0..3 or 4..7) is folded in
+    int pix[2] = {0, 0};
+#pragma unroll
+    for (int tn = 0; tn < T::TN; ++tn) {
+        int n = n0 + wn0 + tn * 32 + l32;
+        if (n >= g.N) n = n0;                              // computed and dropped
+        const int gr = n / cv.row_n, wo = n - gr * cv.row_n;
+        const int b = gr / cv.Hout, ho = gr - b * cv.Hout;
+        pix[tn] = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + lh * 4 * PATCH_PLANE_FLOATS;
+    }
+
+    f32x16 acc[T::TM][T::TN];
+#pragma unroll
+    for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
+
+    if (steps > 0) {
+        PL pl;
+        pl.init(g, m0, v0, tid, patch);
+        // ra[1] holds the stage that the next step stores, at every step that is not the second of a pair
+        f32x4 ra[2][T::A_ITERS], rb_unused[T::B_ITERS];
+        Frag<T> frag[2];
+        // prologue: the first block's patch and the first stage of A
+        pl.load_patch(cb0);
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(w.kbeg, pl.a_off[it]);
+        // margins (and rows no chunk writes) are zero for the whole walk
+        for (int i = tid; i < PATCH_FLOATS / 4; i += T::THREADS)
+            reinterpret_cast<f32x4*>(patch)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+        pl.store_patch();
+        store_stage_a<T>(As, tid, ra[1]);
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(w.kbeg + T::BK, pl.a_off[it]);
+        __syncthreads();
+        // operands of the first group: A from stage 0, B from the patch under tap (0, 0)
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+            frag[0].a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + lh * 4);
+#pragma unroll
+        for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn]];
+
+        // One loop per kind of step: two step bodies chosen inside one loop would make the compiler
+        // copy the accumulators wherever the bodies' register assignments meet, i.e. after every step.
+        int cur = 0, s = 0;
+        auto step_with = [&](const auto& loader, int off_cur, int off_next, f32x4 (&sa)[T::A_ITERS], f32x4 (&fa)[T::A_ITERS]) {
+            using LD = std::remove_cv_t<std::remove_reference_t<decltype(loader)>>;
+            const WalkCtx<T, LD> c{loader, w.kbeg + (s + 2) * T::BK, w.kend,
+                                   As + cur * T::A_STAGE, patch + off_cur,
+                                   As + (cur ^ 1) * T::A_STAGE, patch + off_next,
+                                   tid, a_lane, pix[0], lh, sa, rb_unused, fa, rb_unused, pix[T::TN - 1]};
+            __builtin_amdgcn_sched_barrier(0);
+            step_groups<T, LD>(c, frag, acc);
+            cur ^= 1;
+            ++s;
+        };
+        const int blocks = steps / taps;
+        for (int cb = cb0; cb < cb0 + blocks; ++cb) {
+            int th = 0, tw = 0, off = 0;
+            // offset of the next stage's tap, whose first operands a step reads
+            auto next_tap = [&] {
+                if (++tw == cv.Wf) { tw = 0; ++th; }
+                return th * cv.patch_pitch + tw;
+            };
+            int tap = 0;
+            if ((taps - 1) & 1) {
+                const int off_next = next_tap();
+                step_with(PatchStep<T, PATCH_SINGLE>{pl, cb}, off, off_next, ra[1], ra[1]);
+                off = off_next;
+                ++tap;
+            }
+            for (; tap < taps - 1; tap += 2) {
+                const int off1 = next_tap();
+                step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
+                const int off2 = next_tap();
+                step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off1, off2, ra[0], ra[1]);
+                off = off2;
+            }
+            // (after the last channel block its own patch is fetched once more and never used)
+            step_with(PatchStep<T, PATCH_LAST>{pl, min(cb + 1, last_block)}, off, 0, ra[1], ra[1]);
+        }
+    }
+
+    if (w.tail_tile >= 0) {
+        // a K slice of a tail tile: the whole BM x BN block, tile-local, no masking
+        float* out = g.tail_partial + ((size_t)w.slice * g.tail_tiles + w.tail_tile) * (T::BM * T::BN);
+#pragma unroll
+        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    out[(wm0 + tm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3)) * T::BN + wn0 + tn * 32 + l32] = acc[tm][tn][r];
+        return;
+    }
+    store_c_tile<T, LOAD_IM2COL_ROW>(g, smem, acc, m0, n0, w.slice, wave, wm0, wn0, lane, l32, lh);
+}
+
+// Wt[co][(cb * taps + tap) * 32 + c] = W[co][(cb * 32 + c) * taps + tap], zero for channels past Cin
+__global__ void __launch_bounds__(256) conv_filter_relayout_kernel(const float* __restrict__ W, float* __restrict__ Wt,
+                                                                   int Cout, int Cin, int taps, int kp)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)Cout * kp) return;
+    const int co = (int)(i / kp), k = (int)(i - (size_t)co * kp);
+    const int c = k & 31, bt = k >> 5;
+    const int cb = bt / taps, tap = bt - cb * taps;
+    const int ch = cb * 32 + c;
+    Wt[i] = ch < Cin ? W[((size_t)co * Cin + ch) * taps + tap] : 0.f;
+}
+
+}  // namespace
+
+// Rows and row pitch of the patch for this geometry, or false when the kernel does not take it:
+// stride 1 only, at least two taps, padding of at most 4, whole blocks of 32 channels, and a patch plane of at most 512 floats
+// (56 x 56 maps under a 3 x 3 filter use all of it; wider images keep the staged-copy path).
+bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout, int Wout,
+                         int* rows, int* pitch)
+{
+    if (stride != 1 || Hf * Wf < 2 || pad > 4 || Cin % 32 != 0) return false;
+    const int row_n = (Wout + 3) & ~3;
+    const int bn = TilePatch::BN;
+    const int out_rows = (row_n - 1 + bn - 1) / row_n + 1;               // output rows a tile's pixels can lie in
+    int images = (bn - 1) / (Hout * row_n) + 1;                          // image borders a tile can cross
+    if (images > batch - 1) images = batch - 1;
+    // consecutive output rows of one image are one virtual row apart, the first row of the next
+    // image Hf - 1 more (a padded image has Hout + Hf - 1 rows); a window reaches Hf - 1 rows down
+    const int R = out_rows + (Hf - 1) * images + Hf - 1;
+    const int data = 4 + Win + pad, reach = 4 - pad + row_n + Wf - 1;     // last column written / read, + 1
+    const int P = ((data > reach ? data : reach) + 3) & ~3;
+    if (R * P > PATCH_PLANE_FLOATS) return false;
+    // byte offsets into the input are 32-bit
+    if ((double)batch * Cin * Hin * Win * 4.0 >= 2147483648.0) return false;
+    *rows = R;
+    *pitch = P;
+    return true;
+}
+
+int conv_patch_k(int Cin, int Hf, int Wf) { return (Cin + 31) / 32 * 32 * Hf * Wf; }
+
+hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int taps, hipStream_t stream)
+{
+    const int kp = (Cin + 31) / 32 * 32 * taps;
+    const size_t n = (size_t)Cout * kp;
+    hipLaunchKernelGGL(conv_filter_relayout_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, W, Wt, Cout,
+                       Cin, taps, kp);
+    return hipGetLastError();
+}
+
+hipError_t launch_sgemm_conv_patch(const GemmArgs& args, int grid, hipStream_t stream)
+{
+    using T = TilePatch;
+    auto kern = sgemm_conv_patch_kernel<T>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, patch_smem_bytes<T>());
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::THREADS), patch_smem_bytes<T>(), stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace cake

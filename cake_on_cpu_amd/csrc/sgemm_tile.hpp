@@ -735,13 +735,39 @@ __device__ __forceinline__ int conv_out_map(const ConvGeom& cv, int M, int ldc, 
 // first operands of the new stage come in from LDS, instead of the pipe
 // draining after every barrier.  (By then nobody reads the current buffer any
 // more, and it is only overwritten a whole step later.)
+// Loaders whose B operand is not staged per K step: B is read from a patch of the convolution's
+// input that stays in LDS for a whole block of channels (sgemm_conv_patch.hip).  Such a loader
+// declares PATCH_PLANE, the distance in floats between the planes of two consecutive k of a stage,
+// and may declare END_OF_BLOCK: the step then swaps the patch between its barrier and its last group.
+template <class L, class = void>
+struct patch_plane : std::integral_constant<int, 0> {};
+template <class L>
+struct patch_plane<L, std::void_t<decltype(L::PATCH_PLANE)>> : std::integral_constant<int, L::PATCH_PLANE> {};
+// EARLY_LOADS: that many more load instructions (numbered after the stage's own) go into the
+// step's first operand group, so that what they fetch is there when the patch is swapped.
+template <class L, class = void>
+struct early_loads : std::integral_constant<int, 0> {};
+template <class L>
+struct early_loads<L, std::void_t<decltype(L::EARLY_LOADS)>> : std::integral_constant<int, L::EARLY_LOADS> {};
+// SINGLE_STAGE: the step keeps to one register stage (its loads follow its stores) although the
+// tile has two.
+template <class L, class = void>
+struct single_stage : std::false_type {};
+template <class L>
+struct single_stage<L, std::void_t<decltype(L::SINGLE_STAGE)>> : std::bool_constant<L::SINGLE_STAGE> {};
+template <class L, class = void>
+struct ends_block : std::false_type {};
+template <class L>
+struct ends_block<L, std::void_t<decltype(L::END_OF_BLOCK)>> : std::bool_constant<L::END_OF_BLOCK> {};
+
 template <class T, class L>
 struct Slots {
     static constexpr int NKG = T::WAVE_BK / 8;      // operand groups of 8 k a wave walks per stage
     static constexpr int MFMA_PER_KG = 4 * T::TM * T::TN;
     static constexpr int FRAG_OPS = T::TM + (L::B_ALONG_K ? 1 : 4) * T::TN;   // LDS reads that fill one Frag
     static constexpr int LOAD_OPS = L::NUM_LOADS;               // global load instructions per stage
-    static constexpr int STORE_OPS = T::A_ITERS + T::B_ITERS;   // 16-byte LDS stores per stage
+    static constexpr int PLANE = patch_plane<L>::value;         // > 0: B comes from a resident patch
+    static constexpr int STORE_OPS = T::A_ITERS + (PLANE ? 0 : T::B_ITERS);   // 16-byte LDS stores per stage
     static constexpr int STORE_KG = NKG - 1 - T::STORE_LEAD;
     static_assert(STORE_KG >= 0, "stores must follow the previous step's barrier");
     static_assert(NKG >= 3, "the walk needs three operand groups per K step");
@@ -750,11 +776,14 @@ struct Slots {
     // its groups: issued in one burst by all the waves at once they queue up at
     // the memory pipe and hold back the MFMAs behind them.  With one register
     // stage they have to follow the step's own stores.
-    static constexpr bool SPREAD_LOADS = T::REG_STAGES >= 2;
-    static constexpr int load_begin(int kg) { return SPREAD_LOADS ? kg * LOAD_OPS / NKG : 0; }
+    static constexpr bool SPREAD_LOADS = T::REG_STAGES >= 2 && !single_stage<L>::value;
+    static constexpr int EARLY = early_loads<L>::value;
+    static_assert(EARLY == 0 || !SPREAD_LOADS, "early loads go with one register stage");
+    static constexpr int load_begin(int kg) { return SPREAD_LOADS ? kg * LOAD_OPS / NKG : (kg == 0 ? LOAD_OPS : 0); }
     static constexpr int loads_in(int kg)
     {
-        return SPREAD_LOADS ? (kg + 1) * LOAD_OPS / NKG - kg * LOAD_OPS / NKG : (kg == NKG - 1 ? LOAD_OPS : 0);
+        return SPREAD_LOADS ? (kg + 1) * LOAD_OPS / NKG - kg * LOAD_OPS / NKG
+                            : (kg == NKG - 1 ? LOAD_OPS : kg == 0 ? EARLY : 0);
     }
     // memory instructions riding in group kg: operand reads, then loads, then stores
     static constexpr int ops(int kg) { return FRAG_OPS + loads_in(kg) + (kg == STORE_KG ? STORE_OPS : 0); }
@@ -790,6 +819,7 @@ struct WalkCtx {
     f32x4 (&rb)[T::B_ITERS];
     f32x4 (&la)[T::A_ITERS];  // register stage that this step's global loads fill
     f32x4 (&lb)[T::B_ITERS];
+    int b_lane2 = 0;          // patch loaders: where the lane's second column block starts (b_lane: the first)
 };
 
 // Memory instruction number OP of group KG (compile-time indices, so every
@@ -813,6 +843,11 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
             const f32x4 v = *reinterpret_cast<const f32x4*>(B + c.b_lane + tn * 32 * T::LDA + kk);
 #pragma unroll
             for (int i = 0; i < 4; ++i) next.b[tn][i] = v[i];
+        } else if constexpr (S::PLANE > 0) {
+            // k = plane of the patch; the lane's half (k 0..3 or 4..7 of the group) is part of b_lane
+            constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
+            static_assert(T::TN <= 2, "two column blocks per wave at most");
+            next.b[tn][i] = B[((wrap ? 0 : KG + 1) * 8 + i) * S::PLANE + (tn == 0 ? c.b_lane : c.b_lane2)];
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
@@ -880,6 +915,12 @@ __device__ __forceinline__ void step_groups(const WalkCtx<T, L>& c, Frag<T> (&fr
         if constexpr (KG == Slots<T, L>::NKG - 1) {
             __syncthreads();  // every wave has stored its share of the next stage
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (ends_block<L>::value) {
+                // nobody reads the old patch any more (the last group's operands are in registers)
+                c.ld.swap_patch();
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         mfma_group<T, L, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
         __builtin_amdgcn_sched_barrier(0);

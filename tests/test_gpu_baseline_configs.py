@@ -99,10 +99,11 @@ def test_c5_conv_256x256x56x56_batch32_sampled():
     out = torch.empty((Cout, Bn * H * H), dtype=torch.float32, device="cuda:0")
     cake.conv2d(inp, wt, out, Bn, Cin, H, H, Cout, 3, 3, 1, 1)
     torch.cuda.synchronize()
-    # the reference's own two steps (column matrix first) give the same numbers
+    # the reference's own two steps (column matrix first) give the same numbers up to the order of
+    # the sums (the direct path walks K channel block by channel block): 5e-6 of sum |a||b| <= 2304 / 4
     two_step = torch.empty_like(out)
     cake.conv2d(inp, wt, two_step, Bn, Cin, H, H, Cout, 3, 3, 1, 1, explicit_im2col=True)
-    assert torch.equal(two_step, out)
+    assert float((two_step - out).abs().max()) <= 5e-6 * 576
     # two whole images (first and last) against the naive fp64 convolution
     wh = wt.cpu().numpy()
     for b in (0, Bn - 1):

@@ -143,6 +143,13 @@ CONV_GEOMS = [
     (2, 6, 10, 12, 12, 7, 7, 1, 3),      # 7x7, pad 3: the 16-byte row gather shifts by up to 3 either way
     (2, 8, 16, 16, 16, 5, 5, 1, 2),      # 5x5, pad 2, Wout = 16
     (3, 5, 5, 4, 8, 3, 3, 1, 1),         # Win = 4: the row gather's narrowest image
+    # whole blocks of 32 channels at stride 1: the input read where it lies, a patch of it in LDS
+    (3, 32, 14, 14, 40, 3, 3, 1, 1),     # Wout = 14 (rows of the product padded to 16), tiles across image borders
+    (5, 64, 7, 7, 300, 3, 3, 1, 1),      # 7 x 7 maps: a tile spans three images; two row tiles of filters
+    (2, 32, 13, 9, 33, 3, 3, 1, 0),      # no padding, Win = 9: the last 16 bytes of a row hang over its end
+    (2, 96, 12, 20, 70, 5, 3, 1, 2),     # 5 x 3 filter, pad 2 (the left margin holds 2 zero columns)
+    (2, 32, 30, 30, 16, 2, 2, 1, 1),     # 2 x 2 filter: Wout = 31
+    (1, 32, 56, 56, 24, 3, 3, 1, 1),     # a full-width plane of 56 x 56: every row and column of the patch in use
     (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
     (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
     (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
@@ -271,14 +278,26 @@ def test_conv2d_1x1_many_images(geom, nchw):
 
 
 def test_conv2d_paths_agree_bitwise_layouts():
-    """Same sums in the same order whichever way the columns reach the GEMM."""
-    Bn, Cin, Hin, Win, Cout = 2, 32, 20, 20, 48
+    """The gather from a staged copy sums in the order of the column matrix: same bits as the two
+    steps.  With whole blocks of 32 channels the input is read where it lies and the sum runs
+    channel block by channel block (another order, within the bar), the same on every run."""
+    Bn, Cin, Hin, Win, Cout = 2, 24, 20, 20, 48
     inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 56), oracle.uniform((Cout, Cin, 3, 3), 57)
     a = np.empty((Cout, Bn * 400), np.float32)
     b = np.empty_like(a)
     cake.conv2d(inp, wt, a, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
     cake.conv2d(inp, wt, b, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1, explicit_im2col=True)
     assert np.array_equal(a, b)
+    Cin = 32
+    inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 56), oracle.uniform((Cout, Cin, 3, 3), 57)
+    cake.conv2d(inp, wt, a, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
+    cake.conv2d(inp, wt, b, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1, explicit_im2col=True)
+    _, S = oracle.conv_naive_f64(inp, wt, 1, 1)
+    S = S.transpose(1, 0, 2, 3).reshape(Cout, -1)
+    assert np.max(np.abs(a - b) / S) <= TIGHT
+    again = np.empty_like(a)
+    cake.conv2d(inp, wt, again, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
+    assert np.array_equal(a, again)
 
 
 @pytest.mark.parametrize("geom", [(3, 12, 18, 20, 40, 3, 3, 1, 1), (2, 8, 17, 22, 24, 3, 3, 2, 1),
