@@ -49,6 +49,21 @@ int tail_split_for(int rem, int ksteps, const DeviceModel& dev)
     return split >= 2 ? split : 1;
 }
 
+// Workgroups of this tile that a CU holds at the same time (LDS and wave slots).
+int resident_per_cu(const TileInfo& t, const DeviceModel& dev)
+{
+    return std::max(1, std::min(dev.lds_per_cu / t.lds_bytes, 2048 / t.threads));
+}
+
+// Tiles left over after the rounds that fill every slot of the machine, when they are few enough
+// (at most half a workgroup per CU) to be worth cutting along K; 0 otherwise.
+int thin_tail_tiles(int tiles, const TileInfo& t, const DeviceModel& dev)
+{
+    const long cap = (long)dev.cus * resident_per_cu(t, dev);
+    const int rem = (int)(tiles % cap);
+    return tiles > dev.cus && rem > 0 && rem <= dev.cus / 2 ? rem : 0;
+}
+
 // Modelled time of one tile shape with one split factor.
 double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
 {
@@ -71,12 +86,25 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     // 4352 x 4096 x 1024: 270 against 290 us).
     if (tile_id == TILE_96x128x32_W96x32 && wgs >= 2 * dev.cus && ksteps >= 32) eff = 0.93;
     const double cu_rate = dev.mfma_flops / dev.cus * eff;
-    double rounds = (double)((wgs + dev.cus - 1) / dev.cus);
+    // Time in units of "one workgroup with a CU to itself at the tile's efficiency".  A CU holds
+    // `slots` workgroups at once, each at 1/slots of its rate, so the rounds that fill every slot
+    // cost `slots` units each.  In the last, partial round the fullest CU decides; a four-wave
+    // workgroup of 96 or 128 rows that is alone on its CU there (one wave per SIMD, nothing to hide
+    // its barriers behind) runs about a third slower than the efficiencies above, which were
+    // measured with the CU full (2956 x 7096 x 796 on 128 x 128 tiles: 324 us, on 96 x 128: 250 us;
+    // the 64 x 64 tiles' figures already are those of a workgroup on its own).
+    const int slots = resident_per_cu(t, dev);
+    const long cap = (long)dev.cus * slots;
+    const long rem = wgs % cap;
+    const int on_fullest = (int)((rem + dev.cus - 1) / dev.cus);
+    const double alone = (on_fullest == 1 && slots >= 2 && t.threads <= 256 && t.bm * t.bn >= 96 * 128) ? 1.3 : 1.0;
+    double rounds = (double)(wgs / cap) * slots + on_fullest * alone;
     bool tail = false;
-    if (split == 1 && wgs > dev.cus) {
-        const int ts = tail_split_for((int)(wgs % dev.cus), ksteps, dev);
+    if (split == 1) {
+        const int tt = thin_tail_tiles(tiles, t, dev);
+        const int ts = tt ? tail_split_for(tt, ksteps, dev) : 1;
         if (ts > 1) {
-            rounds = (double)(wgs / dev.cus) + (ceil_div(ksteps, ts) + extra) / (ksteps + extra);
+            rounds = (double)(wgs / cap) * slots + (ceil_div(ksteps, ts) + extra) / (ksteps + extra);
             tail = true;
         }
     }
@@ -85,7 +113,8 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
     // the slices are written, read back and summed by a second kernel
-    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 8e-6;
+    // (the second kernel and the gap in front of it: 1020 x 108 x 731 takes 14.6 us whole, 10.6 us in 4 slices)
+    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 5e-6;
     if (tail) s += 6e-6;  // the second kernel: about 5 us and the gap in front of it
     return s + 3e-6;  // launch
 }
@@ -259,13 +288,14 @@ static int finish_plan(int M, int N, int K, int sched, int tile_id, int split, b
     p.tail_split = 1;
     out->tail_k_per_split = 0;
     const int tiles = p.tiles_m * p.tiles_n;
-    if (p.split_k == 1 && tiles > dev.cus && tail_allowed) {
+    if (p.split_k == 1 && tail_allowed) {
         const int ksteps = ceil_div(K, t.bk);
-        const int ts = tail_split_for(tiles % dev.cus, ksteps, dev);
+        const int tt = thin_tail_tiles(tiles, t, dev);
+        const int ts = tt ? tail_split_for(tt, ksteps, dev) : 1;
         if (ts > 1) {
             out->tail_k_per_split = ceil_div(ksteps, ts) * t.bk;
             p.tail_split = ceil_div(K, out->tail_k_per_split);
-            p.tail_tiles = tiles % dev.cus;
+            p.tail_tiles = tt;
             p.grid = tiles - p.tail_tiles + p.tail_tiles * p.tail_split;
         }
     }
@@ -277,8 +307,7 @@ static int finish_plan(int M, int N, int K, int sched, int tile_id, int split, b
     // Reuse order.  `resident` tiles run at the same time on one XCD and share
     // its L2: a gm x gn block of them re-reads each A panel ceil(tiles_n/gn)
     // times and each B panel ceil(tiles_m/gm) times from HBM.
-    const int slots = std::max(1, std::min(dev.lds_per_cu / t.lds_bytes, 2048 / t.threads));
-    const int resident = std::max(1, dev.cus / dev.xcds * slots);
+    const int resident = std::max(1, dev.cus / dev.xcds * resident_per_cu(t, dev));
     auto traffic = [&](int gm, int gn) {
         return 4.0 * ((double)M * K * ceil_div(p.tiles_n, gn) + (double)K * N * ceil_div(p.tiles_m, gm) +
                       (double)M * N);

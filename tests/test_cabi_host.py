@@ -286,12 +286,13 @@ def test_plan_names_the_kernel_family():
     macro-tile kernel."""
     fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
     assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
-    assert fam(16, 16384, 16384) == 2 and fam(32, 600, 64) == 2 and fam(2, 512, 100) == 2
+    assert fam(16, 16384, 16384) == 2 and fam(32, 600, 256) == 2 and fam(2, 512, 300) == 2
+    assert fam(32, 600, 255) == 0   # a short K walk of few rows stays on the tile
     assert fam(16384, 16, 16384) == 3 and fam(512, 16, 64) == 3 and fam(16384, 32, 16384) == 3
     assert fam(512, 32, 64) == 0 and fam(4096, 17, 4096) == 0   # 17 to 32 columns: only against a large A
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 16384, 16384) == 0
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
-    assert fam(16, 511, 4096) == 0 and fam(16, 4096, 63) == 0 and fam(16, 16, 100000) == 0
+    assert fam(16, 511, 4096) == 0 and fam(16, 4096, 255) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0

@@ -84,9 +84,10 @@ def test_every_tile_shape(tile, shape):
 
 
 TAIL_CASES = [  # (shape M,K,N; tile) -- tile count = a whole number of rounds plus a thin last one
-    ((1100, 520, 1100), (64, 64, 64)), ((1100, 517, 1101), (64, 64, 64)),
-    ((2111, 2111, 2111), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
-    ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)), ((1632, 1024, 2048), (96, 128, 32)),
+    # (a round fills every slot: two workgroups per CU for the four-wave tiles and the K-split 64 x 64 one)
+    ((1472, 520, 1472), (64, 64, 64)), ((1470, 517, 1471), (64, 64, 64)),
+    ((2900, 512, 2900), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
+    ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)), ((3168, 512, 2048), (96, 128, 32)),
 ]
 
 
