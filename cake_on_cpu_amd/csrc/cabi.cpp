@@ -1314,11 +1314,22 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     });
     if (st) return st;
     if (accumulate) out_nchw = 0;   // a single image: [Cout][HW] is its NCHW layout
-    float* prod = out_nchw ? cn : o.dev;
     const bool vec = vec4_loadable(w.dev, cols, K, N);
     const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
+    // NCHW output: with rows of the product a multiple of 4 long the GEMM's epilogue (and its
+    // slice reductions) write the layout themselves, as on the gather path; otherwise the product
+    // goes to [Cout][N] first and a layout pass follows
+    ConvGeom nchw{};
+    const bool fused_nchw = out_nchw && vec && Wout % 4 == 0 && Cout > 48 && K > 64;   // (the macro-tile kernel's shapes)
+    if (fused_nchw) {
+        nchw.in = cols;
+        nchw.Hout = Hout; nchw.Wout = Wout; nchw.row_n = Wout;
+        nchw.out_nchw = 1;
+        out_nchw = 0;
+    }
+    float* prod = out_nchw ? cn : o.dev;
     st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, accumulate, nullptr, mode, mode,
-                  stream, timer);
+                  stream, timer, fused_nchw ? &nchw : nullptr);
     if (st) return st;
     if (out_nchw) {
         st = timer.family(3, [&] { return launch_cn_to_nchw(cn, o.dev, batch, Cout, Hout * Wout, stream); });

@@ -1052,7 +1052,10 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, con
     const float* bias = !PLAIN && g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // a convolution's columns n = (image, output row, column of a row padded to 4) go to
     // [M][batch*Hout*Wout] or NCHW: see conv_out_map
-    const bool conv_out = (B_MODE == LOAD_IM2COL_ROW || B_MODE == LOAD_IM2COL_1X1) && g.partial == nullptr;
+    // (also a plain product whose caller describes its columns as a convolution's: the two-step
+    // path's GEMM writes NCHW itself)
+    const bool conv_out = (B_MODE == LOAD_IM2COL_ROW || B_MODE == LOAD_IM2COL_1X1 || (B_MODE == LOAD_VEC4 && g.conv.in != nullptr)) &&
+                          g.partial == nullptr;
     // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
     // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
     // that a lane owns 4 consecutive columns of a row and C moves in 16-byte pieces: a
