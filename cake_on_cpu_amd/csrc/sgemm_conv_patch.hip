@@ -19,8 +19,8 @@
 //     stage, the channel part an immediate -- no integer work between the MFMAs;
 //   * A (the filters) walks through the usual double-buffered stages; the patch is loaded once per
 //     channel block (8 x 16 bytes per thread for 9 stages, where the gather from a staged copy
-//     issued 2 per stage), at the start of the block's last stage, and swapped in between that
-//     stage's barrier and its last operand group.
+//     issued 2 per stage), at the start of the block's second-to-last stage, and swapped in
+//     between the last stage's barrier and its last operand group.
 // Everything else -- tile raster, tail tiles cut along K, epilogue with the NCHW layout -- is the
 // macro-tile kernel's (sgemm_tile.hpp).
 #include "sgemm_tile.hpp"
@@ -55,7 +55,8 @@ struct PatchLoader {
     unsigned block_bytes;       // bytes of the input between channel blocks
     float* patch;
 
-    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int tid, float* patch_)
+    // v0: virtual row the patch starts at; rows_used: how many of its rows this tile's pixels reach
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid, float* patch_)
     {
         const ConvGeom& cv = g.conv;
         a_base = g.A + (size_t)m0 * g.lda;
@@ -81,7 +82,7 @@ struct PatchLoader {
             const int r = rem / wc, j = rem - r * wc;
             const int v = v0 + r;
             const int b = v / vrows, hi = v - b * vrows - cv.pad;
-            const bool data = q < total && b < cv.batch && hi >= 0 && hi < cv.Hin;
+            const bool data = q < total && r < rows_used && b < cv.batch && hi >= 0 && hi < cv.Hin;
             p_off[it] = data ? (((b * cv.Cin + c) * cv.Hin + hi) * cv.Win + 4 * j) * 4 : BUF_OOB;
             p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : -1;
         }
@@ -129,17 +130,19 @@ struct PatchLoader {
 // One K step as the slot machinery of sgemm_tile.hpp sees it.
 // PAIRED: one of two consecutive taps inside a channel block, which alternate between the two
 // register stages of A so that their loads are dealt over the whole step.
+// PAIRED_FETCH: the second tap of a block's last pair; it also fetches the next block's patch, in
+// its first operand group, so that the patch has a whole step and more to arrive.
 // SINGLE: a tap on its own (a block with an even number of taps starts with one): its loads of A
 // follow its stores, into the registers just stored.
-// LAST: the last tap of a channel block, as SINGLE; it also fetches the next block's patch in its
-// first operand group and swaps it in between its barrier and its last group.
-enum PatchStepKind { PATCH_PAIRED, PATCH_SINGLE, PATCH_LAST };
+// LAST: the last tap of a channel block, as SINGLE; it swaps the fetched patch in between its
+// barrier and its last operand group.
+enum PatchStepKind { PATCH_PAIRED, PATCH_PAIRED_FETCH, PATCH_SINGLE, PATCH_LAST };
 template <class T, int KIND>
 struct PatchStep {
     using PL = PatchLoader<T>;
     static constexpr int NUM_LOADS = T::A_ITERS;
-    static constexpr int EARLY_LOADS = KIND == PATCH_LAST ? PL::PATCH_ITERS : 0;
-    static constexpr bool SINGLE_STAGE = KIND != PATCH_PAIRED;
+    static constexpr int EARLY_LOADS = KIND == PATCH_PAIRED_FETCH ? PL::PATCH_ITERS : 0;
+    static constexpr bool SINGLE_STAGE = KIND == PATCH_SINGLE || KIND == PATCH_LAST;
     static constexpr bool MASK_A_STORES = false;   // K' is a whole number of stages
     static constexpr bool B_ALONG_K = false;
     static constexpr int PATCH_PLANE = PATCH_PLANE_FLOATS;
@@ -206,8 +209,12 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
     if (steps > 0) {
+        // the rows below the last pixel's window are never read: not fetched either
+        const int n_last = min(n0 + T::BN, g.N) - 1;
+        const int g_last = n_last / cv.row_n, img_last = g_last / cv.Hout;
+        const int rows_used = img_last * vrows + (g_last - img_last * cv.Hout) - v0 + cv.Hf;
         PL pl;
-        pl.init(g, m0, v0, tid, patch);
+        pl.init(g, m0, v0, rows_used, tid, patch);
         // ra[1] holds the stage that the next step stores, at every step that is not the second of a pair
         f32x4 ra[2][T::A_ITERS], rb_unused[T::B_ITERS];
         Frag<T> frag[2];
@@ -262,15 +269,20 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
                 off = off_next;
                 ++tap;
             }
-            for (; tap < taps - 1; tap += 2) {
+            // (after the last channel block its own patch is fetched once more and never used)
+            const int fetch = min(cb + 1, last_block);
+            for (; tap < taps - 3; tap += 2) {
                 const int off1 = next_tap();
                 step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
                 const int off2 = next_tap();
                 step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off1, off2, ra[0], ra[1]);
                 off = off2;
             }
-            // (after the last channel block its own patch is fetched once more and never used)
-            step_with(PatchStep<T, PATCH_LAST>{pl, min(cb + 1, last_block)}, off, 0, ra[1], ra[1]);
+            const int off1 = next_tap();
+            step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
+            const int off2 = next_tap();
+            step_with(PatchStep<T, PATCH_PAIRED_FETCH>{pl, fetch}, off1, off2, ra[0], ra[1]);
+            step_with(PatchStep<T, PATCH_LAST>{pl, fetch}, off2, 0, ra[1], ra[1]);
         }
     }
 
@@ -305,12 +317,12 @@ __global__ void __launch_bounds__(256) conv_filter_relayout_kernel(const float* 
 }  // namespace
 
 // Rows and row pitch of the patch for this geometry, or false when the kernel does not take it:
-// stride 1 only, at least two taps, padding of at most 4, whole blocks of 32 channels, and a patch plane of at most 512 floats
+// stride 1 only, at least three taps, padding of at most 4, whole blocks of 32 channels, and a patch plane of at most 512 floats
 // (56 x 56 maps under a 3 x 3 filter use all of it; wider images keep the staged-copy path).
 bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout, int Wout,
                          int* rows, int* pitch)
 {
-    if (stride != 1 || Hf * Wf < 2 || pad > 4 || Cin % 32 != 0) return false;
+    if (stride != 1 || Hf * Wf < 3 || pad > 4 || Cin % 32 != 0) return false;
     const int row_n = (Wout + 3) & ~3;
     const int bn = TilePatch::BN;
     const int out_rows = (row_n - 1 + bn - 1) / row_n + 1;               // output rows a tile's pixels can lie in

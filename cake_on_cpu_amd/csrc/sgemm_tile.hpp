@@ -778,13 +778,15 @@ struct Slots {
     // stage they have to follow the step's own stores.
     static constexpr bool SPREAD_LOADS = T::REG_STAGES >= 2 && !single_stage<L>::value;
     static constexpr int EARLY = early_loads<L>::value;
-    static_assert(EARLY == 0 || !SPREAD_LOADS, "early loads go with one register stage");
-    static constexpr int load_begin(int kg) { return SPREAD_LOADS ? kg * LOAD_OPS / NKG : (kg == 0 ? LOAD_OPS : 0); }
-    static constexpr int loads_in(int kg)
+    // the stage's own loads in group kg, and which of the stage's loads the first of them is
+    static constexpr int own_begin(int kg) { return SPREAD_LOADS ? kg * LOAD_OPS / NKG : 0; }
+    static constexpr int own_in(int kg)
     {
-        return SPREAD_LOADS ? (kg + 1) * LOAD_OPS / NKG - kg * LOAD_OPS / NKG
-                            : (kg == NKG - 1 ? LOAD_OPS : kg == 0 ? EARLY : 0);
+        return SPREAD_LOADS ? (kg + 1) * LOAD_OPS / NKG - kg * LOAD_OPS / NKG : (kg == NKG - 1 ? LOAD_OPS : 0);
     }
+    static constexpr int loads_in(int kg) { return own_in(kg) + (kg == 0 ? EARLY : 0); }
+    // number (as the loader counts them) of load j of group kg: the early ones follow the stage's own
+    static constexpr int load_index(int kg, int j) { return j < own_in(kg) ? own_begin(kg) + j : LOAD_OPS + j - own_in(kg); }
     // memory instructions riding in group kg: operand reads, then loads, then stores
     static constexpr int ops(int kg) { return FRAG_OPS + loads_in(kg) + (kg == STORE_KG ? STORE_OPS : 0); }
 };
@@ -853,7 +855,7 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
         }
     } else if constexpr (OP < N_FRAG + N_LOAD) {
-        c.ld.template load_one<S::load_begin(KG) + OP - N_FRAG>(c.k_next, c.kend, c.la, c.lb);
+        c.ld.template load_one<S::load_index(KG, OP - N_FRAG)>(c.k_next, c.kend, c.la, c.lb);
     } else {
         constexpr int W = OP - N_FRAG - N_LOAD;  // store number W of the stage
         if constexpr (W < T::A_ITERS) {
