@@ -165,12 +165,17 @@ def test_plan_covers_any_shape(M, N, K):
 
 
 def test_plan_tail_split():
-    """A thin last round (few tiles left over after whole rounds of 256 CUs) is cut
-    along K instead: the convolution GEMM leaves 32 of 1568 tiles."""
-    conv = cake.plan(256, 100352, 2304)
-    assert (conv.tile_m, conv.tile_n) == (128, 128) and conv.split_k == 1
-    assert conv.tail_tiles == 1568 % 256 and conv.tail_split == 8
+    """A thin last round (few tiles left over after the rounds that fill every slot of the
+    machine) is cut along K instead: the convolution GEMM leaves 32 of its 1568 tiles of 128 x 128
+    (two workgroups per CU: 512 slots) and 16 of its 784 tiles of 256 x 128."""
+    conv = cake.plan(256, 100352, 2304, cake.NA, (128, 128, 32, 0))
+    assert conv.split_k == 1 and conv.tail_tiles == 1568 % 512 and conv.tail_split == 8
     assert conv.grid == 1568 - 32 + 32 * 8
+    conv = cake.plan(256, 100352, 2304, cake.NA, (256, 128, 32, 0))
+    assert conv.split_k == 1 and conv.tail_tiles == 784 % 256 and conv.tail_split == 15   # 72 K steps in slices of 5
+    assert conv.grid == 784 - 16 + 16 * 15
+    auto = cake.plan(256, 100352, 2304)
+    assert auto.tail_tiles > 0 and auto.grid == auto.tiles_m * auto.tiles_n + auto.tail_tiles * (auto.tail_split - 1)
     assert cake.plan(8192, 8192, 8192).tail_tiles == 0          # whole rounds: nothing to cut
     assert cake.plan(256, 100352, 2304, cake.NA, (128, 128, 32, 1)).tail_tiles == 0   # explicit split is literal
 
