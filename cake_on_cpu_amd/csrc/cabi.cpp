@@ -413,12 +413,13 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         g.A = A; g.B = B; g.C = C;
         g.M = M; g.N = N; g.K = K;
         g.lda = lda; g.ldb = ldb; g.ldc = ldc;
-        g.tiles_m = (M + 63) / 64; g.tiles_n = (N + 63) / 64;
+        const int tn = shortk_tile_n(M, N, K, g_ctx.model.cus);
+        g.tiles_m = (M + 63) / 64; g.tiles_n = (N + tn - 1) / tn;
         g.split_k = 1; g.k_per_split = K;
         g.group = g.tiles_m; g.group_along_n = 0;   // tiles of one column block of B one after the other
         g.accumulate = accumulate;
         g.col_bias = col_bias;
-        return timer.family(0, [&] { return launch_sgemm_shortk(g, g_ctx.model.cus, stream); });
+        return timer.family(0, [&] { return launch_sgemm_shortk(g, tn, g_ctx.model.cus, stream); });
     }
     GemmPlan plan;
     int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec_plan, g_ctx.model, &plan)
@@ -632,13 +633,14 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     if (out->kernel == CAKE_HIP_KERNEL_SHORT_K) {
         // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
         // column blocks of B by at most four resident workgroups per CU
-        out->tile_m = 64; out->tile_n = 64; out->tile_k = 64;
-        out->wave_m = 32; out->wave_n = 32;
+        const int tn = shortk_tile_n(M, N, K, model.cus);
+        out->tile_m = 64; out->tile_n = tn; out->tile_k = 64;
+        out->wave_m = 32; out->wave_n = tn / 2;
         out->threads = 256;
         out->split_k = 1; out->tail_tiles = 0; out->tail_split = 1;
-        out->tiles_m = (M + 63) / 64; out->tiles_n = (N + 63) / 64;
+        out->tiles_m = (M + 63) / 64; out->tiles_n = (N + tn - 1) / tn;
         out->group = out->tiles_m;
-        shortk_launch_shape((long)out->tiles_m * out->tiles_n, model.cus, &out->grid, &out->lds_bytes);
+        shortk_launch_shape((long)out->tiles_m * out->tiles_n, tn, model.cus, &out->grid, &out->lds_bytes);
     }
     return CAKE_HIP_OK;
 }
@@ -1180,14 +1182,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.ldc = out_nchw ? HW : N;                             // [batch][Cout][HW] or [Cout][batch*HW]
         g.b_batch_stride = (size_t)Cin * HW;
         g.c_batch_stride = out_nchw ? (size_t)Cout * HW : (size_t)HW;
+        const int tn = shortk_tile_n(Cout, HW, K, g_ctx.model.cus, batch);
         g.tiles_m = (Cout + 63) / 64;
-        g.tiles_n_per_image = (HW + 63) / 64;
+        g.tiles_n_per_image = (HW + tn - 1) / tn;
         g.tiles_n = g.tiles_n_per_image * batch;
         g.split_k = 1; g.k_per_split = K;
         g.group = g.tiles_m; g.group_along_n = 0;
         g.accumulate = accumulate;
         if ((st = timer.start())) return st;
-        st = timer.family(0, [&] { return launch_sgemm_shortk(g, g_ctx.model.cus, stream); });
+        st = timer.family(0, [&] { return launch_sgemm_shortk(g, tn, g_ctx.model.cus, stream); });
         if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);

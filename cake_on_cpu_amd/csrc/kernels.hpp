@@ -101,9 +101,11 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
 // Products with K <= 64 and many 64 x 64 tiles: workgroups that walk over tiles with the next
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
-bool shortk_applies(int M, int N, int K, int cus, int batch = 1);
-hipError_t launch_sgemm_shortk(const GemmArgs& args, int cus, hipStream_t stream);
-void shortk_launch_shape(long tiles, int cus, int* grid, int* lds_bytes);
+// shortk_tile_n: 0 when the kernel does not apply, else the width of its tiles (64 or 128)
+int shortk_tile_n(int M, int N, int K, int cus, int batch = 1);
+inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1) { return shortk_tile_n(M, N, K, cus, batch) != 0; }
+hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream);
+void shortk_launch_shape(long tiles, int tile_n, int cus, int* grid, int* lds_bytes);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
                                 int accumulate, hipStream_t stream, const ConvGeom* conv = nullptr,

@@ -153,8 +153,9 @@ def test_plan_covers_any_shape(M, N, K):
         tiles = pl.tiles_m * pl.tiles_n
         assert pl.split_k >= 1 and pl.tail_split >= 1 and 0 <= pl.tail_tiles < tiles
         assert not (pl.split_k > 1 and pl.tail_tiles > 0)
-        if pl.kernel == 4:   # short K: resident workgroups, at most four per CU, in whole rows of 8 XCDs
-            assert pl.grid == (min(tiles, 4 * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
+        if pl.kernel == 4:   # short K: resident workgroups, as many as a CU's LDS holds, in whole rows of 8 XCDs
+            per_cu = 3 if pl.tile_n == 128 else 4
+            assert pl.grid == (min(tiles, per_cu * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
         else:
             assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
         assert 1 <= pl.group <= max(pl.tiles_m, pl.tiles_n)
@@ -308,6 +309,11 @@ def test_plan_names_the_kernel_family():
     assert (p.kernel, p.tile_m, p.tile_n, p.tile_k, p.threads, p.split_k, p.tail_tiles) == (4, 64, 64, 64, 256, 1, 0)
     assert (p.tiles_m, p.tiles_n) == (4, 1568) and p.grid == 4 * p.cus and p.grid % 8 == 0
     assert 4 * p.lds_bytes <= 160 * 1024
+    # K up to 24 under many tiles: tiles 128 wide, three workgroups per CU
+    p = cake.plan(16384, 16384, 16)
+    assert (p.kernel, p.tile_m, p.tile_n, p.wave_n, p.threads) == (4, 64, 128, 64, 256)
+    assert (p.tiles_m, p.tiles_n) == (256, 128) and p.grid == 3 * p.cus and 3 * p.lds_bytes <= 160 * 1024
+    assert cake.plan(16384, 16384, 25).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
 
 
 def test_default_schedule_resolves_accumulate_by_the_reference_rule(monkeypatch):

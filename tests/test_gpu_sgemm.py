@@ -191,7 +191,9 @@ def test_tall_matrix_times_few_columns(shape):
 @pytest.mark.parametrize("shape", [(4096, 64, 4096), (3000, 33, 5000), (4100, 63, 3300), (5000, 1, 4000), (2000, 7, 9000),
                                    (256, 64, 100352), (9000, 4, 2111), (3584, 64, 3520), (3584, 65, 3520),
                                    # one to four tiles per CU: every workgroup has a single tile, surplus ones leave early
-                                   (1024, 64, 1024), (2111, 10, 960), (1100, 33, 1500), (960, 7, 1100)],
+                                   (1024, 64, 1024), (2111, 10, 960), (1100, 33, 1500), (960, 7, 1100),
+                                   # K up to 24 under many tiles: tiles 128 wide
+                                   (4096, 16, 8200), (3333, 24, 7777), (8192, 25, 4096)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_short_k_many_tiles(shape):
     """K of at most 64 under at least one 64 x 64 tile per CU: workgroups that walk over tiles with
