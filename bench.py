@@ -87,6 +87,9 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy kernel 3 times (reference point for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--latency-floor", action="store_true",
+                    help="only time 1024 x 1024 x K products for K = 32 .. 1024 and a one-workgroup kernel "
+                         "(what config 1's time is made of: a fixed part and a part per k) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (single-GPU hot path); --gpus must be 1", file=sys.stderr)
@@ -120,8 +123,12 @@ def main() -> int:
         cake.fill_uniform(t, seed)
         return t
 
-    def time_steps(launch, steps, warmup, settle_ms=0.0):
-        """W warm-ups, then K launches between two synchronisations with an event pair per launch.
+    def time_steps(launch, steps, warmup, settle_ms=0.0, each=False):
+        """W warm-ups, then K launches between two synchronisations.  Returns the wall time of the
+        K launches and the average and least launch duration by HIP events on the launch stream:
+        one event pair around the K launches (their duration is the region's over K: a pair costs
+        several microseconds of its own, too much to put around a launch of twenty), or with
+        `each` a pair per launch, which also gives the least.
         settle_ms > 0 keeps launching warm-ups until that much GPU time has passed, so that a
         sub-millisecond kernel is timed at settled clocks like the long ones are."""
         for _ in range(warmup):
@@ -133,17 +140,55 @@ def main() -> int:
                 for _ in range(20):
                     launch()
                 torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        pairs = steps if each else 1
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(pairs)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for a, b in evs:
-            a.record()
-            launch()
-            b.record()
+        if each:
+            for a, b in evs:
+                a.record()
+                launch()
+                b.record()
+        else:
+            evs[0][0].record()
+            for _ in range(steps):
+                launch()
+            evs[0][1].record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-        kernel = [a.elapsed_time(b) * 1e-3 for a, b in evs]
+        kernel = [a.elapsed_time(b) * 1e-3 * pairs / steps for a, b in evs]
         return wall, float(np.mean(kernel)), float(np.min(kernel))
+
+    if args.latency_floor:
+        m = 1024
+        a1, b1 = dev_uniform((m, m), 11), dev_uniform((m, m), 12)
+        c1 = torch.zeros((m, m), dtype=torch.float32, device=dev)
+        one = torch.zeros((64,), dtype=torch.float32, device=dev)
+        rows = []
+
+        def best_of(launch):
+            return min(time_steps(launch, 50, 20, settle_ms=50.0)[1] for _ in range(3))
+
+        rows.append({"kernel": "fill_uniform_kernel, one workgroup",
+                     "us": round(best_of(lambda: _lib.check(lib.cake_hip_fill_uniform(one.data_ptr(), 64, 1, stream), "fill")) * 1e6, 2)})
+        ks = (32, 64, 128, 256, 512, 768, 1024)
+        for k in ks:
+            # dense 1024 x k and k x 1024 operands at the front of the buffers
+            def launch(k=k):
+                _lib.check(lib.cake_hip_sgemm(a1.data_ptr(), b1.data_ptr(), c1.data_ptr(), m, m, k, cake.NA, 0, None,
+                                              stream, None), "cake_hip_sgemm")
+            pl = cake.plan(m, m, k)
+            rows.append({"K": k, "us": round(best_of(launch) * 1e6, 2), "kernel": cake.KERNEL_NAMES[pl.kernel],
+                         "tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "workgroups": pl.grid})
+        # least squares over the K that run the same kernel as K = 1024
+        same = [r for r in rows if r.get("tile") == rows[-1]["tile"] and r.get("kernel") == rows[-1]["kernel"]]
+        xs, ys = np.array([r["K"] for r in same], float), np.array([r["us"] for r in same], float)
+        slope, fixed = np.polyfit(xs, ys, 1) if len(same) >= 2 else (float("nan"), float("nan"))
+        peak_ns_per_k = 2.0 * m * m / (MFMA_PEAK_TFLOPS * 1e12) * 1e9
+        print(json.dumps({"latency_floor_1024x1024xK": rows, "fit_over_K": [int(x) for x in xs],
+                          "fixed_us": round(float(fixed), 2), "ns_per_k": round(float(slope) * 1e3, 2),
+                          "ns_per_k_at_mfma_peak": round(peak_ns_per_k, 2)}))
+        return 0
 
     # ---------------------------------------------------------------- config 2
     n = 8192
@@ -154,7 +199,7 @@ def main() -> int:
     def sgemm_step():
         _lib.check(lib.cake_hip_sgemm(pa, pb, pc, n, n, n, cake.NA, 0, None, stream, None), "cake_hip_sgemm")
 
-    wall, k_avg, k_min = time_steps(sgemm_step, args.steps, args.warmup)
+    wall, k_avg, k_min = time_steps(sgemm_step, args.steps, args.warmup, each=True)
     flops = 2.0 * n * n * n
     value = flops * args.steps / wall / 1e12
     achieved = flops / k_avg / 1e12

@@ -372,7 +372,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
              const ConvGeom* conv = nullptr, const float* col_bias = nullptr,
              const TunedChoice* choice = nullptr)
 {
-    const bool vec = a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4;
+    const bool vec = a_mode == LOAD_VEC4 && (b_mode == LOAD_VEC4 || b_mode == LOAD_VEC4_NCHW);
     const bool vec_plan = vec || (a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4_T);  // planned (and tuned) alike
     // Products with a few rows or columns have streaming kernels of their own; a macro-tile is
     // only used for them on request or when the tuner measured one to be faster.
@@ -631,8 +631,8 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     *out = plan.pub;
     out->kernel = kernel_family(M, N, K, tile_override != nullptr, vec);
     if (out->kernel == CAKE_HIP_KERNEL_SHORT_K) {
-        // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
-        // column blocks of B by at most four resident workgroups per CU
+        // what launch_sgemm_shortk does: 64 x 64 (or 64 x 128) tiles with the whole K in one LDS stage, walked in
+        // column blocks of B by the resident workgroups per CU
         const int tn = shortk_tile_n(M, N, K, model.cus);
         out->tile_m = 64; out->tile_n = tn; out->tile_k = 64;
         out->wave_m = 32; out->wave_n = tn / 2;
@@ -1331,8 +1331,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         out_nchw = 0;
     }
     float* prod = out_nchw ? cn : o.dev;
-    st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, accumulate, nullptr, mode, mode,
-                  stream, timer, fused_nchw ? &nchw : nullptr);
+    st = run_gemm(w.dev, cols, prod, Cout, N, K, K, N, N, CAKE_HIP_NA, accumulate, nullptr, mode,
+                  fused_nchw ? LOAD_VEC4_NCHW : mode, stream, timer, fused_nchw ? &nchw : nullptr);
     if (st) return st;
     if (out_nchw) {
         st = timer.family(3, [&] { return launch_cn_to_nchw(cn, o.dev, batch, Cout, Hout * Wout, stream); });

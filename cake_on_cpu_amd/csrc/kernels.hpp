@@ -92,8 +92,11 @@ enum LoadMode {
     LOAD_VEC4_T = 2, // B only: B handed over as its transpose Bt[N][K] (rows ldb apart), 16-byte loads along k
     LOAD_IM2COL_ROW = 4, // B only: column matrix of a convolution gathered from the staged NCHW input,
                          // one 16-byte load per 4 columns
-    LOAD_IM2COL_1X1 = 5  // the same for a 1 x 1 filter: row k is channel k, tap_stride bytes after row k - 1,
+    LOAD_IM2COL_1X1 = 5, // the same for a 1 x 1 filter: row k is channel k, tap_stride bytes after row k - 1,
                          // so no tap table is read
+    LOAD_VEC4_NCHW = 6   // B only: loaded as LOAD_VEC4 (an explicit column matrix), C's columns placed as a
+                         // convolution's output (GemmArgs::conv describes it).  A mode of its own so that
+                         // the plain product's epilogue carries none of that placement.
 };
 
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,

@@ -4,6 +4,7 @@
 namespace cake {
 
 hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
+hipError_t launch_sgemm_vec_nchw(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_scalar(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_convrow(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
 hipError_t launch_sgemm_vec_nt(int tile_id, const GemmArgs& a, int grid, hipStream_t s);
@@ -40,6 +41,10 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
     if (b_mode == LOAD_VEC4_T) {
         if (a_mode != LOAD_VEC4) return hipErrorInvalidValue;
         return launch_sgemm_vec_nt(tile_id, args, grid, stream);
+    }
+    if (b_mode == LOAD_VEC4_NCHW) {
+        if (a_mode != LOAD_VEC4 || !args.conv.in) return hipErrorInvalidValue;
+        return launch_sgemm_vec_nchw(tile_id, args, grid, stream);
     }
     if (a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4) return launch_sgemm_vec(tile_id, args, grid, stream);
     return launch_sgemm_scalar(tile_id, args, grid, stream);

@@ -1054,9 +1054,8 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, con
     const float* bias = !PLAIN && g.partial == nullptr ? g.col_bias : nullptr;  // split-K adds it in the reduce
     // a convolution's columns n = (image, output row, column of a row padded to 4) go to
     // [M][batch*Hout*Wout] or NCHW: see conv_out_map
-    // (also a plain product whose caller describes its columns as a convolution's: the two-step
-    // path's GEMM writes NCHW itself)
-    const bool conv_out = (B_MODE == LOAD_IM2COL_ROW || B_MODE == LOAD_IM2COL_1X1 || (B_MODE == LOAD_VEC4 && g.conv.in != nullptr)) &&
+    // (LOAD_VEC4_NCHW: the product on an explicit column matrix writes NCHW itself)
+    const bool conv_out = (B_MODE == LOAD_IM2COL_ROW || B_MODE == LOAD_IM2COL_1X1 || B_MODE == LOAD_VEC4_NCHW) &&
                           g.partial == nullptr;
     // The accumulators hold columns of C across lanes (one column per lane, 4 rows per
     // register group).  Each wave turns its block around through LDS, 32 rows at a time, so
@@ -1147,7 +1146,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_tile_kernel(const GemmArgs g
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
-    if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_VEC4)
+    if constexpr (A_MODE == LOAD_VEC4 && (B_MODE == LOAD_VEC4 || B_MODE == LOAD_VEC4_NCHW))
         k_walk_vec<T, VecLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
     else if constexpr (A_MODE == LOAD_VEC4 && B_MODE == LOAD_IM2COL_ROW)
         k_walk_vec<T, ConvRowLoader<T>>(g, As, Bs, m0, n0, kbeg, kend, steps, tid, a_lane, b_lane, lh, acc);
