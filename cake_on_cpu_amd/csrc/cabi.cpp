@@ -1215,16 +1215,20 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.split_k = 1; g.k_per_split = Kp;
         g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
         g.accumulate = accumulate;
-        // tiles of a thin last round are cut along K in whole channel blocks
+        // tiles of a thin last round are cut along K in whole channel blocks, or -- when the plan asks
+        // for more slices than there are blocks and half a block still has the three taps a walk
+        // needs -- in halves of a block's taps (config 5: 16 tiles in 16 slices of 5 and 4 taps)
         int grid = g.tiles_m * g.tiles_n;
         if (plan.pub.tail_tiles > 0) {
             const int block_k = 32 * taps, blocks = Kp / block_k;
-            const int per = (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
-            const int slices = (blocks + per - 1) / per;
+            const bool halves = plan.pub.tail_split > blocks && taps >= 6;
+            const int per = halves ? 1 : (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
+            const int slices = halves ? 2 * blocks : (blocks + per - 1) / per;
             if (slices > 1) {
                 g.tail_tiles = plan.pub.tail_tiles;
                 g.tail_split = slices;
-                g.tail_k_per_split = per * block_k;
+                g.tail_k_per_split = per * block_k;    // (not read for halves: the kernel places them itself)
+                g.conv.tail_halves = halves ? 1 : 0;
                 if ((st = partial_space(g_ctx.splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
                     return st;
                 grid += g.tail_tiles * (slices - 1);

@@ -40,6 +40,8 @@ struct ConvGeom {
     // sgemm_conv_patch.hip only (the input read where it lies, `in` = the NCHW input itself):
     int batch, Hin, Win, pad, Hf, Wf;
     int patch_rows, patch_pitch;   // rows and floats per row of the input patch a workgroup keeps in LDS
+    int tail_halves;               // sgemm_conv_patch.hip: slice s of a tail tile is half h = s & 1 of the taps
+                                   // of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest)
 };
 
 struct GemmArgs {

@@ -180,8 +180,19 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     const WorkItem w = decode_tile(g, blockIdx.x);
     const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
     const int taps = cv.Hf * cv.Wf;
-    const int steps = (w.kend - w.kbeg) / T::BK;          // K slices are whole channel blocks
-    const int cb0 = w.kbeg / (T::BK * taps);
+    // K slices are whole channel blocks, or (tail_halves) the first or second half of one block's taps
+    int kbeg = w.kbeg, kend = w.kend;
+    if (w.tail_tile >= 0 && cv.tail_halves) {
+        const int first = (taps + 1) >> 1, cb = w.slice >> 1;
+        kbeg = (cb * taps + (w.slice & 1) * first) * T::BK;
+        kend = (w.slice & 1) ? (cb + 1) * taps * T::BK : kbeg + first * T::BK;
+    }
+    const int steps = (kend - kbeg) / T::BK;
+    const int cb0 = kbeg / (T::BK * taps);
+    const int tap_lo = kbeg / T::BK - cb0 * taps;         // the first tap of the walk (0 unless half a block)
+    const int tap_n = steps < taps ? steps : taps;        // taps walked per channel block
+    const int th0 = tap_lo / cv.Wf, tw0 = tap_lo - th0 * cv.Wf;
+    const int off0 = th0 * cv.patch_pitch + tw0;
     const int last_block = cv.Cin / PATCH_CHANNELS - 1;
 
     // the tile's first pixel fixes which virtual row the patch starts at
@@ -221,7 +232,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         // prologue: the first block's patch and the first stage of A
         pl.load_patch(cb0);
 #pragma unroll
-        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(w.kbeg, pl.a_off[it]);
+        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(kbeg, pl.a_off[it]);
         // margins (and rows no chunk writes) are zero for the whole walk
         for (int i = tid; i < PATCH_FLOATS / 4; i += T::THREADS)
             reinterpret_cast<f32x4*>(patch)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -229,23 +240,23 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         pl.store_patch();
         store_stage_a<T>(As, tid, ra[1]);
 #pragma unroll
-        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(w.kbeg + T::BK, pl.a_off[it]);
+        for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(kbeg + T::BK, pl.a_off[it]);
         __syncthreads();
-        // operands of the first group: A from stage 0, B from the patch under tap (0, 0)
+        // operands of the first group: A from stage 0, B from the patch under the first tap
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
             frag[0].a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + lh * 4);
 #pragma unroll
         for (int tn = 0; tn < T::TN; ++tn)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn]];
+            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn] + off0];
 
         // One loop per kind of step: two step bodies chosen inside one loop would make the compiler
         // copy the accumulators wherever the bodies' register assignments meet, i.e. after every step.
         int cur = 0, s = 0;
         auto step_with = [&](const auto& loader, int off_cur, int off_next, f32x4 (&sa)[T::A_ITERS], f32x4 (&fa)[T::A_ITERS]) {
             using LD = std::remove_cv_t<std::remove_reference_t<decltype(loader)>>;
-            const WalkCtx<T, LD> c{loader, w.kbeg + (s + 2) * T::BK, w.kend,
+            const WalkCtx<T, LD> c{loader, kbeg + (s + 2) * T::BK, kend,
                                    As + cur * T::A_STAGE, patch + off_cur,
                                    As + (cur ^ 1) * T::A_STAGE, patch + off_next,
                                    tid, a_lane, pix[0], lh, sa, rb_unused, fa, rb_unused, pix[T::TN - 1]};
@@ -254,16 +265,16 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
             cur ^= 1;
             ++s;
         };
-        const int blocks = steps / taps;
+        const int blocks = steps < taps ? 1 : steps / taps;
         for (int cb = cb0; cb < cb0 + blocks; ++cb) {
-            int th = 0, tw = 0, off = 0;
+            int th = th0, tw = tw0, off = off0;
             // offset of the next stage's tap, whose first operands a step reads
             auto next_tap = [&] {
                 if (++tw == cv.Wf) { tw = 0; ++th; }
                 return th * cv.patch_pitch + tw;
             };
             int tap = 0;
-            if ((taps - 1) & 1) {
+            if ((tap_n - 1) & 1) {
                 const int off_next = next_tap();
                 step_with(PatchStep<T, PATCH_SINGLE>{pl, cb}, off, off_next, ra[1], ra[1]);
                 off = off_next;
@@ -271,7 +282,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
             }
             // (after the last channel block its own patch is fetched once more and never used)
             const int fetch = min(cb + 1, last_block);
-            for (; tap < taps - 3; tap += 2) {
+            for (; tap < tap_n - 3; tap += 2) {
                 const int off1 = next_tap();
                 step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
                 const int off2 = next_tap();

@@ -150,6 +150,8 @@ CONV_GEOMS = [
     (2, 96, 12, 20, 70, 5, 3, 1, 2),     # 5 x 3 filter, pad 2 (the left margin holds 2 zero columns)
     (2, 32, 30, 30, 16, 2, 2, 1, 1),     # 2 x 2 filter: Wout = 31
     (1, 32, 56, 56, 24, 3, 3, 1, 1),     # a full-width plane of 56 x 56: every row and column of the patch in use
+    (34, 32, 32, 32, 72, 3, 3, 1, 1),    # 272 tiles: the 16 of the thin last round are cut in halves of the block's 9 taps
+    (34, 64, 32, 32, 40, 5, 3, 1, 2),    # the same with two channel blocks of 15 taps: four slices of 8 and 7 taps
     (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
     (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
     (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
