@@ -42,22 +42,20 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # WRITE_SIZE runs of this script (KiB per dispatch, each scaled by what the same counter reads for a
 # plain 256 MiB copy: FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0000; `--copy-calibration`).  Every entry
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
-KIB = 1024
+# The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": ((4194306 + 262144) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,0>` grid 1048576 (8192^3)"),
-    "sgemm_1024": ((24688 + 4096) * KIB, "row `sgemm_tile_kernel<Tile<64,64,..>,0,0>` (1024^3)"),
-    "sgemm_tall_skinny": ((266447 + 32768) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,0>` grid 131072 (65536 x 1024 x 128)"),
-    "sgemv_16384_rowmajor": ((1049023 + 256) * KIB, "row `sgemv_rowmajor_wg_kernel<2,8>` (GEMV 16384^2, row-major A)"),
-    "sgemv_16384_colmajor": ((1049552 + 576) * KIB, "row `sgemv_colmajor_kernel<true>` + `sgemv_slice_reduce_kernel` (GEMV 16384^2, column-major A)"),
-    "conv_c5_gather": ((100370 + 111537 + 212453 + 116736) * KIB,
-                       "rows `pad_planes_kernel` + `sgemm_tile_kernel<Tile<128,128,..>,0,4>` + `tail_reduce_kernel`"),
-    "conv_c5_two_step": ((112692 + 903172 + 1025061 + 114688 + 100365 + 100352) * KIB,
-                         "rows `im2col_kernel<3>` + `sgemm_tile_kernel<Tile<128,128,..>,0,0>` grid 458752 + `cn_to_nchw_vec_kernel`"),
-    "shortk_256x64x100352": ((25697 + 100352) * KIB, "row `sgemm_shortk_kernel<Tile<64,64,64,32,32>,0,true>` (256 x 100352 x 64)"),
-    "conv_1x1_14x14": ((15519 + 25312) * KIB, "row `sgemm_tile_kernel<Tile<256,128,..>,0,5>` (conv 1x1, 32x256x14x14 -> 1024)"),
-    "fewrows_nn": ((1060242 + 5120) * KIB, "row `sgemm_fewrows_nn_kernel<1,2>` + `splitk_reduce_kernel` (16 x 16384 x 16384)"),
-    "fewrows_nt": ((1060285 + 4119) * KIB, "row `sgemm_fewrows_nt_kernel<true,1>` + `splitk_reduce_kernel` (16384 x 16 x 16384)"),
-    "linear_fwd_8192x4096x4096": (int(1.208e9), "row `sgemm_tile_kernel<Tile<256,128,..>,0,2>` grid 524288 (linear forward)"),
+    "sgemm_8192": (4563245804, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_1024": (29505052, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
+    "sgemm_tall_skinny": (306421102, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
+    "sgemv_16384_rowmajor": (1074462876, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemv_16384_colmajor": (1075318820, "row `sgemv_colmajor_kernel<true>` grid 131072"),
+    "conv_c5_gather": (363982087, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207608827, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129057565, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42284107, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1090915835, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 131072"),
+    "fewrows_nt": (1089942035, "row `sgemm_fewrows_nt_kernel<true, 1>` grid 196608"),
+    "linear_fwd_8192x4096x4096": (1208264570, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -348,9 +346,10 @@ def main() -> int:
             conv_cpu = cpu_leg(conv_cpu_run, cfl * 2 / Bn, "TFLOP/s",
                                "2 of the 32 images: im_2_col + cake_sgemm(KMN) per image as examples/cake_conv.cpp does "
                                "(M=256, K=2304, N=3136 each); median of 3 after a warm-up")
-        # output written as NCHW: inside the GEMM's epilogue on the gather path, a layout pass on the other
-        for fn, label, key in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM, NCHW output", "conv_c5_gather"),
-                               (lib.cake_hip_conv2d_im2col, "im2col kernel, GEMM (the reference's two steps), NCHW layout pass",
+        # output written as NCHW by the GEMM's epilogue on both paths
+        for fn, label, key in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM from the input where it lies, NCHW output",
+                                "conv_c5_gather"),
+                               (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps), NCHW output",
                                 "conv_c5_two_step")):
             _, avg, _ = time_steps(lambda: _lib.check(
                 fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 1,
