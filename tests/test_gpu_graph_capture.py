@@ -83,3 +83,67 @@ def test_captured_sequence_replays_like_eager_calls():
         torch.cuda.synchronize()
         for got, want in zip(captured, eager):
             assert torch.equal(got, want), f"replay {replay}"
+
+
+def test_captured_convolutions_replay_like_eager_calls():
+    """The convolution routes under capture: the input read where it lies (re-laid filters, tail
+    slices summed by a second kernel), the gather from a staged copy (stride 2: staging kernel,
+    tap table) and the reference's two steps (column matrix in a workspace).  A larger eager
+    convolution between the replays grows every one of those workspaces."""
+    dev = torch.device("cuda:0")
+    lib = cake.load()
+    geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: 16 tail tiles in 2 slices
+             (3, 16, 12, 12, 32, 3, 3, 2, 1, lib.cake_hip_conv2d),         # staged copy
+             (2, 8, 16, 16, 24, 3, 3, 1, 1, lib.cake_hip_conv2d_im2col)]   # column matrix first
+    ins, wts = [], []
+    for i, (b, cin, h, w, cout, hf, wf, s, p, _) in enumerate(geoms):
+        ins.append(torch.empty((b, cin, h, w), dtype=torch.float32, device=dev))
+        wts.append(torch.empty((cout, cin, hf, wf), dtype=torch.float32, device=dev))
+        cake.fill_uniform(ins[-1], 300 + i)
+        cake.fill_uniform(wts[-1], 310 + i)
+
+    def outputs():
+        outs = []
+        for b, cin, h, w, cout, hf, wf, s, p, _ in geoms:
+            ho, wo = (h + 2 * p - hf) // s + 1, (w + 2 * p - wf) // s + 1
+            outs.append(torch.zeros((b, cout, ho, wo), dtype=torch.float32, device=dev))
+        return outs
+
+    def run(outs, stream):
+        for (b, cin, h, w, cout, hf, wf, s, p, fn), x, f, o in zip(geoms, ins, wts, outs):
+            assert fn(x.data_ptr(), f.data_ptr(), o.data_ptr(), b, cin, h, w, cout, hf, wf, s, p, 1, None, stream, None) == 0
+
+    side = torch.cuda.Stream()
+    captured = outputs()
+    with torch.cuda.stream(side):
+        run(captured, side.cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(captured, torch.cuda.current_stream().cuda_stream)
+
+    def grow_every_workspace():
+        for b, cin, h, w, cout, s, fn in ((70, 64, 32, 32, 300, 1, lib.cake_hip_conv2d), (8, 32, 40, 40, 64, 2, lib.cake_hip_conv2d),
+                                          (8, 16, 32, 32, 48, 1, lib.cake_hip_conv2d_im2col)):
+            x = torch.empty((b, cin, h, w), dtype=torch.float32, device=dev)
+            f = torch.empty((cout, cin, 3, 3), dtype=torch.float32, device=dev)
+            ho = (h + 2 - 3) // s + 1
+            o = torch.empty((b, cout, ho, ho), dtype=torch.float32, device=dev)
+            assert fn(x.data_ptr(), f.data_ptr(), o.data_ptr(), b, cin, h, w, cout, 3, 3, s, 1, 1, None, None, None) == 0
+        torch.cuda.synchronize()
+
+    for replay in range(4):
+        if replay == 2:
+            grow_every_workspace()
+        for i, t in enumerate(ins):
+            cake.fill_uniform(t, 400 + 10 * replay + i)
+        for t in captured:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = outputs()
+        run(eager, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), f"replay {replay}"
