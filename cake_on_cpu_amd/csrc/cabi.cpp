@@ -1241,6 +1241,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.out_nchw = out_nchw ? 1 : 0;
         cv.batch = batch; cv.Hin = Hin; cv.Win = Win; cv.pad = pad; cv.Hf = Hf; cv.Wf = Wf;
         cv.patch_rows = patch_rows; cv.patch_pitch = patch_pitch;
+        cv.by_row_n = FastDiv::make(row_n); cv.by_hout = FastDiv::make(Hout); cv.by_vrows = FastDiv::make(Hin + 2 * pad);
+        cv.by_channel_chunks = FastDiv::make(patch_rows * ((Win + 3) / 4)); cv.by_row_chunks = FastDiv::make((Win + 3) / 4);
         if ((st = timer.start())) return st;
         if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, taps, stream); }))) return st;
         if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;

@@ -23,6 +23,27 @@ struct IndexTables {
 // Geometry of a convolution whose column matrix B[k][n] is gathered on the fly from a staged
 // copy of the input (conv_stage_input_kernel in misc_kernels.hip: padding written out, rows split
 // into column phases when the stride is above 1):
+// n / d for n < 2^31 as one 32 x 32 -> 64 bit multiply and a shift (division by an invariant
+// integer): with s = ceil(log2 d) and m = floor(2^(31+s) / d) + 1 the error m d - 2^(31+s) is at
+// most d <= 2^s, so n (m d - 2^(31+s)) < 2^(31+s) for every n < 2^31 and the quotient is exact.
+// A hardware division costs tens of vector instructions (a 64-bit one well over a hundred), enough
+// to make a write-bound copy compute-bound -- or, two dozen of them per lane, to put microseconds
+// in front of a tile's first load.
+struct FastDiv {
+    unsigned d, m, sh;
+    __host__ static FastDiv make(unsigned d)
+    {
+        unsigned s = 0;
+        while ((1ull << s) < d) ++s;
+        FastDiv f;
+        f.d = d;
+        f.m = (unsigned)((1ull << (31 + s)) / d + 1);
+        f.sh = 31 + s;
+        return f;
+    }
+    __device__ __forceinline__ unsigned div(unsigned n) const { return (unsigned)(((unsigned long long)n * m) >> sh); }
+};
+
 // k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
 // B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
 struct ConvGeom {
@@ -40,6 +61,9 @@ struct ConvGeom {
     // sgemm_conv_patch.hip only (the input read where it lies, `in` = the NCHW input itself):
     int batch, Hin, Win, pad, Hf, Wf;
     int patch_rows, patch_pitch;   // rows and floats per row of the input patch a workgroup keeps in LDS
+    // divisions by row_n, Hout, rows of a padded image (Hin + 2 pad), 16-byte chunks per patch
+    // channel (patch_rows * ceil(Win / 4)) and chunks per input row
+    FastDiv by_row_n, by_hout, by_vrows, by_channel_chunks, by_row_chunks;
     int tail_halves;               // sgemm_conv_patch.hip: slice s of a tail tile is half h = s & 1 of the taps
                                    // of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest)
 };

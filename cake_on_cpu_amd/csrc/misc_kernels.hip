@@ -11,25 +11,6 @@ namespace cake {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));  // 16 bytes at any 4-byte address
 
-// n / d for n < 2^31 as one 32 x 32 -> 64 bit multiply and a shift (division by an invariant
-// integer): with s = ceil(log2 d) and m = floor(2^(31+s) / d) + 1 the error m d - 2^(31+s) is at
-// most d <= 2^s, so n (m d - 2^(31+s)) < 2^(31+s) for every n < 2^31 and the quotient is exact.
-// A hardware division costs tens of vector instructions (a 64-bit one well over a hundred), enough
-// to make a write-bound copy compute-bound.
-struct FastDiv {
-    unsigned d, m, sh;
-    __host__ static FastDiv make(unsigned d)
-    {
-        unsigned s = 0;
-        while ((1ull << s) < d) ++s;
-        FastDiv f;
-        f.d = d;
-        f.m = (unsigned)((1ull << (31 + s)) / d + 1);
-        f.sh = 31 + s;
-        return f;
-    }
-    __device__ __forceinline__ unsigned div(unsigned n) const { return (unsigned)(((unsigned long long)n * m) >> sh); }
-};
 
 
 // ---------------------------------------------------------------------------

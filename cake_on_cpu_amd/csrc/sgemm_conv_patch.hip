@@ -78,10 +78,10 @@ struct PatchLoader {
 #pragma unroll
         for (int it = 0; it < PATCH_ITERS; ++it) {
             const int q = tid + it * T::THREADS;
-            const int c = q / per_channel, rem = q - c * per_channel;
-            const int r = rem / wc, j = rem - r * wc;
+            const int c = (int)cv.by_channel_chunks.div(q), rem = q - c * per_channel;
+            const int r = (int)cv.by_row_chunks.div(rem), j = rem - r * wc;
             const int v = v0 + r;
-            const int b = v / vrows, hi = v - b * vrows - cv.pad;
+            const int b = (int)cv.by_vrows.div(v), hi = v - b * vrows - cv.pad;
             const bool data = q < total && r < rows_used && b < cv.batch && hi >= 0 && hi < cv.Hin;
             p_off[it] = data ? (((b * cv.Cin + c) * cv.Hin + hi) * cv.Win + 4 * j) * 4 : BUF_OOB;
             p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : -1;
@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
 
     // the tile's first pixel fixes which virtual row the patch starts at
     const int vrows = cv.Hin + 2 * cv.pad;
-    const int g0 = n0 / cv.row_n, img0 = g0 / cv.Hout;
+    const int g0 = (int)cv.by_row_n.div(n0), img0 = (int)cv.by_hout.div(g0);
     const int v0 = img0 * vrows + (g0 - img0 * cv.Hout);
     // where the lane's pixels (one per 32-column block of the wave) sit in the patch under tap (0, 0);
     // the lane's half of an operand group (channels 0..3 or 4..7) is folded in
@@ -206,8 +206,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     for (int tn = 0; tn < T::TN; ++tn) {
         int n = n0 + wn0 + tn * 32 + l32;
         if (n >= g.N) n = n0;                              // computed and dropped
-        const int gr = n / cv.row_n, wo = n - gr * cv.row_n;
-        const int b = gr / cv.Hout, ho = gr - b * cv.Hout;
+        const int gr = (int)cv.by_row_n.div(n), wo = n - gr * cv.row_n;
+        const int b = (int)cv.by_hout.div(gr), ho = gr - b * cv.Hout;
         pix[tn] = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + lh * 4 * PATCH_PLANE_FLOATS;
     }
 
@@ -222,7 +222,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     if (steps > 0) {
         // the rows below the last pixel's window are never read: not fetched either
         const int n_last = min(n0 + T::BN, g.N) - 1;
-        const int g_last = n_last / cv.row_n, img_last = g_last / cv.Hout;
+        const int g_last = (int)cv.by_row_n.div(n_last), img_last = (int)cv.by_hout.div(g_last);
         const int rows_used = img_last * vrows + (g_last - img_last * cv.Hout) - v0 + cv.Hf;
         PL pl;
         pl.init(g, m0, v0, rows_used, tid, patch);
