@@ -1087,12 +1087,18 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, con
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 wbuf[(8 * (r >> 2) + 4 * lh + (r & 3)) * PITCH + tn * 32 + l32] = acc[tm][tn][r];
-        // LDS serves a wave's requests in order, so the reads below see the writes above
+        // LDS serves a wave's requests in order, so the reads below see the writes above.  All of
+        // them are issued before the first store: behind the stores' branches each read would wait
+        // out its own latency.
+        f32x4 turned[32 / ROWS];
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS; ++pass)
+            turned[pass] = *reinterpret_cast<const f32x4*>(wbuf + (pass * ROWS + rd_row) * PITCH + rd_col);
 #pragma unroll
         for (int pass = 0; pass < 32 / ROWS; ++pass) {
             const int lr = pass * ROWS + rd_row;
             const int row = m0 + wm0 + tm * 32 + lr;
-            f32x4 v = *reinterpret_cast<const f32x4*>(wbuf + lr * PITCH + rd_col);
+            f32x4 v = turned[pass];
             if (row < g.M && valid > 0) {
                 float* dst = out + (size_t)row * row_stride + col_off;
                 if (whole) {
