@@ -196,6 +196,40 @@ def test_conv2d_random_geometries():
         done += 1
 
 
+def test_conv2d_random_geometries_whole_channel_blocks():
+    """Seeded random stride-1 geometries with 32, 64 or 96 input channels (the input read where it
+    lies, a patch per channel block in LDS): filters of 3 to 25 taps, square or not, padding 0 to 4
+    (also wider than the filter needs), maps from the filter's size to 60 pixels wide, tiles that
+    straddle image rows and images, against the naive fp64 convolution; NCHW and matrix output,
+    and the same result twice."""
+    rng = np.random.default_rng(1234)
+    done = 0
+    while done < 40:
+        Hf, Wf = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        if Hf * Wf < 3:
+            continue
+        pad = int(rng.integers(0, 5))
+        Hin, Win = int(rng.integers(max(1, Hf - 2 * pad), 40)), int(rng.integers(max(1, Wf - 2 * pad), 61))
+        Bn, Cin, Cout = int(rng.integers(1, 5)), 32 * int(rng.integers(1, 4)), int(rng.integers(1, 300))
+        if Hin * Win * Cin * Bn > 2_000_000:
+            continue
+        nchw = bool(done % 2)
+        print(f"conv2d patch random {done}: b={Bn} Cin={Cin} {Hin}x{Win} Cout={Cout} {Hf}x{Wf} p={pad} nchw={nchw}", flush=True)
+        inp = oracle.uniform((Bn, Cin, Hin, Win), 1700 + done)
+        wt = oracle.uniform((Cout, Cin, Hf, Wf), 1900 + done)
+        ref64, S = oracle.conv_naive_f64(inp, wt, 1, pad)
+        _, _, Hout, Wout = ref64.shape
+        shape = (Bn, Cout, Hout, Wout) if nchw else (Cout, Bn * Hout * Wout)
+        out, again = np.full(shape, np.nan, np.float32), np.full(shape, np.nan, np.float32)
+        cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, Hf, Wf, 1, pad, out_nchw=nchw)
+        cake.conv2d(inp, wt, again, Bn, Cin, Hin, Win, Cout, Hf, Wf, 1, pad, out_nchw=nchw)
+        got = out if nchw else out.reshape(Cout, Bn, Hout, Wout).transpose(1, 0, 2, 3)
+        err = float(np.max(np.abs(got.astype(np.float64) - ref64) / np.maximum(S, 1e-300)))
+        assert err <= TIGHT, (done, err)
+        assert np.array_equal(out, again), done
+        done += 1
+
+
 @pytest.mark.parametrize("geom", CONV_GEOMS, ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
 @pytest.mark.parametrize("explicit", [False, True])
