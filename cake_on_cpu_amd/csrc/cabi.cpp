@@ -1198,8 +1198,23 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // Stride 1 with whole blocks of 32 channels and maps up to about 60 pixels wide: the input is
     // read where it lies, a patch of it per workgroup and channel block kept in LDS with the zero
     // padding around it (sgemm_conv_patch.hip) -- no padded copy, no table of tap offsets.
+    // That kernel has one tile shape, 256 x 128, and one workgroup per CU, so nothing hides a tile's
+    // prologue and epilogue: it is taken where those are small against the tile's K walk and the
+    // tiles fill their rows and the machine -- 64 steps or more, at least three quarters of the
+    // tile rows in use, two rounds of tiles or more (config 5: 840 against 856 us from the staged
+    // copy).  Elsewhere the staged gather with the planner's choice of tile is faster, often by far
+    // (32 x 128 x 56 x 56 -> 256: 440 against 449 us; 64 x 256 x 28 x 28 -> 256: 450 against 538 us;
+    // 32 x 512 x 7 x 7 -> 512: 88 against 534 us).
     int patch_rows = 0, patch_pitch = 0;
-    if (!explicit_cols && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_k(Cin, Hf, Wf)) &&
+    const long patch_tiles_m = (Cout + 255) / 256, patch_tiles_n = ((long)batch * Hout * row_n + 127) / 128;
+    const bool patch_pays = conv_patch_k(Cin, Hf, Wf) / 32 >= 64 && 4L * Cout >= 3L * 256 * patch_tiles_m &&
+                            patch_tiles_m * patch_tiles_n >= 2L * g_ctx.model.cus;
+    // CAKE_HIP_CONV_ROUTE=patch takes that kernel wherever its geometry allows, =staged never
+    // (for tests and measurements; read at every call)
+    const char* route = std::getenv("CAKE_HIP_CONV_ROUTE");
+    const bool patch_wanted = route && !std::strcmp(route, "patch") ? true
+                              : route && !std::strcmp(route, "staged") ? false : patch_pays;
+    if (!explicit_cols && patch_wanted && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_k(Cin, Hf, Wf)) &&
         conv_patch_geometry(batch, Cin, Hin, Win, Hf, Wf, stride, pad, Hout, Wout, &patch_rows, &patch_pitch)) {
         const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n;
         if ((st = g_ctx.conv_filters.reserve((size_t)Cout * Kp * sizeof(float)))) return st;

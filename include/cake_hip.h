@@ -238,7 +238,15 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * without padding needs neither: a plane is then one row of Hin * Win pixels,
  * gathered from the input as it lies, and with at most 64 input channels and
  * enough tiles the images run as one batch of plain products on the short-K
- * kernel.  A batch whose staged input
+ * kernel.  Stride-1 layers with whole blocks of 32 input channels, up to 4
+ * columns of padding and maps up to about 60 pixels wide have a kernel that
+ * reads the input where it lies (no staged copy: a patch of the input per
+ * workgroup and channel block in LDS, zero padding in place); it has a single
+ * 256 x 128 tile and is taken where that pays -- 64 K steps or more, tile rows
+ * at least three quarters full, two rounds of tiles or more.  The environment
+ * variable CAKE_HIP_CONV_ROUTE (read at every call) overrides that choice:
+ * "patch" takes this kernel wherever its geometry allows, "staged" never.
+ * A batch whose staged input
  * would reach 2 GiB, or whose product 2^31 elements, is run in chunks of whole
  * images through the same staged buffer, so input and output may be as large
  * as memory holds; only a single image of 2 GiB takes the two-step path, whose

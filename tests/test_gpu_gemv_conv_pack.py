@@ -196,12 +196,14 @@ def test_conv2d_random_geometries():
         done += 1
 
 
-def test_conv2d_random_geometries_whole_channel_blocks():
-    """Seeded random stride-1 geometries with 32, 64 or 96 input channels (the input read where it
-    lies, a patch per channel block in LDS): filters of 3 to 25 taps, square or not, padding 0 to 4
+def test_conv2d_random_geometries_whole_channel_blocks(monkeypatch):
+    """Seeded random stride-1 geometries with 32, 64 or 96 input channels on the kernel that reads
+    the input where it lies, a patch per channel block in LDS (CAKE_HIP_CONV_ROUTE=patch takes it
+    wherever the geometry allows; by default only large layers do): filters of 3 to 25 taps, square or not, padding 0 to 4
     (also wider than the filter needs), maps from the filter's size to 60 pixels wide, tiles that
     straddle image rows and images, against the naive fp64 convolution; NCHW and matrix output,
     and the same result twice."""
+    monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")
     rng = np.random.default_rng(1234)
     done = 0
     while done < 40:
@@ -232,13 +234,19 @@ def test_conv2d_random_geometries_whole_channel_blocks():
 
 @pytest.mark.parametrize("geom", CONV_GEOMS, ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
-@pytest.mark.parametrize("explicit", [False, True])
-def test_conv2d_matches_oracle(geom, nchw, explicit):
-    """Both convolution paths (column matrix materialised first, as the reference
-    does, or gathered inside the GEMM) against the naive fp64 convolution and
-    against the oracle's own im2col -> cake_sgemm pipeline."""
+@pytest.mark.parametrize("route", ["two steps", "gather", "gather, input where it lies"])
+def test_conv2d_matches_oracle(geom, nchw, route, monkeypatch):
+    """The convolution routes (column matrix materialised first, as the reference does; gathered
+    inside the GEMM by the library's own choice of kernel; gathered from the input where it lies
+    wherever that kernel's geometry allows) against the naive fp64 convolution and against the
+    oracle's own im2col -> cake_sgemm pipeline."""
     Bn, Cin, Hin, Win, Cout, Hf, Wf, stride, pad = geom
-    print(f"conv2d geom={geom} nchw={nchw} explicit={explicit}", flush=True)
+    explicit = route == "two steps"
+    if route == "gather, input where it lies":
+        if Cin % 32 or stride != 1:
+            pytest.skip("that kernel takes whole blocks of 32 channels at stride 1")
+        monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")
+    print(f"conv2d geom={geom} nchw={nchw} route={route}", flush=True)
     inp = oracle.uniform((Bn, Cin, Hin, Win), 54)
     wt = oracle.uniform((Cout, Cin, Hf, Wf), 55)
     ref64, S = oracle.conv_naive_f64(inp, wt, stride, pad)
@@ -313,10 +321,10 @@ def test_conv2d_1x1_many_images(geom, nchw):
     assert np.max(np.abs(two_step - out) / np.maximum(S.max(), 1e-30)) <= TIGHT
 
 
-def test_conv2d_paths_agree_bitwise_layouts():
+def test_conv2d_paths_agree_bitwise_layouts(monkeypatch):
     """The gather from a staged copy sums in the order of the column matrix: same bits as the two
-    steps.  With whole blocks of 32 channels the input is read where it lies and the sum runs
-    channel block by channel block (another order, within the bar), the same on every run."""
+    steps.  The kernel that reads the input where it lies sums channel block by channel block
+    (another order, within the bar), the same on every run."""
     Bn, Cin, Hin, Win, Cout = 2, 24, 20, 20, 48
     inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 56), oracle.uniform((Cout, Cin, 3, 3), 57)
     a = np.empty((Cout, Bn * 400), np.float32)
@@ -326,6 +334,10 @@ def test_conv2d_paths_agree_bitwise_layouts():
     assert np.array_equal(a, b)
     Cin = 32
     inp, wt = oracle.uniform((Bn, Cin, Hin, Win), 56), oracle.uniform((Cout, Cin, 3, 3), 57)
+    cake.conv2d(inp, wt, a, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
+    cake.conv2d(inp, wt, b, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1, explicit_im2col=True)
+    assert np.array_equal(a, b)          # by default a layer this small is gathered from the staged copy
+    monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")
     cake.conv2d(inp, wt, a, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1)
     cake.conv2d(inp, wt, b, Bn, Cin, Hin, Win, Cout, 3, 3, 1, 1, explicit_im2col=True)
     _, S = oracle.conv_naive_f64(inp, wt, 1, 1)

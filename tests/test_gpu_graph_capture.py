@@ -85,11 +85,12 @@ def test_captured_sequence_replays_like_eager_calls():
             assert torch.equal(got, want), f"replay {replay}"
 
 
-def test_captured_convolutions_replay_like_eager_calls():
+def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
     """The convolution routes under capture: the input read where it lies (re-laid filters, tail
     slices summed by a second kernel), the gather from a staged copy (stride 2: staging kernel,
     tap table) and the reference's two steps (column matrix in a workspace).  A larger eager
     convolution between the replays grows every one of those workspaces."""
+    monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")   # layers this small would take the staged copy by themselves
     dev = torch.device("cuda:0")
     lib = cake.load()
     geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: 16 tail tiles in 2 slices
