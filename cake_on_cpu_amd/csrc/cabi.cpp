@@ -631,7 +631,7 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     *out = plan.pub;
     out->kernel = kernel_family(M, N, K, tile_override != nullptr, vec);
     if (out->kernel == CAKE_HIP_KERNEL_SHORT_K) {
-        // what launch_sgemm_shortk does: 64 x 64 (or 64 x 128) tiles with the whole K in one LDS stage, walked in
+        // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
         // column blocks of B by the resident workgroups per CU
         const int tn = shortk_tile_n(M, N, K, model.cus);
         out->tile_m = 64; out->tile_n = tn; out->tile_k = 64;

@@ -56,17 +56,20 @@ int resident_per_cu(const TileInfo& t, const DeviceModel& dev)
     return std::max(1, std::min(dev.lds_per_cu / t.lds_bytes, 2048 / t.threads));
 }
 
-// Tiles left over after the rounds that fill every slot of the machine, when they are few enough
-// (at most half a workgroup per CU) to be worth cutting along K; 0 otherwise.
-int thin_tail_tiles(int tiles, const TileInfo& t, const DeviceModel& dev)
+// Tiles left over when every CU has had the same number of them, when they are few enough (at
+// most half a CU's worth) to be worth cutting along K; 0 otherwise.  Counted per CU, not per
+// resident slot: workgroups that share a CU share its matrix pipes, so what sets the time is how
+// many tiles the fullest CU has, however many of them it holds at once (128 x 25088 x 1152 on
+// 64 x 64 tiles, 784 = 3 x 256 + 16: 63.5 us with the 16 cut, 72.1 us with the 784 counted as
+// less than one round of 1024 slots; 681 x 1544 x 1187: 30.0 against 38.5 us).
+int thin_tail_tiles(int tiles, const DeviceModel& dev)
 {
-    const long cap = (long)dev.cus * resident_per_cu(t, dev);
-    const int rem = (int)(tiles % cap);
+    const int rem = tiles % dev.cus;
     return tiles > dev.cus && rem > 0 && rem <= dev.cus / 2 ? rem : 0;
 }
 
-// Modelled time of one tile shape with one split factor.
-double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
+// Modelled seconds of one workgroup's K walk with a CU to itself.
+double tile_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
 {
     const TileInfo& t = tile_info(tile_id);
     const int tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
@@ -86,37 +89,58 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     // 128 x 128 tile (3000^3: 386 us, where 256 x 128 with its thin last round takes 417 us;
     // 4352 x 4096 x 1024: 270 against 290 us).
     if (tile_id == TILE_96x128x32_W96x32 && wgs >= 2 * dev.cus && ksteps >= 32) eff = 0.93;
-    const double cu_rate = dev.mfma_flops / dev.cus * eff;
-    // Time in units of "one workgroup with a CU to itself at the tile's efficiency".  A CU holds
-    // `slots` workgroups at once, each at 1/slots of its rate, so the rounds that fill every slot
-    // cost `slots` units each.  In the last, partial round the fullest CU decides; a four-wave
-    // workgroup of 96 or 128 rows that is alone on its CU there (one wave per SIMD, nothing to hide
-    // its barriers behind) runs about a third slower than the efficiencies above, which were
-    // measured with the CU full (2956 x 7096 x 796 on 128 x 128 tiles: 324 us, on 96 x 128: 250 us;
-    // the 64 x 64 tiles' figures already are those of a workgroup on its own).
-    const int slots = resident_per_cu(t, dev);
-    const long cap = (long)dev.cus * slots;
-    const long rem = wgs % cap;
-    const int on_fullest = (int)((rem + dev.cus - 1) / dev.cus);
-    const double alone = (on_fullest == 1 && slots >= 2 && t.threads <= 256 && t.bm * t.bn >= 96 * 128) ? 1.3 : 1.0;
-    double rounds = (double)(wgs / cap) * slots + on_fullest * alone;
+    return wg_flops / (dev.mfma_flops / dev.cus * eff);
+}
+
+// What the second kernel of a tail split costs (its launch, the gap in front of it, the slices
+// written and read back): cutting the leftover tiles has to save more than that.
+constexpr double TAIL_SPLIT_SECONDS = 8e-6;
+
+// Slices for the leftover tiles of a thin last round, 1 when cutting them does not pay
+// (1024 x 6272 x 256 on 64 x 64 tiles, 1568 = 6 x 256 + 32 with 5 us per tile: 33.2 us whole,
+// 36.4 us with the 32 cut; 128 x 25088 x 1152, 13 us per tile: 71.8 whole, 61.3 us cut).
+int tail_split_that_pays(int M, int N, int K, int tile_id, const DeviceModel& dev)
+{
+    const TileInfo& t = tile_info(tile_id);
+    const int tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const int ksteps = ceil_div(K, t.bk);
+    const int tt = thin_tail_tiles(tiles, dev);
+    const int ts = tt ? tail_split_for(tt, ksteps, dev) : 1;
+    if (ts <= 1) return 1;
+    const double extra = 64.0 / t.bk;
+    const double saved = (1.0 - (ceil_div(ksteps, ts) + extra) / (ksteps + extra)) * tile_seconds(M, N, K, tile_id, 1, dev);
+    return saved > TAIL_SPLIT_SECONDS ? ts : 1;
+}
+
+// Modelled time of one tile shape with one split factor.
+double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceModel& dev)
+{
+    const TileInfo& t = tile_info(tile_id);
+    const int tiles = ceil_div(M, t.bm) * ceil_div(N, t.bn);
+    const long wgs = (long)tiles * split;
+    const int ksteps = ceil_div(ceil_div(K, split), t.bk);
+    const double extra = 64.0 / t.bk;
+    // Time in units of one tile on a CU: the fullest CU decides.  (Counting rounds in resident
+    // slots, with a penalty for a four-wave workgroup left alone on its CU, was tried and lost on a
+    // set of 130 shapes: 14 of them more than 5 % off the best of four planner variants against 7
+    // for this count.)
+    double rounds = (double)((wgs + dev.cus - 1) / dev.cus);
     bool tail = false;
     if (split == 1) {
-        const int tt = thin_tail_tiles(tiles, t, dev);
-        const int ts = tt ? tail_split_for(tt, ksteps, dev) : 1;
+        const int ts = tail_split_that_pays(M, N, K, tile_id, dev);
         if (ts > 1) {
-            rounds = (double)(wgs / cap) * slots + (ceil_div(ksteps, ts) + extra) / (ksteps + extra);
+            rounds = (double)(wgs / dev.cus) + (ceil_div(ksteps, ts) + extra) / (ksteps + extra);
             tail = true;
         }
     }
-    double s = rounds * wg_flops / cu_rate;
+    double s = rounds * tile_seconds(M, N, K, tile_id, split, dev);
     // never faster than streaming the operands once
     const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
     // the slices are written, read back and summed by a second kernel
     // (the second kernel and the gap in front of it: 1020 x 108 x 731 takes 14.6 us whole, 10.6 us in 4 slices)
     if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 5e-6;
-    if (tail) s += 6e-6;  // the second kernel: about 5 us and the gap in front of it
+    if (tail) s += TAIL_SPLIT_SECONDS;
     return s + 3e-6;  // launch
 }
 
@@ -291,8 +315,8 @@ static int finish_plan(int M, int N, int K, int sched, int tile_id, int split, b
     const int tiles = p.tiles_m * p.tiles_n;
     if (p.split_k == 1 && tail_allowed) {
         const int ksteps = ceil_div(K, t.bk);
-        const int tt = thin_tail_tiles(tiles, t, dev);
-        const int ts = tt ? tail_split_for(tt, ksteps, dev) : 1;
+        const int tt = thin_tail_tiles(tiles, dev);
+        const int ts = tail_split_that_pays(M, N, K, tile_id, dev);
         if (ts > 1) {
             out->tail_k_per_split = ceil_div(ksteps, ts) * t.bk;
             p.tail_split = ceil_div(K, out->tail_k_per_split);

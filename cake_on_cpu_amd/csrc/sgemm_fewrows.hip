@@ -449,9 +449,10 @@ bool fewrows_applies(int M, int N, int K, int lda, int ldb)
     // byte offsets inside a group (15 rows of B plus 256 columns, 47 rows of A) must stay below 2^31
     // 33 to 48 rows only against a large B: at 4096 x 4096 the macro-tile is the faster one (23 against 26 us)
     const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && (double)N * K >= 48.0e6));
-    // (a K walk of fewer than 256 is over before the stream is up to speed: 32 x 6512 x 76 takes
-    // 6.4 us here and 5.1 us on a 64 x 64 tile, 32 x 2882 x 216 7.5 against 6.9 us)
-    return rows_ok && N >= 512 && K >= 256 && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
+    // (a short K walk is over before the stream is up to speed: 32 x 6512 x 76 takes 6.4 us here
+    // and 5.1 us on a 64 x 64 tile, 32 x 2882 x 216 7.5 against 6.9 us; with a single group of 16
+    // rows it pays from a shorter K on, 13 x 2236 x 184: 5.5 against 6.8 us)
+    return rows_ok && N >= 512 && K >= (M <= 16 ? 128 : 256) && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
            (double)lda * 48 * 4 < 2147483648.0;
 }
 

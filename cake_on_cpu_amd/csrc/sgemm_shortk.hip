@@ -17,8 +17,6 @@ namespace cake {
 
 // 64 x 64 tiles of C, 4 waves of 32 x 32; BK is the longest K it takes
 using TileShortK64 = Tile<64, 64, 64, 32, 32>;
-// 64 x 128 tiles, 4 waves of 32 x 64: half the LDS reads of A and half the barriers per product
-using TileShortK128 = Tile<64, 128, 64, 32, 64>;
 
 template <class T>
 static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE) * 4; }  // one stage
@@ -30,7 +28,8 @@ static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE) * 4; 
 // That pays when the matrix work sets the pace (K = 64: 256 x 100352 36.5 -> 35.0 us, 4096^2
 // 26.1 -> 24.5 us, 2048^2 10.0 -> 8.8 us, 8192 x 16384 175 -> 170 us) and costs when the stores do
 // (8192^2 x 48: 75 -> 84 us, x 32: 67 -> 82 us, 16384^2 x 16: 258 -> 291 us, 3000^2 x 48:
-// 15.7 -> 17.2 us), so only K above 56 takes it.
+// 15.7 -> 17.2 us; with an output of a few MB there is nothing to drain: 608 x 1730 x 64
+// 5.8 -> 6.2 us), so only K above 56 with 8 MB of C or more takes it.
 template <class T, int B_MODE, bool PLAIN, bool STREAM_OUT = false>
 __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs g)
 {
@@ -158,17 +157,15 @@ static hipError_t launch_shortk(const GemmArgs& args, int grid, hipStream_t stre
 // from 1 to 16 tiles per CU (1024^2 x 64: 5.3 -> 4.7 us, 3000^2 x 48: 20.1 -> 15.9 us,
 // 4096^2 x 64: 30.5 -> 26.5 us); with up to four tiles per CU every workgroup has one tile and
 // the gain is the single LDS stage and the load-free epilogue.
-// Tiles 128 wide pay from K = 24 down, where the stores of C bound the kernel and fewer, longer
-// row pieces help (16384^2 x 16: 286 -> 268 us, 512 x 20000 x 24: 16.3 -> 16.0 us); with a longer
-// K the three workgroups a CU then holds hide less than four do (256 x 100352 x 64: 46 -> 58 us,
-// 4096^2 x 64: 31 -> 37 us on the same device).
+// Tiles 128 wide (four waves of 32 x 64, three workgroups per CU) were measured against these on
+// the same device from K = 16 to 64 and lost everywhere (16384^2 x 16: 260 against 231 us,
+// 256 x 100352 x 64: 58 against 46 us): the width is a parameter of the launch, with one value.
 int shortk_tile_n(int M, int N, int K, int cus, int batch)
 {
     if (K < 1 || K > 64) return 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64) * batch;
     if (tiles < (long)cus) return 0;
-    const long wide = (long)((M + 63) / 64) * ((N + 127) / 128) * batch;
-    return K <= 24 && wide >= 6L * cus ? 128 : 64;
+    return 64;
 }
 
 // args: tiles_m, tiles_n, group, group_along_n set for 64 x tile_n tiles; split_k = 1, no tail tiles
@@ -178,10 +175,9 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
     if (tiles <= 0) return hipSuccess;
     if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     int grid, lds;
-    if (tile_n != 64 && tile_n != 128) return hipErrorInvalidValue;
+    if (tile_n != 64) return hipErrorInvalidValue;
     shortk_launch_shape(tiles, tile_n, cus, &grid, &lds);
-    if (tile_n == 128) return launch_shortk<TileShortK128, LOAD_VEC4>(args, grid, stream);
-    if (args.K > 56 && !args.accumulate && !args.col_bias)
+    if (args.K > 56 && !args.accumulate && !args.col_bias && (double)args.M * args.N * (args.tiles_n_per_image ? args.tiles_n / args.tiles_n_per_image : 1) >= 2.0e6)
         return launch_shortk_as<TileShortK64, LOAD_VEC4, true, true>(args, grid, stream);
     return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
 }
@@ -189,10 +185,10 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
 // Workgroups launched for `tiles` tiles of 64 x tile_n, and the LDS each of them takes
 void shortk_launch_shape(long tiles, int tile_n, int cus, int* grid, int* lds_bytes)
 {
-    // what the LDS of a CU holds: 35 KB per workgroup with 64-wide tiles, 52 KB with 128-wide ones
-    const long slots = (long)cus * (tile_n == 128 ? 3 : 4);
+    (void)tile_n;
+    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 35 KB per workgroup
     *grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
-    *lds_bytes = tile_n == 128 ? shortk_lds_bytes<TileShortK128>() : shortk_lds_bytes<TileShortK64>();
+    *lds_bytes = shortk_lds_bytes<TileShortK64>();
 }
 
 }  // namespace cake

@@ -78,7 +78,7 @@ enum {
     CAKE_HIP_KERNEL_GEMV = 1,
     CAKE_HIP_KERNEL_STREAM_ROWS = 2, /* few rows of A: B streamed once    */
     CAKE_HIP_KERNEL_STREAM_COLS = 3, /* few columns of B: A streamed once */
-    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K, many tiles: 64 x 64 (K <= 24: 64 x 128) tiles, next tile's operands in flight */
+    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K, many tiles: 64 x 64 tiles, next tile's operands in flight */
 };
 
 /* What the GPU planner decided for one GEMM: the successor of

@@ -166,11 +166,11 @@ def test_plan_covers_any_shape(M, N, K):
 
 
 def test_plan_tail_split():
-    """A thin last round (few tiles left over after the rounds that fill every slot of the
-    machine) is cut along K instead: the convolution GEMM leaves 32 of its 1568 tiles of 128 x 128
-    (two workgroups per CU: 512 slots) and 16 of its 784 tiles of 256 x 128."""
+    """A thin last round (a few tiles left over when every CU has had the same number) is cut
+    along K instead, where that saves more than the second kernel costs: the convolution GEMM
+    leaves 32 of its 1568 tiles of 128 x 128 and 16 of its 784 tiles of 256 x 128."""
     conv = cake.plan(256, 100352, 2304, cake.NA, (128, 128, 32, 0))
-    assert conv.split_k == 1 and conv.tail_tiles == 1568 % 512 and conv.tail_split == 8
+    assert conv.split_k == 1 and conv.tail_tiles == 1568 % 256 and conv.tail_split == 8
     assert conv.grid == 1568 - 32 + 32 * 8
     conv = cake.plan(256, 100352, 2304, cake.NA, (256, 128, 32, 0))
     assert conv.split_k == 1 and conv.tail_tiles == 784 % 256 and conv.tail_split == 15   # 72 K steps in slices of 5
@@ -178,6 +178,8 @@ def test_plan_tail_split():
     auto = cake.plan(256, 100352, 2304)
     assert auto.tail_tiles > 0 and auto.grid == auto.tiles_m * auto.tiles_n + auto.tail_tiles * (auto.tail_split - 1)
     assert cake.plan(8192, 8192, 8192).tail_tiles == 0          # whole rounds: nothing to cut
+    # 64 x 64 tiles: 784 = 3 x 256 + 16 on a walk of 36 steps are cut, 1568 = 6 x 256 + 32 on a walk of 8 are not
+    assert cake.plan(128, 25088, 1152).tail_tiles == 16 and cake.plan(1024, 6272, 256).tail_tiles == 0
     assert cake.plan(256, 100352, 2304, cake.NA, (128, 128, 32, 1)).tail_tiles == 0   # explicit split is literal
 
 
@@ -293,12 +295,13 @@ def test_plan_names_the_kernel_family():
     fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
     assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
     assert fam(16, 16384, 16384) == 2 and fam(32, 600, 256) == 2 and fam(2, 512, 300) == 2
-    assert fam(32, 600, 255) == 0   # a short K walk of few rows stays on the tile
+    assert fam(32, 600, 255) == 0 and fam(17, 4096, 255) == 0   # a short K walk of few rows stays on the tile ...
+    assert fam(16, 4096, 128) == 2 and fam(16, 4096, 127) == 0   # ... a single group of 16 rows streams from K = 128
     assert fam(16384, 16, 16384) == 3 and fam(512, 16, 64) == 3 and fam(16384, 32, 16384) == 3
     assert fam(512, 32, 64) == 0 and fam(4096, 17, 4096) == 0   # 17 to 32 columns: only against a large A
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 16384, 16384) == 0
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
-    assert fam(16, 511, 4096) == 0 and fam(16, 4096, 255) == 0 and fam(16, 16, 100000) == 0
+    assert fam(16, 511, 4096) == 0 and fam(16, 4096, 127) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
@@ -309,11 +312,8 @@ def test_plan_names_the_kernel_family():
     assert (p.kernel, p.tile_m, p.tile_n, p.tile_k, p.threads, p.split_k, p.tail_tiles) == (4, 64, 64, 64, 256, 1, 0)
     assert (p.tiles_m, p.tiles_n) == (4, 1568) and p.grid == 4 * p.cus and p.grid % 8 == 0
     assert 4 * p.lds_bytes <= 160 * 1024
-    # K up to 24 under many tiles: tiles 128 wide, three workgroups per CU
-    p = cake.plan(16384, 16384, 16)
-    assert (p.kernel, p.tile_m, p.tile_n, p.wave_n, p.threads) == (4, 64, 128, 64, 256)
-    assert (p.tiles_m, p.tiles_n) == (256, 128) and p.grid == 3 * p.cus and 3 * p.lds_bytes <= 160 * 1024
-    assert cake.plan(16384, 16384, 25).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
+    # (tiles 128 wide exist but lost every measurement: the choice never takes them)
+    assert cake.plan(16384, 16384, 16).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
 
 
 def test_default_schedule_resolves_accumulate_by_the_reference_rule(monkeypatch):

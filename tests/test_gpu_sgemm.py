@@ -83,9 +83,9 @@ def test_every_tile_shape(tile, shape):
         _check(A, B, Cm, None, (tile, shape, split))
 
 
-TAIL_CASES = [  # (shape M,K,N; tile) -- tile count = a whole number of rounds plus a thin last one
-    # (a round fills every slot: two workgroups per CU for the four-wave tiles and the K-split 64 x 64 one)
-    ((1472, 520, 1472), (64, 64, 64)), ((1470, 517, 1471), (64, 64, 64)),
+TAIL_CASES = [  # (shape M,K,N; tile) -- every CU gets the same number of tiles and a few are left over, on a K
+    # walk long enough for cutting them to pay
+    ((1100, 1500, 1100), (64, 64, 64)), ((1100, 1497, 1099), (64, 64, 32)),
     ((2900, 512, 2900), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
     ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)), ((3168, 512, 2048), (96, 128, 32)),
 ]
@@ -192,7 +192,7 @@ def test_tall_matrix_times_few_columns(shape):
                                    (256, 64, 100352), (9000, 4, 2111), (3584, 64, 3520), (3584, 65, 3520),
                                    # one to four tiles per CU: every workgroup has a single tile, surplus ones leave early
                                    (1024, 64, 1024), (2111, 10, 960), (1100, 33, 1500), (960, 7, 1100),
-                                   # K up to 24 under many tiles: tiles 128 wide
+                                   # K up to 24 under very many tiles
                                    (4096, 16, 8200), (3333, 24, 7777), (8192, 25, 4096)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_short_k_many_tiles(shape):
