@@ -1256,6 +1256,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.out_nchw = out_nchw ? 1 : 0;
         cv.batch = batch; cv.Hin = Hin; cv.Win = Win; cv.pad = pad; cv.Hf = Hf; cv.Wf = Wf;
         cv.patch_rows = patch_rows; cv.patch_pitch = patch_pitch;
+        cv.stream_out = (reinterpret_cast<uintptr_t>(o.dev) & 127) == 0 && (out_nchw ? (Hout * Wout) % 32 == 0 : N % 32 == 0);
         cv.by_row_n = FastDiv::make(row_n); cv.by_hout = FastDiv::make(Hout); cv.by_vrows = FastDiv::make(Hin + 2 * pad);
         cv.by_channel_chunks = FastDiv::make(patch_rows * ((Win + 3) / 4)); cv.by_row_chunks = FastDiv::make((Win + 3) / 4);
         if ((st = timer.start())) return st;

@@ -64,6 +64,8 @@ struct ConvGeom {
     // divisions by row_n, Hout, rows of a padded image (Hin + 2 pad), 16-byte chunks per patch
     // channel (patch_rows * ceil(Win / 4)) and chunks per input row
     FastDiv by_row_n, by_hout, by_vrows, by_channel_chunks, by_row_chunks;
+    int stream_out;                // sgemm_conv_patch.hip: the output's rows are whole 128-byte lines, so it may leave
+                                   // with non-temporal stores (partial lines written that way cost 35-45 %)
     int tail_halves;               // sgemm_conv_patch.hip: slice s of a tail tile is half h = s & 1 of the taps
                                    // of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest)
 };

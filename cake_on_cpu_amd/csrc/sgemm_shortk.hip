@@ -23,14 +23,10 @@ static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE) * 4; 
 
 // PLAIN: C is overwritten and there is no bias, so the epilogue loads nothing and the next
 // tile's operands stay in flight across it
-// STREAM_OUT: C leaves with non-temporal stores.  Ordinary stores leave up to 32 MB of C dirty in
-// the L2s, which the end of the kernel has to wait for; streamed, C drains while the kernel runs.
-// That pays when the matrix work sets the pace (K = 64: 256 x 100352 36.5 -> 35.0 us, 4096^2
-// 26.1 -> 24.5 us, 2048^2 10.0 -> 8.8 us, 8192 x 16384 175 -> 170 us) and costs when the stores do
-// (8192^2 x 48: 75 -> 84 us, x 32: 67 -> 82 us, 16384^2 x 16: 258 -> 291 us, 3000^2 x 48:
-// 15.7 -> 17.2 us; with an output of a few MB there is nothing to drain: 608 x 1730 x 64
-// 5.8 -> 6.2 us), so only K above 56 with 8 MB of C or more takes it.
-template <class T, int B_MODE, bool PLAIN, bool STREAM_OUT = false>
+// (Non-temporal stores for C were measured and left out: where rows of C are whole cache lines
+// they gained 4-6 % on one device and lost 3 % on another, and where they are not -- a row pitch
+// that is no multiple of 128 bytes -- they cost 35-45 %: 4096 x 4100 x 64 27 -> 39 us.)
+template <class T, int B_MODE, bool PLAIN>
 __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs g)
 {
     static_assert(B_MODE == LOAD_VEC4, "row-major operands");
@@ -123,7 +119,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
                 mma_frag<T>(frag[kg & 1], acc);
             }
         }
-        store_c_tile<T, B_MODE, PLAIN, STREAM_OUT>(gt, Bs, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
+        store_c_tile<T, B_MODE, PLAIN>(gt, Bs, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
         if (!more) break;
         t = t_next;
         m0 = m0_next;
@@ -133,10 +129,10 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     }
 }
 
-template <class T, int B_MODE, bool PLAIN, bool STREAM_OUT = false>
+template <class T, int B_MODE, bool PLAIN>
 static hipError_t launch_shortk_as(const GemmArgs& args, int grid, hipStream_t stream)
 {
-    auto kern = sgemm_shortk_kernel<T, B_MODE, PLAIN, STREAM_OUT>;
+    auto kern = sgemm_shortk_kernel<T, B_MODE, PLAIN>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                                        shortk_lds_bytes<T>());
@@ -177,8 +173,6 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
     shortk_launch_shape(tiles, tile_n, cus, &grid, &lds);
-    if (args.K > 56 && !args.accumulate && !args.col_bias && (double)args.M * args.N * (args.tiles_n_per_image ? args.tiles_n / args.tiles_n_per_image : 1) >= 2.0e6)
-        return launch_shortk_as<TileShortK64, LOAD_VEC4, true, true>(args, grid, stream);
     return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
 }
 

@@ -1043,7 +1043,8 @@ __device__ __forceinline__ void k_walk_generic(const GemmArgs& g, float* As, flo
 // the start.  PLAIN: the caller knows that C is overwritten and no bias is added, so the epilogue
 // holds no load at all (a load here would make a kernel that has other loads in flight wait for
 // all of them: the counter of outstanding loads is served in order).
-// STREAM_OUT: whole 16-byte pieces at 16-byte-aligned addresses leave with non-temporal stores.
+// STREAM_OUT: when the caller's geometry says so (ConvGeom::stream_out), whole 16-byte pieces at
+// 16-byte-aligned addresses leave with non-temporal stores.
 template <class T, int B_MODE, bool PLAIN = false, bool STREAM_OUT = false>
 __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, const f32x16 (&acc)[T::TM][T::TN],
                                              int m0, int n0, int slice, int wblk, int wm0, int wn0, int lane,
@@ -1106,7 +1107,7 @@ __device__ __forceinline__ void store_c_tile(const GemmArgs& g, float* smem, con
                     f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst);
                     if (add) v += *d4;
                     if (bias) v += bias_v;
-                    if (STREAM_OUT && (reinterpret_cast<uintptr_t>(dst) & 15) == 0)
+                    if (STREAM_OUT && g.conv.stream_out && (reinterpret_cast<uintptr_t>(dst) & 15) == 0)
                         __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst));
                     else
                         *d4 = v;
