@@ -300,9 +300,19 @@ static int colmajor_slices(int M, int K, int cus)
     const int mblocks = (M + COL_BLOCK_M - 1) / COL_BLOCK_M;
     int want = 2 * cus / mblocks;                  // at most 2 workgroups (8 waves) per CU in one round: more concurrent
                                                     // strided streams than that lose HBM page locality
-    int max_slices = (K + 63) / 64;                // at least 64 k per slice
+    if (want > 64) want = 64;                      // (few columns of y: 1000 x 30000 50 us in 128 slices, 36 us in 64;
+                                                    // 512 x 65536: 70 us in 256 slices, 40 us in 64)
+    int max_slices = (K + 127) / 128;              // at least 128 k per slice (3000^2: 18.8 us in 42 slices, 16.6 in 23)
     if (want > max_slices) want = max_slices;
     if (want < 1) want = 1;
+    // Slices that start a power of two of 8 MB or more apart meet in the same memory channels:
+    // half as many again moves them off that grid (8192^2: 54.8 us in 16 slices, 45.7 in 24;
+    // 8192 x 4096: 36.9 in 16, 25.5 in 24; 16384 x 4096: 51.0 in 8, 42.4 in 12; 32768 x 2048:
+    // 47.9 in 4, 41.8 in 6; 16384^2: 158.8 in 8, 156.9 in 12).
+    if (want >= 4 && (want & (want - 1)) == 0) {
+        const double apart = (double)((K + want - 1) / want) * M * 4.0;
+        if (apart >= 8.0 * 1048576.0 && want * 3 / 2 <= max_slices) want = want * 3 / 2;
+    }
     return want;
 }
 
