@@ -440,7 +440,21 @@ static int nn_cols(int N, int K) { return (double)N * K <= 24.0e6 ? 64 : 128; }
 int fewrows_slices(int M, int N, int K, int cus)
 {
     (void)M;
-    return slices_for((N + nn_cols(N, K) - 1) / nn_cols(N, K), K, cus, 2);
+    // Workgroups = column blocks x slices, up to three per CU.  What decides is how evenly they
+    // fill the CUs: the slice count whose workgroups come closest to whole rounds of one per CU
+    // wins, the smaller count among equals (16 rows, N x K, us by slices: 16384^2 158.7 in 2,
+    // 166.6 in 4; 20000^2 304 in 2, 241 in 3, 259 in 4; 24576^2 427 in 2, 440 in 3, 379 in 4;
+    // 14336^2 140.6 in 2, 172 in 3, 143.5 in 4; 30000 x 12000 229 in 1, 239 in 2).
+    const int blocks = (N + nn_cols(N, K) - 1) / nn_cols(N, K);
+    const int max_slices = std::max(1, std::min((K + FR_K_UNIT - 1) / FR_K_UNIT, std::max(1, 3 * cus / blocks)));
+    int best = 1;
+    double best_fill = 0.0;
+    for (int s = 1; s <= max_slices; ++s) {
+        const long wgs = (long)blocks * s;
+        const double fill = (double)wgs / (double)((wgs + cus - 1) / cus * cus);
+        if (fill > best_fill + 0.03) { best_fill = fill; best = s; }
+    }
+    return best;
 }
 int fewrows_nt_slices(int M, int N, int K, int cus) { return slices_for((N + FR_ROWS - 1) / FR_ROWS, K, cus, M <= 16 ? 3 : 2); }
 
