@@ -44,18 +44,18 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563253643, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
-    "sgemm_1024": (29499944, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
-    "sgemm_tall_skinny": (306425197, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
-    "sgemv_16384_rowmajor": (1074462881, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
-    "sgemv_16384_colmajor": (1075318820, "row `sgemv_colmajor_kernel<true>` grid 131072"),
-    "conv_c5_gather": (353545504, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
-    "conv_c5_two_step": (2207581219, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129072811, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42392854, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
-    "fewrows_nn": (1090903718, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 131072"),
-    "fewrows_nt": (1089930248, "row `sgemm_fewrows_nt_kernel<true, 1>` grid 196608"),
-    "linear_fwd_8192x4096x4096": (1208268384, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "sgemm_8192": (4563310181, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_1024": (29499945, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
+    "sgemm_tall_skinny": (306425198, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
+    "sgemv_16384_rowmajor": (1074462890, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemv_16384_colmajor": (1075843082, "row `sgemv_colmajor_kernel<true>` grid 196608"),
+    "conv_c5_gather": (353529870, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207590196, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129072283, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42392073, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1088107597, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nt": (1089231214, "row `sgemm_fewrows_nt_kernel<true, 1>` grid 196608"),
+    "linear_fwd_8192x4096x4096": (1208266364, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
