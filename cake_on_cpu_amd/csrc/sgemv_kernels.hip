@@ -294,12 +294,26 @@ hipError_t launch_sgemv_rowmajor_multi(const float* A, const float* X, float* Y,
 // column-major
 // ---------------------------------------------------------------------------
 static constexpr int COL_BLOCK_M = 256;  // columns of y per workgroup
+static constexpr int COL_MAX_FILL_SLICES = 3;
 
 static int colmajor_slices(int M, int K, int cus)
 {
     const int mblocks = (M + COL_BLOCK_M - 1) / COL_BLOCK_M;
     int want = 2 * cus / mblocks;                  // at most 2 workgroups (8 waves) per CU in one round: more concurrent
                                                     // strided streams than that lose HBM page locality
+    if (mblocks > cus && mblocks <= 4 * cus) {
+        // More blocks of columns than CUs, up to four per CU (beyond that slices only add traffic:
+        // 300000 x 500, 1172 blocks: 89 us in 1 slice, 93 in 3): the count whose workgroups come closest to whole rounds
+        // of one per CU, the smaller among near-equals, as for the streaming-rows kernel
+        // (70000 x 3000, 274 blocks: 180 us in 1 slice, 154 in 2; 80000 x 8000, 313 blocks: 448 and
+        // 391 us, 373 in 3; 100000 x 2000, 391 blocks: 122 and 136 us).
+        double best = 0.0;
+        for (int s = 1; s <= COL_MAX_FILL_SLICES && s * 128 <= K; ++s) {
+            const long wgs = (long)mblocks * s;
+            const double fill = (double)wgs / (double)((wgs + cus - 1) / cus * cus);
+            if (fill > best + 0.03) { best = fill; want = s; }
+        }
+    }
     if (want > 64) want = 64;                      // (few columns of y: 1000 x 30000 50 us in 128 slices, 36 us in 64;
                                                     // 512 x 65536: 70 us in 256 slices, 40 us in 64)
     int max_slices = (K + 127) / 128;              // at least 128 k per slice (3000^2: 18.8 us in 42 slices, 16.6 in 23)
@@ -324,12 +338,19 @@ size_t sgemv_colmajor_scratch_floats(int M, int K, int cus)
 // grid = (m blocks, k slices).  VEC: each wave covers all 256 columns of the
 // block with one 16-byte load per lane and takes a quarter of the slice's k
 // range; the four waves are summed through LDS in wave order.  Scalar: each
-// thread owns one column over the whole slice.
+// thread owns one column over the whole slice.  A launch of a single slice has `out` = y and
+// adds to it or overwrites it itself (`accumulate`); slices go to the workspace, overwriting.
+//
+// Summing the slices inside this kernel -- every workgroup publishes its partial sums, draws a
+// ticket of its block of columns, and the last one adds them up in slice order -- was measured and
+// costs far more than the second launch it saves (16384^2: 157 -> 293 us, 4096^2: 15 -> 98 us): the
+// device-scope fences it needs write back and invalidate the whole L2 of the workgroup's XCD, and
+// with them the stream of A and the vector x that the other workgroups are reading.
 template <bool VEC>
 __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __restrict__ A,
                                                              const float* __restrict__ x,
                                                              float* __restrict__ out, int M, int K,
-                                                             int k_per_slice)
+                                                             int k_per_slice, int accumulate)
 {
     __shared__ float red[4][COL_BLOCK_M];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -354,7 +375,10 @@ __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __rest
         *reinterpret_cast<f32x4*>(&red[wave][lane * 4]) = acc;
         __syncthreads();
         const int mm = blockIdx.x * COL_BLOCK_M + tid;
-        if (mm < M) dst[mm] = ((red[0][tid] + red[1][tid]) + red[2][tid]) + red[3][tid];
+        if (mm < M) {
+            const float sum = ((red[0][tid] + red[1][tid]) + red[2][tid]) + red[3][tid];
+            dst[mm] = accumulate ? dst[mm] + sum : sum;
+        }
     } else {
         const int m = blockIdx.x * COL_BLOCK_M + tid;
         if (m >= M) return;
@@ -362,7 +386,7 @@ __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __rest
         const float* col = A + (size_t)kbeg * M + m;
 #pragma unroll 8
         for (int k = kbeg; k < kend; ++k, col += M) acc += *col * x[k];
-        dst[m] = acc;
+        dst[m] = accumulate ? dst[m] + acc : acc;
     }
 }
 
@@ -387,12 +411,14 @@ hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M
     k_per_slice = (k_per_slice + 3) & ~3;
     const bool vec = (M % 4 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0);
     const dim3 grid((M + COL_BLOCK_M - 1) / COL_BLOCK_M, slices);
+    float* out = slices == 1 ? y : scratch;          // a single slice needs no second launch
+    const int acc = slices == 1 ? accumulate : 0;
     if (vec)
-        hipLaunchKernelGGL((sgemv_colmajor_kernel<true>), grid, dim3(256), 0, stream, A, x, scratch, M, K, k_per_slice);
+        hipLaunchKernelGGL((sgemv_colmajor_kernel<true>), grid, dim3(256), 0, stream, A, x, out, M, K, k_per_slice, acc);
     else
-        hipLaunchKernelGGL((sgemv_colmajor_kernel<false>), grid, dim3(256), 0, stream, A, x, scratch, M, K, k_per_slice);
+        hipLaunchKernelGGL((sgemv_colmajor_kernel<false>), grid, dim3(256), 0, stream, A, x, out, M, K, k_per_slice, acc);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || slices == 1) return e;
     hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 255) / 256), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
     return hipGetLastError();
 }

@@ -32,6 +32,7 @@ def test_fill_uniform_bit_exact(n, seed):
 # ---------------------------------------------------------------------------
 GEMV_SHAPES = [(1, 1), (8, 1), (13, 2111), (64, 7), (1000, 333), (1024, 1024), (4099, 517),
                (2048, 3000), (300, 70000), (70000, 36),
+               (70000, 400), (70001, 300),     # more blocks of 256 columns than CUs: one launch or a few K slices
                (6, 200000), (9, 65536),        # few long rows: the row-major path cuts K into slices
                (50000, 8), (4097, 20), (333, 31)]  # very short rows: a thread per row
 

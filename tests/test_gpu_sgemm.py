@@ -368,3 +368,31 @@ def test_empty_and_degenerate():
     with pytest.raises(cake.CakeHipError):
         cake.cake_sgemm(np.zeros((4, 4), np.float32), np.zeros((4, 4), np.float32),
                         np.zeros((4, 4), np.float32), 4, 4, 4, 1, None, None, False, False, 1.0, 0.0, 9)
+
+
+def test_calls_from_several_threads_give_the_single_thread_results():
+    """Compute entry points serialise on the library's mutex (they share its workspaces): four
+    threads issuing different products at once -- split-K, tail slices, the streaming kernels,
+    host operands staged through the same buffers -- get bit for bit what one thread gets."""
+    import threading
+    shapes = [(777, 1030, 515), (64, 9000, 70), (1100, 1100, 1500), (16, 4096, 2048), (300, 40, 5000), (2048, 64, 3000),
+              (1, 3000, 3000), (513, 257, 129)]
+    alone = [_run(M, K, N, seedA=10 + i, seedB=20 + i)[2] for i, (M, K, N) in enumerate(shapes)]
+    errors = []
+
+    def worker(t):
+        try:
+            for rep in range(3):
+                for j in range(len(shapes)):
+                    i = (j + 2 * t + rep) % len(shapes)
+                    M, K, N = shapes[i]
+                    got = _run(M, K, N, seedA=10 + i, seedB=20 + i)[2]
+                    if not np.array_equal(got, alone[i]):
+                        errors.append((t, rep, shapes[i]))
+        except Exception as e:     # noqa: BLE001 -- reported by the assertion below
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads: th.start()
+    for th in threads: th.join()
+    assert not errors, errors[:5]
