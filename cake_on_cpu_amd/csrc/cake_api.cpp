@@ -237,6 +237,15 @@ double cake_sgemm_2d_small(float* A, float* B, float* C, int M, int N, int K, in
     return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, 0, 0, 0.f, KMN, 0, 0, 0);
 }
 
+// The timing variant sets sch = KMN and otherwise runs cake_sgemm's steps, packed operands
+// included (src/cake_sgemm.cpp:472-600); K-first assigns C whatever beta says.
+double cake_sgemm_test(float* A, float* B, float* C, int M, int N, int K, int p, cake_cntx_t* cake_cntx,
+                       char* argv[], bool packedA, bool packedB, float alpha, float beta, enum sched sch)
+{
+    (void)alpha; (void)sch;
+    return sgemm_common(A, B, C, M, N, K, p, cake_cntx, argv, packedA, packedB, beta, KMN, 0, 0, 0);
+}
+
 // ---- packing ----------------------------------------------------------------------
 
 size_t cake_sgemm_packed_A_size(int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch)

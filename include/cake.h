@@ -94,6 +94,13 @@ double cake_sgemm_2d_small(float* A, float* B, float* C, int M, int N, int K, in
                            cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0,
                            bool packedB = 0, float alpha = 1, float beta = 0, enum sched sch = NA);
 
+// The reference's timing variant (include/cake.h:39-41, src/cake_sgemm.cpp:472-600): cake_sgemm
+// with the schedule forced to K-first, packedA / packedB honoured, returning the time of the
+// product alone.
+double cake_sgemm_test(float* A, float* B, float* C, int M, int N, int K, int p,
+                       cake_cntx_t* cake_cntx, char* argv[] = NULL, bool packedA = 0,
+                       bool packedB = 0, float alpha = 1, float beta = 0, enum sched sch = NA);
+
 // ---- packing (reference: include/packing.h:6-13,70-72) ----------------------
 
 size_t cake_sgemm_packed_A_size(int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch);

@@ -58,6 +58,9 @@ static void variants_case(cake_cntx_t* cntx)
     cake_sgemm_online(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 0, KMN);
     report("cake_sgemm_online", close_to_naive(A, B, C, M, N, K));
     memset(C, 0, sizeof(float) * M * N);
+    cake_sgemm_test(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 1, NKM);   // K-first whatever is asked: C assigned
+    report("cake_sgemm_test", close_to_naive(A, B, C, M, N, K));
+    memset(C, 0, sizeof(float) * M * N);
     cake_sgemm(A, B, C, M, N, K, p, NULL);  // NULL context, all defaults
     report("cake_sgemm default arguments, NULL context", !cake_sgemm_checker(A, B, C, N, M, K));
     free(A); free(B); free(C);
