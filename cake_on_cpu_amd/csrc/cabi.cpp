@@ -392,7 +392,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     }
     if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
         // a tall A against a few columns of B: the same with A streamed along its rows
-        const int slices = fewrows_nt_slices(N, M, K, g_ctx.model.cus);
+        const int slices = fewrows_nt_slices(N, M, K, lda, true, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
             int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
@@ -1482,7 +1482,7 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
     const bool few_w = !tile_override && !few_x && fewrows_nt_applies(N, M, K, K, K, false);
     if (few_x || few_w) {
         // a few rows on one side: the other operand is streamed once as it lies
-        const int slices = few_x ? fewrows_nt_slices(M, N, K, cus) : fewrows_nt_slices(N, M, K, cus);
+        const int slices = few_x ? fewrows_nt_slices(M, N, K, K, false, cus) : fewrows_nt_slices(N, M, K, K, false, cus);
         float* partial = nullptr;
         if (slices > 1) {
             if ((st = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial))) return st;

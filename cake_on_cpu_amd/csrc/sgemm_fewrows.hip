@@ -28,6 +28,11 @@
 // lane that loads 4 consecutive k of its row (16 bytes) feeds them to 4
 // successive MFMAs: MFMA e of a group of 16 k works on k = 4 (l / 16) + e.
 #include "sgemm_tile.hpp"
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
 
 namespace cake {
 
@@ -230,9 +235,6 @@ __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* _
 // it back in MFMA order: no barrier, LDS operations of one wave complete in order.  The waves
 // of a workgroup take the steps of 32 k in turn, so together they read 512 contiguous bytes of
 // every row at a time.
-static constexpr int NT_STEP = 32;                               // k per step of a wave
-static constexpr int NT_STAGES = 1;                             // steps in flight per wave
-static constexpr int NT_PITCH = 36;                              // floats per staged row: 16-byte reads of 16 rows spread over all banks
 __device__ __forceinline__ f32x4 keep_below(f32x4 v, int valid)  // zero the elements at and past `valid`
 {
     if (valid < 4) v[3] = 0.f;
@@ -243,7 +245,11 @@ __device__ __forceinline__ f32x4 keep_below(f32x4 v, int valid)  // zero the ele
 }
 
 // XG groups of 16 rows of X (M <= 16 XG): every W value staged feeds XG MFMAs.
-template <bool X_KMAJOR, int XG>
+// R rows of W per workgroup (64, 32 or 16), KSTEP k per step of a wave (32 or 64: a load
+// instruction covers 8 rows x 128 bytes or 4 rows x 256 bytes), STAGES steps in flight per wave.
+// Staged rows are KSTEP + 4 floats apart: the 16-byte reads of 16 rows in MFMA order spread
+// over all banks.
+template <bool X_KMAJOR, int XG, int R, int KSTEP, int STAGES>
 __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __restrict__ X,
                                                                const float* __restrict__ W,
                                                                float* __restrict__ out, int M, int N, int K,
@@ -254,18 +260,24 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
                                                                const float* __restrict__ bias_i)
 {
     constexpr int XROWS = 16 * XG;
-    constexpr int WAVE_FLOATS = (FR_ROWS + XROWS) * NT_PITCH;   // 64 rows of W and 16 XG of X
+    constexpr int PITCH = KSTEP + 4;
+    constexpr int LPR = KSTEP / 4;                    // lanes along a row in load order
+    constexpr int RPI = 64 / LPR;                     // rows per load instruction
+    constexpr int NW = R / RPI, NX = XROWS / RPI;     // load instructions per step: W, X (row-major)
+    constexpr int NK = KSTEP / 4;                     // k-major X: 4 k per instruction and group
+    constexpr int WAVE_FLOATS = (R + XROWS) * PITCH;  // R rows of W and 16 XG of X
     __shared__ __align__(16) float smem[4 * WAVE_FLOATS];
-    static_assert(4 * WAVE_FLOATS >= XROWS * FR_ROWS, "the reduction buffer fits the staging memory");
+    static_assert(4 * WAVE_FLOATS >= XROWS * R, "the reduction buffer fits the staging memory");
+    static_assert(R % 16 == 0 && R % RPI == 0 && XROWS % RPI == 0 && (XROWS * R) % 256 == 0, "shape");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 15, lq = lane >> 4;   // MFMA order: row li, k = 4 lq .. + 3 of a group of 16
-    const int lr = lane >> 3, lc = lane & 7;    // load order: row lr of 8, k = 4 lc .. + 3 of the step
-    const int n0 = blockIdx.x * FR_ROWS;
+    const int li = lane & 15, lq = lane >> 4;       // MFMA order: row li, k = 4 lq .. + 3 of a group of 16
+    const int lr = lane / LPR, lc = lane % LPR;     // load order: row lr of RPI, k = 4 lc .. + 3 of the step
+    const int n0 = blockIdx.x * R;
     const int kbeg = blockIdx.y * k_per_slice;
     const int kend = min(K, kbeg + k_per_slice);
-    float* Ws = smem + wave * WAVE_FLOATS;      // [64][NT_PITCH]
-    float* Xs = Ws + FR_ROWS * NT_PITCH;        // [16 XG][NT_PITCH]
+    float* Ws = smem + wave * WAVE_FLOATS;      // [R][PITCH]
+    float* Xs = Ws + R * PITCH;                 // [16 XG][PITCH]
 
     const float* Wb = W + (size_t)n0 * ldw;
     const int rows_left = N - n0;
@@ -274,40 +286,40 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     const int w_off = (lr * ldw + 4 * lc) * 4;
     const int x_off = X_KMAJOR ? (lq * ldx + li) * 4 : (lr * ldx + 4 * lc) * 4;
 
-    f32x4 acc[XG][4];
+    f32x4 acc[XG][R / 16];
 #pragma unroll
     for (int xg = 0; xg < XG; ++xg)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) acc[xg][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < R / 16; ++g) acc[xg][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Rows at and past N (or M) are not masked: what they bring only reaches results that are
     // never written.  Their addresses are kept inside the operands by exact record counts, and
-    // a group of 8 rows that starts past the end gets a count of 0 (records_left must not be asked
+    // a group of rows that starts past the end gets a count of 0 (records_left must not be asked
     // about a start past the end: its difference would wrap to "everything in range").
     // TAIL: the last, partial step of the slice; k at and past kend reads as zero on both sides.
     // live = false: a step past the end of the wave's share, loaded as zeros without a memory
     // access (record count 0), so that the loop below needs no branch
-    auto load_step = [&](int k, bool live, auto tail, f32x4 (&gw)[8], f32x4 (&gx)[2 * XG], float (&gk)[8 * XG]) {
+    auto load_step = [&](int k, bool live, auto tail, f32x4 (&gw)[NW], f32x4 (&gx)[NX], float (&gk)[NK * XG]) {
         constexpr bool TAIL = decltype(tail)::value;
         const int below = kend - (k + 4 * lc);   // of this lane's 4 k, how many lie below kend
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const unsigned used = (unsigned)(8 * t) * (unsigned)ldw + (unsigned)k;
-            const unsigned rec = live && 8 * t < rows_left ? records_left(w_elems, used) : 0u;
-            gw[t] = stream_load_f32x4(Wb + (size_t)(8 * t) * ldw + k, TAIL && below <= 0 ? BUF_OOB : w_off, rec);
+        for (int t = 0; t < NW; ++t) {
+            const unsigned used = (unsigned)(RPI * t) * (unsigned)ldw + (unsigned)k;
+            const unsigned rec = live && RPI * t < rows_left ? records_left(w_elems, used) : 0u;
+            gw[t] = stream_load_f32x4(Wb + (size_t)(RPI * t) * ldw + k, TAIL && below <= 0 ? BUF_OOB : w_off, rec);
             if (TAIL) gw[t] = keep_below(gw[t], below);
         }
         if constexpr (!X_KMAJOR) {
 #pragma unroll
-            for (int t = 0; t < 2 * XG; ++t) {
-                const unsigned used = (unsigned)(8 * t) * (unsigned)ldx + (unsigned)k;
-                const unsigned rec = live && 8 * t < M ? records_left(x_elems, used) : 0u;
-                gx[t] = buffer_load_f32x4(X + (size_t)(8 * t) * ldx + k, TAIL && below <= 0 ? BUF_OOB : x_off, rec);
+            for (int t = 0; t < NX; ++t) {
+                const unsigned used = (unsigned)(RPI * t) * (unsigned)ldx + (unsigned)k;
+                const unsigned rec = live && RPI * t < M ? records_left(x_elems, used) : 0u;
+                gx[t] = buffer_load_f32x4(X + (size_t)(RPI * t) * ldx + k, TAIL && below <= 0 ? BUF_OOB : x_off, rec);
                 if (TAIL) gx[t] = keep_below(gx[t], below);
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {   // k = 4 t + lq of the step, i = 16 xg + li
+            for (int t = 0; t < NK; ++t) {   // k = 4 t + lq of the step, i = 16 xg + li
                 const unsigned used = (unsigned)(k + 4 * t) * (unsigned)ldx;
                 const unsigned rec = live && (!TAIL || k + 4 * t < kend) ? records_left(x_elems, used) : 0u;
                 const int off = TAIL && k + 4 * t + lq >= kend ? BUF_OOB : x_off;
@@ -318,30 +330,30 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the loads in front of the MFMAs they overlap
     };
-    auto store_step = [&](const f32x4 (&gw)[8], const f32x4 (&gx)[2 * XG], const float (&gk)[8 * XG]) {
+    auto store_step = [&](const f32x4 (&gw)[NW], const f32x4 (&gx)[NX], const float (&gk)[NK * XG]) {
 #pragma unroll
-        for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(Ws + (8 * t + lr) * NT_PITCH + 4 * lc) = gw[t];
+        for (int t = 0; t < NW; ++t) *reinterpret_cast<f32x4*>(Ws + (RPI * t + lr) * PITCH + 4 * lc) = gw[t];
         if constexpr (!X_KMAJOR) {
 #pragma unroll
-            for (int t = 0; t < 2 * XG; ++t) *reinterpret_cast<f32x4*>(Xs + (8 * t + lr) * NT_PITCH + 4 * lc) = gx[t];
+            for (int t = 0; t < NX; ++t) *reinterpret_cast<f32x4*>(Xs + (RPI * t + lr) * PITCH + 4 * lc) = gx[t];
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t)
+            for (int t = 0; t < NK; ++t)
 #pragma unroll
-                for (int xg = 0; xg < XG; ++xg) Xs[(16 * xg + li) * NT_PITCH + 4 * t + lq] = gk[XG * t + xg];
+                for (int xg = 0; xg < XG; ++xg) Xs[(16 * xg + li) * PITCH + 4 * t + lq] = gk[XG * t + xg];
         }
         __builtin_amdgcn_sched_barrier(0);
     };
     auto compute_step = [&]() {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < KSTEP / 16; ++u) {
             f32x4 x[XG];
 #pragma unroll
             for (int xg = 0; xg < XG; ++xg)
-                x[xg] = *reinterpret_cast<const f32x4*>(Xs + (16 * xg + li) * NT_PITCH + 16 * u + 4 * lq);
+                x[xg] = *reinterpret_cast<const f32x4*>(Xs + (16 * xg + li) * PITCH + 16 * u + 4 * lq);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const f32x4 w = *reinterpret_cast<const f32x4*>(Ws + (16 * g + li) * NT_PITCH + 16 * u + 4 * lq);
+            for (int g = 0; g < R / 16; ++g) {
+                const f32x4 w = *reinterpret_cast<const f32x4*>(Ws + (16 * g + li) * PITCH + 16 * u + 4 * lq);
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
 #pragma unroll
@@ -353,26 +365,35 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
     };
 
     {
-        // The wave's steps are wave, wave + 4, ... below `full`; NT_STAGES of them are in flight.
-        f32x4 gw[NT_STAGES][8], gx[NT_STAGES][2 * XG];
-        float gk[NT_STAGES][8 * XG];
-        const int full = (kend - kbeg) / NT_STEP;
+        // The wave's steps are wave, wave + 4, ... below `full`; STAGES of them are in flight.
+        f32x4 gw[STAGES][NW], gx[STAGES][NX];
+        float gk[STAGES][NK * XG];
+        const int full = (kend - kbeg) / KSTEP;
         const int mine = full > wave ? (full - wave + 3) >> 2 : 0;
-        auto step_k = [&](int j) { return kbeg + NT_STEP * (wave + 4 * j); };
+        // Workgroups start their walk at different steps and wrap around: rows of W are a power
+        // of two apart more often than not, and workgroups that all read the same k of their rows
+        // at the same time meet in the same memory channels (a pure read of 8192 x 8192 in this
+        // shape: 56 us from a common start, 38 us rotated).
+        const int rot = full > 0 ? (int)((blockIdx.x * 7u) % (unsigned)full) : 0;
+        auto step_k = [&](int j) {
+            int s = wave + 4 * j + rot;
+            if (s >= full) s -= full;
+            return kbeg + KSTEP * s;
+        };
         if (mine > 0) {
 #pragma unroll
-            for (int i = 0; i < NT_STAGES; ++i) load_step(step_k(i), i < mine, std::false_type{}, gw[i], gx[i], gk[i]);
-            for (int j = 0; j < mine; j += NT_STAGES) {
+            for (int i = 0; i < STAGES; ++i) load_step(step_k(i), i < mine, std::false_type{}, gw[i], gx[i], gk[i]);
+            for (int j = 0; j < mine; j += STAGES) {
 #pragma unroll
-                for (int i = 0; i < NT_STAGES; ++i) {
+                for (int i = 0; i < STAGES; ++i) {
                     store_step(gw[i], gx[i], gk[i]);
-                    load_step(step_k(j + i + NT_STAGES), j + i + NT_STAGES < mine, std::false_type{}, gw[i], gx[i], gk[i]);
+                    load_step(step_k(j + i + STAGES), j + i + STAGES < mine, std::false_type{}, gw[i], gx[i], gk[i]);
                     compute_step();
                 }
             }
         }
-        if (((kend - kbeg) & (NT_STEP - 1)) && wave == (full & 3)) {
-            load_step(kbeg + NT_STEP * full, true, std::true_type{}, gw[0], gx[0], gk[0]);
+        if (((kend - kbeg) & (KSTEP - 1)) && wave == (full & 3)) {
+            load_step(kbeg + KSTEP * full, true, std::true_type{}, gw[0], gx[0], gk[0]);
             store_step(gw[0], gx[0], gk[0]);
             compute_step();
         }
@@ -387,24 +408,25 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
 #pragma unroll
             for (int xg = 0; xg < XG; ++xg)
 #pragma unroll
-                for (int g = 0; g < 4; ++g)
+                for (int g = 0; g < R / 16; ++g)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        float* p = red + (16 * xg + 4 * lq + r) * FR_ROWS + 16 * g + li;
+                        float* p = red + (16 * xg + 4 * lq + r) * R + 16 * g + li;
                         *p = w == 0 ? acc[xg][g][r] : *p + acc[xg][g][r];
                     }
         }
     }
     __syncthreads();
-    const int n = n0 + (tid & 63);
+    constexpr int PER_THREAD = XROWS * R / 256;     // rows of C' per thread: thread (tid / R) owns PER_THREAD of them
+    const int n = n0 + tid % R;
     if (n >= N) return;
     float* dst = out + (size_t)blockIdx.y * out_slice_stride + (long long)n * ld_n;
     const float bn = bias_n ? bias_n[n] : 0.f;
 #pragma unroll
-    for (int r = 0; r < 4 * XG; ++r) {
-        const int i = 4 * XG * (tid >> 6) + r;
+    for (int r = 0; r < PER_THREAD; ++r) {
+        const int i = PER_THREAD * (tid / R) + r;
         if (i >= M) break;
-        float v = red[i * FR_ROWS + (tid & 63)];
+        float v = red[i * R + tid % R];
         if (accumulate) v += dst[i * ld_i];
         if (bias_n) v += bn;
         if (bias_i) v += bias_i[i];
@@ -456,7 +478,61 @@ int fewrows_slices(int M, int N, int K, int cus)
     }
     return best;
 }
-int fewrows_nt_slices(int M, int N, int K, int cus) { return slices_for((N + FR_ROWS - 1) / FR_ROWS, K, cus, M <= 16 ? 3 : 2); }
+// Shape of the nt kernel for a product: rows of W per workgroup (64 with steps of 32 k, 32 or 16
+// with steps of 64 k and two of them in flight) and K slices.  Every pair is priced by a small model
+// of what a sweep of 48 products showed (16 and 32 rows of X, W from 2048^2 to 20000^2, both
+// layouts of X; us on one device) and the cheapest is taken:
+//  * the stream of W runs at the rate of a plain read times how evenly the workgroups fill the
+//    CUs -- rounds of one per CU, and rounds of as many as the LDS lets a CU hold (16 x 8192 x 8192:
+//    32 rows in 256 workgroups 41.5, 64 rows in 2 x 128: 45.0; 16 x 10000 x 10000: 64 rows in 3 slices,
+//    471 workgroups, 91; in 1 slice, 157 workgroups, 102);
+//  * two groups of 16 rows of X want more than one workgroup per CU (32 x 16384 x 16384: 512
+//    workgroups 202, 256 workgroups 223);
+//  * fewer rows per workgroup fetch X more often: 16 rows cost 8-10 % over 64 with X in rows, twice
+//    that with X k-major, whose loads are single floats (16 x 16384 x 16384: 64 rows 153, 32 rows 161);
+//  * K slices cost the kernel that adds them up, and more with every slice (16 x 4096 x 4096: 16 rows
+//    in one slice 14.1, 64 rows in 4 slices 17.6; 16 x 1024 x 8192: 16 rows in 4 slices 12.1, 64 rows
+//    in 16 slices 15.4);
+//  * a workgroup spends about 1.5 us before its stream is up to speed, so short rows want few
+//    workgroups (16 x 100000 x 512: 64 rows 36.9, 32 rows 42.4: rows of up to 1024 k keep 64 rows
+//    per workgroup when that fills the device);
+//  * rows of W that are not 16-byte aligned cost the 128-byte pieces of the 64-row shape more
+//    (16 x 16385 x 4097: 32 rows 60.6, 64 rows 66.8).
+// Over the sweep the choice is within 1.7 % of the best shape measured on average, 15 % at worst.
+struct NtConfig { int rows, kstep, stages, slices; };
+static NtConfig nt_config(int M, int N, int K, int ldw, bool x_kmajor, int cus)
+{
+    static const NtConfig shapes[3] = {{64, 32, 1, 1}, {32, 64, 2, 1}, {16, 64, 2, 1}};
+    const int groups = M <= 16 ? 1 : 2;
+    const double stream_us = (double)N * K * 4.0 / 7.0e6;
+    const double need = groups == 2 ? 1.5 * cus : 1.0 * cus;
+    NtConfig best = shapes[0];
+    double best_us = 1e30;
+    for (const NtConfig& shape : shapes) {
+        const long blocks = (N + shape.rows - 1) / shape.rows;
+        // rows too short to pay for a workgroup's start twice as often, and 64-row blocks fill the device anyway
+        if (shape.rows < 64 && K <= 1024 && (N + 63) / 64 >= cus) continue;
+        const long lds = (long)(shape.rows + 16 * groups) * (shape.kstep + 4) * 16;
+        const long resident = std::max(1L, std::min(4L, 163840L / lds)) * cus;
+        const double refetch = 1.0 + (x_kmajor ? 0.6 : 0.3) * 16.0 * groups / shape.rows;
+        const double unaligned = shape.rows == 64 && ldw % 4 != 0 ? 1.15 : 1.0;
+        const int max_slices = std::max(1, std::min((K + FR_K_UNIT - 1) / FR_K_UNIT, (int)((3L * cus + blocks - 1) / blocks)));
+        for (int s = 1; s <= max_slices; ++s) {
+            int used;
+            (void)slice_length(K, s, &used);
+            if (used != s) continue;     // the rounding of slices to whole units gives this count no launch of its own
+            const long wgs = blocks * s;
+            const double per_cu = wgs < cus ? (double)wgs / cus : (double)wgs / (double)((wgs + cus - 1) / cus * cus);
+            const double per_round = wgs > resident ? (double)wgs / (double)((wgs + resident - 1) / resident * resident) : 1.0;
+            const double busy = std::min(per_cu, per_round) * std::pow(std::min(1.0, wgs / need), 0.2);
+            const double rounds = (double)((wgs + resident - 1) / resident);     // every round starts its stream anew
+            const double us = stream_us / busy * refetch * unaligned + 1.5 * rounds + (s > 1 ? 4.5 + 0.4 * s : 0.0);
+            if (us < best_us) { best_us = us; best = shape; best.slices = s; }
+        }
+    }
+    return best;
+}
+int fewrows_nt_slices(int M, int N, int K, int ldw, bool x_kmajor, int cus) { return nt_config(M, N, K, ldw, x_kmajor, cus).slices; }
 
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
@@ -514,8 +590,9 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
                                    int accumulate, const float* bias, int cus, hipStream_t stream)
 {
     int used;
-    const int k_per = slice_length(K, fewrows_nt_slices(M, N, K, cus), &used);
-    const dim3 grid((N + FR_ROWS - 1) / FR_ROWS, used), block(256);
+    const NtConfig cfg = nt_config(M, N, K, ldw, x_kmajor, cus);
+    const int k_per = slice_length(K, cfg.slices, &used);
+    const dim3 grid((N + cfg.rows - 1) / cfg.rows, used), block(256);
     const bool split = used > 1;
     float* out = split ? partial : C;
     const long long ld_i = c_is_n_by_m ? 1 : (split ? N : ldc);
@@ -523,10 +600,21 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
     const size_t stride = split ? (size_t)M * N : 0;
     const float* bias_n = split || c_is_n_by_m ? nullptr : bias;
     const float* bias_i = split || !c_is_n_by_m ? nullptr : bias;
-    auto kernel = M <= 16 ? (x_kmajor ? sgemm_fewrows_nt_kernel<true, 1> : sgemm_fewrows_nt_kernel<false, 1>)
-                          : (x_kmajor ? sgemm_fewrows_nt_kernel<true, 2> : sgemm_fewrows_nt_kernel<false, 2>);
-    hipLaunchKernelGGL(kernel, grid, block, 0, stream, X, W, out, M, N, K, ldx, ldw, k_per, ld_i, ld_n, stride,
-                       split ? 0 : accumulate, bias_n, bias_i);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, X, W, out, M, N, K, ldx, ldw, k_per, ld_i, ld_n, stride,
+                           split ? 0 : accumulate, bias_n, bias_i);
+    };
+    auto pick = [&](auto rows, auto kstep, auto stages) {
+        constexpr int R = decltype(rows)::value, KS = decltype(kstep)::value, ST = decltype(stages)::value;
+        if (M <= 16) x_kmajor ? launch(sgemm_fewrows_nt_kernel<true, 1, R, KS, ST>) : launch(sgemm_fewrows_nt_kernel<false, 1, R, KS, ST>);
+        else x_kmajor ? launch(sgemm_fewrows_nt_kernel<true, 2, R, KS, ST>) : launch(sgemm_fewrows_nt_kernel<false, 2, R, KS, ST>);
+    };
+    using std::integral_constant;
+    switch (cfg.rows) {
+    case 64: pick(integral_constant<int, 64>{}, integral_constant<int, 32>{}, integral_constant<int, 1>{}); break;
+    case 32: pick(integral_constant<int, 32>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}); break;
+    default: pick(integral_constant<int, 16>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}); break;
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !split) return e;
     return c_is_n_by_m ? launch_splitk_reduce(partial, C, N, M, ldc, used, accumulate, stream, nullptr, bias)
