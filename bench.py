@@ -44,18 +44,19 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563310181, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_8192": (4563250475, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
     "sgemm_1024": (29499945, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
-    "sgemm_tall_skinny": (306425198, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
-    "sgemv_16384_rowmajor": (1074462890, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemm_tall_skinny": (306425197, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
+    "sgemv_16384_rowmajor": (1074462898, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
     "sgemv_16384_colmajor": (1075843082, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (353529870, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
-    "conv_c5_two_step": (2207590196, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129072283, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42392073, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
-    "fewrows_nn": (1088107597, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nt": (1089231214, "row `sgemm_fewrows_nt_kernel<true, 1>` grid 196608"),
-    "linear_fwd_8192x4096x4096": (1208266364, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "conv_c5_gather": (353530347, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207581038, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129071987, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42381920, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1087401126, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nt": (1083204967, "row `sgemm_fewrows_nt_kernel<true, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083255167, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_8192x4096x4096": (1208263672, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -295,7 +296,7 @@ def main() -> int:
         gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
                    "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
         gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
-                   "sgemm_fewrows_nt_kernel + splitk_reduce_kernel")
+                   "sgemm_fewrows_nt_kernel")
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
@@ -406,8 +407,8 @@ def main() -> int:
                                         stream, None), "linear_forward"), 50, 5, 40.0)
         extras.append({"workload": "linear forward, batch 16, 16384->16384, bias",
                        "us": round(avg * 1e6, 2), "tflops": round(2.0 * Sm * Sn * Sk / avg / 1e12, 2),
-                       "kernel": "sgemm_fewrows_nt_kernel + splitk_reduce_kernel",
-                       "roofline": roofline("hbm", sby, avg, "fewrows_nt")})
+                       "kernel": "sgemm_fewrows_nt_kernel",
+                       "roofline": roofline("hbm", sby, avg, "linear_fwd_16x16384x16384")})
         out["extras"] = extras
 
     # -------------------------------------------------------------- CPU baseline
