@@ -42,6 +42,8 @@ LINEAR_SHAPES = [(1, 1, 1), (7, 5, 3), (64, 96, 48), (33, 130, 257), (128, 10, 9
                  (8, 1024, 4096), (3, 333, 1030), (16, 4099, 2048), (1, 64, 512), (13, 16390, 600), (16, 70, 5000),
                  (32, 1024, 2048), (20, 333, 1030), (17, 4099, 513), (33, 1024, 2048), (48, 2048, 1000), (40, 513, 600),
                  (49, 1024, 2048), (200, 1000, 4099), (64, 4096, 1000), (130, 77, 260), (131, 77, 260),
+                 # the streaming kernel's three shapes: 16, 32 and 64 rows of w per workgroup, ragged everywhere
+                 (16, 1003, 4100), (16, 777, 8200), (30, 1000, 8190), (9, 300, 16400), (24, 2050, 4097),
                  # 2 samples on long rows: one matrix-vector sweep over w for both
                  (2, 2048, 1024), (2, 4096, 2050), (2, 2052, 4097), (2, 16384, 2051), (2, 2048, 1023),
                  # a single sample: the row-major matrix-vector kernels (long rows, K slices, short rows, odd K)

@@ -69,7 +69,8 @@ def test_reference_shape_grid_against_the_oracle():
 
 @pytest.mark.parametrize("shape", [(1, 4096, 3000), (3000, 4096, 1), (1, 20000, 9), (2, 2048, 1024), (8, 1000, 2048),
                                    (32, 2111, 600), (2048, 1000, 8), (600, 2111, 32), (33, 1024, 2048), (2048, 1024, 33),
-                                   (2111, 2111, 2111), (4099, 64, 515), (515, 4100, 4099)],
+                                   (2111, 2111, 2111), (4099, 64, 515), (515, 4100, 4099),
+                                   (16, 777, 8200), (8200, 777, 16), (4100, 1003, 13), (13, 1003, 4100), (16400, 300, 20)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_default_routes(shape):
     """One row on either side (matrix-vector sweep), two rows (two-vector sweep), up to 32 rows on
