@@ -479,7 +479,9 @@ int fewrows_slices(int M, int N, int K, int cus)
     return best;
 }
 // Shape of the nt kernel for a product: rows of W per workgroup (64 with steps of 32 k, 32 or 16
-// with steps of 64 k and two of them in flight) and K slices.  Every pair is priced by a small model
+// with steps of 64 k and two of them in flight; with two groups of rows of X, whose matrix work per
+// byte of W is twice as long, two steps of 32 k in flight for 64 and 32 rows: 32 x 16384 x 16384
+// 208 -> 189 us, 32 x 8192 x 8192 60 -> 54 us) and K slices.  Every pair is priced by a small model
 // of what a sweep of 48 products showed (16 and 32 rows of X, W from 2048^2 to 20000^2, both
 // layouts of X; us on one device) and the cheapest is taken:
 //  * the stream of W runs at the rate of a plain read times how evenly the workgroups fill the
@@ -502,8 +504,10 @@ int fewrows_slices(int M, int N, int K, int cus)
 struct NtConfig { int rows, kstep, stages, slices; };
 static NtConfig nt_config(int M, int N, int K, int ldw, bool x_kmajor, int cus)
 {
-    static const NtConfig shapes[3] = {{64, 32, 1, 1}, {32, 64, 2, 1}, {16, 64, 2, 1}};
+    static const NtConfig shapes1[3] = {{64, 32, 1, 1}, {32, 64, 2, 1}, {16, 64, 2, 1}};
+    static const NtConfig shapes2[3] = {{64, 32, 2, 1}, {32, 32, 2, 1}, {16, 64, 2, 1}};   // two groups: two steps in flight throughout
     const int groups = M <= 16 ? 1 : 2;
+    const NtConfig (&shapes)[3] = groups == 1 ? shapes1 : shapes2;
     const double stream_us = (double)N * K * 4.0 / 7.0e6;
     const double need = groups == 2 ? 1.5 * cus : 1.0 * cus;
     NtConfig best = shapes[0];
@@ -527,7 +531,12 @@ static NtConfig nt_config(int M, int N, int K, int ldw, bool x_kmajor, int cus)
             const double busy = std::min(per_cu, per_round) * std::pow(std::min(1.0, wgs / need), 0.2);
             const double rounds = (double)((wgs + resident - 1) / resident);     // every round starts its stream anew
             const double us = stream_us / busy * refetch * unaligned + 1.5 * rounds + (s > 1 ? 4.5 + 0.4 * s : 0.0);
-            if (us < best_us) { best_us = us; best = shape; best.slices = s; }
+            if (us < best_us) {
+                best_us = us; best = shape; best.slices = s;
+                // a second step in flight pays once a wave has a dozen steps to walk (32 x 3000 x 5000 in
+                // 5 slices of 64 rows: 24.2 us with one step in flight, 26.7 with two)
+                if (shape.rows == 64 && slice_length(K, s, &used) < 1536) best.stages = 1;
+            }
         }
     }
     return best;
@@ -610,9 +619,11 @@ hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, flo
         else x_kmajor ? launch(sgemm_fewrows_nt_kernel<true, 2, R, KS, ST>) : launch(sgemm_fewrows_nt_kernel<false, 2, R, KS, ST>);
     };
     using std::integral_constant;
-    switch (cfg.rows) {
-    case 64: pick(integral_constant<int, 64>{}, integral_constant<int, 32>{}, integral_constant<int, 1>{}); break;
-    case 32: pick(integral_constant<int, 32>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}); break;
+    switch (cfg.rows * 1000 + cfg.kstep * 10 + cfg.stages) {
+    case 64321: pick(integral_constant<int, 64>{}, integral_constant<int, 32>{}, integral_constant<int, 1>{}); break;
+    case 64322: pick(integral_constant<int, 64>{}, integral_constant<int, 32>{}, integral_constant<int, 2>{}); break;
+    case 32642: pick(integral_constant<int, 32>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}); break;
+    case 32322: pick(integral_constant<int, 32>{}, integral_constant<int, 32>{}, integral_constant<int, 2>{}); break;
     default: pick(integral_constant<int, 16>{}, integral_constant<int, 64>{}, integral_constant<int, 2>{}); break;
     }
     hipError_t e = hipGetLastError();
