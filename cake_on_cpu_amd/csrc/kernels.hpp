@@ -133,6 +133,8 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t str
 // Products with K <= 64 and many 64 x 64 tiles: workgroups that walk over tiles with the next
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
 // shortk_tile_n: 0 when the kernel does not apply, else the width of its tiles (64)
+// tile rows per band of the short-K kernel's tile sequence (group of the launch arguments)
+int shortk_band_rows(int tiles_m, int N);
 int shortk_tile_n(int M, int N, int K, int cus, int batch = 1);
 inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1) { return shortk_tile_n(M, N, K, cus, batch) != 0; }
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream);

@@ -164,6 +164,11 @@ int shortk_tile_n(int M, int N, int K, int cus, int batch)
     return 64;
 }
 
+int shortk_band_rows(int tiles_m, int N)
+{
+    return tiles_m <= 16 ? tiles_m : N >= 12288 ? 4 : N >= 6144 ? 8 : 16;
+}
+
 // args: tiles_m, tiles_n, group, group_along_n set for 64 x tile_n tiles; split_k = 1, no tail tiles
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream)
 {
