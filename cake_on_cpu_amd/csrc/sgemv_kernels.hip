@@ -54,8 +54,25 @@ __global__ void __launch_bounds__(256) sgemv_rowmajor_kernel(const float* __rest
     if (VEC) {
         const int K4 = K >> 2;
         const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+        // Rows are a power of two of bytes apart more often than not, and the same k of the ROWS rows
+        // of a wave then lies in the same memory channel: each row is walked one step further along
+        // than the one before (whole steps of 64 lanes, wrapping around; the rest of a row after them).
+        const int whole = K4 >> 6;
+        const int skew = whole >= ROWS ? 1 : 0;    // (so that one subtraction wraps every row)
 #pragma unroll 4
-        for (int c = lane; c < K4; c += 64) {
+        for (int i = 0; i < whole; ++i) {
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                int it = i + r * skew;
+                if (it >= whole) it -= whole;
+                const int c = it * 64 + lane;
+                const f32x4 xv = x4[c];
+                const f32x4 av = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(rowp[r]) + c);
+                acc[r] += av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
+            }
+        }
+        const int c = whole * 64 + lane;
+        if (c < K4) {
             const f32x4 xv = x4[c];
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) {
