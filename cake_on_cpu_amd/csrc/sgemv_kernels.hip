@@ -272,7 +272,7 @@ hipError_t launch_sgemv_rowmajor(const float* A, const float* x, float* y, int M
             hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2, slices), dim3(512), 0, stream, A, x, scratch, M, K, 0, k4_per);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) return e;
-            hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 255) / 256), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
+            hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 63) / 64), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
             return hipGetLastError();
         }
         hipLaunchKernelGGL((sgemv_rowmajor_wg_kernel<2, 8>), dim3((M + 1) / 2), dim3(512), 0, stream, A, x, y, M, K, accumulate, K / 4);
@@ -331,8 +331,13 @@ static int colmajor_slices(int M, int K, int cus)
             if (fill > best + 0.03) { best = fill; want = s; }
         }
     }
-    if (want > 64) want = 64;                      // (few columns of y: 1000 x 30000 50 us in 128 slices, 36 us in 64;
-                                                    // 512 x 65536: 70 us in 256 slices, 40 us in 64)
+    // Few blocks of columns: up to 64 slices, more when one or two blocks would otherwise leave most
+    // CUs idle (us by slices, with the slices added up by four waves per 64 columns -- one thread per
+    // column adding them in turn had made every count above 64 slower: 256 x 262144 88 in 64, 49 in
+    // 191, 55 in 255; 300 x 100000 44 in 64, 31 in 127; 512 x 131072 52 in 64, 43 in 96, 45 in 127;
+    // 1024 x 65536 42 in 64, 47 in 96; 1000 x 30000 24 in 64, 28 in 96; 2048 x 32768 42 in 64, 48 in 96).
+    const int most = mblocks == 1 ? 192 : mblocks == 2 ? 128 : 64;
+    if (want > most) want = most;
     int max_slices = (K + 127) / 128;              // at least 128 k per slice (3000^2: 18.8 us in 42 slices, 16.6 in 23)
     if (want > max_slices) want = max_slices;
     if (want < 1) want = 1;
@@ -410,13 +415,26 @@ __global__ void __launch_bounds__(256) sgemv_colmajor_kernel(const float* __rest
 __global__ void sgemv_slice_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int M,
                                           int slices, int accumulate)
 {
-    const int m = blockIdx.x * 256 + threadIdx.x;
-    if (m >= M) return;
+    // 64 columns per workgroup; its four waves each add every fourth slice, several loads in
+    // flight, and meet in LDS in wave order: a fixed order, so the same sums from run to run.
+    // (One thread per column adding all slices in turn took as long as the slices' loads one after
+    // the other: 256 columns in 255 slices 105 us for a product that the main kernel does in 40.)
+    __shared__ float red[4][64];
+    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int m = blockIdx.x * 64 + c;
+    float acc = 0.f;
+    if (m < M) {
+#pragma unroll 8
+        for (int s = g; s < slices; s += 4) acc += part[(size_t)s * M + m];
+    }
+    red[g][c] = acc;
+    __syncthreads();
     // the slices first, then one addition to what y held: y += A.x rounds the same way whether
     // or not K was cut into slices
-    float acc = 0.f;
-    for (int s = 0; s < slices; ++s) acc += part[(size_t)s * M + m];
-    y[m] = accumulate ? y[m] + acc : acc;
+    if (g == 0 && m < M) {
+        const float sum = ((red[0][c] + red[1][c]) + red[2][c]) + red[3][c];
+        y[m] = accumulate ? y[m] + sum : sum;
+    }
 }
 
 hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M, int K,
@@ -436,7 +454,7 @@ hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M
         hipLaunchKernelGGL((sgemv_colmajor_kernel<false>), grid, dim3(256), 0, stream, A, x, out, M, K, k_per_slice, acc);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || slices == 1) return e;
-    hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 255) / 256), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
+    hipLaunchKernelGGL(sgemv_slice_reduce_kernel, dim3((M + 63) / 64), dim3(256), 0, stream, scratch, y, M, slices, accumulate);
     return hipGetLastError();
 }
 
