@@ -88,6 +88,8 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
             dst = C + (size_t)row * row_stride + off;
         }
         float acc = accumulate ? *dst : 0.f;
+        // (unrolled: the loads of several slices are in flight together, the additions keep their order)
+#pragma unroll 8
         for (int s = 0; s < splits; ++s) acc += partial[(size_t)s * total + i];
         if (col_bias) acc += col_bias[col];
         *dst = acc;
