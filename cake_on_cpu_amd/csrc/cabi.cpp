@@ -91,7 +91,7 @@ struct Context {
     cake_hip_device_t info{};
     DeviceModel model;
     DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
-    DeviceBuffer splitk, gemv, conv, conv_taps, conv_filters, tables, unpacked, linear;
+    DeviceBuffer splitk, gemv, conv, conv_taps, conv_filters, tables, unpacked, linear, turned;
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
     // host <-> device transfers of large host operands: two pinned buffers, a stream, an event each
@@ -391,15 +391,32 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         });
     }
     if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
-        // a tall A against a few columns of B: the same with A streamed along its rows
-        const int slices = fewrows_nt_slices(N, M, K, lda, true, g_ctx.model.cus);
+        // a tall A against a few columns of B: the same with A streamed along its rows.
+        // Against 200 million elements of A and more, up to 16 columns of B (K x N, about a megabyte)
+        // are first turned into N rows of K: the kernel then loads them 16 bytes per lane instead of 4
+        // and stages them with a quarter of the LDS stores, which is worth more than the small kernel
+        // in front (16384 x 16 x 16384: 174 -> 158 us; below that size and with 17 to 32 columns it
+        // costs 3-6 %: 16384 x 8 x 4096 44.8 -> 46.3 us, 8192 x 32 x 8192 58.4 -> 61.9 us).  Not in a
+        // call that must not allocate.
+        const bool turn = !g_noalloc_call && ldb == N && N <= 16 && (double)M * K >= 200.0e6 &&
+                          fewrows_nt_applies(N, M, K, K, lda, false);
+        const float* Bx = B;
+        if (turn) {
+            int st2 = g_ctx.turned.reserve((size_t)K * N * sizeof(float));
+            if (st2) return st2;
+            float* bt = static_cast<float*>(g_ctx.turned.ptr);
+            st2 = timer.family(4, [&] { return launch_transpose(B, bt, K, N, stream); });
+            if (st2) return st2;
+            Bx = bt;
+        }
+        const int slices = fewrows_nt_slices(N, M, K, lda, !turn, g_ctx.model.cus);
         float* partial = nullptr;
         if (slices > 1) {
             int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
             if (st2) return st2;
         }
         return timer.family(0, [&] {
-            return launch_sgemm_fewrows_nt(B, A, C, partial, N, M, K, ldb, lda, ldc, true, true, accumulate,
+            return launch_sgemm_fewrows_nt(Bx, A, C, partial, N, M, K, turn ? K : ldb, lda, ldc, !turn, true, accumulate,
                                            col_bias, g_ctx.model.cus, stream);
         });
     }
@@ -523,7 +540,7 @@ int cake_hip_init(int device)
     if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
     for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
         if (!*e) HIP_TRY(hipEventCreate(e));
-    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.conv_filters, &c.tables, &c.unpacked, &c.linear})
+    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.conv_filters, &c.tables, &c.unpacked, &c.linear, &c.turned})
         b->keep_old = true;
     // this device's copy of the file-scope scratch array (every device has its own, at its own address)
     if (device < MAX_DEVICES && !g_noalloc_ptr[device]) {
@@ -543,7 +560,7 @@ int cake_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     for (DeviceBuffer& b : g_ctx.stage) b.release();
     g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
-    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.conv_taps.release(); g_ctx.conv_filters.release();
+    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.turned.release(); g_ctx.conv_taps.release(); g_ctx.conv_filters.release();
     for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1], &g_ctx.copy_done[0], &g_ctx.copy_done[1]}) {
         if (*e) (void)hipEventDestroy(*e);
         *e = nullptr;

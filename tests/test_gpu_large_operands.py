@@ -73,7 +73,7 @@ def test_matrix_vector_products(big):
     _check(y[rows][:, None], big[:, rows].double().t().contiguous(), x.double()[:, None], "column-major gemv")
 
 
-@pytest.mark.parametrize("N", [16, 48, 200], ids=lambda n: f"N{n}")
+@pytest.mark.parametrize("N", [9, 16, 48, 200], ids=lambda n: f"N{n}")
 def test_large_a(big, N):
     """C = big . B: few columns (streaming kernel for N <= 32) and macro-tiles."""
     B = _filled((R, N), 903)
