@@ -138,8 +138,10 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
     // the slices are written, read back and summed by a second kernel
-    // (the second kernel and the gap in front of it: 1020 x 108 x 731 takes 14.6 us whole, 10.6 us in 4 slices)
-    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 5e-6;
+    // (the second kernel and the gap in front of it: 1020 x 108 x 731 takes 14.6 us whole, 10.6 us in 4 slices;
+    // 3.5 us since that kernel keeps the loads of eight slices in flight -- with 5 us the choice was more than 5 %
+    // off the best of three settings on 6 of 130 shapes, 140 x 2611 x 830 by 16 %, with 3.5 us on none)
+    if (split > 1) s += 4.0 * (double)M * N * (split + 1) / (0.5 * dev.hbm_bytes_per_s) + 3.5e-6;
     if (tail) s += TAIL_SPLIT_SECONDS;
     return s + 3e-6;  // launch
 }
