@@ -44,19 +44,19 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563246891, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
-    "sgemm_1024": (29499945, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
+    "sgemm_8192": (4563259370, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_1024": (29499946, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
     "sgemm_tall_skinny": (306425198, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
     "sgemv_16384_rowmajor": (1074454701, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
     "sgemv_16384_colmajor": (1075863560, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (353517469, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
-    "conv_c5_two_step": (2207584865, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129071991, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42389192, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
-    "fewrows_nn": (1087403161, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nt": (1083204983, "row `sgemm_fewrows_nt_kernel<true, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_16x16384x16384": (1083255143, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_8192x4096x4096": (1208266657, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "conv_c5_gather": (353527701, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207582716, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129072005, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42396240, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1087403164, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nt": (1083225741, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083225741, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_8192x4096x4096": (1208262372, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -296,7 +296,7 @@ def main() -> int:
         gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
                    "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
         gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
-                   "sgemm_fewrows_nt_kernel")
+                   "transpose_kernel (B into 16 rows) + sgemm_fewrows_nt_kernel")
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
