@@ -607,9 +607,30 @@ int cake_hip_free(void* ptr)
     return CAKE_HIP_OK;
 }
 
+// true for ordinary (pageable) host memory: neither device memory nor host memory the runtime knows
+static bool is_pageable_host(const void* p)
+{
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return attr.type == hipMemoryTypeUnregistered;
+}
+
+// Large copies from or to pageable memory travel through the library's pinned buffers like the
+// operands of a compute call (a plain hipMemcpy of 256 MB: 30 GB/s to the device, 17.5 GB/s back).
+// Both wait for the device first, as hipMemcpy on the null stream does for its own stream.
 int cake_hip_memcpy_h2d(void* dst, const void* src, size_t bytes)
 {
     if (bytes && (!dst || !src)) return fail(CAKE_HIP_ERR_ARG, "NULL pointer");
+    if (bytes >= PIN_THRESHOLD && is_pageable_host(src)) {
+        int st = ensure_init();
+        if (st) return st;
+        std::lock_guard<std::mutex> lock(g_mutex);
+        HIP_TRY(hipDeviceSynchronize());
+        return host_to_device(dst, src, bytes);
+    }
     HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
     return CAKE_HIP_OK;
 }
@@ -617,6 +638,13 @@ int cake_hip_memcpy_h2d(void* dst, const void* src, size_t bytes)
 int cake_hip_memcpy_d2h(void* dst, const void* src, size_t bytes)
 {
     if (bytes && (!dst || !src)) return fail(CAKE_HIP_ERR_ARG, "NULL pointer");
+    if (bytes >= PIN_THRESHOLD && is_pageable_host(dst)) {
+        int st = ensure_init();
+        if (st) return st;
+        std::lock_guard<std::mutex> lock(g_mutex);
+        HIP_TRY(hipDeviceSynchronize());
+        return device_to_host(dst, src, bytes);
+    }
     HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return CAKE_HIP_OK;
 }
