@@ -422,7 +422,7 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         // in front (16384 x 16 x 16384: 174 -> 158 us; below that size and with 17 to 32 columns it
         // costs 3-6 %: 16384 x 8 x 4096 44.8 -> 46.3 us, 8192 x 32 x 8192 58.4 -> 61.9 us).  Not in a
         // call that must not allocate.
-        const bool turn = !g_noalloc_call && ldb == N && N <= 16 && (double)M * K >= 200.0e6 &&
+        const bool turn = !g_noalloc_call && ldb == N && N <= 16 && (double)M * K >= 200.0e6 && K <= 64 * 65535 &&   // (what the transpose kernel's grid takes)
                           fewrows_nt_applies(N, M, K, K, lda, false);
         const float* Bx = B;
         if (turn) {
