@@ -314,6 +314,11 @@ def test_plan_names_the_kernel_family():
     assert 4 * p.lds_bytes <= 160 * 1024
     # (tiles 128 wide exist but lost every measurement: the choice never takes them)
     assert cake.plan(16384, 16384, 16).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
+    # the tile sequence runs in bands: all tile rows of a product up to 16 of them, else 4, 8 or 16
+    # tile rows, lower for wider products
+    assert p.group == 4 and cake.plan(1024, 50176, 64).group == 16
+    assert cake.plan(16384, 16384, 16).group == 4 and cake.plan(8192, 8192, 32).group == 8
+    assert cake.plan(16384, 4096, 16).group == 16
 
 
 def test_default_schedule_resolves_accumulate_by_the_reference_rule(monkeypatch):
