@@ -1,6 +1,6 @@
 // sgemm_fewrows.hip -- products in which one operand has at most 32 rows or
-// columns ("a few vectors times a matrix": small-batch linear layers, blocks of
-// matrix-vector products).
+// columns, or A up to 64 rows against a large B ("a few vectors times a matrix":
+// small-batch linear layers, blocks of matrix-vector products).
 //
 // Such a product is bound by reading the large operand once from HBM, not by
 // arithmetic, and a 64-row macro-tile would spend most of the matrix pipe on
@@ -11,7 +11,7 @@
 // so every wave keeps its loads in flight on its own.  The small operand comes
 // from L2 with one load per 4 to 16 loads of the large one.
 //
-//   sgemm_fewrows_nn_kernel   C[M<=32][N] = A[M][K] . B[K][N]      streams B (n contiguous),
+//   sgemm_fewrows_nn_kernel   C[M<=64][N] = A[M][K] . B[K][N]      streams B (n contiguous),
 //                             straight from global memory into MFMA operands
 //   sgemm_fewrows_nt_kernel   C'[i<=32][n] = sum_k X[i][k] W[n][k]  streams W (k contiguous)
 //                             through a wave-private LDS area that turns rows into MFMA
@@ -67,8 +67,12 @@ __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0
 // B value loaded feeds MG MFMAs, so the arithmetic per byte grows with MG.  One and two groups
 // (up to 32 rows) stay bound by memory; three (up to 48 rows) need about as long for the matrix
 // work as for the memory and still beat the 64-row macro-tile on large operands (48 x 16384 x
-// 16384: 220 us against 289 us); four groups (up to 64 rows) are bound by the matrix pipe and
-// were measured no faster than the macro-tile, so they are not instantiated.
+// 16384: 220 us against 289 us).  Four groups (up to 64 rows) are bound by the matrix pipe: against
+// 100 million elements of B and more they are 4 to 11 % ahead of the macro-tile (64 x 16384 x
+// 16384: 265-277 us against 288-298 us; 64 x 10240 x 10240: 121 against 137 us), below that behind
+// it (64 x 8192 x 8192: 76 against 73 us).  The matrix pipe is busy in 85-88 % of that launch's
+// cycles, and the cycles themselves are slower: with the pipe and a 4 TB/s stream both running the
+// device clocks about a tenth below what it holds for 8192^3.
 template <int MG, int NJ>
 __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
                                                                const float* __restrict__ B,
@@ -545,14 +549,15 @@ int fewrows_nt_slices(int M, int N, int K, int ldw, bool x_kmajor, int cus) { re
 
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
-    // byte offsets inside a group (15 rows of B plus 256 columns, 47 rows of A) must stay below 2^31
-    // 33 to 48 rows only against a large B: at 4096 x 4096 the macro-tile is the faster one (23 against 26 us)
-    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && (double)N * K >= 48.0e6));
+    // byte offsets inside a group (15 rows of B plus 256 columns, 63 rows of A) must stay below 2^31
+    // 33 to 48 rows only against a large B: at 4096 x 4096 the macro-tile is the faster one (23 against
+    // 26 us); 49 to 64 rows against a larger one still
+    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && (double)N * K >= 48.0e6) || (M <= 64 && (double)N * K >= 100.0e6));
     // (a short K walk is over before the stream is up to speed: 32 x 6512 x 76 takes 6.4 us here
     // and 5.1 us on a 64 x 64 tile, 32 x 2882 x 216 7.5 against 6.9 us; with a single group of 16
     // rows it pays from a shorter K on, 13 x 2236 x 184: 5.5 against 6.8 us)
     return rows_ok && N >= 512 && K >= (M <= 16 ? 128 : 256) && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
-           (double)lda * 48 * 4 < 2147483648.0;
+           (double)lda * 64 * 4 < 2147483648.0;
 }
 
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
@@ -582,7 +587,8 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
     const size_t stride = used > 1 ? (size_t)M * N : 0;
     auto kernel = M <= 16 ? (cols == 128 ? sgemm_fewrows_nn_kernel<1, 2> : sgemm_fewrows_nn_kernel<1, 1>)
                 : M <= 32 ? (cols == 128 ? sgemm_fewrows_nn_kernel<2, 2> : sgemm_fewrows_nn_kernel<2, 1>)
-                          : (cols == 128 ? sgemm_fewrows_nn_kernel<3, 2> : sgemm_fewrows_nn_kernel<3, 1>);
+                : M <= 48 ? (cols == 128 ? sgemm_fewrows_nn_kernel<3, 2> : sgemm_fewrows_nn_kernel<3, 1>)
+                          : (cols == 128 ? sgemm_fewrows_nn_kernel<4, 2> : sgemm_fewrows_nn_kernel<4, 1>);
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
                        out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();
