@@ -44,19 +44,20 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563259370, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
-    "sgemm_1024": (29499946, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
-    "sgemm_tall_skinny": (306425198, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
-    "sgemv_16384_rowmajor": (1074454701, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemm_8192": (4563254155, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_1024": (29499945, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
+    "sgemm_tall_skinny": (306425197, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
+    "sgemv_16384_rowmajor": (1074454677, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
     "sgemv_16384_colmajor": (1075863560, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (353527701, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
-    "conv_c5_two_step": (2207582716, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129072005, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42396240, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
-    "fewrows_nn": (1087403164, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nt": (1083225741, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_16x16384x16384": (1083225741, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_8192x4096x4096": (1208262372, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "conv_c5_gather": (353502885, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207579283, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129072441, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42353755, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1087406236, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nn_64rows": (1128385571, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
+    "fewrows_nt": (1083220551, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083220551, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_8192x4096x4096": (1208268524, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -257,7 +258,7 @@ def main() -> int:
     if not args.no_extras:
         extras = []
 
-        def gemm_extra(name, M, N, K, traffic_key=None, streaming_kernel=None, cpu=False):
+        def gemm_extra(name, M, N, K, traffic_key=None, streaming_kernel=None, cpu=False, bound="hbm"):
             a, b = dev_uniform((M, K), 1), dev_uniform((K, N), 2)
             c = torch.zeros((M, N), dtype=torch.float32, device=dev)
             p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
@@ -269,8 +270,9 @@ def main() -> int:
             e = {"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
                  "compulsory_GBps": round(by / avg / 1e9, 1), "kernel_family": cake.KERNEL_NAMES[pl.kernel]}
             if streaming_kernel:   # few rows or columns: bound by reading the large operand once
-                e["kernel"] = streaming_kernel
-                e["roofline"] = roofline("hbm", by, avg, traffic_key)
+                e["kernel"] = streaming_kernel   # (or, from 49 rows on, by the matrix pipe)
+                e["roofline"] = (roofline("hbm", by, avg, traffic_key) if bound == "hbm" else
+                                 roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by))
             else:
                 e.update({"tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
                           "schedule": cake.SCHED_NAMES[pl.sched]})
@@ -297,6 +299,8 @@ def main() -> int:
                    "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
         gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
                    "transpose_kernel (B into 16 rows) + sgemm_fewrows_nt_kernel")
+        gemm_extra("sgemm 64 rows: M=64 K=16384 N=16384", 64, 16384, 16384, "fewrows_nn_64rows",
+                   "sgemm_fewrows_nn_kernel<4, 2> + splitk_reduce_kernel", bound="mfma")
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)

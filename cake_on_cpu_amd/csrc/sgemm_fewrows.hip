@@ -52,7 +52,6 @@ __device__ __forceinline__ float load_f32(const float* base, int byte_offset, un
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
 }
 
-static constexpr int FR_ROWS = 64;      // nt: rows of W per workgroup
 static constexpr int FR_K_UNIT = 256;   // K slices are multiples of this: 64 k per wave
 
 // The part of [kbeg, kend) that wave `wave` of 4 walks: quarters rounded up to 16 k
@@ -70,9 +69,10 @@ __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0
 // 16384: 220 us against 289 us).  Four groups (up to 64 rows) are bound by the matrix pipe: against
 // 100 million elements of B and more they are 4 to 11 % ahead of the macro-tile (64 x 16384 x
 // 16384: 265-277 us against 288-298 us; 64 x 10240 x 10240: 121 against 137 us), below that behind
-// it (64 x 8192 x 8192: 76 against 73 us).  The matrix pipe is busy in 85-88 % of that launch's
-// cycles, and the cycles themselves are slower: with the pipe and a 4 TB/s stream both running the
-// device clocks about a tenth below what it holds for 8192^3.
+// it (64 x 8192 x 8192: 76 against 73 us).  The matrix pipe is busy in 84-85 % of that launch's
+// cycles (counters); more loads in flight, a load behind every piece of B that the MFMAs are done
+// with instead of behind the whole unit, and leaving the scheduling to the compiler did not
+// raise that.
 template <int MG, int NJ>
 __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
                                                                const float* __restrict__ B,
@@ -436,17 +436,6 @@ __global__ void __launch_bounds__(256) sgemm_fewrows_nt_kernel(const float* __re
         if (bias_i) v += bias_i[i];
         dst[i * ld_i] = v;
     }
-}
-
-// K slices so that at most `per_cu` workgroups of 4 waves land on every CU: one round of
-// workgroups that all run from start to end (a few more than fit would leave a second, nearly
-// empty round: 16 x 12288 x 12288 took 112 us with 576 workgroups, 99 us with 480)
-static int slices_for(int blocks, int K, int cus, int per_cu)
-{
-    int want = per_cu * cus / blocks;
-    const int max_slices = (K + FR_K_UNIT - 1) / FR_K_UNIT;
-    if (want > max_slices) want = max_slices;
-    return want < 1 ? 1 : want;
 }
 
 static int slice_length(int K, int slices, int* used)
