@@ -146,8 +146,8 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, in
 
 // scratch: at least sgemv_rowmajor_scratch_floats(M, K, cus) floats (0 for most shapes), or nullptr
 size_t sgemv_rowmajor_scratch_floats(int M, int K, int cus);
-// Products in which one operand has few rows or columns (up to 64 rows of A, up to 32 columns of
-// B), bound by streaming the other one: see sgemm_fewrows.hip.
+// Products in which one operand has few rows or columns (up to 112 rows of A, up to 32 columns
+// of B), which stream the other one once: see sgemm_fewrows.hip.
 bool fewrows_applies(int M, int N, int K, int lda, int ldb);
 int fewrows_slices(int M, int N, int K, int cus);
 hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float* partial, int M, int N,

@@ -1,5 +1,5 @@
 // sgemm_fewrows.hip -- products in which one operand has at most 32 rows or
-// columns, or A up to 64 rows against a large B ("a few vectors times a matrix":
+// columns, or A up to 112 rows against a large B ("a few vectors times a matrix":
 // small-batch linear layers, blocks of matrix-vector products).
 //
 // Such a product is bound by reading the large operand once from HBM, not by
@@ -11,7 +11,7 @@
 // so every wave keeps its loads in flight on its own.  The small operand comes
 // from L2 with one load per 4 to 16 loads of the large one.
 //
-//   sgemm_fewrows_nn_kernel   C[M<=64][N] = A[M][K] . B[K][N]      streams B (n contiguous),
+//   sgemm_fewrows_nn_kernel   C[M<=112][N] = A[M][K] . B[K][N]      streams B (n contiguous),
 //                             straight from global memory into MFMA operands
 //   sgemm_fewrows_nt_kernel   C'[i<=32][n] = sum_k X[i][k] W[n][k]  streams W (k contiguous)
 //                             through a wave-private LDS area that turns rows into MFMA
@@ -73,6 +73,14 @@ __device__ __forceinline__ void wave_part(int kbeg, int kend, int wave, int& kw0
 // cycles (counters); more loads in flight, a load behind every piece of B that the MFMAs are done
 // with instead of behind the whole unit, and leaving the scheduling to the compiler did not
 // raise that.
+// Five and seven groups (65 to 80 and 97 to 112 rows) run on 64 columns per workgroup with four
+// units in flight, which is what the registers hold.  They win where the macro-tiles would pad
+// the rows to 96 or 128: 80 x 16384 x 16384 320 us against 374 us, 72 x 8192 x 8192 89 against
+// 98 us, 112 x 16384 x 16384 430 against 475 us (N x K, us for 65/72/80 rows, tiles -> here:
+// 8192 x 4096 54-56 -> 50-52, 4096 x 4096 31-32 -> 31-33, 2048 x 2048 16 -> 16-18; for 104/112
+// rows: 12288 x 12288 278-281 -> 254-256, 8192 x 8192 124-125 -> 120-122, 8192 x 4096 63 -> 69).
+// Six groups tie with the 96-row macro-tile, which pads nothing there (96 x 16384 x 16384: 374
+// against 388 us, 8192 x 8192: 106 against 102 us), and are not instantiated.
 template <int MG, int NJ>
 __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* __restrict__ A,
                                                                const float* __restrict__ B,
@@ -82,7 +90,7 @@ __global__ void __launch_bounds__(256, 2) sgemm_fewrows_nn_kernel(const float* _
                                                                int accumulate, const float* __restrict__ col_bias)
 {
     constexpr int COLS = 64 * NJ;                     // columns of B per workgroup
-    constexpr int STAGES = 8 / NJ;                    // units in flight per wave: 16 loads of B
+    constexpr int STAGES = MG > 4 ? 4 : 8 / NJ;       // units in flight per wave: 16 loads of B (8 from five groups on)
     __shared__ __align__(16) float red[16 * MG * COLS];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -448,19 +456,19 @@ static int slice_length(int K, int slices, int* used)
 
 // Columns of B per workgroup of the nn kernel: 128, or 64 for small products, which then spread
 // over more workgroups with fewer K slices (measured: 16 x 4096 x 4096 17 us against 21 us;
-// 256 columns were slower throughout, 16 x 8192 x 8192: 63 us against 49 us).
-static int nn_cols(int N, int K) { return (double)N * K <= 24.0e6 ? 64 : 128; }
+// 256 columns were slower throughout, 16 x 8192 x 8192: 63 us against 49 us), and for more than
+// 64 rows, whose sums leave registers for no more.
+static int nn_cols(int M, int N, int K) { return M > 64 || (double)N * K <= 24.0e6 ? 64 : 128; }
 
 // workgroups per CU: what the registers of the nn kernel and the LDS of the nt kernel allow
 int fewrows_slices(int M, int N, int K, int cus)
 {
-    (void)M;
     // Workgroups = column blocks x slices, up to three per CU.  What decides is how evenly they
     // fill the CUs: the slice count whose workgroups come closest to whole rounds of one per CU
     // wins, the smaller count among equals (16 rows, N x K, us by slices: 16384^2 158.7 in 2,
     // 166.6 in 4; 20000^2 304 in 2, 241 in 3, 259 in 4; 24576^2 427 in 2, 440 in 3, 379 in 4;
     // 14336^2 140.6 in 2, 172 in 3, 143.5 in 4; 30000 x 12000 229 in 1, 239 in 2).
-    const int blocks = (N + nn_cols(N, K) - 1) / nn_cols(N, K);
+    const int blocks = (N + nn_cols(M, N, K) - 1) / nn_cols(M, N, K);
     const int max_slices = std::max(1, std::min((K + FR_K_UNIT - 1) / FR_K_UNIT, std::max(1, 3 * cus / blocks)));
     int best = 1;
     double best_fill = 0.0;
@@ -538,15 +546,18 @@ int fewrows_nt_slices(int M, int N, int K, int ldw, bool x_kmajor, int cus) { re
 
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
-    // byte offsets inside a group (15 rows of B plus 256 columns, 63 rows of A) must stay below 2^31
+    // byte offsets inside a group (15 rows of B plus 256 columns, 111 rows of A) must stay below 2^31
     // 33 to 48 rows only against a large B: at 4096 x 4096 the macro-tile is the faster one (23 against
-    // 26 us); 49 to 64 rows against a larger one still
-    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && (double)N * K >= 48.0e6) || (M <= 64 && (double)N * K >= 100.0e6));
+    // 26 us); 49 to 64 rows against a larger one still; 65 to 80 and 97 to 112 rows where the
+    // macro-tiles would pad to 96 and 128 (81 to 96 rows fill the 96-row tile)
+    const double big = (double)N * K;
+    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && big >= 48.0e6) || (M <= 64 && big >= 100.0e6) ||
+                                    (M > 64 && M <= 80 && big >= 30.0e6) || (M > 96 && M <= 112 && big >= 64.0e6));
     // (a short K walk is over before the stream is up to speed: 32 x 6512 x 76 takes 6.4 us here
     // and 5.1 us on a 64 x 64 tile, 32 x 2882 x 216 7.5 against 6.9 us; with a single group of 16
     // rows it pays from a shorter K on, 13 x 2236 x 184: 5.5 against 6.8 us)
     return rows_ok && N >= 512 && K >= (M <= 16 ? 128 : 256) && (double)ldb * 16 * 4 + 1024 < 2147483648.0 &&
-           (double)lda * 64 * 4 < 2147483648.0;
+           (double)lda * 112 * 4 < 2147483648.0;
 }
 
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
@@ -567,9 +578,10 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
                                 int K, int lda, int ldb, int ldc, int accumulate, const float* col_bias,
                                 int cus, hipStream_t stream)
 {
+    if (M > 112) return hipErrorInvalidValue;   // seven groups of 16 rows are the most there are
     int used;
     const int k_per = slice_length(K, fewrows_slices(M, N, K, cus), &used);
-    const int cols = nn_cols(N, K);
+    const int cols = nn_cols(M, N, K);
     const dim3 grid((N + cols - 1) / cols, used), block(256);
     float* out = used > 1 ? partial : C;
     const int out_ld = used > 1 ? N : ldc;
@@ -577,7 +589,8 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
     auto kernel = M <= 16 ? (cols == 128 ? sgemm_fewrows_nn_kernel<1, 2> : sgemm_fewrows_nn_kernel<1, 1>)
                 : M <= 32 ? (cols == 128 ? sgemm_fewrows_nn_kernel<2, 2> : sgemm_fewrows_nn_kernel<2, 1>)
                 : M <= 48 ? (cols == 128 ? sgemm_fewrows_nn_kernel<3, 2> : sgemm_fewrows_nn_kernel<3, 1>)
-                          : (cols == 128 ? sgemm_fewrows_nn_kernel<4, 2> : sgemm_fewrows_nn_kernel<4, 1>);
+                : M <= 64 ? (cols == 128 ? sgemm_fewrows_nn_kernel<4, 2> : sgemm_fewrows_nn_kernel<4, 1>)
+                : M <= 80 ? sgemm_fewrows_nn_kernel<5, 1> : sgemm_fewrows_nn_kernel<7, 1>;
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, M, N, K, lda, ldb, k_per,
                        out_ld, stride, used > 1 ? 0 : accumulate, used > 1 ? nullptr : col_bias);
     hipError_t e = hipGetLastError();

@@ -290,7 +290,7 @@ def test_tune_table_load_lookup_save_clear(tmp_path):
 
 def test_plan_names_the_kernel_family():
     """Single rows or columns go to the matrix-vector kernels, up to 32 rows or columns against a
-    wide operand (up to 48 rows against a large one, up to 64 against a larger one still) to the
+    wide operand (more rows against a large one, up to 112 where tiles would pad them) to the
     streaming kernels, the rest (and anything with a tile override) to the macro-tile kernel."""
     fam = lambda M, N, K, tile=None: cake.plan(M, N, K, tile=tile).kernel
     assert fam(1, 4096, 4096) == 1 and fam(4096, 1, 4096) == 1
@@ -300,7 +300,11 @@ def test_plan_names_the_kernel_family():
     assert fam(16384, 16, 16384) == 3 and fam(512, 16, 64) == 3 and fam(16384, 32, 16384) == 3
     assert fam(512, 32, 64) == 0 and fam(4096, 17, 4096) == 0   # 17 to 32 columns: only against a large A
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 8192, 8192) == 0
-    assert fam(49, 16384, 16384) == 2 and fam(64, 10240, 10240) == 2 and fam(64, 9000, 9000) == 0 and fam(65, 16384, 16384) == 0
+    assert fam(49, 16384, 16384) == 2 and fam(64, 10240, 10240) == 2 and fam(64, 9000, 9000) == 0
+    # 65 to 80 and 97 to 112 rows, which the macro-tiles would pad to 96 and 128
+    assert fam(65, 16384, 16384) == 2 and fam(80, 8192, 4096) == 2 and fam(80, 4096, 4096) == 0
+    assert fam(81, 16384, 16384) == 0 and fam(96, 16384, 16384) == 0
+    assert fam(97, 8192, 8192) == 2 and fam(112, 16384, 16384) == 2 and fam(112, 8192, 4096) == 0 and fam(113, 16384, 16384) == 0
     assert fam(33, 4096, 4096) == 0 and fam(16384, 33, 16384) == 0
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 127) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0

@@ -154,13 +154,16 @@ def test_very_long_k_takes_the_element_loader():
                                    (17, 300, 1000), (32, 1000, 2048), (33, 777, 2050), (48, 2111, 1030),
                                    (64, 4096, 1024), (50, 65, 513), (65, 300, 1000), (40, 300, 1000), (47, 4099, 600),
                                    (48, 16384, 4096), (33, 12000, 4100), (41, 7000, 7001), (49, 1000, 2048),
-                                   (64, 8192, 12288), (49, 12301, 8200), (57, 10001, 10003)],
+                                   (64, 8192, 12288), (49, 12301, 8200), (57, 10001, 10003),
+                                   (65, 5000, 6100), (80, 4099, 8200), (73, 7001, 4500), (97, 8200, 8000),
+                                   (112, 9001, 7300), (105, 4100, 16000)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_few_rows_times_wide_matrix(shape):
     """Up to 32 rows of A against a wide B, up to 48 against a large one, up to 64 against 100
-    million elements and more: the streaming kernels (B read once, one to four groups of 16-row
-    MFMAs; other products with more than 32 rows take the tile kernel), with K slices summed in
-    order, ragged N and K, accumulation, and run-to-run identical sums."""
+    million elements and more, 65 to 80 and 97 to 112 where macro-tiles would pad the rows: the
+    streaming kernels (B read once, one to seven groups of 16-row MFMAs; other products with
+    more than 32 rows take the tile kernel), with K slices summed in order, ragged N and K,
+    accumulation, and run-to-run identical sums."""
     M, K, N = shape
     print(f"sgemm few rows M={M} K={K} N={N}", flush=True)
     A, B, Cm = _run(M, K, N)
