@@ -415,15 +415,11 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         });
     }
     if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
-        // a tall A against a few columns of B: the same with A streamed along its rows.
-        // Against 200 million elements of A and more, up to 16 columns of B (K x N, about a megabyte)
-        // are first turned into N rows of K: the kernel then loads them 16 bytes per lane instead of 4
-        // and stages them with a quarter of the LDS stores, which is worth more than the small kernel
-        // in front (16384 x 16 x 16384: 174 -> 158 us; below that size and with 17 to 32 columns it
-        // costs 3-6 %: 16384 x 8 x 4096 44.8 -> 46.3 us, 8192 x 32 x 8192 58.4 -> 61.9 us).  Not in a
-        // call that must not allocate.
-        const bool turn = !g_noalloc_call && ldb == N && N <= 16 && (double)M * K >= 200.0e6 && K <= 64 * 65535 &&   // (what the transpose kernel's grid takes)
-                          fewrows_nt_applies(N, M, K, K, lda, false);
+        // a tall A against a few columns of B: the same with A streamed along its rows.  Up to 16
+        // columns of B (K x N, small next to A) are turned into N rows of K first where
+        // fewrows_nt_turn_pays says so.  Not in a call that must not allocate.
+        const bool turn = !g_noalloc_call && ldb == N && K <= 64 * 65535 &&   // (what the transpose kernel's grid takes)
+                          fewrows_nt_turn_pays(N, M, K, lda, g_ctx.model.cus) && fewrows_nt_applies(N, M, K, K, lda, false);
         const float* Bx = B;
         if (turn) {
             int st2 = g_ctx.turned.reserve((size_t)K * N * sizeof(float));

@@ -155,6 +155,7 @@ hipError_t launch_sgemm_fewrows(const float* A, const float* B, float* C, float*
                                 int cus, hipStream_t stream);
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor);
 int fewrows_nt_slices(int M, int N, int K, int ldw, bool x_kmajor, int cus);
+bool fewrows_nt_turn_pays(int cols, int rows, int K, int lda, int cus);
 hipError_t launch_sgemm_fewrows_nt(const float* X, const float* W, float* C, float* partial, int M, int N,
                                    int K, int ldx, int ldw, int ldc, bool x_kmajor, bool c_is_n_by_m,
                                    int accumulate, const float* bias, int cus, hipStream_t stream);

@@ -544,6 +544,26 @@ static NtConfig nt_config(int M, int N, int K, int ldw, bool x_kmajor, int cus)
 }
 int fewrows_nt_slices(int M, int N, int K, int ldw, bool x_kmajor, int cus) { return nt_config(M, N, K, ldw, x_kmajor, cus).slices; }
 
+// A tall A (rows x K, row pitch lda) against up to 16 columns of B (K x cols): whether to turn B
+// into `cols` rows of K first, so that the kernel loads it 16 bytes at a time and stages it with a
+// quarter of the LDS stores.  That costs a small kernel in front (about 3 us) and pays where
+// workgroups of fewer than 64 rows, which fetch B more often, would fetch it k-major at twice the
+// price: a single K slice, rows of 4096 k and more (us, B as it lies -> turned: 8192 x 16 x 4096
+// 30.7 -> 27.0, 4096 x 16 x 4096 20.8 -> 18.1, 8192 x 16 x 8192 48.7 -> 45.7, 7000 x 16 x 7000
+// 53.2 -> 48.6; not with 64-row workgroups, K slices or short rows: 16384 x 16 x 4096 45.1 ->
+// 45.6, 10000 x 16 x 10000 91.7 -> 96.5, 32768 x 16 x 1024 24.2 -> 27.0, 3000 x 16 x 5000 20 -> 24),
+// and against 200 million elements and more with rows of 16384 k (16384 x 16 x 16384: 166 -> 158).
+// Over 28 products from 2048^2 to 20000^2 the choice is 0.6 % off the better of the two on
+// average and 4.5 % at worst.
+bool fewrows_nt_turn_pays(int cols, int rows, int K, int lda, int cus)
+{
+    if (cols > 16 || K < 4096) return false;
+    if (K >= 16384 && (double)rows * K >= 200.0e6) return true;
+    if (rows < 4096 || lda % 4 != 0) return false;
+    const NtConfig turned = nt_config(cols, rows, K, lda, false, cus);
+    return turned.slices == 1 && turned.rows < 64;
+}
+
 bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 {
     // byte offsets inside a group (15 rows of B plus 256 columns, 111 rows of A) must stay below 2^31
@@ -568,7 +588,9 @@ bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
     // 74-78 us against 69 us; 16384 x 16384: 205 against 270 us).  X as the rows of a small batch
     // (a linear layer, W as it lies): up to 32 rows; a third group of 16 was measured and lost to
     // the macro-tile kernel that reads W along k (48 x 8192 x 8192: 82 against 72 us).
-    const bool rows_ok = M <= 16 || (M <= 32 && (!x_kmajor || (double)N * K >= 50.0e6));
+    // (rows of W that are not 16-byte aligned cost two groups more than the macro-tile between 50
+    // and 100 million elements: 16385 x 32 x 4097 91 against 74 us)
+    const bool rows_ok = M <= 16 || (M <= 32 && (!x_kmajor || ((double)N * K >= 50.0e6 && (ldw % 4 == 0 || (double)N * K >= 100.0e6))));
     return M >= 1 && rows_ok && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
            (double)ldx * 32 * 4 + (x_kmajor ? 128 : 0) < 2147483648.0;
 }

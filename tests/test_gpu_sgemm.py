@@ -178,7 +178,9 @@ def test_few_rows_times_wide_matrix(shape):
                                    (16384, 2111, 16), (1024, 16384, 16), (600, 100, 1), (515, 65, 9),
                                    (1000, 300, 17), (5000, 4099, 4), (4096, 1000, 24), (2050, 777, 32),
                                    (513, 65, 31), (1000, 300, 33), (4096, 1000, 40), (2050, 777, 48), (513, 65, 47),
-                                   (1000, 300, 49)],
+                                   (1000, 300, 49),
+                                   # up to 16 columns against rows of 4096 k and more: B is turned into rows first
+                                   (4097, 4100, 13), (8200, 4096, 16), (5000, 8192, 7), (4100, 4101, 16)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_tall_matrix_times_few_columns(shape):
     """Up to 48 columns of B against a tall A: A streamed once along its rows (49 columns take the
