@@ -582,15 +582,21 @@ bool fewrows_applies(int M, int N, int K, int lda, int ldb)
 
 bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
 {
-    // 64 rows of W, and 32 rows (or 32 k) of X, within 2^31 bytes of the block's origin
-    // X as the few columns of a product (k-major): up to 16 columns win against the 64 x 64
-    // macro-tile at every size, 17 to 32 only from about 50 million elements of W on (8192 x 8192:
-    // 74-78 us against 69 us; 16384 x 16384: 205 against 270 us).  X as the rows of a small batch
-    // (a linear layer, W as it lies): up to 32 rows; a third group of 16 was measured and lost to
-    // the macro-tile kernel that reads W along k (48 x 8192 x 8192: 82 against 72 us).
-    // (rows of W that are not 16-byte aligned cost two groups more than the macro-tile between 50
-    // and 100 million elements: 16385 x 32 x 4097 91 against 74 us)
-    const bool rows_ok = M <= 16 || (M <= 32 && (!x_kmajor || ((double)N * K >= 50.0e6 && (ldw % 4 == 0 || (double)N * K >= 100.0e6))));
+    // 64 rows of W, and 32 rows (or 32 k) of X, within 2^31 bytes of the block's origin.
+    // X as the rows of a small batch (a linear layer, W as it lies): up to 32 rows; a third group
+    // of 16 was measured and lost to the macro-tile kernel that reads W along k (48 x 8192 x 8192:
+    // 82 against 72 us).
+    // X as the few columns of a product (k-major), against the 128 x 32 macro-tile with its K
+    // slices (us, here / tile): 17 to 32 columns from 100 million elements of W on (16384 x 32 x
+    // 8192 102 / 140, 32768 x 32 x 4096 97 / 123, 16384 x 32 x 16384 190 / 213; below: 16384 x 32 x
+    // 4096 68 / 47, 8192 x 32 x 8192 59 / 53, 100000 x 20 x 512 62 / 41, 8192 x 32 x 4096 38 / 26);
+    // up to 16 columns everywhere but between 8 and 60 million elements with rows of 2048 to
+    // 8192 k (8192 x 8 x 4096 27 / 25, 4096 x 16 x 4096 18 / 16, 3000 x 8 x 3000 17.5 / 13, 2048 x 16 x
+    // 8192 22 / 17; outside: 16384 x 16 x 4096 45 / 45, 1000 x 5 x 1000 8.8 / 11.8, 4096 x 8 x 1024
+    // 7.7 / 9.4, 1024 x 16 x 16384 21 / 23).
+    const double big = (double)N * K;
+    const bool cols_ok = M <= 16 ? !(big >= 8.0e6 && big <= 60.0e6 && K >= 2048 && K <= 8192) : (M <= 32 && big >= 100.0e6);
+    const bool rows_ok = x_kmajor ? cols_ok : M <= 32;
     return M >= 1 && rows_ok && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
            (double)ldx * 32 * 4 + (x_kmajor ? 128 : 0) < 2147483648.0;
 }

@@ -299,6 +299,17 @@ def test_plan_names_the_kernel_family():
     assert fam(16, 4096, 128) == 2 and fam(16, 4096, 127) == 0   # ... a single group of 16 rows streams from K = 128
     assert fam(16384, 16, 16384) == 3 and fam(512, 16, 64) == 3 and fam(16384, 32, 16384) == 3
     assert fam(512, 32, 64) == 0 and fam(4096, 17, 4096) == 0   # 17 to 32 columns: only against a large A
+    assert fam(16384, 32, 4096) == 0 and fam(16384, 32, 8192) == 3   # (from 100 million elements on)
+    # few columns on the macro-tiles get the 128 x 32 tile, with slices of about 1024 k and a workgroup per CU
+    p = cake.plan(8192, 32, 4096)
+    assert (p.kernel, p.tile_m, p.tile_n, p.split_k) == (0, 128, 32, 4)
+    p = cake.plan(8192, 24, 8192)
+    assert (p.tile_m, p.tile_n, p.split_k) == (128, 32, 8)       # rows of 8192 floats: two workgroups per CU
+    p = cake.plan(32768, 32, 1024)
+    assert (p.tile_m, p.tile_n, p.split_k) == (128, 32, 1)
+    p = cake.plan(8192, 16, 4096)                                  # up to 16 columns: in the mid sizes only
+    assert (p.kernel, p.tile_m, p.tile_n) == (0, 128, 32) and fam(16384, 16, 4096) == 3 and fam(4096, 8, 1024) == 3
+    assert cake.plan(8192, 64, 4096).tile_n == 64
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 8192, 8192) == 0
     assert fam(49, 16384, 16384) == 2 and fam(64, 10240, 10240) == 2 and fam(64, 9000, 9000) == 0
     # 65 to 80 and 97 to 112 rows, which the macro-tiles would pad to 96 and 128

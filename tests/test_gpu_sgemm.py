@@ -67,7 +67,7 @@ def test_edge_shapes_with_2111(shape):
         _check(A, B, Cm, ref, (shape, sch))
 
 
-TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64), (96, 128, 32)]
+TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64), (96, 128, 32), (128, 32, 32)]
 
 
 @pytest.mark.parametrize("tile", TILES, ids=lambda t: "x".join(map(str, t)))
@@ -88,6 +88,7 @@ TAIL_CASES = [  # (shape M,K,N; tile) -- every CU gets the same number of tiles 
     ((1100, 1500, 1100), (64, 64, 64)), ((1100, 1497, 1099), (64, 64, 32)),
     ((2900, 512, 2900), (128, 128, 32)), ((4352, 1024, 2048), (256, 128, 32)),
     ((2048, 1024, 4352), (128, 256, 32)), ((4352, 512, 4096), (256, 256, 32)), ((3168, 512, 2048), (96, 128, 32)),
+    ((33000, 1536, 30), (128, 32, 32)),
 ]
 
 
@@ -180,11 +181,16 @@ def test_few_rows_times_wide_matrix(shape):
                                    (513, 65, 31), (1000, 300, 33), (4096, 1000, 40), (2050, 777, 48), (513, 65, 47),
                                    (1000, 300, 49),
                                    # up to 16 columns against rows of 4096 k and more: B is turned into rows first
-                                   (4097, 4100, 13), (8200, 4096, 16), (5000, 8192, 7), (4100, 4101, 16)],
+                                   (4097, 4100, 13), (8200, 4096, 16), (5000, 8192, 7), (4100, 4101, 16),
+                                   # 17 to 32 columns below 100 million elements of A, up to 16 in the mid sizes: the 128 x 32
+                                   # tile with its own K-slice rule
+                                   (8200, 4096, 32), (5000, 4099, 20), (4097, 2050, 17), (16400, 2048, 31), (3000, 3000, 8),
+                                   (33000, 1000, 24), (2049, 8200, 16)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_tall_matrix_times_few_columns(shape):
-    """Up to 48 columns of B against a tall A: A streamed once along its rows (49 columns take the
-    tile kernel), ragged M and K, K slices summed in order, accumulation, run-to-run identical sums."""
+    """Few columns of B against a tall A: A streamed once along its rows, or on the 128 x 32
+    macro-tile in its K slices; ragged M and K, K slices summed in order, accumulation, run-to-run
+    identical sums."""
     M, K, N = shape
     print(f"sgemm few columns M={M} K={K} N={N}", flush=True)
     A, B, Cm = _run(M, K, N)
