@@ -106,6 +106,7 @@ enum TileId {
     TILE_64x64x64_W32x32,         // 8 waves, two per 32x32 block of C (one per K half): small shapes, one workgroup per CU
     TILE_96x128x32_W96x32,        // 4 waves side by side, each 96 rows tall: products with 65..96 (or 129..192) rows
     TILE_128x32x32_W32x32,        // 4 waves on top of each other: products with up to 32 columns (or 65..96), which wider tiles would pad
+    TILE_32x128x32_W32x32,        // 4 waves side by side: products with up to 32 rows, which taller tiles would pad
     TILE_COUNT
 };
 

@@ -29,6 +29,7 @@ double tile_efficiency(int tile_id)
         case TILE_128x128x32_W64x64: return 0.93;
         case TILE_96x128x32_W96x32: return 0.86;  // 0.90 on a long K walk (192 x 16384^2); rated lower so that it is taken where it
                                                   // saves a quarter of padded rows, not for 512 rows as 6 x 96 (measured 68 against 60 us)
+        case TILE_32x128x32_W32x32:
         case TILE_128x32x32_W32x32: return 0.82;  // as the 64 x 64 tile per MFMA; rated below it so that it is taken where it saves padded columns
         case TILE_64x64x32_W32x32: return 0.85;  // one wave per SIMD per workgroup, 16 MFMAs between barriers
         default: return 0.80;  // 64x64x64 with two waves per block of C: see model_seconds
@@ -113,21 +114,24 @@ int tail_split_that_pays(int M, int N, int K, int tile_id, const DeviceModel& de
     return saved > TAIL_SPLIT_SECONDS ? ts : 1;
 }
 
-// K slices for the 128 x 32 tile.  Its products are bound by reading A, not by the matrix pipe
-// (13 FLOP per byte), so what counts is how many workgroups keep loads in flight and how long
-// each one's walk is, which the round count below does not see: at least one workgroup per CU
-// -- two where rows of A are 8192 floats and longer, whose power-of-two pitch puts workgroups
-// that walk in step into the same memory channels -- and slices of about 1024 k rather than 2048
-// while that still adds workgroups (us by slices 1/2/4/8/16: 8192 x 32 x 4096 69 40 26 27 34;
-// 4096 x 32 x 4096 69 39 24 16 19; 8192 x 32 x 8192 160 84 69 53 60; 4096 x 16 x 8192 133 72 40 35
-// 28; 16384 x 32 x 4096 82 54 47 56 67; 16384 x 32 x 2048 37 26 29 36 43; 32768 x 32 x 1024 23 29 37).
-int narrow_tile_split(int M, int N, int K, const DeviceModel& dev)
+// K slices for the 128 x 32 and 32 x 128 tiles.  Their products are bound by reading the large
+// operand, not by the matrix pipe (13 FLOP per byte), so what counts is how many workgroups keep
+// loads in flight and how long each one's walk is, which the round count below does not see: at
+// least one workgroup per CU -- two for a K of 8192 and more while slices stay 512 k long (rows a
+// power of two apart put workgroups that walk in step into the same memory channels) -- and
+// slices of about 1024 k rather than 2048 while that still adds workgroups (us by slices
+// 1/2/4/8/16: 8192 x 32 x 4096 69 40 26 27 34; 4096 x 32 x 4096 69 39 24 16 19; 8192 x 32 x 8192 160
+// 84 69 53 60; 4096 x 16 x 8192 133 72 40 35 28; 16384 x 32 x 4096 82 54 47 56 67; 16384 x 32 x 2048
+// 37 26 29 36 43; 32768 x 32 x 1024 23 29 37; a linear layer at batch 32, 4096 -> 4096 66 38 24 16 19,
+// 11008 -> 4096 170 91 51 35 38, 8192 -> 2048 127 69 39 23 17).
+int narrow_tile_split(int M, int N, int K, int tile_id, const DeviceModel& dev)
 {
-    const TileInfo& t = tile_info(TILE_128x32x32_W32x32);
+    const TileInfo& t = tile_info(tile_id);
     const long tiles = (long)ceil_div(M, t.bm) * ceil_div(N, t.bn);
-    const long want = (K >= 8192 ? 2L : 1L) * dev.cus;
     int split = 1;
-    while (tiles * split < want && K / (2 * split) >= 256) split *= 2;
+    while (tiles * split < dev.cus && K / (2 * split) >= 256) split *= 2;
+    if (K >= 8192)
+        while (tiles * split < 2L * dev.cus && K / (2 * split) >= 512) split *= 2;
     if (K / split >= 2048 && tiles * split < 2L * dev.cus) split *= 2;
     return split;
 }
@@ -157,7 +161,8 @@ double model_seconds(int M, int N, int K, int tile_id, int split, const DeviceMo
     // never faster than streaming the operands once
     const double bytes = 4.0 * ((double)M * K + (double)K * N + (double)M * N);
     s = std::max(s, bytes / (0.7 * dev.hbm_bytes_per_s));
-    if (tile_id == TILE_128x32x32_W32x32 && split != narrow_tile_split(M, N, K, dev)) s *= 1.3;   // see there
+    if ((tile_id == TILE_128x32x32_W32x32 || tile_id == TILE_32x128x32_W32x32) && split != narrow_tile_split(M, N, K, tile_id, dev))
+        s *= 1.3;   // see there
     // the slices are written, read back and summed by a second kernel
     // (the second kernel and the gap in front of it: 1020 x 108 x 731 takes 14.6 us whole, 10.6 us in 4 slices;
     // 3.5 us since that kernel keeps the loads of eight slices in flight -- with 5 us the choice was more than 5 %

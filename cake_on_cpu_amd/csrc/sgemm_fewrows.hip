@@ -571,7 +571,13 @@ bool fewrows_applies(int M, int N, int K, int lda, int ldb)
     // 26 us); 49 to 64 rows against a larger one still; 65 to 80 and 97 to 112 rows where the
     // macro-tiles would pad to 96 and 128 (81 to 96 rows fill the 96-row tile)
     const double big = (double)N * K;
-    const bool rows_ok = M >= 1 && (M <= 32 || (M <= 48 && big >= 48.0e6) || (M <= 64 && big >= 100.0e6) ||
+    // 17 to 32 rows stream from 100 million elements of B on; below, the 32 x 128 macro-tile in its
+    // K slices is ahead at every size (us, here / tile: 32 x 8192 x 8192 52 / 46, 32 x 4096 x 4096
+    // 20 / 16, 32 x 3333 x 3333 24 / 14.5, 32 x 1000 x 1000 12 / 11; 32 x 10000 x 10000 81 on either).
+    // Up to 16 rows stay here: the tile gains and loses 5-10 % from size to size (16 x 6144 x 6144
+    // 34 / 31, 16 x 11008 x 4096 37 / 38.5, 8 x 9000 x 3000 27 / 30, 16 x 8192 x 1024 10 / 12).
+    const bool few = M <= 16 || (M <= 32 && (big >= 100.0e6 || N < 1024));   // (a B of few columns has too few tiles: 24 x 640 x 20000 19 / 21)
+    const bool rows_ok = M >= 1 && (few || (M > 32 && M <= 48 && big >= 48.0e6) || (M > 48 && M <= 64 && big >= 100.0e6) ||
                                     (M > 64 && M <= 80 && big >= 30.0e6) || (M > 96 && M <= 112 && big >= 64.0e6));
     // (a short K walk is over before the stream is up to speed: 32 x 6512 x 76 takes 6.4 us here
     // and 5.1 us on a 64 x 64 tile, 32 x 2882 x 216 7.5 against 6.9 us; with a single group of 16
@@ -596,7 +602,12 @@ bool fewrows_nt_applies(int M, int N, int K, int ldx, int ldw, bool x_kmajor)
     // 7.7 / 9.4, 1024 x 16 x 16384 21 / 23).
     const double big = (double)N * K;
     const bool cols_ok = M <= 16 ? !(big >= 8.0e6 && big <= 60.0e6 && K >= 2048 && K <= 8192) : (M <= 32 && big >= 100.0e6);
-    const bool rows_ok = x_kmajor ? cols_ok : M <= 32;
+    // X as rows, 17 to 32 of them: from 100 million elements of W on, and for small layers and short
+    // rows; between, the 32 x 128 macro-tile that reads W along k is ahead (us, here / tile: 32 x 8192
+    // x 8192 56 / 50, 32 x 4096 x 11008 45 / 38, 32 x 14336 x 4096 56 / 41, 32 x 4096 x 4096 22 / 16.5, 32 x
+    // 100000 x 512 59 / 42; 32 x 1000 x 1000 9.8 / 11.2, 32 x 512 x 512 5.7 / 9.2, 32 x 8192 x 1024 11.5 / 12.9)
+    const bool batch_ok = M <= 16 || (M <= 32 && (big >= 100.0e6 || big < 4.0e6 || (K < 2048 && big < 30.0e6)));
+    const bool rows_ok = x_kmajor ? cols_ok : batch_ok;
     return M >= 1 && rows_ok && N >= 512 && K >= 64 && (double)ldw * 64 * 4 < 2147483648.0 &&
            (double)ldx * 32 * 4 + (x_kmajor ? 128 : 0) < 2147483648.0;
 }

@@ -15,6 +15,7 @@ hipError_t launch_sgemm_conv1x1(int tile_id, const GemmArgs& a, int grid, hipStr
         case TILE_64x64x64_W32x32: return launch_tile<Tile64x64x64, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
         case TILE_96x128x32_W96x32: return launch_tile<Tile96x128x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
         case TILE_128x32x32_W32x32: return launch_tile<Tile128x32x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
+        case TILE_32x128x32_W32x32: return launch_tile<Tile32x128x32, LOAD_VEC4, LOAD_IM2COL_1X1>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }

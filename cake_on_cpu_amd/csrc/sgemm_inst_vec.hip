@@ -14,6 +14,7 @@ hipError_t launch_sgemm_vec(int tile_id, const GemmArgs& a, int grid, hipStream_
         case TILE_64x64x64_W32x32: return launch_tile<Tile64x64x64, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         case TILE_96x128x32_W96x32: return launch_tile<Tile96x128x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         case TILE_128x32x32_W32x32: return launch_tile<Tile128x32x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
+        case TILE_32x128x32_W32x32: return launch_tile<Tile32x128x32, LOAD_VEC4, LOAD_VEC4>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }

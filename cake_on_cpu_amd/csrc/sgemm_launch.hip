@@ -21,7 +21,7 @@ const TileInfo& tile_info(int tile_id)
     static const TileInfo table[TILE_COUNT] = {
         info_of<Tile256x256x32>(), info_of<Tile256x128x32>(),
         info_of<Tile128x256x32>(), info_of<Tile128x128x32>(), info_of<Tile64x64x32>(),
-        info_of<Tile64x64x64>(), info_of<Tile96x128x32>(), info_of<Tile128x32x32>(),
+        info_of<Tile64x64x64>(), info_of<Tile96x128x32>(), info_of<Tile128x32x32>(), info_of<Tile32x128x32>(),
     };
     return table[tile_id < 0 || tile_id >= TILE_COUNT ? TILE_64x64x32_W32x32 : tile_id];
 }
@@ -64,6 +64,7 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& a, hipStream_t stream
         case TILE_64x64x64_W32x32: hipLaunchKernelGGL(tail_reduce_kernel<Tile64x64x64>, grid, block, 0, stream, a); break;
         case TILE_96x128x32_W96x32: hipLaunchKernelGGL(tail_reduce_kernel<Tile96x128x32>, grid, block, 0, stream, a); break;
         case TILE_128x32x32_W32x32: hipLaunchKernelGGL(tail_reduce_kernel<Tile128x32x32>, grid, block, 0, stream, a); break;
+        case TILE_32x128x32_W32x32: hipLaunchKernelGGL(tail_reduce_kernel<Tile32x128x32>, grid, block, 0, stream, a); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

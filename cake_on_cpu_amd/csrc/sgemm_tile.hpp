@@ -1267,5 +1267,6 @@ using Tile64x64x32 = Tile<64, 64, 32, 32, 32, 2, 2>;
 using Tile64x64x64 = Tile<64, 64, 64, 32, 32, 2, 2, 2>;
 using Tile96x128x32 = Tile<96, 128, 32, 96, 32, 2>;
 using Tile128x32x32 = Tile<128, 32, 32, 32, 32, 2>;
+using Tile32x128x32 = Tile<32, 128, 32, 32, 32, 2>;
 
 }  // namespace cake

@@ -69,8 +69,9 @@ typedef struct cake_hip_cpu_cntx_t {
 /* Kernel families of cake_hip_plan_t.kernel.  Dense row-major operands without a tile override:
  * a product with a single row or column runs on the matrix-vector kernels, one with at most 32
  * rows of A (K >= 256) or columns of B (K >= 64) and at least 512 of the other on the streaming kernels
- * (few columns only where those are ahead of the 128 x 32 macro-tile: 17 to 32 from 100 million elements
- * of A on, up to 16 outside 8 to 60 million elements with rows of 2048 to 8192 floats),
+ * where those are ahead of the 32 x 128 and 128 x 32 macro-tiles: 17 to 32 rows or columns from 100
+ * million elements of the other operand on (rows also against fewer than 1024 columns), up to 16 rows
+ * always, up to 16 columns outside 8 to 60 million elements with rows of 2048 to 8192 floats;
  * as does one with 33 to 48 rows of A against a B of 48 million elements or more, 49 to 64
  * rows against 100 million, 65 to 80 against 30 million, 97 to 112 against 64 million,
  * one with K <= 64 and at least one tile of 64 x 64 per CU on workgroups that walk over tiles

@@ -310,6 +310,10 @@ def test_plan_names_the_kernel_family():
     p = cake.plan(8192, 16, 4096)                                  # up to 16 columns: in the mid sizes only
     assert (p.kernel, p.tile_m, p.tile_n) == (0, 128, 32) and fam(16384, 16, 4096) == 3 and fam(4096, 8, 1024) == 3
     assert cake.plan(8192, 64, 4096).tile_n == 64
+    # 17 to 32 rows below 100 million elements of B: the 32 x 128 tile (not against a narrow B)
+    p = cake.plan(32, 8192, 8192)
+    assert (p.kernel, p.tile_m, p.tile_n, p.split_k) == (0, 32, 128, 8)
+    assert fam(24, 4096, 4096) == 0 and fam(32, 16384, 8192) == 2 and fam(16, 4096, 4096) == 2 and fam(32, 640, 20000) == 2
     assert fam(33, 16384, 16384) == 2 and fam(48, 8192, 8192) == 2 and fam(49, 8192, 8192) == 0
     assert fam(49, 16384, 16384) == 2 and fam(64, 10240, 10240) == 2 and fam(64, 9000, 9000) == 0
     # 65 to 80 and 97 to 112 rows, which the macro-tiles would pad to 96 and 128

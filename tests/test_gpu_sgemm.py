@@ -67,7 +67,7 @@ def test_edge_shapes_with_2111(shape):
         _check(A, B, Cm, ref, (shape, sch))
 
 
-TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64), (96, 128, 32), (128, 32, 32)]
+TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64, 32), (64, 64, 64), (96, 128, 32), (128, 32, 32), (32, 128, 32)]
 
 
 @pytest.mark.parametrize("tile", TILES, ids=lambda t: "x".join(map(str, t)))
