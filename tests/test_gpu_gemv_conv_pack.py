@@ -140,6 +140,8 @@ CONV_GEOMS = [
     (1, 16, 9, 12, 10, 1, 1, 1, 0),      # 1x1 filter, Wout = 12
     (2, 4, 12, 14, 9, 5, 3, 1, 2),       # 5x3 filter, pad 2, Wout = 16
     (4, 32, 14, 8, 64, 3, 3, 1, 1),      # Wout = 8
+    (8, 64, 56, 56, 24, 1, 1, 1, 0),     # few output channels, many pixels: the 32-row tile
+    (4, 96, 28, 28, 20, 3, 3, 1, 1),     # the same with a 3x3 filter
     (1, 4, 6, 8, 5, 3, 3, 3, 2),         # stride 3, pad 2, Wout = 4
     (2, 6, 10, 12, 12, 7, 7, 1, 3),      # 7x7, pad 3: the 16-byte row gather shifts by up to 3 either way
     (2, 8, 16, 16, 16, 5, 5, 1, 2),      # 5x5, pad 2, Wout = 16
