@@ -44,20 +44,21 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563254155, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
-    "sgemm_1024": (29499945, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
-    "sgemm_tall_skinny": (306425197, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
-    "sgemv_16384_rowmajor": (1074454677, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemm_8192": (4563232461, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_1024": (29500957, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
+    "sgemm_tall_skinny": (306412911, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
+    "sgemv_16384_rowmajor": (1074454684, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
     "sgemv_16384_colmajor": (1075863560, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (353502885, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
-    "conv_c5_two_step": (2207579283, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129072441, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42353755, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
-    "fewrows_nn": (1087406236, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nn_64rows": (1128385571, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
-    "fewrows_nt": (1083220551, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_16x16384x16384": (1083220551, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_8192x4096x4096": (1208268524, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "conv_c5_gather": (353534876, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1> >` grid 524288"),
+    "conv_c5_two_step": (2207575967, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129072691, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (42423885, "row `sgemm_tile_kernel<Tile<64, 64, 32, 32, 32, 2, 2, 1>, 0, 5>` grid 401408"),
+    "fewrows_nn": (1087400095, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nn_64rows": (1128387615, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
+    "narrow_tile_32cols": (288886752, "row `sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0>` grid 131072"),
+    "fewrows_nt": (1083225758, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083225758, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_8192x4096x4096": (1208268729, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -301,6 +302,8 @@ def main() -> int:
                    "transpose_kernel (B into 16 rows) + sgemm_fewrows_nt_kernel")
         gemm_extra("sgemm 64 rows: M=64 K=16384 N=16384", 64, 16384, 16384, "fewrows_nn_64rows",
                    "sgemm_fewrows_nn_kernel<4, 2> + splitk_reduce_kernel", bound="mfma")
+        gemm_extra("sgemm 32 columns (a low-rank projection): M=16384 K=4096 N=32", 16384, 32, 4096, "narrow_tile_32cols",
+                   "sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0> in 4 K slices + splitk_reduce_kernel")
 
         m = 16384
         Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
