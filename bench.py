@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fp32 GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras] [--all-extras]
 
 A step is one cake_sgemm of BASELINE config 2 (M = K = N = 8192, row-major fp32,
 A and B uniform[-1,1) from seeds 1 and 2), operands resident in HBM, launched
@@ -16,10 +16,18 @@ timed steps between two synchronisations.  Prints ONE JSON line:
   cpu_baseline   the CPU restatement of the reference cake_sgemm (oracle/, kind
                  "port") on this host's physical cores, same inputs, full 8192^3
                  product once after a small warm-up
-  extras         the other BASELINE configs and a few more workloads (not bench
-                 lines: reported for information), each with a roofline object
-                 of its own and, for the BASELINE configs, the CPU restatement
-                 of the reference's call timed beside it
+  extras         the other four BASELINE configs (not bench lines: reported for
+                 information), each with a roofline object of its own and the CPU
+                 restatement of the reference's call timed beside it; with
+                 --all-extras a dozen more workloads (the short-K, streaming and
+                 1 x 1 kernels, the linear layer) and, in every roofline object,
+                 the row of profiles/ its traffic figure was read from
+
+Bandwidth-bound workloads (the matrix-vector products, the streaming kernels)
+are timed twice: `same_buffer`, every launch on the same operand, and
+`rotating`, consecutive launches on four different 1 GiB operands, so that no
+launch finds part of its operand in the 256 MB memory-side cache from the launch
+before.  Their roofline is computed from the rotating run.
 """
 from __future__ import annotations
 
@@ -62,6 +70,9 @@ MEASURED_TRAFFIC = {
 }
 
 
+VERBOSE = False    # --all-extras: name the profile row behind every traffic figure
+
+
 def roofline(bound, work, seconds, traffic_key=None, **more):
     """The roofline object of one workload: `work` algorithmic FLOPs (bound "mfma") or bytes (bound
     "hbm") per launch over the measured seconds per launch, against the published peak."""
@@ -72,7 +83,7 @@ def roofline(bound, work, seconds, traffic_key=None, **more):
     traffic, source = MEASURED_TRAFFIC.get(traffic_key, (None, None))
     r = {"bound": bound, "achieved": round(achieved, 3 if bound == "mfma" else 1), "peak": peak, "unit": unit,
          "frac": round(achieved / peak, 4), "traffic": traffic, key: work}
-    if source:
+    if source and VERBOSE:
         r["traffic_source"] = "profiles/all_kernels_hbm_traffic_pmc.md, " + source
     r.update(more)
     return r
@@ -85,6 +96,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--all-extras", action="store_true",
+                    help="also time the workloads outside BASELINE.json (short K, streaming kernels, 1 x 1 convolution, "
+                         "linear layer) and name the profile row of every traffic figure")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy kernel 3 times (reference point for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -92,6 +106,8 @@ def main() -> int:
                     help="only time 1024 x 1024 x K products for K = 32 .. 1024 and a one-workgroup kernel "
                          "(what config 1's time is made of: a fixed part and a part per k) and exit")
     args = ap.parse_args()
+    global VERBOSE
+    VERBOSE = args.all_extras
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (single-GPU hot path); --gpus must be 1", file=sys.stderr)
         return 2
@@ -159,6 +175,26 @@ def main() -> int:
         wall = time.perf_counter() - t0
         kernel = [a.elapsed_time(b) * 1e-3 * pairs / steps for a, b in evs]
         return wall, float(np.mean(kernel)), float(np.min(kernel))
+
+    ROTATE = 4
+
+    def time_rotating(launch_on, steps, warmup, settle_ms):
+        """`launch_on(i)` launches on operand i of ROTATE.  Returns the average launch duration with
+        every launch on operand 0 and with consecutive launches on different operands."""
+        same = time_steps(lambda: launch_on(0), steps, warmup, settle_ms)[1]
+        turn = [0]
+
+        def next_one():
+            launch_on(turn[0] % ROTATE)
+            turn[0] += 1
+        return same, time_steps(next_one, steps, warmup, settle_ms)[1]
+
+    def rotating_operand(elems, seed):
+        """ROTATE operands of `elems` floats in one allocation; operand 0 is the stream `seed`."""
+        whole = torch.empty((ROTATE * elems,), dtype=torch.float32, device=dev)
+        for r in range(ROTATE):
+            cake.fill_uniform(whole[r * elems:(r + 1) * elems], seed if r == 0 else 1000 * r + seed)
+        return whole
 
     if args.latency_floor:
         m = 1024
@@ -256,117 +292,8 @@ def main() -> int:
         return {"value": round(work / secs / scale, 4), "unit": unit, "cores": p_cores, "kind": "port",
                 "seconds": round(secs, 5), "sample": sample}
 
-    if not args.no_extras:
-        extras = []
-
-        def gemm_extra(name, M, N, K, traffic_key=None, streaming_kernel=None, cpu=False, bound="hbm"):
-            a, b = dev_uniform((M, K), 1), dev_uniform((K, N), 2)
-            c = torch.zeros((M, N), dtype=torch.float32, device=dev)
-            p3 = (a.data_ptr(), b.data_ptr(), c.data_ptr())
-            _, avg, _ = time_steps(lambda: _lib.check(
-                lib.cake_hip_sgemm(p3[0], p3[1], p3[2], M, N, K, cake.NA, 0, None, stream, None), name), 50, 5, 40.0)
-            pl = cake.plan(M, N, K)
-            fl = 2.0 * M * N * K
-            by = 4.0 * (M * K + K * N + M * N)
-            e = {"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
-                 "compulsory_GBps": round(by / avg / 1e9, 1), "kernel_family": cake.KERNEL_NAMES[pl.kernel]}
-            if streaming_kernel:   # few rows or columns: bound by reading the large operand once
-                e["kernel"] = streaming_kernel   # (or, from 49 rows on, by the matrix pipe)
-                e["roofline"] = (roofline("hbm", by, avg, traffic_key) if bound == "hbm" else
-                                 roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by))
-            else:
-                e.update({"tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
-                          "schedule": cake.SCHED_NAMES[pl.sched]})
-                e["roofline"] = roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by)
-            if cpu:
-                Ah, Bh = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
-                dims = {}
-
-                def run():
-                    _, secs, x = oracle.cake_sgemm(Ah, Bh, p_cores, cpu_cx, return_time=True)
-                    dims["x"] = x
-                    return secs
-                e["cpu_baseline"] = cpu_leg(run, fl, "TFLOP/s", "")
-                if e["cpu_baseline"]:
-                    x = dims["x"]
-                    e["cpu_baseline"]["sample"] = (f"the full product, cake_sgemm with the reference's default schedule "
-                                                   f"({oracle.SCHED_NAMES[x.sch]}, m_c=k_c={x.m_c}, n_c={x.n_c}); median of 3 after a warm-up")
-            extras.append(e)
-
-        gemm_extra("sgemm 1024^3 (configs[0])", 1024, 1024, 1024, "sgemm_1024", cpu=True)
-        gemm_extra("sgemm tall-skinny M=65536 K=1024 N=128 (configs[2])", 65536, 128, 1024, "sgemm_tall_skinny", cpu=True)
-        gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64, "shortk_256x64x100352")
-        gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
-                   "sgemm_fewrows_nn_kernel + splitk_reduce_kernel")
-        gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
-                   "transpose_kernel (B into 16 rows) + sgemm_fewrows_nt_kernel")
-        gemm_extra("sgemm 64 rows: M=64 K=16384 N=16384", 64, 16384, 16384, "fewrows_nn_64rows",
-                   "sgemm_fewrows_nn_kernel<4, 2> + splitk_reduce_kernel", bound="mfma")
-        gemm_extra("sgemm 32 columns (a low-rank projection): M=16384 K=4096 N=32", 16384, 32, 4096, "narrow_tile_32cols",
-                   "sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0> in 4 K slices + splitk_reduce_kernel")
-
-        m = 16384
-        Ag, xg = dev_uniform((m * m,), 1), dev_uniform((m,), 3)
-        yg = torch.zeros((m,), dtype=torch.float32, device=dev)
-        gbytes = 4.0 * (m * m + m + m)
-        gemv_cpu = None
-        if not args.no_cpu:
-            # cake_sgemv as examples/cake_gemv.cpp runs it: column-major A, m_r = 8, y accumulates
-            Agh, xgh = oracle.uniform((m, m), 1), oracle.uniform(m, 3)
-            gcx = oracle.query_cntx()
-            gcx.mr = 8
-            gemv_cpu = cpu_leg(lambda: oracle.cake_sgemv(Agh, xgh, p_cores, gcx, M=m, K=m, return_time=True)[1], gbytes, "GB/s",
-                               "the full 16384 x 16384 cake_sgemv (column-major A, the reference's own layout); median of 3 after a warm-up")
-            del Agh
-        for col, label, key in ((0, "row-major A (configs[3])", "sgemv_16384_rowmajor"),
-                                (1, "column-major A (cake_sgemv's own layout)", "sgemv_16384_colmajor")):
-            _, avg, _ = time_steps(lambda: _lib.check(
-                lib.cake_hip_sgemv(Ag.data_ptr(), xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None), "sgemv"), 50, 10, 40.0)
-            extras.append({"workload": f"sgemv 16384x16384 {label}", "us": round(avg * 1e6, 2),
-                           "GBps": round(gbytes / avg / 1e9, 1), "roofline": roofline("hbm", gbytes, avg, key),
-                           "cpu_baseline": gemv_cpu})
-        del Ag
-
-        Bn, Cc, H = 32, 256, 56
-        inp, wt = dev_uniform((Bn, Cc, H, H), 5), dev_uniform((Cc, Cc, 3, 3), 4)
-        oc = torch.empty((Cc, Bn * H * H), dtype=torch.float32, device=dev)
-        ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
-        ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
-        cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
-        cby = 4.0 * (Bn * Cc * H * H + Cc * Cc * 9 + Bn * Cc * H * H)      # input + weights + output
-        conv_cpu = None
-        if not args.no_cpu:
-            # the reference's sequence for one image (examples/cake_conv.cpp:1007-1066): im_2_col of the
-            # zero-padded CHW image, then cake_sgemm (which packs both operands); 2 of the 32 images
-            imgs = oracle.uniform((2, Cc, H, H), 5)
-            wh = oracle.uniform((Cc, Cc * 9), 4)
-            padded = np.zeros((2, Cc, H + 2, H + 2), np.float32)
-            padded[:, :, 1:-1, 1:-1] = imgs
-
-            def conv_cpu_run():
-                total = 0.0
-                for b in range(2):
-                    t0 = time.perf_counter()
-                    cols = oracle.im_2_col(padded[b], 3, 3, H, H)
-                    total += time.perf_counter() - t0
-                    total += oracle.cake_sgemm(wh, cols, p_cores, cpu_cx, sch=oracle.KMN, return_time=True)[1]
-                return total
-            conv_cpu = cpu_leg(conv_cpu_run, cfl * 2 / Bn, "TFLOP/s",
-                               "2 of the 32 images: im_2_col + cake_sgemm(KMN) per image as examples/cake_conv.cpp does "
-                               "(M=256, K=2304, N=3136 each); median of 3 after a warm-up")
-        # output written as NCHW by the GEMM's epilogue on both paths
-        for fn, label, key in ((lib.cake_hip_conv2d, "columns gathered inside the GEMM from the input where it lies, NCHW output",
-                                "conv_c5_gather"),
-                               (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps), NCHW output",
-                                "conv_c5_two_step")):
-            _, avg, _ = time_steps(lambda: _lib.check(
-                fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 1,
-                   ws.data_ptr(), stream, None), "conv2d"), 20, 3, 40.0)
-            extras.append({"workload": f"conv 3x3 s1 p1, batch 32, 256->256 ch, 56x56 (configs[4]): {label}",
-                           "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
-                           "roofline": roofline("mfma", cfl, avg, key, algorithmic_bytes_per_launch=cby),
-                           "cpu_baseline": conv_cpu})
-        del inp, oc, ws
+    def more_extras():
+        extras = other_extras
         # a 1 x 1 layer: planes read in place (no staged copy, no tap table), NCHW output
         Pb, Pc, Ph, Po = 32, 256, 14, 1024
         pin, pw = dev_uniform((Pb, Pc, Ph, Ph), 6), dev_uniform((Po, Pc), 7)
@@ -406,17 +333,153 @@ def main() -> int:
         del lx, lg, ly, lgx
         # a small batch: the weights are streamed once as they lie, no transposed copy
         Sm, Sk, Sn = 16, 16384, 16384
-        sx, sw, sb = dev_uniform((Sm, Sk), 15), dev_uniform((Sn, Sk), 16), dev_uniform((Sn,), 17)
+        sx, sw, sb = dev_uniform((Sm, Sk), 15), rotating_operand(Sn * Sk, 16), dev_uniform((Sn,), 17)
         sy = torch.empty((Sm, Sn), dtype=torch.float32, device=dev)
         sby = 4.0 * (Sm * Sk + Sn * Sk + Sn + Sm * Sn)
-        _, avg, _ = time_steps(lambda: _lib.check(
-            lib.cake_hip_linear_forward(sx.data_ptr(), sw.data_ptr(), sb.data_ptr(), sy.data_ptr(), Sm, Sn, Sk,
+        same, avg = time_rotating(lambda i: _lib.check(
+            lib.cake_hip_linear_forward(sx.data_ptr(), sw.data_ptr() + 4 * Sn * Sk * i, sb.data_ptr(), sy.data_ptr(), Sm, Sn, Sk,
                                         stream, None), "linear_forward"), 50, 5, 40.0)
         extras.append({"workload": "linear forward, batch 16, 16384->16384, bias",
-                       "us": round(avg * 1e6, 2), "tflops": round(2.0 * Sm * Sn * Sk / avg / 1e12, 2),
-                       "kernel": "sgemm_fewrows_nt_kernel",
-                       "roofline": roofline("hbm", sby, avg, "linear_fwd_16x16384x16384")})
-        out["extras"] = extras
+                       "us": round(avg * 1e6, 2), "us_same_buffer": round(same * 1e6, 2),
+                       "tflops": round(2.0 * Sm * Sn * Sk / avg / 1e12, 2), "kernel": "sgemm_fewrows_nt_kernel",
+                       "roofline": roofline("hbm", sby, avg, "linear_fwd_16x16384x16384",
+                                            timed_on=f"{ROTATE} rotating weight matrices",
+                                            frac_same_buffer=round(sby / same / 1e9 / HBM_PEAK_GBPS, 4))})
+
+    if not args.no_extras:
+
+        def gemm_extra(name, M, N, K, traffic_key=None, streaming_kernel=None, cpu=False, bound="hbm", rotate=None):
+            """rotate: "A" or "B" -- the operand that is streamed once, timed on ROTATE different copies."""
+            a = rotating_operand(M * K, 1) if rotate == "A" else dev_uniform((M, K), 1)
+            b = rotating_operand(K * N, 2) if rotate == "B" else dev_uniform((K, N), 2)
+            c = torch.zeros((M, N), dtype=torch.float32, device=dev)
+            pc = c.data_ptr()
+
+            def launch_on(i):
+                pa = a.data_ptr() + (4 * M * K * i if rotate == "A" else 0)
+                pb = b.data_ptr() + (4 * K * N * i if rotate == "B" else 0)
+                _lib.check(lib.cake_hip_sgemm(pa, pb, pc, M, N, K, cake.NA, 0, None, stream, None), name)
+            same = None
+            if rotate:
+                same, avg = time_rotating(launch_on, 50, 5, 40.0)
+            else:
+                _, avg, _ = time_steps(lambda: launch_on(0), 50, 5, 40.0)
+            pl = cake.plan(M, N, K)
+            fl = 2.0 * M * N * K
+            by = 4.0 * (M * K + K * N + M * N)
+            e = {"workload": name, "us": round(avg * 1e6, 2), "tflops": round(fl / avg / 1e12, 2),
+                 "compulsory_GBps": round(by / avg / 1e9, 1), "kernel_family": cake.KERNEL_NAMES[pl.kernel]}
+            more = {}
+            if same is not None:
+                e["us_same_buffer"] = round(same * 1e6, 2)
+                more = {"timed_on": f"{ROTATE} rotating operands", "frac_same_buffer": round(by / same / 1e9 / HBM_PEAK_GBPS, 4)}
+            if streaming_kernel:   # few rows or columns: bound by reading the large operand once
+                e["kernel"] = streaming_kernel   # (or, from 49 rows on, by the matrix pipe)
+                e["roofline"] = (roofline("hbm", by, avg, traffic_key, **more) if bound == "hbm" else
+                                 roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by))
+            else:
+                e.update({"tile": f"{pl.tile_m}x{pl.tile_n}x{pl.tile_k}", "split_k": pl.split_k,
+                          "schedule": cake.SCHED_NAMES[pl.sched]})
+                e["roofline"] = roofline("mfma", fl, avg, traffic_key, algorithmic_bytes_per_launch=by)
+            if cpu:
+                Ah, Bh = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+                dims = {}
+
+                def run():
+                    _, secs, x = oracle.cake_sgemm(Ah, Bh, p_cores, cpu_cx, return_time=True)
+                    dims["x"] = x
+                    return secs
+                e["cpu_baseline"] = cpu_leg(run, fl, "TFLOP/s", "")
+                if e["cpu_baseline"]:
+                    x = dims["x"]
+                    e["cpu_baseline"]["sample"] = (f"full product, reference default schedule "
+                                                   f"{oracle.SCHED_NAMES[x.sch]}, m_c={x.m_c}, n_c={x.n_c}; median of 3")
+            del a, b, c
+            return e
+
+        baseline_extras, other_extras = [], []
+        baseline_extras.append(gemm_extra("configs[0] sgemm 1024^3", 1024, 1024, 1024, "sgemm_1024", cpu=True))
+        baseline_extras.append(gemm_extra("configs[2] sgemm tall-skinny M=65536 K=1024 N=128", 65536, 128, 1024,
+                                          "sgemm_tall_skinny", cpu=True))
+        if args.all_extras:
+            other_extras.append(gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64, "shortk_256x64x100352"))
+            other_extras.append(gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
+                                           "sgemm_fewrows_nn_kernel + splitk_reduce_kernel", rotate="B"))
+            other_extras.append(gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",
+                                           "transpose_kernel (B into 16 rows) + sgemm_fewrows_nt_kernel", rotate="A"))
+            other_extras.append(gemm_extra("sgemm 64 rows: M=64 K=16384 N=16384", 64, 16384, 16384, "fewrows_nn_64rows",
+                                           "sgemm_fewrows_nn_kernel<4, 2> + splitk_reduce_kernel", bound="mfma"))
+            other_extras.append(gemm_extra("sgemm 32 columns (a low-rank projection): M=16384 K=4096 N=32", 16384, 32, 4096,
+                                           "narrow_tile_32cols",
+                                           "sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0> in 4 K slices + splitk_reduce_kernel"))
+
+        m = 16384
+        Ag, xg = rotating_operand(m * m, 1), dev_uniform((m,), 3)
+        yg = torch.zeros((m,), dtype=torch.float32, device=dev)
+        gbytes = 4.0 * (m * m + m + m)
+        gemv_cpu = None
+        if not args.no_cpu:
+            # cake_sgemv as examples/cake_gemv.cpp runs it: column-major A, m_r = 8, y accumulates
+            Agh, xgh = oracle.uniform((m, m), 1), oracle.uniform(m, 3)
+            gcx = oracle.query_cntx()
+            gcx.mr = 8
+            gemv_cpu = cpu_leg(lambda: oracle.cake_sgemv(Agh, xgh, p_cores, gcx, M=m, K=m, return_time=True)[1], gbytes, "GB/s",
+                               "full 16384^2 cake_sgemv, column-major A (the reference's layout); median of 3")
+            del Agh
+        for col, label, key in ((0, "configs[3] sgemv 16384^2, row-major A", "sgemv_16384_rowmajor"),
+                                (1, "configs[3] sgemv 16384^2, column-major A (cake_sgemv's layout)", "sgemv_16384_colmajor")):
+            same, avg = time_rotating(lambda i: _lib.check(
+                lib.cake_hip_sgemv(Ag.data_ptr() + 4 * m * m * i, xg.data_ptr(), yg.data_ptr(), m, m, col, 0, stream, None),
+                "sgemv"), 60, 12, 40.0)
+            baseline_extras.append({"workload": label, "us": round(avg * 1e6, 2), "us_same_buffer": round(same * 1e6, 2),
+                                    "GBps": round(gbytes / avg / 1e9, 1),
+                                    "roofline": roofline("hbm", gbytes, avg, key, timed_on=f"{ROTATE} rotating 1 GiB matrices",
+                                                         frac_same_buffer=round(gbytes / same / 1e9 / HBM_PEAK_GBPS, 4)),
+                                    "cpu_baseline": gemv_cpu if col else None})
+        del Ag
+
+        Bn, Cc, H = 32, 256, 56
+        inp, wt = dev_uniform((Bn, Cc, H, H), 5), dev_uniform((Cc, Cc, 3, 3), 4)
+        oc = torch.empty((Cc, Bn * H * H), dtype=torch.float32, device=dev)
+        ws_bytes = lib.cake_hip_conv2d_workspace(Bn, Cc, H, H, Cc, 3, 3, 1, 1)
+        ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
+        cfl = 2.0 * Cc * (Cc * 9) * (Bn * H * H)
+        cby = 4.0 * (Bn * Cc * H * H + Cc * Cc * 9 + Bn * Cc * H * H)      # input + weights + output
+        conv_cpu = None
+        if not args.no_cpu:
+            # the reference's sequence for one image (examples/cake_conv.cpp:1007-1066): im_2_col of the
+            # zero-padded CHW image, then cake_sgemm (which packs both operands); 2 of the 32 images
+            imgs = oracle.uniform((2, Cc, H, H), 5)
+            wh = oracle.uniform((Cc, Cc * 9), 4)
+            padded = np.zeros((2, Cc, H + 2, H + 2), np.float32)
+            padded[:, :, 1:-1, 1:-1] = imgs
+
+            def conv_cpu_run():
+                total = 0.0
+                for b in range(2):
+                    t0 = time.perf_counter()
+                    cols = oracle.im_2_col(padded[b], 3, 3, H, H)
+                    total += time.perf_counter() - t0
+                    total += oracle.cake_sgemm(wh, cols, p_cores, cpu_cx, sch=oracle.KMN, return_time=True)[1]
+                return total
+            conv_cpu = cpu_leg(conv_cpu_run, cfl * 2 / Bn, "TFLOP/s",
+                               "2 of the 32 images: im_2_col + cake_sgemm(KMN) per image, as examples/cake_conv.cpp; median of 3")
+        # output written as NCHW by the GEMM's epilogue on both paths
+        for fn, label, key in ((lib.cake_hip_conv2d, "input read where it lies (no column matrix)", "conv_c5_gather"),
+                               (lib.cake_hip_conv2d_im2col, "im2col kernel, then GEMM (the reference's two steps)",
+                                "conv_c5_two_step")):
+            _, avg, _ = time_steps(lambda: _lib.check(
+                fn(inp.data_ptr(), wt.data_ptr(), oc.data_ptr(), Bn, Cc, H, H, Cc, 3, 3, 1, 1, 1,
+                   ws.data_ptr(), stream, None), "conv2d"), 20, 3, 40.0)
+            baseline_extras.append({"workload": f"configs[4] conv 3x3 s1 p1, batch 32, 256->256, 56x56, NCHW out: {label}",
+                                    "ms": round(avg * 1e3, 4), "tflops": round(cfl / avg / 1e12, 2),
+                                    "roofline": roofline("mfma", cfl, avg, key, algorithmic_bytes_per_launch=cby),
+                                    "cpu_baseline": conv_cpu if fn == lib.cake_hip_conv2d_im2col else None})
+        del inp, oc, ws
+        if args.all_extras:
+            more_extras()
+        # the BASELINE configs last: the end of a long line is what a log keeps
+        out["extras"] = other_extras + baseline_extras
 
     # -------------------------------------------------------------- CPU baseline
     if not args.no_cpu:

@@ -16,6 +16,7 @@ CXX_LIB_PATH = LIB_DIR / "libcake.so"
 KMN, MKN, NKM, NA = 0, 1, 2, 3
 SCHED_NAMES = {KMN: "KMN", MKN: "MKN", NKM: "NKM", NA: "NA"}
 # Plan.kernel: which kernel family cake_hip_sgemm runs for a shape
+CONV_NONE, CONV_SHORTK_BATCH, CONV_PATCH, CONV_GATHER, CONV_TWO_STEP = range(5)   # cake_hip_last_conv_route
 KERNEL_NAMES = {0: "macro-tile", 1: "matrix-vector", 2: "streaming, few rows", 3: "streaming, few columns",
                 4: "short K, tiles walked by resident workgroups"}
 
@@ -88,6 +89,13 @@ SIGNATURES = {
     "cake_hip_plan": (_i, [_i, _i, _i, _i, C.POINTER(_i), C.POINTER(Plan)]),
     "cake_hip_init_block_dims": (_i, [_i, _i, _i, _i, _cx, _i, _i, _i, _i, _bd]),
     "cake_hip_derive_schedule": (_i, [_i, _i, _i, _i, _i, _cx]),
+    "cake_hip_grid_dims_2d": (_i, [_i] * 5),
+    "cake_hip_init_block_dims_2d": (_i, [_i, _i, _i, _i, _cx, _i, C.c_float, _i, _i, _i, _bd]),
+    "cake_hip_init_block_dims_2d_small": (_i, [_i, _i, _i, _i, _cx, _i, C.c_float, _bd]),
+    "cake_hip_init_block_dims_conv": (_i, [_i] * 10 + [_cx, _bd]),
+    "cake_hip_packed_filters_size": (C.c_size_t, [_i, _i, _i, _i, _bd, _cx]),
+    "cake_hip_pack_filters": (_i, [_fp, _fp, _i, _i, _i, _i, _bd, _cx, C.c_void_p, _dp]),
+    "cake_hip_sconv_packed": (_i, [_fp, _fp, _fp] + [_i] * 10 + [_bd, _cx, C.c_void_p, _dp]),
     "cake_hip_sgemm": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _i, C.POINTER(_i), C.c_void_p, _dp]),
     "cake_hip_sgemm_noalloc": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _i, C.c_void_p]),
     "cake_hip_sgemm_packed": (_i, [_fp, _fp, _fp, _i, _i, _i, _i, _bd, _cx, _i, _i, _i, C.c_void_p, _dp]),
@@ -116,6 +124,12 @@ SIGNATURES = {
     "cake_hip_tune_clear": (_i, []),
     "cake_hip_tune_count": (_i, []),
     "cake_hip_fill_uniform": (_i, [_fp, C.c_size_t, C.c_uint64, C.c_void_p]),
+    "cake_hip_last_conv_route": (_i, []),
+    "cake_hip_ctx_create": (_i, [C.POINTER(C.c_void_p)]),
+    "cake_hip_ctx_destroy": (_i, [C.c_void_p]),
+    "cake_hip_ctx_set_current": (_i, [C.c_void_p]),
+    "cake_hip_ctx_get_current": (C.c_void_p, []),
+    "cake_hip_ctx_stream": (C.c_void_p, [C.c_void_p]),
     "cake_hip_last_kernel_seconds": (_i, [C.POINTER(C.c_double * 5)]),
 }
 

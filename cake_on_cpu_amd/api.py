@@ -134,6 +134,38 @@ def init_block_dims(M, N, K, p, cake_cntx: CpuCntx, sch=NA, argv=None, type_size
     return x
 
 
+def grid_dims_2d(M, N, K, p, ncores=0) -> int:
+    """pn of the reference's pm x pn grid of cores (src/block_sizing.cpp:596-634): the factor of p
+    closest to sqrt(p N / M).  Host arithmetic."""
+    return load().cake_hip_grid_dims_2d(M, N, K, p, ncores)
+
+
+def init_block_dims_2d(M, N, K, p, cake_cntx: CpuCntx, sch=NA, argv=None, type_size=4,
+                       mcu=0, kcu=0, ncu=0) -> BlkDims:
+    """init_block_dims_2d (include/tiling.h:43-45, src/block_sizing.cpp:639-779)."""
+    x = BlkDims()
+    check(load().cake_hip_init_block_dims_2d(M, N, K, p, C.byref(cake_cntx), sch, float(type_size), mcu, kcu, ncu,
+                                             C.byref(x)), "init_block_dims_2d")
+    return x
+
+
+def init_block_dims_2d_small(M, N, K, p, cake_cntx: CpuCntx, sch=NA, argv=None, type_size=4) -> BlkDims:
+    """init_block_dims_2d_small (include/tiling.h:47-49, src/block_sizing.cpp:785-841)."""
+    x = BlkDims()
+    check(load().cake_hip_init_block_dims_2d_small(M, N, K, p, C.byref(cake_cntx), sch, float(type_size), C.byref(x)),
+          "init_block_dims_2d_small")
+    return x
+
+
+def init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cake_cntx: CpuCntx, sch=KMN,
+                         argv=None, density=0.0, type_size=4) -> BlkDims:
+    """init_block_dims_conv (examples/cake_conv.cpp:333-425): blocks of the direct convolution, K-first."""
+    x = BlkDims()
+    check(load().cake_hip_init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, C.byref(cake_cntx),
+                                               C.byref(x)), "init_block_dims_conv")
+    return x
+
+
 def plan(M, N, K, sch=NA, tile=None) -> Plan:
     """The GPU planner's decision for one product (tile, wave layout, reuse order, split-K)."""
     out = Plan()
@@ -314,25 +346,86 @@ def conv2d(inp, weights, out, batch, Cin, Hin, Win, Cout, Hf, Wf, stride=1, pad=
     return secs.value
 
 
+def pack_filters(A, A_p, M, K, p, x, cake_cntx, taps=9) -> float:
+    """pack_filters (examples/cake_conv.cpp:536-610): filters A[M = Cout][K = Cin * taps] into the K-first
+    blocks of init_block_dims_conv; A_p holds x.M_padded * K floats.  The reference is written for
+    3 x 3 filters (taps = 9)."""
+    _need(A, M * K, "filters")
+    _need(A_p, x.M_padded * K, "packed filters")
+    secs = C.c_double(0.0)
+    check(load().cake_hip_pack_filters(_ptr(A, "filters"), _ptr(A_p, "packed filters"), M, K // taps, taps, p,
+                                       C.byref(x), C.byref(cake_cntx), _stream(A, A_p), C.byref(secs)), "pack_filters")
+    return secs.value
+
+
 def cake_sconv(A, B, Cm, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cake_cntx=None, argv=None,
                packedA=False, sch=NA) -> float:
     """cake_sconv (examples/cake_conv.cpp:5-8,765-848): C[Cout][Hout][Wout] += A[Cout][Cin][Hf][Wf] * B[Cin][Hin][Win],
-    one CHW image, no padding; p, cake_cntx and sch are accepted and unused (the reference always
-    runs it K-first).  Returns seconds."""
-    if packedA:
-        raise ValueError("cake_sconv: filters packed by the reference's pack_filters are not supported")
-    _need(A, Cout * Cin * Hf * Wf, "filters")
+    one CHW image, no padding; sch is accepted and unused (the reference always runs it K-first).
+    With packedA the filters are in the layout of pack_filters for the blocks that
+    init_block_dims_conv derives from the same geometry, p and cake_cntx (:791-799).  Returns seconds."""
     _need(B, Cin * Hin * Win, "input")
     _need(Cm, Cout * Hout * Wout, "output")
     secs = C.c_double(0.0)
+    if packedA:
+        cx = cake_cntx if cake_cntx is not None else _default_cntx()
+        x = init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cx)
+        _need(A, x.M_padded * Cin * Hf * Wf, "packed filters")
+        check(load().cake_hip_sconv_packed(_ptr(A, "filters"), _ptr(B, "input"), _ptr(Cm, "output"), Wf, Hf, Win, Hin,
+                                           Wout, Hout, Cin, Cout, s, p, C.byref(x), C.byref(cx), _stream(A, B, Cm),
+                                           C.byref(secs)), "cake_sconv")
+        return secs.value
+    _need(A, Cout * Cin * Hf * Wf, "filters")
     check(load().cake_hip_sconv(_ptr(A, "filters"), _ptr(B, "input"), _ptr(Cm, "output"), Wf, Hf, Win, Hin, Wout, Hout,
                                 Cin, Cout, s, _stream(A, B, Cm), C.byref(secs)), "cake_sconv")
     return secs.value
 
 
+def last_conv_route() -> int:
+    """Which route this thread's last convolution call took (_lib.CONV_*)."""
+    return load().cake_hip_last_conv_route()
+
+
 # ----------------------------------------------------------------------------
-# transpose and the linear layer (include/util.h:32, src/linear.cpp:12-107)
+# device contexts
 # ----------------------------------------------------------------------------
+class Context:
+    """A device context of its own (cake_hip_ctx_create): workspaces, events and a stream that calls
+    made while it is current do not share with the default context or with other contexts.
+
+        with cake.Context() as ctx:          # current on this thread inside the block
+            cake.cake_sgemm(...)             # device operands: enqueued on ctx.stream unless torch's
+                                             # current stream is passed by the operands
+    """
+
+    def __init__(self):
+        h = C.c_void_p()
+        check(load().cake_hip_ctx_create(C.byref(h)), "cake_hip_ctx_create")
+        self.handle = h.value
+        self._before = []
+
+    @property
+    def stream(self) -> int:
+        return load().cake_hip_ctx_stream(self.handle) or 0
+
+    def make_current(self) -> None:
+        check(load().cake_hip_ctx_set_current(self.handle), "cake_hip_ctx_set_current")
+
+    def __enter__(self):
+        self._before.append(load().cake_hip_ctx_get_current())
+        self.make_current()
+        return self
+
+    def __exit__(self, *exc):
+        check(load().cake_hip_ctx_set_current(self._before.pop()), "cake_hip_ctx_set_current")
+        return False
+
+    def destroy(self) -> None:
+        if self.handle:
+            check(load().cake_hip_ctx_destroy(self.handle), "cake_hip_ctx_destroy")
+            self.handle = None
+
+
 def transpose_mat(A_old, At, K, N, Kt=0, Nt=0) -> float:
     """At[n][k] = A_old[k][n] for a K x N matrix (src/transpose.cpp:5-29; the
     blocking arguments Kt, Nt are accepted and unused).  Returns seconds."""

@@ -34,6 +34,16 @@ int init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cx, int sch
 // src/block_sizing.cpp:434-462
 int derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_cpu_cntx_t* cx);
 
+// src/block_sizing.cpp:596-841: sizing for the reference's 2-D grid of cores
+int grid_dims_2d(int M, int N, int K, int p, int ncores);
+int init_block_dims_2d(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cx, int sched, float type_size,
+                       int mcu, int kcu, int ncu, cake_hip_blk_dims_t* out);
+int init_block_dims_2d_small(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cx, int sched, float type_size,
+                             cake_hip_blk_dims_t* out);
+// examples/cake_conv.cpp:262-420: blocks of the direct convolution (K-first)
+int init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s, int p,
+                         cake_hip_cpu_cntx_t* cx, cake_hip_blk_dims_t* out);
+
 // Padded extents of the packed operands (src/pack_helper.cpp:5-87).
 CAKE_HD int padded_rows(const PackGeom& g)
 {
@@ -108,6 +118,22 @@ CAKE_HD int64_t packed_a_offset(const PackGeom& g, int row, int col)
                        : (int64_t)mb * mspan * g.K + (int64_t)k.block * g.p * d.k_c * rows;
     return base + (int64_t)k.core * k.slice * rows + (int64_t)panel * mr * k.length +
            (int64_t)k.inner * mr + j;
+}
+
+// Offset of filter element (row = output channel, channel, tap) in the layout of the reference's
+// pack_filters (examples/cake_conv.cpp:430-454,536-610): K-first blocks of A with K = input
+// channels, and inside an m_r panel the taps outermost, [m-blk][channel-blk][core][m_r-panel][tap][channel][m_r].
+// g.d from init_block_dims_conv, g.K = Cin.  row < padded rows (d.M_padded), channel < Cin.
+CAKE_HD int64_t packed_filter_offset(const PackGeom& g, int row, int channel, int tap, int taps)
+{
+    const cake_hip_blk_dims_t& d = g.d;
+    const int mr = g.mr;
+    SplitPos m = split_pos(row, g.p, d.m_c, d.Mb, d.m_pad, mr * d.mr_rem, d.m_c1, d.p_l, d.m_c1_last_core);
+    const int kb = channel / d.k_c, i = channel - kb * d.k_c;
+    const int kc = (d.k_pad && kb == d.Kb - 1) ? d.k_c1 : d.k_c;
+    const int panel = m.inner / mr, j = m.inner - panel * mr;
+    return ((int64_t)m.block * g.p * d.m_c * g.K + (int64_t)kb * m.span * d.k_c + (int64_t)m.core * m.slice * kc +
+            (int64_t)panel * mr * kc) * taps + (int64_t)tap * kc * mr + (int64_t)i * mr + j;
 }
 
 // Offset of B(row = k, col = n) in the packed B.

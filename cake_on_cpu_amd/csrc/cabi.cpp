@@ -24,6 +24,7 @@ using namespace cake;
 
 thread_local std::string g_last_error;
 thread_local double g_family_seconds[5] = {0, 0, 0, 0, 0};
+thread_local int g_last_conv_route = CAKE_HIP_CONV_NONE;
 
 int fail(int status, const char* fmt, ...)
 {
@@ -44,30 +45,52 @@ int fail(int status, const char* fmt, ...)
     } while (0)
 
 // Grow-only device buffer.  A workspace that kernels of device-operand calls use (`keep_old`) is
-// never freed when it grows: a caller may have captured earlier launches in a HIP graph, which
-// holds the old address, so the outgrown allocation is kept until shutdown.  Such a buffer at
-// least doubles, which bounds everything kept to the size of the live one.  Staging copies of
-// host operands are only touched by synchronous calls and are freed at once.
+// not freed when it grows: a caller may have captured earlier launches in a HIP graph, which
+// holds the old address, so the outgrown allocation is kept until shutdown.  Such a buffer asks
+// for at least twice its size, which bounds everything kept to the size of the live one (old
+// blocks + live block < 2 x live block, i.e. at most 4 x the largest request while the doubling
+// succeeds).  When memory does not allow that it falls back in steps: the request with a little
+// slack, then the bare request, and as the last resort it waits for the device, gives the
+// outgrown blocks and the present one back and asks again -- graphs captured before that point
+// then hold addresses that are gone and must be captured anew (the call still succeeds whenever
+// the request itself fits).  Staging copies of host operands are only touched by synchronous
+// calls and are freed at once.
 struct DeviceBuffer {
     void* ptr = nullptr;
     size_t cap = 0;
     bool keep_old = false;
     std::vector<void*> outgrown;
+    static void* try_alloc(size_t bytes)
+    {
+        void* fresh = nullptr;
+        if (hipMalloc(&fresh, bytes) == hipSuccess) return fresh;
+        (void)hipGetLastError();
+        return nullptr;
+    }
     int reserve(size_t bytes)
     {
         if (bytes <= cap) return CAKE_HIP_OK;
-        size_t want = bytes + (bytes >> 3) + 256;
-        if (keep_old && want < 2 * cap) want = 2 * cap;
-        void* fresh = nullptr;
+        const size_t slack = bytes + (bytes >> 3) + 256;
         if (!keep_old && ptr) {
             (void)hipFree(ptr);
             ptr = nullptr;
             cap = 0;
         }
-        if (hipMalloc(&fresh, want) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(CAKE_HIP_ERR_ALLOC, "device allocation of %zu bytes failed", want);
+        size_t want = keep_old && slack < 2 * cap ? 2 * cap : slack;
+        void* fresh = try_alloc(want);
+        if (!fresh && want > slack) fresh = try_alloc(want = slack);
+        if (!fresh) fresh = try_alloc(want = bytes + 256);
+        if (!fresh && (ptr || !outgrown.empty())) {
+            (void)hipDeviceSynchronize();   // nothing in flight may still use the blocks given back
+            for (void* q : outgrown) (void)hipFree(q);
+            outgrown.clear();
+            if (ptr) (void)hipFree(ptr);
+            ptr = nullptr;
+            cap = 0;
+            fresh = try_alloc(want = slack);
+            if (!fresh) fresh = try_alloc(want = bytes + 256);
         }
+        if (!fresh) return fail(CAKE_HIP_ERR_ALLOC, "device allocation of %zu bytes failed", bytes + 256);
         if (ptr) outgrown.push_back(ptr);
         ptr = fresh;
         cap = want;
@@ -85,13 +108,20 @@ struct DeviceBuffer {
 
 enum { STAGE_SLOTS = 6 };
 
+// Everything a compute call needs besides its operands: workspaces, events, the pinned buffers
+// and streams of host-operand transfers.  One default context exists per process (it is what
+// cake_hip_init sets up); cake_hip_ctx_create makes further ones.  A context has a mutex of its
+// own, so calls on different contexts run side by side, on different streams; calls on one
+// context take turns because they share its workspaces.
 struct Context {
+    std::recursive_mutex mutex;        // one compute call at a time per context (an entry point may call another)
     std::atomic<bool> ready{false};
     int device = 0;
     cake_hip_device_t info{};
     DeviceModel model;
     DeviceBuffer stage[STAGE_SLOTS];  // device copies of host operands
     DeviceBuffer splitk, gemv, conv, conv_taps, conv_filters, tables, unpacked, linear, turned;
+    hipStream_t own_stream = nullptr;   // what a NULL stream argument means on this context (default context: the null stream)
     hipEvent_t ev[2] = {nullptr, nullptr};
     hipEvent_t fam[2] = {nullptr, nullptr};
     std::vector<hipEvent_t> fam_pool;   // event pairs of the kernel families of one timed call, created on demand
@@ -101,30 +131,75 @@ struct Context {
     void* pinned[4] = {nullptr, nullptr, nullptr, nullptr};
     hipStream_t copy_stream = nullptr, copy_back_stream = nullptr;
     hipEvent_t copy_done[2] = {nullptr, nullptr};
+    // cake_hip_sgemm_noalloc in progress (set under `mutex`): partial sums and the turned operand
+    // are carved from the file-scope array, `noalloc_used` bytes of it so far
+    bool noalloc_call = false;
+    size_t noalloc_used = 0;
+
+    DeviceBuffer* compute_buffers[9] = {&splitk, &gemv, &conv, &conv_taps, &conv_filters, &tables, &unpacked, &linear, &turned};
+    int create_events()
+    {
+        for (hipEvent_t* e : {&ev[0], &ev[1], &fam[0], &fam[1]})
+            if (!*e) HIP_TRY(hipEventCreate(e));
+        for (DeviceBuffer* b : compute_buffers) b->keep_old = true;
+        return CAKE_HIP_OK;
+    }
+    void release_all()
+    {
+        for (DeviceBuffer& b : stage) b.release();
+        for (DeviceBuffer* b : compute_buffers) b->release();
+        for (hipEvent_t e : fam_pool) (void)hipEventDestroy(e);
+        fam_pool.clear();
+        for (hipEvent_t* e : {&ev[0], &ev[1], &fam[0], &fam[1], &copy_done[0], &copy_done[1]}) {
+            if (*e) (void)hipEventDestroy(*e);
+            *e = nullptr;
+        }
+        for (void*& p : pinned) {
+            if (p) (void)hipHostFree(p);
+            p = nullptr;
+        }
+        for (hipStream_t* cs : {&copy_stream, &copy_back_stream, &own_stream}) {
+            if (*cs) (void)hipStreamDestroy(*cs);
+            *cs = nullptr;
+        }
+    }
 };
 
-Context g_ctx;
-std::mutex g_mutex;  // one compute call at a time: the workspaces are shared
+Context g_default_ctx;
+thread_local Context* t_current_ctx = nullptr;   // set by cake_hip_ctx_set_current; nullptr: the default context
+std::mutex g_ctx_registry_mutex;
+std::vector<Context*> g_created_ctx;             // contexts from cake_hip_ctx_create that are still alive
+
+inline Context& cur() { return t_current_ctx ? *t_current_ctx : g_default_ctx; }
+
+// the stream argument of an entry point: NULL means the current context's own stream
+inline hipStream_t pick_stream(void* stream_)
+{
+    return stream_ ? static_cast<hipStream_t>(stream_) : cur().own_stream;
+}
 
 // Partial sums (K slices of split-K, tail-split and streaming products, slices of the
 // matrix-vector kernels) of cake_hip_sgemm_noalloc: a file-scope array instead of a buffer from
 // hipMalloc.  The name is a host-side handle, not a device address; cake_hip_init asks the runtime
 // for the address on each device it is called for and the kernels only ever get that pointer.
+// Every context on a device shares the device's one array.
 constexpr size_t NOALLOC_SCRATCH_BYTES = 64u << 20;
 static __device__ __align__(256) unsigned char noalloc_scratch[NOALLOC_SCRATCH_BYTES];
 enum { MAX_DEVICES = 64 };
-float* g_noalloc_ptr[MAX_DEVICES] = {nullptr};
-bool g_noalloc_call = false;   // set (under g_mutex) while cake_hip_sgemm_noalloc runs
+unsigned char* g_noalloc_ptr[MAX_DEVICES] = {nullptr};
 
-// Where the partial sums of the current call go: `buf` (grown when needed), or the file-scope array
-// during cake_hip_sgemm_noalloc, which never grows.
-int partial_space(DeviceBuffer& buf, size_t bytes, float** out)
+// Scratch memory of the current call: `buf` (grown when needed), or the next piece of the
+// file-scope array during cake_hip_sgemm_noalloc, which never grows.
+int scratch_space(DeviceBuffer& buf, size_t bytes, float** out)
 {
-    if (g_noalloc_call) {
-        if (bytes > NOALLOC_SCRATCH_BYTES)
+    Context& c = cur();
+    if (c.noalloc_call) {
+        const size_t at = (c.noalloc_used + 255) & ~(size_t)255;
+        if (bytes > NOALLOC_SCRATCH_BYTES || at + bytes > NOALLOC_SCRATCH_BYTES)
             return fail(CAKE_HIP_ERR_RANGE, "this product needs %zu bytes of partial sums; cake_hip_sgemm_noalloc has %zu",
-                        bytes, (size_t)NOALLOC_SCRATCH_BYTES);
-        *out = g_noalloc_ptr[g_ctx.device];
+                        at + bytes, (size_t)NOALLOC_SCRATCH_BYTES);
+        *out = reinterpret_cast<float*>(g_noalloc_ptr[c.device] + at);
+        c.noalloc_used = at + bytes;
         return CAKE_HIP_OK;
     }
     int st = buf.reserve(bytes);
@@ -135,7 +210,8 @@ int partial_space(DeviceBuffer& buf, size_t bytes, float** out)
 
 int ensure_init()
 {
-    if (g_ctx.ready) return CAKE_HIP_OK;
+    if (cur().ready) return CAKE_HIP_OK;
+    if (&cur() != &g_default_ctx) return fail(CAKE_HIP_ERR_ARG, "the current context has been destroyed");
     return cake_hip_init(0);
 }
 
@@ -167,10 +243,10 @@ constexpr int PIN_THREADS = 8;
 static int pinned_ready()
 {
     for (int i = 0; i < 2; ++i) {
-        if (!g_ctx.pinned[i]) HIP_TRY(hipHostMalloc(&g_ctx.pinned[i], PIN_CHUNK, hipHostMallocDefault));
-        if (!g_ctx.copy_done[i]) HIP_TRY(hipEventCreateWithFlags(&g_ctx.copy_done[i], hipEventDisableTiming));
+        if (!cur().pinned[i]) HIP_TRY(hipHostMalloc(&cur().pinned[i], PIN_CHUNK, hipHostMallocDefault));
+        if (!cur().copy_done[i]) HIP_TRY(hipEventCreateWithFlags(&cur().copy_done[i], hipEventDisableTiming));
     }
-    if (!g_ctx.copy_stream) HIP_TRY(hipStreamCreateWithFlags(&g_ctx.copy_stream, hipStreamNonBlocking));
+    if (!cur().copy_stream) HIP_TRY(hipStreamCreateWithFlags(&cur().copy_stream, hipStreamNonBlocking));
     return CAKE_HIP_OK;
 }
 
@@ -179,8 +255,8 @@ static int pinned_both_ways_ready()
     int st = pinned_ready();
     if (st) return st;
     for (int i = 2; i < 4; ++i)
-        if (!g_ctx.pinned[i]) HIP_TRY(hipHostMalloc(&g_ctx.pinned[i], PIN_CHUNK, hipHostMallocDefault));
-    if (!g_ctx.copy_back_stream) HIP_TRY(hipStreamCreateWithFlags(&g_ctx.copy_back_stream, hipStreamNonBlocking));
+        if (!cur().pinned[i]) HIP_TRY(hipHostMalloc(&cur().pinned[i], PIN_CHUNK, hipHostMallocDefault));
+    if (!cur().copy_back_stream) HIP_TRY(hipStreamCreateWithFlags(&cur().copy_back_stream, hipStreamNonBlocking));
     return CAKE_HIP_OK;
 }
 
@@ -207,12 +283,12 @@ static int host_to_device(void* dev, const void* host, size_t bytes)
     for (size_t off = 0; off < bytes; off += PIN_CHUNK, ++i) {
         const size_t n = bytes - off < PIN_CHUNK ? bytes - off : PIN_CHUNK;
         const int b = i & 1;
-        if (i >= 2) HIP_TRY(hipEventSynchronize(g_ctx.copy_done[b]));   // the buffer's last transfer is over
-        parallel_memcpy(g_ctx.pinned[b], static_cast<const char*>(host) + off, n);
-        HIP_TRY(hipMemcpyAsync(static_cast<char*>(dev) + off, g_ctx.pinned[b], n, hipMemcpyHostToDevice, g_ctx.copy_stream));
-        HIP_TRY(hipEventRecord(g_ctx.copy_done[b], g_ctx.copy_stream));
+        if (i >= 2) HIP_TRY(hipEventSynchronize(cur().copy_done[b]));   // the buffer's last transfer is over
+        parallel_memcpy(cur().pinned[b], static_cast<const char*>(host) + off, n);
+        HIP_TRY(hipMemcpyAsync(static_cast<char*>(dev) + off, cur().pinned[b], n, hipMemcpyHostToDevice, cur().copy_stream));
+        HIP_TRY(hipEventRecord(cur().copy_done[b], cur().copy_stream));
     }
-    HIP_TRY(hipStreamSynchronize(g_ctx.copy_stream));
+    HIP_TRY(hipStreamSynchronize(cur().copy_stream));
     return CAKE_HIP_OK;
 }
 
@@ -228,16 +304,16 @@ static int device_to_host(void* host, const void* dev, size_t bytes)
     auto chunk_bytes = [&](size_t c) { return bytes - c * PIN_CHUNK < PIN_CHUNK ? bytes - c * PIN_CHUNK : PIN_CHUNK; };
     auto issue = [&](size_t c) -> hipError_t {
         const int b = (int)(c & 1);
-        hipError_t e = hipMemcpyAsync(g_ctx.pinned[b], static_cast<const char*>(dev) + c * PIN_CHUNK, chunk_bytes(c),
-                                      hipMemcpyDeviceToHost, g_ctx.copy_stream);
-        return e != hipSuccess ? e : hipEventRecord(g_ctx.copy_done[b], g_ctx.copy_stream);
+        hipError_t e = hipMemcpyAsync(cur().pinned[b], static_cast<const char*>(dev) + c * PIN_CHUNK, chunk_bytes(c),
+                                      hipMemcpyDeviceToHost, cur().copy_stream);
+        return e != hipSuccess ? e : hipEventRecord(cur().copy_done[b], cur().copy_stream);
     };
     HIP_TRY(issue(0));
     for (size_t c = 0; c < chunks; ++c) {
         // the other buffer was emptied in the previous round: fill it while this one is copied out
         if (c + 1 < chunks) HIP_TRY(issue(c + 1));
-        HIP_TRY(hipEventSynchronize(g_ctx.copy_done[c & 1]));
-        parallel_memcpy(static_cast<char*>(host) + c * PIN_CHUNK, g_ctx.pinned[c & 1], chunk_bytes(c));
+        HIP_TRY(hipEventSynchronize(cur().copy_done[c & 1]));
+        parallel_memcpy(static_cast<char*>(host) + c * PIN_CHUNK, cur().pinned[c & 1], chunk_bytes(c));
     }
     return CAKE_HIP_OK;
 }
@@ -250,9 +326,9 @@ int stage_in(const float* p, size_t bytes, int slot, bool copy, Operand* op)
         op->host = nullptr;
         return CAKE_HIP_OK;
     }
-    int st = g_ctx.stage[slot].reserve(bytes);
+    int st = cur().stage[slot].reserve(bytes);
     if (st) return st;
-    op->dev = static_cast<float*>(g_ctx.stage[slot].ptr);
+    op->dev = static_cast<float*>(cur().stage[slot].ptr);
     op->host = const_cast<float*>(p);
     if (copy) {
         // an earlier call may have left kernels in flight that still read this slot (device
@@ -275,26 +351,26 @@ struct Timer {
     hipStream_t stream;
     double* out;
     bool on;
-    int pairs = 0;              // event pairs of g_ctx.fam_pool in use by this call
+    int pairs = 0;              // event pairs of cur().fam_pool in use by this call
     int family_of[32];
     Timer(hipStream_t s, double* o) : stream(s), out(o), on(o != nullptr) {}
     int start()
     {
         for (double& f : g_family_seconds) f = 0;
-        if (on) HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
+        if (on) HIP_TRY(hipEventRecord(cur().ev[0], stream));
         return CAKE_HIP_OK;
     }
     int stop()
     {
         if (!on) return CAKE_HIP_OK;
-        HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));
-        HIP_TRY(hipEventSynchronize(g_ctx.ev[1]));
+        HIP_TRY(hipEventRecord(cur().ev[1], stream));
+        HIP_TRY(hipEventSynchronize(cur().ev[1]));
         float ms = 0;
-        HIP_TRY(hipEventElapsedTime(&ms, g_ctx.ev[0], g_ctx.ev[1]));
+        HIP_TRY(hipEventElapsedTime(&ms, cur().ev[0], cur().ev[1]));
         *out = ms * 1e-3;
         // the families' events were recorded before ev[1] on the same stream: all of them are over
         for (int i = 0; i < pairs; ++i) {
-            HIP_TRY(hipEventElapsedTime(&ms, g_ctx.fam_pool[2 * i], g_ctx.fam_pool[2 * i + 1]));
+            HIP_TRY(hipEventElapsedTime(&ms, cur().fam_pool[2 * i], cur().fam_pool[2 * i + 1]));
             g_family_seconds[family_of[i]] += ms * 1e-3;
         }
         pairs = 0;
@@ -308,25 +384,25 @@ struct Timer {
     {
         const bool pooled = on && pairs < 32;
         if (pooled) {
-            while ((int)g_ctx.fam_pool.size() < 2 * pairs + 2) {
+            while ((int)cur().fam_pool.size() < 2 * pairs + 2) {
                 hipEvent_t e = nullptr;
                 HIP_TRY(hipEventCreate(&e));
-                g_ctx.fam_pool.push_back(e);
+                cur().fam_pool.push_back(e);
             }
-            HIP_TRY(hipEventRecord(g_ctx.fam_pool[2 * pairs], stream));
+            HIP_TRY(hipEventRecord(cur().fam_pool[2 * pairs], stream));
         } else if (on) {
-            HIP_TRY(hipEventRecord(g_ctx.fam[0], stream));
+            HIP_TRY(hipEventRecord(cur().fam[0], stream));
         }
         hipError_t e = launch();
         if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
         if (pooled) {
-            HIP_TRY(hipEventRecord(g_ctx.fam_pool[2 * pairs + 1], stream));
+            HIP_TRY(hipEventRecord(cur().fam_pool[2 * pairs + 1], stream));
             family_of[pairs++] = which;
         } else if (on) {   // more families than the pool holds: wait for this one here
-            HIP_TRY(hipEventRecord(g_ctx.fam[1], stream));
-            HIP_TRY(hipEventSynchronize(g_ctx.fam[1]));
+            HIP_TRY(hipEventRecord(cur().fam[1], stream));
+            HIP_TRY(hipEventSynchronize(cur().fam[1]));
             float ms = 0;
-            HIP_TRY(hipEventElapsedTime(&ms, g_ctx.fam[0], g_ctx.fam[1]));
+            HIP_TRY(hipEventElapsedTime(&ms, cur().fam[0], cur().fam[1]));
             g_family_seconds[which] += ms * 1e-3;
         }
         return CAKE_HIP_OK;
@@ -367,13 +443,13 @@ int check_geom(const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, int 
     return CAKE_HIP_OK;
 }
 
-// Device index tables for one packed operand, carved from g_ctx.tables at `at`.
+// Device index tables for one packed operand, carved from cur().tables at `at`.
 int build_tables(int which, const PackGeom& g, size_t* at, IndexTables* out, hipStream_t stream)
 {
     const int Mp = padded_rows(g), Np = padded_cols(g);
     const size_t nrows = (which == 1) ? g.K : Mp;
     const size_t ncols = (which == 0) ? g.K : Np;
-    int4* base = reinterpret_cast<int4*>(static_cast<char*>(g_ctx.tables.ptr) + *at);
+    int4* base = reinterpret_cast<int4*>(static_cast<char*>(cur().tables.ptr) + *at);
     out->row = base;
     out->col = base + nrows;
     *at += (nrows + ncols) * sizeof(int4);
@@ -403,41 +479,41 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     const bool streaming_ok = vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, true, nullptr);
     if (streaming_ok && fewrows_applies(M, N, K, lda, ldb)) {
         // a few rows of A against a wide B: bound by reading B, served by the streaming kernel
-        const int slices = fewrows_slices(M, N, K, g_ctx.model.cus);
+        const int slices = fewrows_slices(M, N, K, cur().model.cus);
         float* partial = nullptr;
         if (slices > 1) {
-            int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
+            int st2 = scratch_space(cur().splitk, (size_t)slices * M * N * sizeof(float), &partial);
             if (st2) return st2;
         }
         return timer.family(0, [&] {
             return launch_sgemm_fewrows(A, B, C, partial, M, N, K, lda, ldb, ldc, accumulate, col_bias,
-                                        g_ctx.model.cus, stream);
+                                        cur().model.cus, stream);
         });
     }
     if (streaming_ok && fewrows_nt_applies(N, M, K, ldb, lda, true)) {
         // a tall A against a few columns of B: the same with A streamed along its rows.  Up to 16
         // columns of B (K x N, small next to A) are turned into N rows of K first where
-        // fewrows_nt_turn_pays says so.  Not in a call that must not allocate.
-        const bool turn = !g_noalloc_call && ldb == N && K <= 64 * 65535 &&   // (what the transpose kernel's grid takes)
-                          fewrows_nt_turn_pays(N, M, K, lda, g_ctx.model.cus) && fewrows_nt_applies(N, M, K, K, lda, false);
+        // fewrows_nt_turn_pays says so.
+        const bool turn = ldb == N && K <= 64 * 65535 &&   // (what the transpose kernel's grid takes)
+                          fewrows_nt_turn_pays(N, M, K, lda, cur().model.cus) && fewrows_nt_applies(N, M, K, K, lda, false);
         const float* Bx = B;
         if (turn) {
-            int st2 = g_ctx.turned.reserve((size_t)K * N * sizeof(float));
+            float* bt = nullptr;
+            int st2 = scratch_space(cur().turned, (size_t)K * N * sizeof(float), &bt);
             if (st2) return st2;
-            float* bt = static_cast<float*>(g_ctx.turned.ptr);
             st2 = timer.family(4, [&] { return launch_transpose(B, bt, K, N, stream); });
             if (st2) return st2;
             Bx = bt;
         }
-        const int slices = fewrows_nt_slices(N, M, K, lda, !turn, g_ctx.model.cus);
+        const int slices = fewrows_nt_slices(N, M, K, lda, !turn, cur().model.cus);
         float* partial = nullptr;
         if (slices > 1) {
-            int st2 = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial);
+            int st2 = scratch_space(cur().splitk, (size_t)slices * M * N * sizeof(float), &partial);
             if (st2) return st2;
         }
         return timer.family(0, [&] {
             return launch_sgemm_fewrows_nt(Bx, A, C, partial, N, M, K, turn ? K : ldb, lda, ldc, !turn, true, accumulate,
-                                           col_bias, g_ctx.model.cus, stream);
+                                           col_bias, cur().model.cus, stream);
         });
     }
     // A short K under many tiles of C: workgroups that walk over tiles, the next tile's operands in flight
@@ -445,12 +521,12 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     // tile's columns in the image, paid per tile instead of once per workgroup, cost more than
     // the overlap gives -- 1 x 1, 64 -> 256 channels on 56 x 56: 56 us against 50 us)
     if (vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, vec_plan, nullptr) &&
-        shortk_applies(M, N, K, g_ctx.model.cus)) {
+        shortk_applies(M, N, K, cur().model.cus)) {
         GemmArgs g{};
         g.A = A; g.B = B; g.C = C;
         g.M = M; g.N = N; g.K = K;
         g.lda = lda; g.ldb = ldb; g.ldc = ldc;
-        const int tn = shortk_tile_n(M, N, K, g_ctx.model.cus);
+        const int tn = shortk_tile_n(M, N, K, cur().model.cus);
         g.tiles_m = (M + 63) / 64; g.tiles_n = (N + tn - 1) / tn;
         g.split_k = 1; g.k_per_split = K;
         // The tile sequence runs down bands of tile rows.  Up to 16 tile rows make one band: a
@@ -466,11 +542,11 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         g.group_along_n = 0;
         g.accumulate = accumulate;
         g.col_bias = col_bias;
-        return timer.family(0, [&] { return launch_sgemm_shortk(g, tn, g_ctx.model.cus, stream); });
+        return timer.family(0, [&] { return launch_sgemm_shortk(g, tn, cur().model.cus, stream); });
     }
     GemmPlan plan;
-    int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec_plan, g_ctx.model, &plan)
-                    : plan_gemm(M, N, K, sched, tile_override, vec_plan, g_ctx.model, &plan);
+    int st = choice ? plan_gemm_choice(M, N, K, sched, *choice, vec_plan, cur().model, &plan)
+                    : plan_gemm(M, N, K, sched, tile_override, vec_plan, cur().model, &plan);
     if (st) return fail(st, "no tile matches the requested override");
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C;
@@ -488,12 +564,12 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     g.tail_k_per_split = plan.tail_k_per_split;
     g.tail_partial = nullptr;
     if (plan.pub.tail_tiles > 0) {
-        st = partial_space(g_ctx.splitk, (size_t)plan.pub.tail_tiles * plan.pub.tail_split * plan.pub.tile_m *
+        st = scratch_space(cur().splitk, (size_t)plan.pub.tail_tiles * plan.pub.tail_split * plan.pub.tile_m *
                                              plan.pub.tile_n * sizeof(float), &g.tail_partial);
         if (st) return st;
     }
     if (plan.pub.split_k > 1) {
-        st = partial_space(g_ctx.splitk, (size_t)plan.pub.split_k * M * N * sizeof(float), &g.partial);
+        st = scratch_space(cur().splitk, (size_t)plan.pub.split_k * M * N * sizeof(float), &g.partial);
         if (st) return st;
     }
     st = timer.family(0, [&] { return launch_sgemm(plan.tile_id, a_mode, b_mode, g, plan.pub.grid, stream); });
@@ -530,8 +606,9 @@ const char* cake_hip_last_error(void) { return g_last_error.c_str(); }
 
 int cake_hip_init(int device)
 {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (g_ctx.ready && g_ctx.device == device) return CAKE_HIP_OK;
+    Context& c = g_default_ctx;
+    std::lock_guard<std::recursive_mutex> lock(c.mutex);
+    if (c.ready && c.device == device) return CAKE_HIP_OK;
     int count = 0;
     if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
         (void)hipGetLastError();
@@ -543,7 +620,6 @@ int cake_hip_init(int device)
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(CAKE_HIP_ERR_ARCH, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
-    Context& c = g_ctx;
     c.device = device;
     c.info = cake_hip_device_t{};
     c.info.device = device;
@@ -558,15 +634,13 @@ int cake_hip_init(int device)
     c.model = DeviceModel{};
     if (c.info.cus > 0) c.model.cus = c.info.cus;
     if (c.info.lds_bytes_per_cu >= 64 * 1024) c.model.lds_per_cu = c.info.lds_bytes_per_cu;
-    for (hipEvent_t* e : {&c.ev[0], &c.ev[1], &c.fam[0], &c.fam[1]})
-        if (!*e) HIP_TRY(hipEventCreate(e));
-    for (DeviceBuffer* b : {&c.splitk, &c.gemv, &c.conv, &c.conv_taps, &c.conv_filters, &c.tables, &c.unpacked, &c.linear, &c.turned})
-        b->keep_old = true;
+    int st = c.create_events();
+    if (st) return st;
     // this device's copy of the file-scope scratch array (every device has its own, at its own address)
     if (device < MAX_DEVICES && !g_noalloc_ptr[device]) {
         void* at = nullptr;
         HIP_TRY(hipGetSymbolAddress(&at, HIP_SYMBOL(noalloc_scratch)));
-        g_noalloc_ptr[device] = static_cast<float*>(at);
+        g_noalloc_ptr[device] = static_cast<unsigned char*>(at);
     }
     if (const char* tuned = std::getenv("CAKE_HIP_TUNE_FILE")) (void)tune_load(tuned);  // optional
     c.ready = true;
@@ -575,28 +649,101 @@ int cake_hip_init(int device)
 
 int cake_hip_shutdown(void)
 {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (!g_ctx.ready) return CAKE_HIP_OK;
+    Context& c = g_default_ctx;
+    std::lock_guard<std::recursive_mutex> lock(c.mutex);
+    if (!c.ready) return CAKE_HIP_OK;
     (void)hipDeviceSynchronize();
-    for (DeviceBuffer& b : g_ctx.stage) b.release();
-    g_ctx.splitk.release(); g_ctx.gemv.release(); g_ctx.conv.release();
-    g_ctx.tables.release(); g_ctx.unpacked.release(); g_ctx.linear.release(); g_ctx.turned.release(); g_ctx.conv_taps.release(); g_ctx.conv_filters.release();
-    for (hipEvent_t e : g_ctx.fam_pool) (void)hipEventDestroy(e);
-    g_ctx.fam_pool.clear();
-    for (hipEvent_t* e : {&g_ctx.ev[0], &g_ctx.ev[1], &g_ctx.fam[0], &g_ctx.fam[1], &g_ctx.copy_done[0], &g_ctx.copy_done[1]}) {
-        if (*e) (void)hipEventDestroy(*e);
-        *e = nullptr;
-    }
-    for (void*& p : g_ctx.pinned) {
-        if (p) (void)hipHostFree(p);
-        p = nullptr;
-    }
-    for (hipStream_t* cs : {&g_ctx.copy_stream, &g_ctx.copy_back_stream}) {
-        if (*cs) (void)hipStreamDestroy(*cs);
-        *cs = nullptr;
-    }
-    g_ctx.ready = false;
+    c.release_all();
+    c.ready = false;
     return CAKE_HIP_OK;
+}
+
+int cake_hip_ctx_create(cake_hip_ctx_t* out)
+{
+    if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
+    *out = nullptr;
+    if (!g_default_ctx.ready) {
+        int st = cake_hip_init(0);
+        if (st) return st;
+    }
+    Context* c = new (std::nothrow) Context;
+    if (!c) return fail(CAKE_HIP_ERR_ALLOC, "out of host memory");
+    c->device = g_default_ctx.device;
+    c->info = g_default_ctx.info;
+    c->model = g_default_ctx.model;
+    int st = c->create_events();
+    if (st == CAKE_HIP_OK && hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        st = fail(CAKE_HIP_ERR_HIP, "hipStreamCreateWithFlags failed");
+    }
+    if (st) {
+        c->release_all();
+        delete c;
+        return st;
+    }
+    c->ready = true;
+    {
+        std::lock_guard<std::mutex> lock(g_ctx_registry_mutex);
+        g_created_ctx.push_back(c);
+    }
+    *out = c;
+    return CAKE_HIP_OK;
+}
+
+static Context* find_created(cake_hip_ctx_t h)
+{
+    std::lock_guard<std::mutex> lock(g_ctx_registry_mutex);
+    for (Context* c : g_created_ctx)
+        if (c == h) return c;
+    return nullptr;
+}
+
+int cake_hip_ctx_destroy(cake_hip_ctx_t h)
+{
+    if (!h) return CAKE_HIP_OK;
+    Context* c = find_created(h);
+    if (!c) return fail(CAKE_HIP_ERR_ARG, "not a context from cake_hip_ctx_create (or destroyed already)");
+    if (t_current_ctx == c) t_current_ctx = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_ctx_registry_mutex);
+        for (size_t i = 0; i < g_created_ctx.size(); ++i)
+            if (g_created_ctx[i] == c) {
+                g_created_ctx.erase(g_created_ctx.begin() + i);
+                break;
+            }
+    }
+    {
+        // a call on another thread that still holds the context finishes first; the work it and
+        // earlier calls enqueued (on the context's stream or a caller's) may still read the workspaces
+        std::lock_guard<std::recursive_mutex> lock(c->mutex);
+        (void)hipDeviceSynchronize();
+        c->release_all();
+        c->ready = false;
+    }
+    // The husk (a few hundred bytes, no device resources) is kept: a thread that still has the
+    // context current then gets an error from its next call instead of touching freed memory.
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_ctx_set_current(cake_hip_ctx_t h)
+{
+    if (!h) {
+        t_current_ctx = nullptr;
+        return CAKE_HIP_OK;
+    }
+    Context* c = find_created(h);
+    if (!c) return fail(CAKE_HIP_ERR_ARG, "not a context from cake_hip_ctx_create (or destroyed already)");
+    t_current_ctx = c;
+    return CAKE_HIP_OK;
+}
+
+cake_hip_ctx_t cake_hip_ctx_get_current(void) { return t_current_ctx; }
+
+void* cake_hip_ctx_stream(cake_hip_ctx_t h)
+{
+    if (!h) return nullptr;
+    Context* c = find_created(h);
+    return c ? c->own_stream : nullptr;
 }
 
 int cake_hip_device_info(cake_hip_device_t* out)
@@ -604,7 +751,7 @@ int cake_hip_device_info(cake_hip_device_t* out)
     if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
     int st = ensure_init();
     if (st) return st;
-    *out = g_ctx.info;
+    *out = cur().info;
     return CAKE_HIP_OK;
 }
 
@@ -649,7 +796,7 @@ int cake_hip_memcpy_h2d(void* dst, const void* src, size_t bytes)
     if (bytes >= PIN_THRESHOLD && is_pageable_host(src)) {
         int st = ensure_init();
         if (st) return st;
-        std::lock_guard<std::mutex> lock(g_mutex);
+        std::lock_guard<std::recursive_mutex> lock(cur().mutex);
         HIP_TRY(hipDeviceSynchronize());
         return host_to_device(dst, src, bytes);
     }
@@ -663,7 +810,7 @@ int cake_hip_memcpy_d2h(void* dst, const void* src, size_t bytes)
     if (bytes >= PIN_THRESHOLD && is_pageable_host(dst)) {
         int st = ensure_init();
         if (st) return st;
-        std::lock_guard<std::mutex> lock(g_mutex);
+        std::lock_guard<std::recursive_mutex> lock(cur().mutex);
         HIP_TRY(hipDeviceSynchronize());
         return device_to_host(dst, src, bytes);
     }
@@ -692,7 +839,7 @@ static int kernel_family(int M, int N, int K, bool tile_forced, bool vec)
     if (vec && !tune_lookup(M, N, K, true, nullptr)) {
         if (fewrows_applies(M, N, K, K, N)) return CAKE_HIP_KERNEL_STREAM_ROWS;
         if (fewrows_nt_applies(N, M, K, N, K, true)) return CAKE_HIP_KERNEL_STREAM_COLS;
-        if (shortk_applies(M, N, K, g_ctx.ready ? g_ctx.model.cus : DeviceModel{}.cus)) return CAKE_HIP_KERNEL_SHORT_K;
+        if (shortk_applies(M, N, K, cur().ready ? cur().model.cus : DeviceModel{}.cus)) return CAKE_HIP_KERNEL_SHORT_K;
     }
     return CAKE_HIP_KERNEL_TILE;
 }
@@ -701,7 +848,7 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
 {
     if (!out) return fail(CAKE_HIP_ERR_ARG, "out is NULL");
     GemmPlan plan;
-    const DeviceModel model = g_ctx.ready ? g_ctx.model : DeviceModel{};
+    const DeviceModel model = cur().ready ? cur().model : DeviceModel{};
     const bool vec = vec4_loadable(nullptr, nullptr, K, N);
     int st = plan_gemm(M, N, K, sched, tile_override, vec, model, &plan);
     if (st) return fail(st, "cake_hip_plan: bad shape, schedule or tile override");
@@ -736,6 +883,32 @@ int cake_hip_derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_
     return derive_schedule(M, N, K, p, mc, cntx);
 }
 
+int cake_hip_grid_dims_2d(int M, int N, int K, int p, int ncores) { return grid_dims_2d(M, N, K, p, ncores); }
+
+int cake_hip_init_block_dims_2d(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx, int sched, float type_size,
+                                int mcu, int kcu, int ncu, cake_hip_blk_dims_t* out)
+{
+    int st = init_block_dims_2d(M, N, K, p, cntx, sched, type_size, mcu, kcu, ncu, out);
+    if (st) return fail(st, "cake_hip_init_block_dims_2d: invalid argument");
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_init_block_dims_2d_small(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx, int sched,
+                                      float type_size, cake_hip_blk_dims_t* out)
+{
+    int st = init_block_dims_2d_small(M, N, K, p, cntx, sched, type_size, out);
+    if (st) return fail(st, "cake_hip_init_block_dims_2d_small: invalid argument");
+    return CAKE_HIP_OK;
+}
+
+int cake_hip_init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s,
+                                  int p, cake_hip_cpu_cntx_t* cntx, cake_hip_blk_dims_t* out)
+{
+    int st = init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cntx, out);
+    if (st) return fail(st, "cake_hip_init_block_dims_conv: invalid argument");
+    return CAKE_HIP_OK;
+}
+
 // Rows of A (and of C) per block of the pipelined host path: about a quarter of the rows, whole
 // macro-tile rows, and a block of either matrix fits a pinned buffer.  0: rows too long for this path.
 static int host_row_block(int M, int K, int N)
@@ -759,10 +932,10 @@ static int sgemm_host_pipelined(const float* A, const float* b_dev, float* C, in
     const int nblk = (M + RB - 1) / RB;
     int st = pinned_both_ways_ready();
     if (st) return st;
-    if ((st = g_ctx.stage[0].reserve((size_t)M * K * 4))) return st;
-    if ((st = g_ctx.stage[2].reserve((size_t)M * N * 4))) return st;
-    float* a_dev = static_cast<float*>(g_ctx.stage[0].ptr);
-    float* c_dev = static_cast<float*>(g_ctx.stage[2].ptr);
+    if ((st = cur().stage[0].reserve((size_t)M * K * 4))) return st;
+    if ((st = cur().stage[2].reserve((size_t)M * N * 4))) return st;
+    float* a_dev = static_cast<float*>(cur().stage[0].ptr);
+    float* c_dev = static_cast<float*>(cur().stage[2].ptr);
     HIP_TRY(hipDeviceSynchronize());   // nothing of an earlier call still uses the staging slots
 
     struct Events {
@@ -783,11 +956,11 @@ static int sgemm_host_pipelined(const float* A, const float* b_dev, float* C, in
     for (int i = 0; i < nblk + 2; ++i) {
         if (i < nblk) {
             const size_t off = (size_t)i * RB * K, bytes = (size_t)rows_of(i) * K * 4;
-            void* pin = g_ctx.pinned[i & 1];
+            void* pin = cur().pinned[i & 1];
             if (i >= 2) HIP_TRY(hipEventSynchronize(up[i - 2]));   // the buffer's last transfer is over
             parallel_memcpy(pin, A + off, bytes);
-            HIP_TRY(hipMemcpyAsync(a_dev + off, pin, bytes, hipMemcpyHostToDevice, g_ctx.copy_stream));
-            HIP_TRY(hipEventRecord(up[i], g_ctx.copy_stream));
+            HIP_TRY(hipMemcpyAsync(a_dev + off, pin, bytes, hipMemcpyHostToDevice, cur().copy_stream));
+            HIP_TRY(hipEventRecord(up[i], cur().copy_stream));
             HIP_TRY(hipStreamWaitEvent(stream, up[i], 0));
             const float* ai = a_dev + off;
             float* ci = c_dev + (size_t)i * RB * N;
@@ -798,15 +971,15 @@ static int sgemm_host_pipelined(const float* A, const float* b_dev, float* C, in
         }
         if (i >= 1 && i - 1 < nblk) {   // block i - 1 starts its way back (its buffer was emptied one round ago)
             const int j = i - 1;
-            HIP_TRY(hipStreamWaitEvent(g_ctx.copy_back_stream, done[j], 0));
-            HIP_TRY(hipMemcpyAsync(g_ctx.pinned[2 + (j & 1)], c_dev + (size_t)j * RB * N, (size_t)rows_of(j) * N * 4,
-                                   hipMemcpyDeviceToHost, g_ctx.copy_back_stream));
-            HIP_TRY(hipEventRecord(back[j], g_ctx.copy_back_stream));
+            HIP_TRY(hipStreamWaitEvent(cur().copy_back_stream, done[j], 0));
+            HIP_TRY(hipMemcpyAsync(cur().pinned[2 + (j & 1)], c_dev + (size_t)j * RB * N, (size_t)rows_of(j) * N * 4,
+                                   hipMemcpyDeviceToHost, cur().copy_back_stream));
+            HIP_TRY(hipEventRecord(back[j], cur().copy_back_stream));
         }
         if (i >= 2) {                   // block i - 2 has arrived: out to the caller's C
             const int j = i - 2;
             HIP_TRY(hipEventSynchronize(back[j]));
-            parallel_memcpy(C + (size_t)j * RB * N, g_ctx.pinned[2 + (j & 1)], (size_t)rows_of(j) * N * 4);
+            parallel_memcpy(C + (size_t)j * RB * N, cur().pinned[2 + (j & 1)], (size_t)rows_of(j) * N * 4);
         }
     }
     return timer.stop();
@@ -827,13 +1000,13 @@ static int sgemm_on_device(const float* A, const float* B, float* C, int M, int 
     } else if ((M == 1 || N == 1) && !tile_override) {
         // A product with a single row or column is a matrix-vector product: C[M] = A[M][K] . B[K]
         // reads A row-major; C[N] = A[K] . B[K][N] is B read as a column-major N x K matrix.
-        const size_t floats = N == 1 ? sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus)
-                                     : sgemv_colmajor_scratch_floats(N, K, g_ctx.model.cus);
+        const size_t floats = N == 1 ? sgemv_rowmajor_scratch_floats(M, K, cur().model.cus)
+                                     : sgemv_colmajor_scratch_floats(N, K, cur().model.cus);
         float* scratch = nullptr;
-        if (floats && (st = partial_space(g_ctx.gemv, floats * sizeof(float), &scratch))) return st;
+        if (floats && (st = scratch_space(cur().gemv, floats * sizeof(float), &scratch))) return st;
         st = timer.family(2, [&] {
-            return N == 1 ? launch_sgemv_rowmajor(A, B, C, M, K, accumulate, scratch, g_ctx.model.cus, stream)
-                          : launch_sgemv_colmajor(B, A, C, N, K, accumulate, scratch, g_ctx.model.cus, stream);
+            return N == 1 ? launch_sgemv_rowmajor(A, B, C, M, K, accumulate, scratch, cur().model.cus, stream)
+                          : launch_sgemv_colmajor(B, A, C, N, K, accumulate, scratch, cur().model.cus, stream);
         });
         if (st) return st;
     } else {
@@ -858,8 +1031,8 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
         return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand a, b, c;
     // large host operands: transfers and arithmetic overlap block by block
@@ -890,18 +1063,20 @@ int cake_hip_sgemm_noalloc(const float* A, const float* B, float* C, int M, int 
     if (!fits_int((double)M * K) || !fits_int((double)K * N) || !fits_int((double)M * N))
         return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
     // nothing is set up here: events, device model and the scratch address come from cake_hip_init
-    if (!g_ctx.ready)
+    Context& c = cur();
+    std::lock_guard<std::recursive_mutex> lock(c.mutex);
+    if (!c.ready)
         return fail(CAKE_HIP_ERR_NO_DEVICE, "cake_hip_sgemm_noalloc needs cake_hip_init to have run: it sets nothing up itself");
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (g_ctx.device >= MAX_DEVICES || !g_noalloc_ptr[g_ctx.device])
-        return fail(CAKE_HIP_ERR_NO_DEVICE, "no scratch address for device %d", g_ctx.device);
+    if (c.device >= MAX_DEVICES || !g_noalloc_ptr[c.device])
+        return fail(CAKE_HIP_ERR_NO_DEVICE, "no scratch address for device %d", c.device);
     if (!is_device_pointer(A) || !is_device_pointer(B) || !is_device_pointer(C))
         return fail(CAKE_HIP_ERR_ARG, "cake_hip_sgemm_noalloc takes device memory only (host operands need staging buffers)");
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = pick_stream(stream_);
     Timer untimed(stream, nullptr);
-    g_noalloc_call = true;
+    c.noalloc_call = true;
+    c.noalloc_used = 0;
     const int st = sgemm_on_device(A, B, C, M, N, K, sched, accumulate, nullptr, stream, untimed);
-    g_noalloc_call = false;
+    c.noalloc_call = false;
     return st;
 }
 
@@ -958,15 +1133,15 @@ static int pack_common(int which, int dir, const float* src, float* dst, int M, 
     if (rows <= 0 || cols <= 0) return fail(CAKE_HIP_ERR_ARG, "empty operand");
     if (!fits_int((double)rows_p * cols_p)) return fail(CAKE_HIP_ERR_RANGE, "packed operand exceeds 2^31 elements");
     if ((st = ensure_init())) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     const size_t plain_bytes = (size_t)rows * cols * 4, packed_bytes = (size_t)rows_p * cols_p * 4;
     Operand in, out;
     if ((st = stage_in(src, dir == 0 ? plain_bytes : packed_bytes, 0, true, &in))) return st;
     // unpack writes only the real extent of C; a staged C must start from the caller's values
     if ((st = stage_in(dst, dir == 0 ? packed_bytes : plain_bytes, 1, false, &out))) return st;
-    if ((st = g_ctx.tables.reserve(tables_bytes(which, g)))) return st;
+    if ((st = cur().tables.reserve(tables_bytes(which, g)))) return st;
 
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
@@ -1025,21 +1200,21 @@ int cake_hip_sgemm_packed(const float* A, const float* B, float* C, int M, int N
     if (!fits_int((double)a_elems) || !fits_int((double)b_elems) || !fits_int((double)M * N))
         return fail(CAKE_HIP_ERR_RANGE, "operand exceeds 2^31 elements");
     if ((st = ensure_init())) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand a, b, c;
     if ((st = stage_in(A, a_elems * 4, 0, true, &a))) return st;
     if ((st = stage_in(B, b_elems * 4, 1, true, &b))) return st;
     if ((st = stage_in(C, (size_t)M * N * 4, 2, accumulate != 0, &c))) return st;
-    if ((st = g_ctx.tables.reserve((packedA ? tables_bytes(0, g) : 0) + (packedB ? tables_bytes(1, g) : 0)))) return st;
+    if ((st = cur().tables.reserve((packedA ? tables_bytes(0, g) : 0) + (packedB ? tables_bytes(1, g) : 0)))) return st;
     // A packed operand is first copied back to row-major order (one pass at HBM speed through
     // the index tables); the product then runs on the row-major kernel, which is several times
     // faster than gathering packed elements inside the K walk.
     const size_t ua_floats = packedA ? (((size_t)M * K + 63) & ~(size_t)63) : 0;
     const size_t ub_floats = packedB ? (size_t)K * N : 0;
-    if ((st = g_ctx.unpacked.reserve((ua_floats + ub_floats) * sizeof(float)))) return st;
-    float* ua = static_cast<float*>(g_ctx.unpacked.ptr);
+    if ((st = cur().unpacked.reserve((ua_floats + ub_floats) * sizeof(float)))) return st;
+    float* ua = static_cast<float*>(cur().unpacked.ptr);
     float* ub = ua + ua_floats;
 
     Timer timer(stream, seconds);
@@ -1073,17 +1248,17 @@ int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K, int a
     if (!fits_int((double)M * K)) return fail(CAKE_HIP_ERR_RANGE, "matrix of %dx%d exceeds 2^31 elements", M, K);
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand a, xv, yv;
     if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
     if ((st = stage_in(x, (size_t)K * 4, 1, true, &xv))) return st;
     if ((st = stage_in(y, (size_t)M * 4, 2, accumulate != 0, &yv))) return st;
     if (K > 0) {
-        const size_t floats = a_col_major ? sgemv_colmajor_scratch_floats(M, K, g_ctx.model.cus)
-                                          : sgemv_rowmajor_scratch_floats(M, K, g_ctx.model.cus);
-        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
+        const size_t floats = a_col_major ? sgemv_colmajor_scratch_floats(M, K, cur().model.cus)
+                                          : sgemv_rowmajor_scratch_floats(M, K, cur().model.cus);
+        if (floats && (st = cur().gemv.reserve(floats * sizeof(float)))) return st;
     }
     Timer timer(stream, seconds);
     if ((st = timer.start())) return st;
@@ -1095,9 +1270,9 @@ int cake_hip_sgemv(const float* A, const float* x, float* y, int M, int K, int a
     } else {
         st = timer.family(2, [&] {
             return a_col_major ? launch_sgemv_colmajor(a.dev, xv.dev, yv.dev, M, K, accumulate,
-                                                       static_cast<float*>(g_ctx.gemv.ptr), g_ctx.model.cus, stream)
+                                                       static_cast<float*>(cur().gemv.ptr), cur().model.cus, stream)
                                : launch_sgemv_rowmajor(a.dev, xv.dev, yv.dev, M, K, accumulate,
-                                                       static_cast<float*>(g_ctx.gemv.ptr), g_ctx.model.cus, stream);
+                                                       static_cast<float*>(cur().gemv.ptr), cur().model.cus, stream);
         });
         if (st) return st;
     }
@@ -1127,8 +1302,8 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
         return fail(CAKE_HIP_ERR_RANGE, "column matrix %gx%g out of range", krows, ncols);
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
     Operand i, o;
     if ((st = stage_in(in, (size_t)batch * Cin * Hin * Win * 4, 0, true, &i))) return st;
     if ((st = stage_in(cols, (size_t)(krows * ncols) * 4, 1, false, &o))) return st;
@@ -1188,6 +1363,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
                          void* workspace, void* stream_, double* seconds, int explicit_cols, int accumulate = 0)
 {
     if (seconds) *seconds = 0;
+    g_last_conv_route = CAKE_HIP_CONV_NONE;
     int Hout, Wout;
     if (batch <= 0 || Cin <= 0 || Cout <= 0 || Hin <= 0 || Win <= 0 ||
         conv_out_dims(Hin, Win, Hf, Wf, stride, pad, &Hout, &Wout))
@@ -1211,8 +1387,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const int K = (int)K_d, N = (int)ncols_d;
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand i, w, o;
     if ((st = stage_in(in, (size_t)in_elems * 4, 0, true, &i))) return st;
@@ -1249,8 +1425,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // (64 -> 256 channels on 32 x 56 x 56: 50 -> 43 us).
     const int HW = Hout * Wout;
     if (!explicit_cols && Hf == 1 && Wf == 1 && stride == 1 && pad == 0 &&
-        shortk_applies(Cout, HW, K, g_ctx.model.cus, batch) &&
-        (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch >= 12L * g_ctx.model.cus &&   // measured from there on
+        shortk_applies(Cout, HW, K, cur().model.cus, batch) &&
+        (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch >= 12L * cur().model.cus &&   // measured from there on
         vec4_loadable(w.dev, i.dev, K, HW)) {
         GemmArgs g{};
         g.A = w.dev; g.B = i.dev; g.C = o.dev;
@@ -1259,15 +1435,16 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.ldc = out_nchw ? HW : N;                             // [batch][Cout][HW] or [Cout][batch*HW]
         g.b_batch_stride = (size_t)Cin * HW;
         g.c_batch_stride = out_nchw ? (size_t)Cout * HW : (size_t)HW;
-        const int tn = shortk_tile_n(Cout, HW, K, g_ctx.model.cus, batch);
+        const int tn = shortk_tile_n(Cout, HW, K, cur().model.cus, batch);
         g.tiles_m = (Cout + 63) / 64;
         g.tiles_n_per_image = (HW + tn - 1) / tn;
         g.tiles_n = g.tiles_n_per_image * batch;
         g.split_k = 1; g.k_per_split = K;
         g.group = g.tiles_m; g.group_along_n = 0;
         g.accumulate = accumulate;
+        g_last_conv_route = CAKE_HIP_CONV_SHORTK_BATCH;
         if ((st = timer.start())) return st;
-        st = timer.family(0, [&] { return launch_sgemm_shortk(g, tn, g_ctx.model.cus, stream); });
+        st = timer.family(0, [&] { return launch_sgemm_shortk(g, tn, cur().model.cus, stream); });
         if (st) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);
@@ -1285,7 +1462,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     int patch_rows = 0, patch_pitch = 0;
     const long patch_tiles_m = (Cout + 255) / 256, patch_tiles_n = ((long)batch * Hout * row_n + 127) / 128;
     const bool patch_pays = conv_patch_k(Cin, Hf, Wf) / 32 >= 64 && 4L * Cout >= 3L * 256 * patch_tiles_m &&
-                            patch_tiles_m * patch_tiles_n >= 2L * g_ctx.model.cus;
+                            patch_tiles_m * patch_tiles_n >= 2L * cur().model.cus;
     // CAKE_HIP_CONV_ROUTE=patch takes that kernel wherever its geometry allows, =staged never
     // (for tests and measurements; read at every call)
     const char* route = std::getenv("CAKE_HIP_CONV_ROUTE");
@@ -1294,11 +1471,12 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if (!explicit_cols && patch_wanted && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_k(Cin, Hf, Wf)) &&
         conv_patch_geometry(batch, Cin, Hin, Win, Hf, Wf, stride, pad, Hout, Wout, &patch_rows, &patch_pitch)) {
         const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n;
-        if ((st = g_ctx.conv_filters.reserve((size_t)Cout * Kp * sizeof(float)))) return st;
-        float* wt = static_cast<float*>(g_ctx.conv_filters.ptr);
+        g_last_conv_route = CAKE_HIP_CONV_PATCH;
+        if ((st = cur().conv_filters.reserve((size_t)Cout * Kp * sizeof(float)))) return st;
+        float* wt = static_cast<float*>(cur().conv_filters.ptr);
         const int tile[4] = {256, 128, 32, 0};
         GemmPlan plan;
-        if ((st = plan_gemm(Cout, Np, Kp, CAKE_HIP_NA, tile, true, g_ctx.model, &plan))) return fail(st, "conv2d: no plan");
+        if ((st = plan_gemm(Cout, Np, Kp, CAKE_HIP_NA, tile, true, cur().model, &plan))) return fail(st, "conv2d: no plan");
         GemmArgs g{};
         g.A = wt; g.B = nullptr; g.C = o.dev;
         g.M = Cout; g.N = Np; g.K = Kp;
@@ -1321,7 +1499,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
                 g.tail_split = slices;
                 g.tail_k_per_split = per * block_k;    // (not read for halves: the kernel places them itself)
                 g.conv.tail_halves = halves ? 1 : 0;
-                if ((st = partial_space(g_ctx.splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
+                if ((st = scratch_space(cur().splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
                     return st;
                 grid += g.tail_tiles * (slices - 1);
             }
@@ -1344,19 +1522,20 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         return stage_out(o, stream);
     }
     if (implicit) {
+        g_last_conv_route = CAKE_HIP_CONV_GATHER;
         float* staged = nullptr;
         if (sg.copy) {
             char* ws = static_cast<char*>(workspace);
             if (!ws) {
-                if ((st = g_ctx.conv.reserve((size_t)sg.elems * 4 + 256))) return st;
-                ws = static_cast<char*>(g_ctx.conv.ptr);
+                if ((st = cur().conv.reserve((size_t)sg.elems * 4 + 256))) return st;
+                ws = static_cast<char*>(cur().conv.ptr);
             } else if (!is_device_pointer(ws)) {
                 return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
             }
             staged = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
         }
-        if ((st = g_ctx.conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
-        int* taps = static_cast<int*>(g_ctx.conv_taps.ptr);
+        if ((st = cur().conv_taps.reserve(((size_t)K + CONV_TAP_TABLE_EXTRA) * sizeof(int)))) return st;
+        int* taps = static_cast<int*>(cur().conv_taps.ptr);
         if ((st = timer.start())) return st;
         const bool one_by_one = Hf == 1 && Wf == 1;   // row k is channel k: no table of tap offsets
         if (!one_by_one) {
@@ -1399,10 +1578,11 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
 
     if (!fits_int(K_d * ncols_d) || !fits_int(Cout * ncols_d) || !fits_int(in_elems) || K > 65535)
         return fail(CAKE_HIP_ERR_RANGE, "column matrix %gx%g out of range", K_d, ncols_d);
+    g_last_conv_route = CAKE_HIP_CONV_TWO_STEP;
     char* ws = static_cast<char*>(workspace);
     if (!ws) {
-        if ((st = g_ctx.conv.reserve(cake_hip_conv2d_workspace(batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)))) return st;
-        ws = static_cast<char*>(g_ctx.conv.ptr);
+        if ((st = cur().conv.reserve(cake_hip_conv2d_workspace(batch, Cin, Hin, Win, Cout, Hf, Wf, stride, pad)))) return st;
+        ws = static_cast<char*>(cur().conv.ptr);
     } else if (!is_device_pointer(ws)) {
         return fail(CAKE_HIP_ERR_ARG, "workspace must be device memory");
     }
@@ -1470,6 +1650,77 @@ int cake_hip_sconv(const float* filters, const float* in, float* out, int Wf, in
     return conv2d_common(in, filters, out, 1, Cin, Hin, Win, Cout, Hf, Wf, stride, 0, 0, nullptr, stream, seconds, 0, 1);
 }
 
+// ---- filters in the reference's packed layout ------------------------------------------
+
+static int filter_geom(int Cout, int Cin, int taps, int p, const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx,
+                       PackGeom* g)
+{
+    int st = check_geom(d, cx, p, CAKE_HIP_KMN);
+    if (st) return st;
+    if (Cout <= 0 || Cin <= 0 || taps <= 0) return fail(CAKE_HIP_ERR_ARG, "empty filters");
+    *g = make_geom(Cout, 0, Cin, p, d, cx, CAKE_HIP_KMN);
+    // the block dims must be those of this Cout, Cin and p (init_block_dims_conv): the index map reads them
+    if (d->sch != CAKE_HIP_KMN || padded_rows(*g) != d->M_padded || d->M_padded < Cout ||
+        d->Kb != Cin / d->k_c + (Cin % d->k_c != 0) || (d->k_pad && d->k_c1 != Cin % d->k_c))
+        return fail(CAKE_HIP_ERR_ARG, "block dims do not belong to %d x %d filters on %d cores", Cout, Cin, p);
+    if (!fits_int((double)d->M_padded * Cin * taps)) return fail(CAKE_HIP_ERR_RANGE, "packed filters exceed 2^31 elements");
+    return CAKE_HIP_OK;
+}
+
+size_t cake_hip_packed_filters_size(int Cout, int Cin, int taps, int p, const cake_hip_blk_dims_t* d,
+                                    const cake_hip_cpu_cntx_t* cx)
+{
+    PackGeom g;
+    if (filter_geom(Cout, Cin, taps, p, d, cx, &g)) return 0;
+    return (size_t)d->M_padded * Cin * taps * sizeof(float);
+}
+
+int cake_hip_pack_filters(const float* filters, float* filters_p, int Cout, int Cin, int taps, int p,
+                          const cake_hip_blk_dims_t* d, const cake_hip_cpu_cntx_t* cx, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    PackGeom g;
+    int st = filter_geom(Cout, Cin, taps, p, d, cx, &g);
+    if (st) return st;
+    if (!filters || !filters_p) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
+    Operand in, out;
+    if ((st = stage_in(filters, (size_t)Cout * Cin * taps * 4, 0, true, &in))) return st;
+    if ((st = stage_in(filters_p, (size_t)d->M_padded * Cin * taps * 4, 1, false, &out))) return st;
+    Timer timer(stream, seconds);
+    if ((st = timer.start())) return st;
+    if ((st = timer.family(4, [&] { return launch_filter_layout(in.dev, out.dev, g, Cout, Cin, taps, 1, stream); }))) return st;
+    if ((st = timer.stop())) return st;
+    return stage_out(out, stream);
+}
+
+int cake_hip_sconv_packed(const float* filters_p, const float* in, float* out, int Wf, int Hf, int Win, int Hin,
+                          int Wout, int Hout, int Cin, int Cout, int stride, int p, const cake_hip_blk_dims_t* d,
+                          const cake_hip_cpu_cntx_t* cx, void* stream_, double* seconds)
+{
+    if (seconds) *seconds = 0;
+    if (Wf <= 0 || Hf <= 0 || !fits_int((double)Wf * Hf)) return fail(CAKE_HIP_ERR_ARG, "bad convolution geometry");
+    const int taps = Wf * Hf;
+    PackGeom g;
+    int st = filter_geom(Cout, Cin, taps, p, d, cx, &g);
+    if (st) return st;
+    if (!filters_p) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
+    if ((st = ensure_init())) return st;
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);   // held across the unpacking and the convolution
+    hipStream_t stream = pick_stream(stream_);
+    Operand fp;
+    // (slot 3: the convolution stages its own operands in slots 0 to 2)
+    if ((st = stage_in(filters_p, (size_t)d->M_padded * Cin * taps * 4, 3, true, &fp))) return st;
+    if ((st = cur().unpacked.reserve((size_t)Cout * Cin * taps * sizeof(float)))) return st;
+    float* plain = static_cast<float*>(cur().unpacked.ptr);
+    // the filters go back to [Cout][Cin][Hf][Wf] (a few megabytes at most), then the convolution runs as cake_hip_sconv does
+    hipError_t e = launch_filter_layout(fp.dev, plain, g, Cout, Cin, taps, 0, stream);
+    if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "filter unpack launch failed: %s", hipGetErrorString(e));
+    return cake_hip_sconv(plain, in, out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, stride, stream_, seconds);
+}
+
 int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* stream_, double* seconds)
 {
     if (seconds) *seconds = 0;
@@ -1480,8 +1731,8 @@ int cake_hip_transpose(const float* src, float* dst, int rows, int cols, void* s
     if (!fits_int((double)rows * cols)) return fail(CAKE_HIP_ERR_RANGE, "matrix of %dx%d exceeds 2^31 elements", rows, cols);
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
     Operand in, out;
     const size_t bytes = (size_t)rows * cols * 4;
     if ((st = stage_in(src, bytes, 0, true, &in))) return st;
@@ -1531,7 +1782,7 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
         hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, accumulate, stream, nullptr, bias);
         return e == hipSuccess ? CAKE_HIP_OK : fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
     }
-    const int cus = g_ctx.model.cus;
+    const int cus = cur().model.cus;
     if ((M == 1 || N == 1) && !tile_override && !(bias && accumulate)) {
         // y = W . x (one row of X), or C[:, 0] = X . w (one row of W): the matrix is read row-major at
         // 7.2 TB/s where the streaming kernel reaches 6.4.  A bias goes first and the product is
@@ -1540,8 +1791,8 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
         const float* vec = M == 1 ? X : W;
         const int rows = M == 1 ? N : M;
         const size_t floats = sgemv_rowmajor_scratch_floats(rows, K, cus);
-        if (floats && (st = g_ctx.gemv.reserve(floats * sizeof(float)))) return st;
-        float* scratch = static_cast<float*>(g_ctx.gemv.ptr);
+        if (floats && (st = cur().gemv.reserve(floats * sizeof(float)))) return st;
+        float* scratch = static_cast<float*>(cur().gemv.ptr);
         if (bias) {   // C[m][n] = bias[n], by a kernel (no copy or memset node for a captured graph)
             hipError_t e = launch_splitk_reduce(nullptr, C, M, N, N, 0, 0, stream, nullptr, bias);
             if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "fill failed: %s", hipGetErrorString(e));
@@ -1562,7 +1813,7 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
         const int slices = few_x ? fewrows_nt_slices(M, N, K, K, false, cus) : fewrows_nt_slices(N, M, K, K, false, cus);
         float* partial = nullptr;
         if (slices > 1) {
-            if ((st = partial_space(g_ctx.splitk, (size_t)slices * M * N * sizeof(float), &partial))) return st;
+            if ((st = scratch_space(cur().splitk, (size_t)slices * M * N * sizeof(float), &partial))) return st;
         }
         return timer.family(0, [&] {
             return few_x ? launch_sgemm_fewrows_nt(X, W, C, partial, M, N, K, K, K, N, false, false, accumulate, bias, cus, stream)
@@ -1572,8 +1823,8 @@ static int gemm_nt(const float* X, const float* W, float* C, int M, int N, int K
     if ((double)K * 256 * 4 < 2147483648.0)
         return run_gemm(X, W, C, M, N, K, K, K, N, CAKE_HIP_NA, accumulate, tile_override, LOAD_VEC4, LOAD_VEC4_T,
                         stream, timer, nullptr, bias);
-    if ((st = g_ctx.linear.reserve((size_t)N * K * 4))) return st;
-    float* wt = static_cast<float*>(g_ctx.linear.ptr);
+    if ((st = cur().linear.reserve((size_t)N * K * 4))) return st;
+    float* wt = static_cast<float*>(cur().linear.ptr);
     st = timer.family(4, [&] { return launch_transpose(W, wt, N, K, stream); });
     if (st) return st;
     const int mode = vec4_loadable(X, wt, K, N) ? LOAD_VEC4 : LOAD_SCALAR;
@@ -1592,8 +1843,8 @@ int cake_hip_sgemm_nt(const float* A, const float* Bt, float* C, int M, int N, i
         return fail(CAKE_HIP_ERR_RANGE, "operand of %dx%dx%d exceeds 2^31 elements", M, K, N);
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
     Operand a, b, c;
     if ((st = stage_in(A, (size_t)M * K * 4, 0, true, &a))) return st;
     if ((st = stage_in(Bt, (size_t)N * K * 4, 1, true, &b))) return st;
@@ -1614,8 +1865,8 @@ int cake_hip_linear_forward(const float* x, const float* w, const float* bias, f
     if (M == 0 || N == 0) return CAKE_HIP_OK;
     if (!y || (K > 0 && (!x || !w))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
     if ((st = ensure_init())) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand xo, wo, bo, yo;
     if ((st = stage_in(x, (size_t)M * K * 4, 0, true, &xo))) return st;
@@ -1638,8 +1889,8 @@ int cake_hip_linear_forward_wt(const float* x, const float* wt, const float* bia
     if (M == 0 || N == 0) return CAKE_HIP_OK;
     if (!y || (K > 0 && (!x || !wt))) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
     if ((st = ensure_init())) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand xo, wo, bo, yo;
     if ((st = stage_in(x, (size_t)M * K * 4, 0, true, &xo))) return st;
@@ -1664,8 +1915,8 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
     if (grad_x && !w && N > 0) return fail(CAKE_HIP_ERR_ARG, "grad_x needs w");
     if (grad_w && !x && M > 0) return fail(CAKE_HIP_ERR_ARG, "grad_w needs x");
     if ((st = ensure_init())) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
 
     Operand go, xo, wo, gxo, gwo, gbo;
     if ((st = stage_in(grad_y, (size_t)M * N * 4, 0, true, &go))) return st;
@@ -1677,9 +1928,9 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
     // workspace: grad_y transposed (N x M), then a vector of M ones, then the GEMV's slice partials
     const size_t gt_floats = grad_w ? (((size_t)M * N + 63) & ~(size_t)63) : 0;
     const size_t ones_floats = grad_bias ? (((size_t)M + 63) & ~(size_t)63) : 0;
-    const size_t gemv_floats = grad_bias && M > 0 && N > 0 ? sgemv_colmajor_scratch_floats(N, M, g_ctx.model.cus) : 0;
-    if ((st = g_ctx.linear.reserve((gt_floats + ones_floats + gemv_floats) * 4 + 256))) return st;
-    float* gt = static_cast<float*>(g_ctx.linear.ptr);
+    const size_t gemv_floats = grad_bias && M > 0 && N > 0 ? sgemv_colmajor_scratch_floats(N, M, cur().model.cus) : 0;
+    if ((st = cur().linear.reserve((gt_floats + ones_floats + gemv_floats) * 4 + 256))) return st;
+    float* gt = static_cast<float*>(cur().linear.ptr);
     float* ones = gt + gt_floats;
     float* gemv_scratch = ones + ones_floats;
 
@@ -1703,7 +1954,7 @@ int cake_hip_linear_backward(const float* grad_y, const float* x, const float* w
             st = timer.family(2, [&] {
                 hipError_t e = launch_fill_value(ones, (size_t)M, 1.f, stream);
                 if (e != hipSuccess) return e;
-                return launch_sgemv_colmajor(go.dev, ones, gbo.dev, N, M, 0, gemv_scratch, g_ctx.model.cus, stream);
+                return launch_sgemv_colmajor(go.dev, ones, gbo.dev, N, M, 0, gemv_scratch, cur().model.cus, stream);
             });
             if (st) return st;
         }
@@ -1728,16 +1979,16 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     if (!(budget_seconds > 0)) budget_seconds = 2.0;
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = nullptr;
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = cur().own_stream;
 
     // synthetic operands in the staging slots (what a host caller's operands would use)
-    if ((st = g_ctx.stage[0].reserve((size_t)M * K * 4))) return st;
-    if ((st = g_ctx.stage[1].reserve((size_t)K * N * 4))) return st;
-    if ((st = g_ctx.stage[2].reserve((size_t)M * N * 4))) return st;
-    float* A = static_cast<float*>(g_ctx.stage[0].ptr);
-    float* B = static_cast<float*>(g_ctx.stage[1].ptr);
-    float* C = static_cast<float*>(g_ctx.stage[2].ptr);
+    if ((st = cur().stage[0].reserve((size_t)M * K * 4))) return st;
+    if ((st = cur().stage[1].reserve((size_t)K * N * 4))) return st;
+    if ((st = cur().stage[2].reserve((size_t)M * N * 4))) return st;
+    float* A = static_cast<float*>(cur().stage[0].ptr);
+    float* B = static_cast<float*>(cur().stage[1].ptr);
+    float* C = static_cast<float*>(cur().stage[2].ptr);
     HIP_TRY(launch_fill_uniform(A, (size_t)M * K, 1, stream));
     HIP_TRY(launch_fill_uniform(B, (size_t)K * N, 2, stream));
     const bool vec = vec4_loadable(A, B, K, N);
@@ -1750,15 +2001,15 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
         double est = 0, best_batch = 1e30;
         for (int pass = 0; pass < 4; ++pass) {
             const int reps = pass == 0 ? 1 : (est < 2e-4 ? 20 : est < 5e-3 ? 5 : 2);
-            HIP_TRY(hipEventRecord(g_ctx.ev[0], stream));
+            HIP_TRY(hipEventRecord(cur().ev[0], stream));
             for (int r = 0; r < reps; ++r) {
                 int e = run_gemm(A, B, C, M, N, K, K, N, N, CAKE_HIP_NA, 0, nullptr, mode, mode, stream, untimed, nullptr, nullptr, c);
                 if (e) return e;
             }
-            HIP_TRY(hipEventRecord(g_ctx.ev[1], stream));
-            HIP_TRY(hipEventSynchronize(g_ctx.ev[1]));
+            HIP_TRY(hipEventRecord(cur().ev[1], stream));
+            HIP_TRY(hipEventSynchronize(cur().ev[1]));
             float ms = 0;
-            HIP_TRY(hipEventElapsedTime(&ms, g_ctx.ev[0], g_ctx.ev[1]));
+            HIP_TRY(hipEventElapsedTime(&ms, cur().ev[0], cur().ev[1]));
             est = ms * 1e-3 / reps;
             if (pass > 0 && est < best_batch) best_batch = est;
         }
@@ -1770,7 +2021,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     GemmPlan model_plan;
     {
         const int any[4] = {0, 0, 0, 0};
-        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, any, vec, g_ctx.model, &model_plan))) return st;
+        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, any, vec, cur().model, &model_plan))) return st;
     }
     TunedChoice best{model_plan.tile_id, model_plan.pub.split_k, 1, 0.0};
     if ((st = measure(&best, &best.seconds))) return st;
@@ -1778,7 +2029,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     // to beat it: that kernel is the default here, and the table keeps no entry when it wins
     // (the same holds for the short-K kernel that walks over tiles)
     const bool streaming = vec && (fewrows_applies(M, N, K, K, N) || fewrows_nt_applies(N, M, K, N, K, true) ||
-                                   shortk_applies(M, N, K, g_ctx.model.cus));
+                                   shortk_applies(M, N, K, cur().model.cus));
     double streaming_seconds = 0;
     if (streaming) {
         tune_erase(M, N, K, true);
@@ -1791,7 +2042,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     bool out_of_time = false;
     for (int id = 0; id < TILE_COUNT && !out_of_time; ++id) {
         const TileInfo& t = tile_info(id);
-        if (t.lds_bytes > g_ctx.model.lds_per_cu) continue;
+        if (t.lds_bytes > cur().model.lds_per_cu) continue;
         const int max_split = std::max(1, K / (4 * t.bk));
         for (int split = 1; split <= max_split && split <= 1024; split *= 2) {
             for (int tail = (split == 1 ? 1 : 0); tail >= 0; --tail) {
@@ -1801,7 +2052,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
                 TunedChoice c{id, split, tail, 0.0};
                 if (tail) {  // only a distinct candidate when the tile count leaves a thin round
                     GemmPlan probe;
-                    if (plan_gemm_choice(M, N, K, CAKE_HIP_NA, c, vec, g_ctx.model, &probe) || probe.pub.tail_tiles == 0)
+                    if (plan_gemm_choice(M, N, K, CAKE_HIP_NA, c, vec, cur().model, &probe) || probe.pub.tail_tiles == 0)
                         continue;
                 }
                 // skip candidates the model already puts far behind: a split whose slices alone outweigh the product
@@ -1836,7 +2087,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
         if (best_seconds) *best_seconds = streaming_seconds;
         if (best_plan) {
             GemmPlan plan;
-            if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
+            if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, cur().model, &plan))) return st;
             *best_plan = plan.pub;
             best_plan->kernel = kernel_family(M, N, K, false, vec);
         }
@@ -1851,7 +2102,7 @@ int cake_hip_autotune(int M, int N, int K, double budget_seconds, cake_hip_plan_
     if (best_seconds) *best_seconds = best.seconds;
     if (best_plan) {
         GemmPlan plan;
-        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, g_ctx.model, &plan))) return st;
+        if ((st = plan_gemm(M, N, K, CAKE_HIP_NA, nullptr, vec, cur().model, &plan))) return st;
         *best_plan = plan.pub;
         best_plan->kernel = kernel_family(M, N, K, false, vec);
     }
@@ -1889,14 +2140,16 @@ int cake_hip_fill_uniform(float* dst, size_t n, uint64_t seed, void* stream_)
     if (!dst) return fail(CAKE_HIP_ERR_ARG, "NULL operand");
     int st = ensure_init();
     if (st) return st;
-    std::lock_guard<std::mutex> lock(g_mutex);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    std::lock_guard<std::recursive_mutex> lock(cur().mutex);
+    hipStream_t stream = pick_stream(stream_);
     Operand o;
     if ((st = stage_in(dst, n * 4, 0, false, &o))) return st;
     hipError_t e = launch_fill_uniform(o.dev, n, seed, stream);
     if (e != hipSuccess) return fail(CAKE_HIP_ERR_HIP, "fill launch failed: %s", hipGetErrorString(e));
     return stage_out(o, stream);
 }
+
+int cake_hip_last_conv_route(void) { return g_last_conv_route; }
 
 int cake_hip_last_kernel_seconds(double out[5])
 {

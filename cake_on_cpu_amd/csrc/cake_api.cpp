@@ -10,6 +10,8 @@
 #include <math.h>
 #include <time.h>
 
+#include <mutex>
+
 #include "cake_hip.h"
 
 namespace {
@@ -60,6 +62,49 @@ long popen_number(const char* cmd)
     return got ? atol(buf) : -1;
 }
 
+// Device-side state per cake_cntx_t.  The reference keeps its kernel library's context in
+// cake_cntx_t::blis_cntx (include/common.h:139); here that field names the device context
+// (workspaces, events, stream: cake_hip_ctx_create) the cntx works on, so that host threads that each
+// use a cntx of their own do not wait for each other.  A cntx cannot be told when it is freed (callers
+// free() it, examples/cake_sgemm_test.cpp:87), so contexts are not owned by it: they come from a
+// small pool that lives as long as the process.  The first cntx seen works on the library's default
+// context, the following ones on up to three created contexts, handed out in turn; whatever the
+// field holds is only ever compared with the pool's entries, never followed.
+enum { CONTEXT_POOL = 4 };
+std::mutex g_pool_mutex;
+char g_default_marker;                    // its address stands for the default context
+void* g_pool[CONTEXT_POOL] = {&g_default_marker, NULL, NULL, NULL};
+int g_pool_made = 1, g_pool_next = 0;
+
+cake_hip_ctx_t context_of(cake_cntx_t* c)
+{
+    if (!c) return NULL;
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    void* mine = NULL;
+    for (int i = 0; i < g_pool_made; ++i)
+        if (c->blis_cntx == g_pool[i]) mine = g_pool[i];
+    if (!mine) {
+        if (g_pool_next >= g_pool_made && g_pool_made < CONTEXT_POOL) {
+            cake_hip_ctx_t fresh = NULL;
+            if (cake_hip_ctx_create(&fresh) == CAKE_HIP_OK && fresh) g_pool[g_pool_made++] = fresh;
+        }
+        mine = g_pool[g_pool_next % g_pool_made];
+        g_pool_next = (g_pool_next + 1) % CONTEXT_POOL;
+        c->blis_cntx = mine;
+    }
+    return mine == &g_default_marker ? NULL : mine;
+}
+
+// makes a cntx's device context the calling thread's for the duration of one call
+struct OnContextOf {
+    cake_hip_ctx_t before;
+    explicit OnContextOf(cake_cntx_t* c) : before(cake_hip_ctx_get_current())
+    {
+        (void)cake_hip_ctx_set_current(context_of(c));
+    }
+    ~OnContextOf() { (void)cake_hip_ctx_set_current(before); }
+};
+
 // macro-tile override from the caller's mcu,kcu,ncu when such a tile exists
 const int* tile_from_user(int M, int N, int K, int sch, int mcu, int kcu, int ncu, int out[4])
 {
@@ -75,6 +120,7 @@ double sgemm_common(float* A, float* B, float* C, int M, int N, int K, int p, ca
 {
     (void)argv;
     if (cntx == NULL) cntx = cake_query_cntx();  // leaked, as in the reference (:14-16)
+    OnContextOf on(cntx);
     const double t0 = wall_seconds();
     if (packedA || packedB) {
         blk_dims_t x;
@@ -94,6 +140,8 @@ double sgemm_common(float* A, float* B, float* C, int M, int N, int K, int p, ca
             blk_dims_t x;
             init_block_dims(M, N, K, p, &x, cntx, sch, argv, 4, mcu, kcu, ncu);
             resolved = x.sch;
+        } else if (sch == NA) {
+            resolved = KMN;   // nothing to size for an empty product: K-first, which assigns C
         }
         const int accumulate = (resolved != KMN) && (beta != 0);
         int ov[4];
@@ -194,6 +242,61 @@ cache_dims_t* get_cache_dims(int M, int N, int K, int p, cake_cntx_t* cake_cntx,
     return r;
 }
 
+int grid_dims_2d(int M, int N, int K, int p, int ncores) { return cake_hip_grid_dims_2d(M, N, K, p, ncores); }
+
+void init_block_dims_2d(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch,
+                        char* argv[], float type_size, int mcu, int kcu, int ncu)
+{
+    (void)argv;
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    cake_hip_blk_dims_t d;
+    die_on(cake_hip_init_block_dims_2d(M, N, K, p, &cx, sch, type_size, mcu, kcu, ncu, &d), "init_block_dims_2d");
+    memcpy(x, &d, sizeof d);
+    cake_cntx->alpha_n = cx.alpha_n;
+}
+
+void init_block_dims_2d_small(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch,
+                              char* argv[], float type_size)
+{
+    (void)argv;
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    cake_hip_blk_dims_t d;
+    die_on(cake_hip_init_block_dims_2d_small(M, N, K, p, &cx, sch, type_size, &d), "init_block_dims_2d_small");
+    memcpy(x, &d, sizeof d);
+}
+
+void init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s, int p,
+                          blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch, char* argv[], float density,
+                          float type_size)
+{
+    (void)argv; (void)density; (void)type_size;
+    if (sch != KMN && sch != MKN && sch != NKM) {
+        printf("unknown schedule\n");
+        exit(1);
+    }
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    cake_hip_blk_dims_t d;
+    die_on(cake_hip_init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &cx, &d), "init_block_dims_conv");
+    if (sch != KMN) {   // the reference sizes m_c, k_c, n_c and fills in nothing else for these (cake_conv.cpp:404-416)
+        cake_hip_blk_dims_t only = cake_hip_blk_dims_t();
+        only.m_c = d.m_c; only.k_c = d.k_c; only.n_c = d.n_c;
+        d = only;
+    }
+    d.sch = sch;
+    memcpy(x, &d, sizeof d);
+}
+
+cache_dims_t* get_cache_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s,
+                                  int p, cake_cntx_t* cake_cntx, enum sched sch, char* argv[], float density,
+                                  float type_size)
+{
+    blk_dims_t x;
+    init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &x, cake_cntx, KMN, argv, density, type_size);
+    cache_dims_t* r = (cache_dims_t*)malloc(sizeof(cache_dims_t));
+    r->m_c = x.m_c; r->k_c = x.k_c; r->n_c = x.n_c; r->sch = sch;
+    return r;
+}
+
 enum sched derive_schedule(int M, int N, int K, int p, int mc_ret, cake_cntx_t* cake_cntx)
 {
     cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
@@ -273,6 +376,7 @@ double pack_A(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cnt
 {
     cake_hip_blk_dims_t d = to_abi(x);
     cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    OnContextOf on(cake_cntx);
     const double t0 = wall_seconds();
     die_on(cake_hip_pack_a(A, A_p, M, K, p, &d, &cx, sch, NULL, NULL), "pack_A");
     die_on(cake_hip_synchronize(), "pack_A");
@@ -283,6 +387,7 @@ void pack_B(float* B, float* B_p, int K, int N, int p, blk_dims_t* x, cake_cntx_
 {
     cake_hip_blk_dims_t d = to_abi(x);
     cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    OnContextOf on(cake_cntx);
     die_on(cake_hip_pack_b(B, B_p, K, N, p, &d, &cx, sch, NULL, NULL), "pack_B");
 }
 
@@ -290,6 +395,7 @@ void pack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cntx_
 {
     cake_hip_blk_dims_t d = to_abi(x);
     cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    OnContextOf on(cake_cntx);
     die_on(cake_hip_pack_c(C, C_p, M, N, p, &d, &cx, sch, NULL, NULL), "pack_C");
 }
 
@@ -297,6 +403,7 @@ void unpack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cnt
 {
     cake_hip_blk_dims_t d = to_abi(x);
     cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    OnContextOf on(cake_cntx);
     die_on(cake_hip_unpack_c(C, C_p, M, N, p, &d, &cx, sch, NULL, NULL), "unpack_C");
 }
 
@@ -305,7 +412,8 @@ void unpack_C(float* C, float* C_p, int M, int N, int p, blk_dims_t* x, cake_cnt
 double cake_sgemv(float* A, float* B, float* C, int M, int K, int p, cake_cntx_t* cake_cntx,
                   char* argv[], bool packedA, float alpha, float beta, enum sched sch)
 {
-    (void)p; (void)cake_cntx; (void)argv; (void)packedA; (void)alpha; (void)beta; (void)sch;
+    (void)p; (void)argv; (void)packedA; (void)alpha; (void)beta; (void)sch;
+    OnContextOf on(cake_cntx);
     const double t0 = wall_seconds();
     double dev_s = 0;
     // column-major A, accumulate into y: examples/cake_gemv.cpp:89-140
@@ -333,17 +441,37 @@ float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
 
 // ---- direct convolution --------------------------------------------------------------
 
+// pack_filters (examples/cake_conv.cpp:536-610) is written for 3 x 3 filters: K = Cin * 9
+double pack_filters(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx)
+{
+    cake_hip_blk_dims_t d = to_abi(x);
+    cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+    OnContextOf on(cake_cntx);
+    const double t0 = wall_seconds();
+    die_on(cake_hip_pack_filters(A, A_p, M, K / 9, 9, p, &d, &cx, NULL, NULL), "pack_filters");
+    die_on(cake_hip_synchronize(), "pack_filters");
+    return wall_seconds() - t0;
+}
+
 double cake_sconv(float* A, float* B, float* C, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
                   int Cin, int Cout, int s, int p, cake_cntx_t* cake_cntx, char* argv[], bool packedA,
                   enum sched sch)
 {
-    (void)p; (void)cake_cntx; (void)argv; (void)sch;   // always K-first in the reference (cake_conv.cpp:790)
-    if (packedA) {
-        printf("cake_sconv: filters packed by pack_filters are not supported; pass them as [Cout][Cin][Hf][Wf]\n");
-        exit(1);
-    }
+    (void)sch;   // always K-first in the reference (cake_conv.cpp:790)
+    if (cake_cntx == NULL) cake_cntx = cake_query_cntx();  // leaked, as in the reference (:770-772)
+    OnContextOf on(cake_cntx);
     const double t0 = wall_seconds();
-    die_on(cake_hip_sconv(A, B, C, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, NULL, NULL), "cake_sconv");
+    if (packedA) {
+        // A was written by pack_filters for the blocks the reference derives here (:791-799)
+        blk_dims_t x;
+        init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &x, cake_cntx, KMN, argv, 0, 4);
+        cake_hip_blk_dims_t d = to_abi(&x);
+        cake_hip_cpu_cntx_t cx = to_abi(cake_cntx);
+        die_on(cake_hip_sconv_packed(A, B, C, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &d, &cx, NULL, NULL),
+               "cake_sconv");
+    } else {
+        die_on(cake_hip_sconv(A, B, C, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, NULL, NULL), "cake_sconv");
+    }
     return wall_seconds() - t0;
 }
 

@@ -217,6 +217,9 @@ hipError_t launch_build_index_tables(int which, const PackGeom& g, int4* row_tab
 // dst_packed[offset(r,c)] = (r,c) inside the matrix ? src[r*ld + c] : 0   over the padded extent.
 // fast / rows_fast: the short axis of a micro-panel (A: mr rows, rows_fast; B and C: nr columns),
 // which the packed layout stores fastest; 0 selects the element-wise kernel.
+// filters between [Cout][Cin][taps] and the reference's pack_filters layout (g.d from init_block_dims_conv, g.K = Cin)
+hipError_t launch_filter_layout(const float* src, float* dst, const PackGeom& g, int Cout, int Cin, int taps,
+                                int to_packed, hipStream_t stream);
 hipError_t launch_pack(const float* src, float* dst_packed, int rows, int cols, int ld,
                        int rows_padded, int cols_padded, IndexTables tab, int fast, bool rows_fast,
                        hipStream_t stream);

@@ -100,6 +100,40 @@ hipError_t launch_fill_value(float* dst, size_t n, float value, hipStream_t stre
 }
 
 // ---------------------------------------------------------------------------
+// Filters in the layout of the reference's pack_filters (examples/cake_conv.cpp:536-610) and
+// back.  A thread owns one (padded row, channel) pair and walks its taps: on the plain side those
+// are `taps` consecutive floats, on the packed side they lie m_r * k_c floats apart.  Filters are a
+// few megabytes at most, so this is a plain index-map kernel.
+//   to_packed != 0: packed[off(r, c, t)] = r < Cout ? plain[r][c][t] : 0   for r < padded rows
+//   to_packed == 0: plain[r][c][t] = packed[off(r, c, t)]                  for r < Cout
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) filter_layout_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                            PackGeom g, int Cout, int Cin, int taps, int rows,
+                                                            int to_packed)
+{
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)rows * Cin) return;
+    const int r = (int)(idx / Cin), c = (int)(idx - (size_t)r * Cin);
+    const size_t plain = ((size_t)r * Cin + c) * taps;
+    for (int t = 0; t < taps; ++t) {
+        const int64_t off = packed_filter_offset(g, r, c, t, taps);
+        if (to_packed) dst[off] = r < Cout ? src[plain + t] : 0.f;
+        else dst[plain + t] = src[off];
+    }
+}
+
+hipError_t launch_filter_layout(const float* src, float* dst, const PackGeom& g, int Cout, int Cin, int taps,
+                                int to_packed, hipStream_t stream)
+{
+    const int rows = to_packed ? g.d.M_padded : Cout;
+    const size_t threads = (size_t)rows * Cin;
+    if (threads == 0) return hipSuccess;
+    hipLaunchKernelGGL(filter_layout_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, src, dst, g,
+                       Cout, Cin, taps, rows, to_packed);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // zero padding of image planes: the convolution's gather then needs no edge
 // tests.  Output rows are `pitch` floats apart (a multiple of 4, >= Win + 2 pad),
 // so every thread writes one aligned float4; reads run along image rows.  One

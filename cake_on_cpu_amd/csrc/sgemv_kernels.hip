@@ -354,7 +354,9 @@ static int colmajor_slices(int M, int K, int cus)
 
 size_t sgemv_colmajor_scratch_floats(int M, int K, int cus)
 {
-    return (size_t)colmajor_slices(M, K, cus) * (size_t)M;
+    // a single slice writes y itself and touches no workspace
+    const int slices = colmajor_slices(M, K, cus);
+    return slices > 1 ? (size_t)slices * (size_t)M : 0;
 }
 
 // grid = (m blocks, k slices).  VEC: each wave covers all 256 columns of the

@@ -37,7 +37,7 @@ typedef struct blk_dims_t {
 } blk_dims_t;
 
 typedef struct cake_cntx_t {
-    void* blis_cntx;      // unused here; kept so the layout matches
+    void* blis_cntx;      // names the device context this cntx works on (set on first use; zero it in a cntx you build yourself)
     double alpha_n;
     double peak_dram_bw;  // bytes/s of the device the library runs on
     double peak_flops;    // fp32 matrix FLOP/s of that device
@@ -71,6 +71,17 @@ cache_dims_t* get_cache_dims(int M, int N, int K, int p, cake_cntx_t* cake_cntx,
 void init_block_dims(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx,
                      enum sched sch, char* argv[], float type_size = 4,
                      int mcu = 0, int kcu = 0, int ncu = 0);
+
+// Block sizing of the reference's 2-D grid of cores (include/tiling.h:43-51,
+// src/block_sizing.cpp:596-841): host arithmetic, as in the reference.  grid_dims_2d returns pn,
+// the factor of p closest to sqrt(p N / M); the reference's generated factor table is replaced by
+// a divisibility test, so `ncores` is not read.
+int grid_dims_2d(int M, int N, int K, int p, int ncores);
+void init_block_dims_2d(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx,
+                        enum sched sch, char* argv[], float type_size = 4,
+                        int mcu = 0, int kcu = 0, int ncu = 0);
+void init_block_dims_2d_small(int M, int N, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx,
+                              enum sched sch, char* argv[], float type_size = 4);
 
 // ---- GEMM (reference: include/cake.h:12-14,36-47) ---------------------------
 
@@ -128,11 +139,22 @@ float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
 // Direct convolution of one CHW image (reference: examples/cake_conv.cpp:5-8,765-848):
 // C[Cout][Hout][Wout] += A[Cout][Cin][Hf][Wf] * B[Cin][Hin][Win], no padding,
 // Hout = (Hin - Hf) / s + 1 and Wout = (Win - Wf) / s + 1.  On the GPU the windows are gathered
-// inside the product, so there is no column matrix either.  packedA (filters from the
-// reference's file-local pack_filters) is not offered: the call prints a message and exits.
+// inside the product, so there is no column matrix either.  With packedA the filters are in the
+// layout of pack_filters for the blocks of init_block_dims_conv (same Cout, Cin, p and cntx), as in
+// the reference (:791-799); they are brought back to [Cout][Cin][Hf][Wf] on the device first.
 double cake_sconv(float* A, float* B, float* C, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
                   int Cin, int Cout, int s, int p, cake_cntx_t* cake_cntx, char* argv[] = NULL,
                   bool packedA = 0, enum sched sch = NA);
+// examples/cake_conv.cpp:10-18,262-420: blocks of that convolution (K-first only), and
+// examples/cake_conv.cpp:536-610: 3 x 3 filters, A[M = Cout][K = Cin * 9], into those blocks;
+// A_p holds x->M_padded * K floats.  Returns seconds.
+cache_dims_t* get_cache_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout,
+                                  int s, int p, cake_cntx_t* cake_cntx, enum sched sch, char* argv[],
+                                  float density = 0, float type_size = 4);
+void init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s, int p,
+                          blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch, char* argv[],
+                          float density = 0, float type_size = 4);
+double pack_filters(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx);
 void conv_gemm_checker(float* conv, float* gemm, int M, int N);    // cake_conv.cpp:1216
 
 // ---- test helpers (reference: include/util.h) -------------------------------

@@ -128,6 +128,32 @@ int cake_hip_device_info(cake_hip_device_t* out);
 const char* cake_hip_strerror(int status);
 const char* cake_hip_last_error(void);
 
+/* ---- contexts ------------------------------------------------------------ */
+/* A context owns what a compute call needs besides its operands: the workspaces (split-K and
+ * streaming slices, the convolution's column matrix or staged input, staging copies of host
+ * operands, pinned transfer buffers), its timing events and a stream of its own.  The library has
+ * one default context, which cake_hip_init sets up and every entry point uses unless the calling
+ * thread has made another one current.  Calls on one context take turns (they share its
+ * workspaces); calls on different contexts hold different locks and, given different streams and
+ * device operands, run side by side on the device.  This is the device-side state the reference
+ * keeps per cake_cntx_t in its blis_cntx field (include/common.h:138-151); the C++ layer hangs a
+ * context off that field.
+ *
+ * cake_hip_ctx_create needs an initialised library (it calls cake_hip_init(0) when none is) and
+ * makes a context for the device of the default one, with a non-blocking stream of its own.
+ * cake_hip_ctx_set_current(ctx) makes it the calling thread's context (NULL: back to the default);
+ * from then on a NULL `stream` argument means the context's own stream (cake_hip_ctx_stream), where
+ * on the default context it means the HIP null stream.  cake_hip_ctx_destroy waits for the device
+ * and frees the context's device memory, events and stream; a thread that still has it current
+ * gets CAKE_HIP_ERR_ARG from its next call.  cake_hip_sgemm_noalloc on any context uses the
+ * device's one scratch array. */
+typedef void* cake_hip_ctx_t;
+int cake_hip_ctx_create(cake_hip_ctx_t* out);
+int cake_hip_ctx_destroy(cake_hip_ctx_t ctx);
+int cake_hip_ctx_set_current(cake_hip_ctx_t ctx);
+cake_hip_ctx_t cake_hip_ctx_get_current(void);
+void* cake_hip_ctx_stream(cake_hip_ctx_t ctx);
+
 /* ---- device memory for callers without a HIP runtime of their own ------- */
 int cake_hip_malloc(void** ptr, size_t bytes);
 int cake_hip_free(void* ptr);
@@ -155,6 +181,24 @@ int cake_hip_init_block_dims(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cn
  * reuse order for a CB block of side p*mc.  Returns KMN, MKN or NKM. */
 int cake_hip_derive_schedule(int M, int N, int K, int p, int mc, const cake_hip_cpu_cntx_t* cntx);
 
+/* Block sizing of the reference's 2-D grid of cores: grid_dims_2d, init_block_dims_2d and
+ * init_block_dims_2d_small (include/tiling.h:43-51, src/block_sizing.cpp:596-841).  Host integer
+ * arithmetic; no device is needed.  grid_dims_2d returns pn, the number of cores along N (pm = p / pn):
+ * the factor of p closest to sqrt(p N / M).  The reference reads the factors of p from a table
+ * generated at build time for the machine's core count (python/grid_gen.py); here divisibility is
+ * tested directly and `ncores` is not used.  Fields of blk_dims_t that the reference leaves
+ * unset are zero. */
+int cake_hip_grid_dims_2d(int M, int N, int K, int p, int ncores);
+int cake_hip_init_block_dims_2d(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx, int sched,
+                                float type_size, int mcu, int kcu, int ncu, cake_hip_blk_dims_t* out);
+int cake_hip_init_block_dims_2d_small(int M, int N, int K, int p, cake_hip_cpu_cntx_t* cntx, int sched,
+                                      float type_size, cake_hip_blk_dims_t* out);
+/* Blocks of the direct convolution: get_cache_dims_conv + init_block_dims_conv
+ * (examples/cake_conv.cpp:262-420): m_c output channels per core, k_c input channels, n_c rows of
+ * the output image; always K-first.  cntx->alpha_n is read (cake_query_cntx sets 1.0). */
+int cake_hip_init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout,
+                                  int s, int p, cake_hip_cpu_cntx_t* cntx, cake_hip_blk_dims_t* out);
+
 /* ---- GEMM ---------------------------------------------------------------- */
 /* C[MxN] = A[MxK] . B[KxN], all row-major fp32: cake_sgemm
  * (src/cake_sgemm.cpp:9-175).  accumulate != 0 starts from the existing C
@@ -165,10 +209,11 @@ int cake_hip_sgemm(const float* A, const float* B, float* C, int M, int N, int K
 
 /* cake_hip_sgemm for callers that must not allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
- * The same kernels as cake_hip_sgemm run on the planner's own choice of tile; the partial sums
- * that split-K, tail-split and streaming products and the matrix-vector kernels need go into a
- * 64 MiB array that is part of the library's device image instead of a buffer that grows, and the
- * call makes no hipMalloc or hipFree.  A, B and C must be device memory; cake_hip_init must have run
+ * The same kernels as cake_hip_sgemm run on the planner's own choice of tile, with the same slice
+ * counts, so the results are the same bits; the partial sums that split-K, tail-split and
+ * streaming products and the matrix-vector kernels need, and the few columns of B that a tall
+ * product turns into rows first, go into a 64 MiB array that is part of the library's device image
+ * instead of buffers that grow, and the call makes no hipMalloc or hipFree.  A, B and C must be device memory; cake_hip_init must have run
  * (it looks up the array's address on its device); a product whose partial sums would not fit
  * returns CAKE_HIP_ERR_RANGE and touches nothing.  Every call on a device uses that device's one
  * array: calls that overlap on one device (different streams) race, calls on one stream do not. */
@@ -271,6 +316,17 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
                            int stride, int pad, int out_nchw, void* workspace,
                            void* stream, double* seconds);
 
+/* Which of the routes above the calling thread's last convolution call took (cake_hip_conv2d,
+ * cake_hip_conv2d_im2col, cake_hip_sconv); CAKE_HIP_CONV_NONE when it failed its argument checks. */
+enum {
+    CAKE_HIP_CONV_NONE = 0,
+    CAKE_HIP_CONV_SHORTK_BATCH = 1, /* 1 x 1 layer as a batch of plain products on the short-K kernel */
+    CAKE_HIP_CONV_PATCH = 2,        /* input read where it lies, a patch per channel block in LDS     */
+    CAKE_HIP_CONV_GATHER = 3,       /* columns gathered inside the product (staged copy where needed) */
+    CAKE_HIP_CONV_TWO_STEP = 4      /* column matrix written out, then the product                    */
+};
+int cake_hip_last_conv_route(void);
+
 /* out[Cout][Hout][Wout] += filters[Cout][Cin][Hf][Wf] * in[Cin][Hin][Win]: the direct convolution
  * of one CHW image without padding, cake_sconv (examples/cake_conv.cpp:5-8,765-848), whose
  * micro-kernel starts from the values out already holds (:36-47).  Runs as cake_hip_conv2d does
@@ -278,6 +334,24 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
  * (Hin - Hf) / stride + 1 and (Win - Wf) / stride + 1. */
 int cake_hip_sconv(const float* filters, const float* in, float* out, int Wf, int Hf, int Win, int Hin,
                    int Wout, int Hout, int Cin, int Cout, int stride, void* stream, double* seconds);
+
+/* Filters [Cout][Cin][taps] (taps = Hf * Wf) into the layout of the reference's pack_filters
+ * (examples/cake_conv.cpp:430-454,536-610; it is written for 3 x 3 filters, taps = 9): K-first
+ * blocks over output channels and input channels, and inside an m_r panel
+ * [tap][channel][m_r]; rows past Cout are zero.  dims from cake_hip_init_block_dims_conv for the
+ * same Cout, Cin, p and cntx.  The size in bytes is M_padded * Cin * taps * 4. */
+size_t cake_hip_packed_filters_size(int Cout, int Cin, int taps, int p, const cake_hip_blk_dims_t* dims,
+                                    const cake_hip_cpu_cntx_t* cntx);
+int cake_hip_pack_filters(const float* filters, float* filters_p, int Cout, int Cin, int taps, int p,
+                          const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx, void* stream,
+                          double* seconds);
+/* cake_hip_sconv with the filters in that layout: cake_sconv with packedA = 1
+ * (examples/cake_conv.cpp:797-799).  The filters are copied back to [Cout][Cin][Hf][Wf] in a
+ * library workspace first (one small kernel). */
+int cake_hip_sconv_packed(const float* filters_p, const float* in, float* out, int Wf, int Hf, int Win, int Hin,
+                          int Wout, int Hout, int Cin, int Cout, int stride, int p,
+                          const cake_hip_blk_dims_t* dims, const cake_hip_cpu_cntx_t* cntx, void* stream,
+                          double* seconds);
 
 /* ---- transpose and the linear layer ---------------------------------------- */
 /* dst[c][r] = src[r][c] for a rows x cols row-major matrix; dst is cols x rows.

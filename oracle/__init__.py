@@ -102,6 +102,8 @@ def lib():
         "orc_max_rel_err": (C.c_double, [_fp, _dp, _dp, C.c_size_t]),
         "orc_gemv_f64": (None, [_fp, _fp, i, i, i, _dp, _dp]),
         "orc_conv_naive_f64": (None, [_fp, _fp, _dp, _dp] + [i] * 11),
+        "orc_init_block_dims_conv": (None, [i] * 10 + [bp, cp]),
+        "orc_pack_filters": (None, [_fp, _fp, i, i, i, i, bp, cp]),
         "orc_sizeof_blk_dims": (i, []),
     }
     for name, (res, args) in sig.items():
@@ -196,6 +198,22 @@ def pack_C(Cm, p, x, cx, sch) -> np.ndarray:
 def unpack_C(Cp, M, N, p, x, cx, sch, into=None) -> np.ndarray:
     out = np.zeros((M, N), dtype=np.float32) if into is None else into
     lib().orc_unpack_C(_f(out), _f(Cp), M, N, p, C.byref(x), C.byref(cx), sch)
+    return out
+
+
+def init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cx: Cntx) -> BlkDims:
+    """Blocks of the reference's direct convolution (examples/cake_conv.cpp:262-425), K-first."""
+    x = BlkDims()
+    lib().orc_init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, C.byref(x), C.byref(cx))
+    return x
+
+
+def pack_filters(F, Cin, taps, p, x, cx) -> np.ndarray:
+    """F[Cout][Cin*taps] in the layout of the reference's pack_filters (examples/cake_conv.cpp:536-610)."""
+    Cout = F.shape[0]
+    assert F.size == Cout * Cin * taps
+    out = np.full(x.M_padded * Cin * taps, np.nan, dtype=np.float32)
+    lib().orc_pack_filters(_f(np.ascontiguousarray(F.reshape(Cout, -1))), _f(out), Cout, Cin, taps, p, C.byref(x), C.byref(cx))
     return out
 
 

@@ -33,6 +33,10 @@
  *   The outputs of the compiled reference parts on seeded inputs are also
  *   committed (tests/golden/reference_vectors.npz), so the packing, kernel, gemv
  *   and im_2_col comparisons run where the reference sources are absent too.
+ *   orc_init_block_dims_conv / orc_pack_filters
+ *       - bit-exact against the reference's init_block_dims_conv and pack_filters
+ *         (oracle/_ref) and their committed outputs, a hand-computed block table,
+ *         and the permutation property (every filter value lands exactly once).
  *   The linear layer (oracle/__init__.py, a caller of orc_cake_sgemm) is pinned
  *   against torch.nn.functional.linear and its autograd in fp64.
  *   No function here is "parity unpinned".
@@ -968,6 +972,91 @@ void orc_conv_naive_f64(const float *in, const float *wt, double *out, double *S
                     out[o] = acc;
                     if (S) S[o] = s;
                 }
+}
+
+/* ------------------------------------------------------------------------ */
+/* Blocks of the direct convolution and the packed filters of cake_sconv.    */
+/*   get_cache_dims_conv   examples/cake_conv.cpp:262-329                     */
+/*   init_block_dims_conv  examples/cake_conv.cpp:333-425 (K-first case)      */
+/*   pack_filters          examples/cake_conv.cpp:536-610                     */
+/*   pack_ob_A_single_buf_conv  examples/cake_conv.cpp:430-454                */
+/* Pinned bit for bit against those functions compiled from the reference    */
+/* (oracle/_ref) and their committed outputs (tests/golden), and by a        */
+/* hand-computed block table.                                                 */
+/* ------------------------------------------------------------------------ */
+void orc_init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout,
+                              int s, int p, orc_blk_dims *x, const orc_cntx *cx)
+{
+    (void)Hin; (void)s;
+    const int mr = cx->mr;
+    memset(x, 0, sizeof *x);
+    /* output channels per core: an even share, whole m_r panels */
+    int share = (int)ceil((double)Cout / p);
+    share -= share % mr;
+    int mc = share;
+    if (Cout < p * mr) mc = mr;
+    else if (Cout < p * share) {
+        int a = Cout / p;
+        mc = a < mr ? mr : a + (mr - a % mr);
+    }
+    /* rows of the output image per block, then the channels that still fit the L2 */
+    int rows = (int)floor((cx->alpha_n * p * mc) / Wout);
+    if (rows == 0) rows = 1;
+    int ck = (int)ceil((((double)cx->L2) / 4.0 - (double)rows * Wout * mc) /
+                       ((double)mc * Wf * Hf + (double)rows * Win));
+    if (ck > Cin) ck = Cin;
+    else if (ck < 0) ck = 128;
+    if (ck == 0) ck = 1;   /* the reference would go on to divide by it */
+    x->m_c = mc; x->k_c = ck; x->n_c = rows; x->sch = ORC_KMN;
+
+    const int block_rows = p * mc;
+    const int left = Cout % block_rows;
+    x->m_pad = left != 0;
+    x->k_pad = Cin % ck != 0;
+    x->n_pad = Hout % rows != 0;
+    x->mr_rem = ceil_ratio(left, mr);
+    int panels = ceil_ratio(x->mr_rem, p);
+    x->p_l = panels ? ceil_ratio(x->mr_rem, panels) : 0;
+    x->m_c1 = panels * mr;
+    x->m_c1_last_core = (panels - (x->p_l * panels - x->mr_rem)) * mr;
+    x->k_c1 = Cin % ck;
+    x->n_c1 = Hout % rows;
+    x->Mb = Cout / block_rows + x->m_pad;
+    x->Kb = Cin / ck + x->k_pad;
+    x->Nb = Hout / rows + x->n_pad;
+    x->M_padded = mr * x->mr_rem + (Cout / block_rows) * block_rows;
+    x->N_padded = (Hout - Hout % rows) + x->n_c1;
+}
+
+/* F[Cout][Cin][taps] -> K-first blocks whose m_r panels hold [tap][channel][m_r]. */
+void orc_pack_filters(const float *F, float *Fp, int Cout, int Cin, int taps, int p,
+                      const orc_blk_dims *x, const orc_cntx *cx)
+{
+    const int mr = cx->mr;
+    const size_t K = (size_t)Cin * taps;
+    size_t off = 0;
+    for (int mb = 0; mb < x->Mb; ++mb) {
+        int last = (mb == x->Mb - 1) && x->m_pad;
+        split_t sp = split_of(last, p, x->p_l, x->m_c, mr * x->mr_rem);
+        int slice = last ? x->m_c1 : x->m_c;
+        for (int kb = 0; kb < x->Kb; ++kb) {
+            int kc = ((kb == x->Kb - 1) && x->k_pad) ? x->k_c1 : x->k_c;
+            for (int core = 0; core < sp.used; ++core) {
+                int rows = last ? (core == x->p_l - 1 ? x->m_c1_last_core : x->m_c1) : x->m_c;
+                size_t row0 = (size_t)mb * p * x->m_c + (size_t)core * slice;
+                float *dst = Fp + off + (size_t)core * slice * kc * taps;
+                for (int panel = 0; panel < rows; panel += mr)
+                    for (int t = 0; t < taps; ++t)
+                        for (int c = 0; c < kc; ++c)
+                            for (int j = 0; j < mr; ++j) {
+                                size_t r = row0 + panel + j;
+                                *dst++ = r < (size_t)Cout
+                                             ? F[r * K + ((size_t)kb * x->k_c + c) * taps + t] : 0.f;
+                            }
+            }
+            off += (size_t)sp.span * kc * taps;
+        }
+    }
 }
 
 int orc_sizeof_blk_dims(void) { return (int)sizeof(orc_blk_dims); }

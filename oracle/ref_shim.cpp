@@ -18,6 +18,11 @@ void schedule_mvm(float* A_p, float* B_p, float* C_p, int M, int K, int p,
 float* im_2_col(float* In, int Wf, int Hf, int Win, int Hin, int Wout, int Hout,
                 int Cin, int Cout, int s);
 
+void init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout, int s, int p,
+                          blk_dims_t* x, cake_cntx_t* cake_cntx, enum sched sch, char* argv[], float density,
+                          float type_size);
+double pack_filters(float* A, float* A_p, int M, int K, int p, blk_dims_t* x, cake_cntx_t* cake_cntx);
+
 #define EXPORT extern "C" __attribute__((visibility("default")))
 
 namespace {
@@ -115,4 +120,29 @@ EXPORT void ref_im_2_col(float* In, float* out, int Wf, int Hf, int Win, int Hin
     float* m = im_2_col(In, Wf, Hf, Win, Hin, Wout, Hout, Cin, 1, 1);
     memcpy(out, m, sizeof(float) * (size_t)Cin * Wf * Hf * Wout * Hout);
     free(m);
+}
+
+// 26 ints in blk_dims_t field order out of the reference's struct (fields the reference leaves
+// unset are zeroed first, so that the comparison is defined)
+EXPORT void ref_init_block_dims_conv(int Wf, int Hf, int Win, int Hin, int Wout, int Hout, int Cin, int Cout,
+                                     int s, int p, int mr, int nr, int L2, double alpha_n, int* dims_out)
+{
+    blk_dims_t x;
+    memset(&x, 0, sizeof x);
+    cake_cntx_t c = cntx_from(mr, nr);
+    c.L2 = L2;
+    c.alpha_n = alpha_n;
+    init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &x, &c, KMN, NULL, 0, 4);
+    const int* f = reinterpret_cast<const int*>(&x);
+    for (int i = 0; i < 25; ++i) dims_out[i] = f[i];
+    dims_out[25] = (int)x.sch;
+}
+
+// 3 x 3 filters only: the reference's pack_filters has Wf = Hf = 3 written into it
+EXPORT void ref_pack_filters(float* F, float* F_p, int Cout, int K, int p, const int* dims, int mr, int nr)
+{
+    blk_dims_t x = dims_from(dims);
+    cake_cntx_t c = cntx_from(mr, nr);
+    omp_set_num_threads(p);
+    pack_filters(F, F_p, Cout, K, p, &x, &c);
 }

@@ -5,6 +5,8 @@
 // case and "ALL PASS" at the end; exit status 0 only if every case passed.
 #include <math.h>
 
+#include <thread>
+
 #include "cake.h"
 
 static int failures = 0;
@@ -150,6 +152,90 @@ static void sconv_case(cake_cntx_t* cntx, int Cin, int Cout, int Hin, int Win, i
     free(F); free(In); free(Out); free(Bm); free(C);
 }
 
+// cake_sconv with packedA: the reference's sequence (examples/cake_conv.cpp:791-805) -- blocks from
+// init_block_dims_conv, a buffer of cake_sgemm_packed_A_size bytes, pack_filters, then the call.
+static void packed_sconv_case(cake_cntx_t* cntx, int Cin, int Cout, int Hin, int Win)
+{
+    const int Hf = 3, Wf = 3, Hout = Hin - 2, Wout = Win - 2, p = 4, s = 1;
+    const int M = Cout, K = Cin * 9, N = Hout * Wout;
+    float* F = (float*)malloc(sizeof(float) * M * K);
+    float* In = (float*)malloc(sizeof(float) * Cin * Hin * Win);
+    rand_init(F, M, K);
+    rand_init(In, Cin, Hin * Win);
+    float* plain = (float*)calloc((size_t)M * N, sizeof(float));
+    float* packed = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_sconv(F, In, plain, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cntx);
+    blk_dims_t x;
+    init_block_dims_conv(Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, &x, cntx, KMN, NULL);
+    const size_t bytes = cake_sgemm_packed_A_size(Cout, K, p, &x, cntx, KMN);
+    float* F_p = (float*)malloc(bytes);
+    pack_filters(F, F_p, Cout, K, p, &x, cntx);
+    // the layout, from its definition: the first m_r panel of the first block holds [tap][channel][m_r]
+    bool layout = bytes == sizeof(float) * (size_t)x.M_padded * K;
+    const int kc = x.Kb == 1 && x.k_pad ? x.k_c1 : x.k_c;
+    for (int t = 0; t < 9 && layout; ++t)
+        for (int c = 0; c < kc; ++c)
+            for (int j = 0; j < cntx->mr; ++j) {
+                const float want = j < Cout ? F[(size_t)j * K + c * 9 + t] : 0.f;
+                if (F_p[((size_t)t * kc + c) * cntx->mr + j] != want) layout = false;
+            }
+    cake_sconv(F_p, In, packed, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, s, p, cntx, NULL, 1);
+    char what[128];
+    snprintf(what, sizeof what, "pack_filters layout, %d->%d channels", Cin, Cout);
+    report(what, layout);
+    snprintf(what, sizeof what, "cake_sconv packedA=1 equals packedA=0, %d->%d on %dx%d", Cin, Cout, Hin, Win);
+    report(what, memcmp(plain, packed, sizeof(float) * M * N) == 0);
+    free(F); free(In); free(plain); free(packed); free(F_p);
+}
+
+// The 2-D block sizing is host arithmetic; 3000^3 on 8 cores with L1 = 32 KiB, L2 = 1 MiB, worked
+// out by hand from src/block_sizing.cpp:639-779: a 4 x 2 grid of 354 x 368 blocks, k_c = 368.
+static void dims_2d_case(cake_cntx_t* cntx)
+{
+    cake_cntx_t c = *cntx;
+    c.mr = 6; c.nr = 16; c.L1 = 32 << 10; c.L2 = 1 << 20; c.ncores = 8;
+    report("grid_dims_2d", grid_dims_2d(3000, 3000, 3000, 8, 8) == 2 && grid_dims_2d(1000, 1600, 1, 10, 10) == 5);
+    blk_dims_t x;
+    init_block_dims_2d(3000, 3000, 3000, 8, &x, &c, KMN, NULL);
+    report("init_block_dims_2d", x.pm == 4 && x.pn == 2 && x.m_c == 354 && x.n_c == 368 && x.k_c == 368 && x.Mb == 3 &&
+                                     x.Nb == 5 && x.Kb == 9 && x.m_c1 == 42 && x.n_c1 == 32 && x.N_padded == 3008);
+    init_block_dims_2d_small(100, 200, 500, 8, &x, &c, KMN, NULL);
+    report("init_block_dims_2d_small", x.pm == 2 && x.pn == 4 && x.m_c == 54 && x.n_c == 64 && x.k_c == 54 &&
+                                           x.m_c1 == 48 && x.n_c1 == 16 && x.Kb == 10);
+}
+
+// Two host threads, each with a cntx of its own: each cntx works on a device context of its own
+// (its blis_cntx field names it), so the calls do not take turns; the results are those of the same
+// calls made one after the other.
+static void two_cntx_case()
+{
+    const int M = 700, K = 900, N = 500, p = 4;
+    float* A = (float*)malloc(sizeof(float) * M * K);
+    float* B = (float*)malloc(sizeof(float) * K * N);
+    rand_init(A, M, K);
+    rand_init(B, K, N);
+    float* alone = (float*)calloc((size_t)M * N, sizeof(float));
+    cake_cntx_t* c0 = cake_query_cntx();
+    cake_sgemm(A, B, alone, M, N, K, p, c0);
+    cake_cntx_t* cx[2] = {cake_query_cntx(), cake_query_cntx()};
+    float* C[2] = {(float*)calloc((size_t)M * N, sizeof(float)), (float*)calloc((size_t)M * N, sizeof(float))};
+    bool same[2] = {true, true};
+    std::thread t[2];
+    for (int i = 0; i < 2; ++i)
+        t[i] = std::thread([&, i] {
+            for (int rep = 0; rep < 5; ++rep) {
+                cake_sgemm(A, B, C[i], M, N, K, p, cx[i]);
+                if (memcmp(C[i], alone, sizeof(float) * M * N) != 0) same[i] = false;
+            }
+        });
+    for (int i = 0; i < 2; ++i) t[i].join();
+    report("two threads, a cntx each: results of the single calls", same[0] && same[1]);
+    report("each cntx names a device context of its own", cx[0]->blis_cntx && cx[1]->blis_cntx &&
+                                                              cx[0]->blis_cntx != cx[1]->blis_cntx &&
+                                                              c0->blis_cntx != cx[0]->blis_cntx);
+    free(A); free(B); free(alone); free(C[0]); free(C[1]); free(c0); free(cx[0]); free(cx[1]);
+}
+
 // beta with the default schedule: whether C is added to follows the schedule init_block_dims
 // resolves from the caller's cntx and p (src/cake_sgemm.cpp:34-35,114), not the device's tiling.
 static void beta_case(int M, int K, int N, int p, cake_cntx_t* cntx)
@@ -180,6 +266,25 @@ static void beta_case(int M, int K, int N, int p, cake_cntx_t* cntx)
     cake_sgemm_online(A, B, C, M, N, K, p, cntx, NULL, 0, 0, 1, 1, MKN);
     report("cake_sgemm_online beta=1 sch=MKN assigns C", memcmp(C, P, sizeof(float) * M * N) == 0);
     free(A); free(B); free(C0); free(C); free(P);
+}
+
+// K = 0: the sum is empty.  With sch = NA there is nothing to size a block for and the product is
+// K-first, which assigns (C becomes zero whatever beta says); M-first asked for by name keeps C.
+static void empty_k_case(cake_cntx_t* cntx)
+{
+    const int M = 5, N = 7;
+    float A[1] = {0}, B[1] = {0};
+    float C[M * N];
+    for (int i = 0; i < M * N; ++i) C[i] = 3.f;
+    cake_sgemm(A, B, C, M, N, 0, 4, cntx, NULL, 0, 0, 1, 1);
+    bool zero = true;
+    for (int i = 0; i < M * N; ++i) zero = zero && C[i] == 0.f;
+    report("cake_sgemm K=0 beta=1 sch=NA assigns zero", zero);
+    for (int i = 0; i < M * N; ++i) C[i] = 3.f;
+    cake_sgemm(A, B, C, M, N, 0, 4, cntx, NULL, 0, 0, 1, 1, MKN);
+    bool kept = true;
+    for (int i = 0; i < M * N; ++i) kept = kept && C[i] == 3.f;
+    report("cake_sgemm K=0 beta=1 sch=MKN keeps C", kept);
 }
 
 // examples/cake_gemv.cpp main: column-major A, mr = 8, y accumulates
@@ -248,10 +353,15 @@ int main(int argc, char** argv)
         beta_case(1024, 1024, 1024, 8, &fixed);
         beta_case(200, 300, 3000, 4, &fixed);
         beta_case(300, 3000, 300, 4, &fixed);
+        empty_k_case(&fixed);
     }
     conv_case(cntx);
     sconv_case(cntx, 16, 24, 34, 34, 3, 3);
     sconv_case(cntx, 5, 130, 21, 37, 5, 3);
+    packed_sconv_case(cntx, 16, 24, 34, 34);
+    packed_sconv_case(cntx, 40, 100, 21, 37);
+    dims_2d_case(cntx);
+    two_cntx_case();
     gemv_case(cntx, 1024, 777);
     gemv_case(cntx, 37, 5);
     transpose_case(130, 77);

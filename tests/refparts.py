@@ -38,6 +38,10 @@ def lib():
         L.ref_schedule_mvm.argtypes = [_fp, _fp, _fp, i, i, i, _ip, i]
         L.ref_im_2_col.restype = None
         L.ref_im_2_col.argtypes = [_fp, _fp, i, i, i, i, i, i, i]
+        L.ref_init_block_dims_conv.restype = None
+        L.ref_init_block_dims_conv.argtypes = [i] * 13 + [C.c_double, _ip]
+        L.ref_pack_filters.restype = None
+        L.ref_pack_filters.argtypes = [_fp, _fp, i, i, i, _ip, i, i]
         assert L.ref_sizeof_blk_dims() == C.sizeof(oracle.BlkDims)
         _lib = L
     return _lib

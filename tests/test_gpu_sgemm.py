@@ -206,7 +206,10 @@ def test_tall_matrix_times_few_columns(shape):
                                    # one to four tiles per CU: every workgroup has a single tile, surplus ones leave early
                                    (1024, 64, 1024), (2111, 10, 960), (1100, 33, 1500), (960, 7, 1100),
                                    # K up to 24 under very many tiles
-                                   (4096, 16, 8200), (3333, 24, 7777), (8192, 25, 4096)],
+                                   (4096, 16, 8200), (3333, 24, 7777), (8192, 25, 4096),
+                                   # more than 16 tile rows against 12288 columns and more: bands of 4 tile rows,
+                                   # 18 and 19 tile rows (neither a multiple of 4), ragged everything
+                                   (1100, 16, 12300), (1160, 24, 12417)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_short_k_many_tiles(shape):
     """K of at most 64 under at least one 64 x 64 tile per CU: workgroups that walk over tiles with
@@ -375,6 +378,17 @@ def test_empty_and_degenerate():
     out = np.full((4, 3), 7.0, np.float32)
     cake.cake_sgemm(np.zeros((4, 0), np.float32), np.zeros((0, 3), np.float32), out, 4, 3, 0, 1)
     assert not out.any()               # empty sum assigns zero in K-first
+    # an empty sum under the default schedule is K-first as well: beta = 1 still assigns ...
+    out = np.full((4, 3), 7.0, np.float32)
+    cake.cake_sgemm(np.zeros((4, 0), np.float32), np.zeros((0, 3), np.float32), out, 4, 3, 0, 1, None, None,
+                    False, False, 1.0, 1.0)
+    assert not out.any()
+    # ... and only an explicit M-first or N-first schedule keeps the C it starts from
+    for sch in (cake.MKN, cake.NKM):
+        out = np.full((4, 3), 7.0, np.float32)
+        cake.cake_sgemm(np.zeros((4, 0), np.float32), np.zeros((0, 3), np.float32), out, 4, 3, 0, 1, None, None,
+                        False, False, 1.0, 1.0, sch)
+        assert (out == 7.0).all()
     sq = np.zeros((4, 4), np.float32)
     with pytest.raises(cake.CakeHipError):
         cake.cake_sgemm(sq, sq, sq.copy(), -1, 3, 5, 1)

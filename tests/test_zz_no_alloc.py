@@ -23,6 +23,8 @@ CASES = {
     "tail_split": [(1100, 512, 1100), (700, 300, 650)],
     "stream_rows": [(16, 4096, 4096), (9, 2048, 1500)],
     "stream_cols": [(4096, 4096, 24), (3000, 1024, 7)],
+    # up to 16 columns of B that are turned into rows first: the turned copy comes from the same array
+    "stream_cols_turned": [(8200, 4096, 16), (4100, 4096, 9)],
     "single_row": [(1, 5000, 3000), (1, 700, 900)],
     "single_column": [(3000, 9000, 1), (1200, 8200, 1)],
     "no_partial_sums": [(2111, 300, 960), (96, 111, 10)],
@@ -55,8 +57,11 @@ def test_noalloc_equals_cake_hip_sgemm_twice_in_a_row(kind):
             tA, tB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
             want, got = torch.from_numpy(C0).cuda(), torch.from_numpy(C0).cuda()
             _plain(tA, tB, want, M, N, K, cake.NA, acc)
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info()[0]
             _noalloc(tA, tB, got, M, N, K, cake.NA, acc)
             torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
             got_h, want_h = got.cpu().numpy(), want.cpu().numpy()
             assert np.array_equal(got_h, want_h), (kind, call, acc)
             C64, S = oracle.gemm_f64(A, B)
@@ -70,8 +75,10 @@ def test_noalloc_equals_cake_hip_sgemm_twice_in_a_row(kind):
 def test_noalloc_rejects_what_does_not_fit_and_host_memory():
     import torch
     _lib.check(cake.load().cake_hip_init(0), "cake_hip_init")
-    # a single row against 20 M columns: the column-major matrix-vector kernel wants 80 MB of slices
-    M, K, N = 1, 4, 20_000_000
+    # 640 x 16384 x 4096 runs in 8 K slices of 640 x 4096 floats: 80 MiB of partial sums
+    M, K, N = 640, 16384, 4096
+    pl = cake.plan(M, N, K)
+    assert pl.split_k * M * N * 4 > 64 << 20, (pl.split_k, "the shape no longer needs more than the array holds")
     tA = torch.zeros((M, K), dtype=torch.float32, device="cuda")
     tB = torch.zeros((K, N), dtype=torch.float32, device="cuda")
     tC = torch.full((M, N), 7.0, dtype=torch.float32, device="cuda")
