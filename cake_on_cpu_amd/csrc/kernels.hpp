@@ -33,6 +33,7 @@ struct FastDiv {
     unsigned d, m, sh;
     __host__ static FastDiv make(unsigned d)
     {
+        if (d == 0) d = 1;
         unsigned s = 0;
         while ((1ull << s) < d) ++s;
         FastDiv f;
@@ -94,6 +95,9 @@ struct GemmArgs {
     // all images, tiles_n_per_image of them per image.  0 = a single product.
     int tiles_n_per_image;
     size_t b_batch_stride, c_batch_stride;
+    // sgemm_shortk.hip: divisions of the tile walk as multiplications (filled in by its launcher):
+    // by tiles per band, by tile rows of a whole band, by those of the last band, by column tiles per image
+    FastDiv by_band, by_group, by_last_group, by_image_tiles;
 };
 
 // Macro-tile shapes the planner can choose from.

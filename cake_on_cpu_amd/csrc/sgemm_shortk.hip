@@ -18,19 +18,31 @@ namespace cake {
 // 64 x 64 tiles of C, 4 waves of 32 x 32; BK is the longest K it takes
 using TileShortK64 = Tile<64, 64, 64, 32, 32>;
 
+// one stage of each operand and, behind them, 8 rows of staging per wave for the epilogue that overwrites C
 template <class T>
-static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE) * 4; }  // one stage
+static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE + T::WAVES_M * T::WAVES_N * 8 * (T::WN + 4)) * 4; }
 
 // PLAIN: C is overwritten and there is no bias, so the epilogue loads nothing and the next
 // tile's operands stay in flight across it
 // (Non-temporal stores for C were measured and left out: where rows of C are whole cache lines
 // they gained 4-6 % on one device and lost 3 % on another, and where they are not -- a row pitch
 // that is no multiple of 128 bytes -- they cost 35-45 %: 4096 x 4100 x 64 27 -> 39 us.)
+//
+// What a workgroup does between two tiles is a chain that nothing of its own overlaps (the other
+// workgroups of the CU fill the matrix pipe meanwhile), so the chain is kept short:
+//   * a thread's chunk offsets do not depend on the tile: rows of A at and past M fall outside the
+//     buffer's record count, which is set per tile; columns of B at and past N bring in values of
+//     the next row, which only reach columns of the tile that are never stored; chunks at and past
+//     K are out of range from the start.  Placing a tile is scalar work: three divisions by
+//     invariants (multiplications with reciprocals from the host), two base addresses, two
+//     record counts;
+//   * the next tile's operands are waited for right after the tile's MFMAs and before its stores
+//     are issued: loads and stores share one counter of outstanding operations, so a wait placed
+//     after the stores would wait for their round trip to memory as well.
 template <class T, int B_MODE, bool PLAIN>
 __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs g)
 {
     static_assert(B_MODE == LOAD_VEC4, "row-major operands");
-    using L = VecLoader<T>;
     static_assert(T::KSPLIT == 1, "one wave per block of C");
     static_assert(T::WAVES_M * T::WAVES_N * 32 * (T::WN + 4) <= T::B_STAGE, "the epilogue's staging blocks fit B's stage");
     extern __shared__ __align__(16) float smem[];
@@ -55,37 +67,81 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
     const int tiles = first + (tiles_all >> 3) + (xcd < (tiles_all & 7) ? 1 : 0);   // end of this XCD's run
     int t = first + (blockIdx.x >> 3);
     if (t >= tiles) return;                   // before any barrier: the whole workgroup leaves
-    // tile number -> origin of the tile and, for a batch of products, the image's B and C
-    GemmArgs gt = g, gt_next = g;
-    auto place = [&](int tile, GemmArgs& ga, int& m0_, int& n0_) {
-        int tile_m, tile_n;
-        raster_tile(g, tile, tile_m, tile_n);
-        if (g.tiles_n_per_image) {
-            const int b = tile_n / g.tiles_n_per_image;
-            tile_n -= b * g.tiles_n_per_image;
-            ga.B = g.B + (size_t)b * g.b_batch_stride;
-            ga.C = g.C + (size_t)b * g.c_batch_stride;
-        }
-        m0_ = tile_m * T::BM;
-        n0_ = tile_n * T::BN;
-    };
-    int m0, n0;
-    place(t, gt, m0, n0);
 
-    L ld;
+    // per thread, for every tile: where its chunks lie relative to the tile's origin
+    int a_off[T::A_ITERS], b_off[T::B_ITERS];
+#pragma unroll
+    for (int it = 0; it < T::A_ITERS; ++it) {
+        const int c = tid + it * T::THREADS, k = (c % (T::BK / 4)) * 4;
+        a_off[it] = k < g.K ? ((c / (T::BK / 4)) * g.lda + k) * 4 : BUF_OOB;
+    }
+#pragma unroll
+    for (int it = 0; it < T::B_ITERS; ++it) {
+        const int c = tid + it * T::THREADS, k = c / (T::BN / 4);
+        b_off[it] = k < g.K ? (k * g.ldb + (c % (T::BN / 4)) * 4) * 4 : BUF_OOB;
+    }
+    const bool ragged_k = (g.K & 3) != 0;     // then an A chunk can straddle K and is masked when it is stored
+
+    // tile number -> origin of the tile, the operands' base addresses and record counts
+    struct Place {
+        int m0, n0;
+        const float* a;
+        const float* b;
+        float* c;
+        unsigned a_bytes, b_bytes;
+    };
+    auto place = [&](int tile) {
+        // raster_tile with the grouped dimension along M, its divisions by invariants
+        const int band_sz = g.group * g.tiles_n;
+        const int band = (int)g.by_band.div((unsigned)tile), rem = tile - band * band_sz;
+        const int row0 = band * g.group;
+        const bool whole_band = g.tiles_m - row0 >= g.group;
+        const int gsz = whole_band ? g.group : g.tiles_m - row0;
+        int tile_n = (int)(whole_band ? g.by_group.div((unsigned)rem) : g.by_last_group.div((unsigned)rem));
+        const int tile_m = row0 + rem - tile_n * gsz;
+        Place p;
+        p.b = g.B;
+        p.c = g.C;
+        if (g.tiles_n_per_image) {
+            const int img = (int)g.by_image_tiles.div((unsigned)tile_n);
+            tile_n -= img * g.tiles_n_per_image;
+            p.b += (size_t)img * g.b_batch_stride;
+            p.c += (size_t)img * g.c_batch_stride;
+        }
+        p.m0 = tile_m * T::BM;
+        p.n0 = tile_n * T::BN;
+        p.a = g.A + (size_t)p.m0 * g.lda;
+        p.b += p.n0;
+        p.a_bytes = records_left(clamp_elems((long long)(g.M - 1 - p.m0) * g.lda + g.K), 0u);
+        p.b_bytes = records_left(clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0), 0u);
+        return p;
+    };
     f32x4 ra[T::A_ITERS], rb[T::B_ITERS];
-    ld.init(gt, m0, n0, tid);
-    ld.load_first_stage(g.K, ra, rb);
-    // A's stage outlives a tile (the epilogue turns C around inside B's stage): a workgroup whose
-    // next tile has the same rows of A -- every time when the walk's stride is a multiple of
-    // tiles_m -- neither loads nor stores them again
+    auto load_a = [&](const Place& p) {
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = buffer_load_f32x4(p.a, a_off[it], p.a_bytes);
+    };
+    auto load_b = [&](const Place& p) {
+#pragma unroll
+        for (int it = 0; it < T::B_ITERS; ++it) rb[it] = buffer_load_f32x4(p.b, b_off[it], p.b_bytes);
+    };
+
+    Place cur = place(t);
+    load_a(cur);
+    load_b(cur);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): from here on the loop waits for loads where it says so
+    GemmArgs gt = g;                      // what the epilogue that reads C sees: C and, for a batch, the image's part of it
+    // A's stage outlives a tile (no epilogue touches it): a workgroup whose next tile has the same
+    // rows of A -- every time when the walk's stride is a multiple of tiles_m -- neither loads nor
+    // stores them again
     bool a_fresh = true;
     for (;;) {
-        __syncthreads();   // every wave is done with the staging reads of the previous tile's epilogue
+        __syncthreads();   // every wave has read the previous tile's last operands (and is done with staging reads inside B's stage)
         if (a_fresh) {     // the same for every thread of the workgroup
-            // an A chunk that straddles K is loaded whole: zero its tail (chunks past K read as zero)
+            if (ragged_k) {
 #pragma unroll
-            for (int it = 0; it < T::A_ITERS; ++it) ra[it] = a_chunk_below<T>(ra[it], it, tid, 0, g.K);
+                for (int it = 0; it < T::A_ITERS; ++it) ra[it] = a_chunk_below<T>(ra[it], it, tid, 0, g.K);
+            }
             store_stage_a<T>(As, tid, ra);
         }
         store_stage_b<T>(Bs, tid, rb);
@@ -94,13 +150,12 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
         // the next tile's operands start their way into the registers just emptied
         const int t_next = t + stride;
         const bool more = t_next < tiles;   // the same for every thread of the workgroup
-        int m0_next = 0, n0_next = 0;
+        Place nxt = cur;
         if (more) {
-            place(t_next, gt_next, m0_next, n0_next);
-            ld.init(gt_next, m0_next, n0_next, tid);
-            a_fresh = m0_next != m0;
-            if (a_fresh) ld.load_first_stage(g.K, ra, rb);
-            else ld.load_first_stage_b(g.K, ra, rb);
+            nxt = place(t_next);
+            a_fresh = nxt.m0 != cur.m0;
+            if (a_fresh) load_a(nxt);
+            load_b(nxt);
         }
 
         f32x16 acc[T::TM][T::TN];
@@ -119,13 +174,55 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
                 mma_frag<T>(frag[kg & 1], acc);
             }
         }
-        store_c_tile<T, B_MODE, PLAIN>(gt, Bs, acc, m0, n0, 0, wave, wm0, wn0, lane, l32, lh);
+        if (PLAIN) {
+            // the next tile's operands have had the tile's MFMAs to arrive; no store is outstanding
+            // but the previous tile's, issued a whole tile ago
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (PLAIN) {
+            // The wave turns its block around in pieces of 8 rows through a staging block of its own,
+            // next to the operand stages: no barrier in front of the epilogue, so a wave that has
+            // finished its MFMAs stores while the others of the workgroup are still multiplying.
+            static_assert(T::TM == 1 && T::TN == 1 && T::WN == 32, "one 32 x 32 block of C per wave");
+            constexpr int PITCH = T::WN + 4;
+            float* stg = smem + T::A_STAGE + T::B_STAGE + wave * (8 * PITCH);
+            const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
+            const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+            float* dst = cur.c + (size_t)row * g.ldc + col;
+            const int rows = g.M - row, valid = min(4, g.N - col);
+            // LDS serves a wave's requests in order: a piece's read sees its writes, and the next
+            // piece's writes come after it.  All four pieces are therefore issued back to back and
+            // the stores follow as the reads return.
+            f32x4 v[4];
+#pragma unroll
+            for (int P = 0; P < 4; ++P) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) stg[(4 * lh + j) * PITCH + l32] = acc[0][0][4 * P + j];
+                v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int P = 0; P < 4; ++P) {
+                if (8 * P < rows && valid > 0) {
+                    float* d = dst + (size_t)(8 * P) * g.ldc;
+                    if (valid == 4) {
+                        *reinterpret_cast<f32x4_u*>(d) = v[P];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (e < valid) d[e] = v[P][e];
+                    }
+                }
+            }
+        } else {
+            gt.C = cur.c;
+            store_c_tile<T, B_MODE, PLAIN>(gt, Bs, acc, cur.m0, cur.n0, 0, wave, wm0, wn0, lane, l32, lh);
+        }
         if (!more) break;
         t = t_next;
-        m0 = m0_next;
-        n0 = n0_next;
-        gt.B = gt_next.B;
-        gt.C = gt_next.C;
+        cur = nxt;
     }
 }
 
@@ -178,14 +275,23 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
     shortk_launch_shape(tiles, tile_n, cus, &grid, &lds);
-    return launch_shortk<TileShortK64, LOAD_VEC4>(args, grid, stream);
+    GemmArgs a2 = args;
+    {
+        const int group = args.group > 0 ? args.group : 1;
+        const int nbands = (args.tiles_m + group - 1) / group;
+        a2.by_band = FastDiv::make((unsigned)(group * args.tiles_n));
+        a2.by_group = FastDiv::make((unsigned)group);
+        a2.by_last_group = FastDiv::make((unsigned)(args.tiles_m - (nbands - 1) * group));
+        a2.by_image_tiles = FastDiv::make((unsigned)args.tiles_n_per_image);
+    }
+    return launch_shortk<TileShortK64, LOAD_VEC4>(a2, grid, stream);
 }
 
 // Workgroups launched for `tiles` tiles of 64 x tile_n, and the LDS each of them takes
 void shortk_launch_shape(long tiles, int tile_n, int cus, int* grid, int* lds_bytes)
 {
     (void)tile_n;
-    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 35 KB per workgroup
+    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 39.5 KB per workgroup
     *grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
     *lds_bytes = shortk_lds_bytes<TileShortK64>();
 }
