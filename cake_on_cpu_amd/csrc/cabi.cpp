@@ -858,13 +858,13 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
         // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
         // column blocks of B by the resident workgroups per CU
         const int tn = shortk_tile_n(M, N, K, model.cus);
-        out->tile_m = 64; out->tile_n = tn; out->tile_k = 64;
+        out->tile_m = 64; out->tile_n = tn; out->tile_k = K <= 32 ? 32 : 64;
         out->wave_m = 32; out->wave_n = tn / 2;
         out->threads = 256;
         out->split_k = 1; out->tail_tiles = 0; out->tail_split = 1;
         out->tiles_m = (M + 63) / 64; out->tiles_n = (N + tn - 1) / tn;
         out->group = shortk_band_rows(out->tiles_m, N);
-        shortk_launch_shape((long)out->tiles_m * out->tiles_n, tn, model.cus, &out->grid, &out->lds_bytes);
+        shortk_launch_shape((long)out->tiles_m * out->tiles_n, tn, K, model.cus, &out->grid, &out->lds_bytes);
     }
     return CAKE_HIP_OK;
 }

@@ -144,7 +144,7 @@ int shortk_band_rows(int tiles_m, int N);
 int shortk_tile_n(int M, int N, int K, int cus, int batch = 1);
 inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1) { return shortk_tile_n(M, N, K, cus, batch) != 0; }
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream);
-void shortk_launch_shape(long tiles, int tile_n, int cus, int* grid, int* lds_bytes);
+void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int* lds_bytes);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,
                                 int accumulate, hipStream_t stream, const ConvGeom* conv = nullptr,

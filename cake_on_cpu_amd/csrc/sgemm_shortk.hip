@@ -245,6 +245,218 @@ static hipError_t launch_shortk(const GemmArgs& args, int grid, hipStream_t stre
                                               : launch_shortk_as<T, B_MODE, false>(args, grid, stream);
 }
 
+// C overwritten, no bias: the same walk with B loaded straight into LDS (buffer loads with the
+// LDS bit: a wave's 64 lanes x 16 bytes land in 1 KB of consecutive LDS, lane by lane, so a lane
+// asks for the chunk that belongs at its place: 4 rows of 64 columns per instruction, rows
+// unpadded -- the 4-byte operand reads of a half-wave cover 32 consecutive floats of a row either
+// way).  B has two buffers: while tile t is multiplied out of one, tile t + 1 arrives in the
+// other, without passing through registers and without a store pass, and one barrier per tile is
+// left (two when the rows of A change).  A's rows are unpadded as well, their 16-byte chunks
+// swizzled (chunk c of row r sits at c ^ (r & 7)) so that the 16-byte operand reads of 8
+// consecutive rows still hit 8 different bank groups.  With stages of 32 k that is 29 KB of LDS and
+// 84 registers: five workgroups share a CU, and products with K up to 32 that overwrite C run
+// here (against the kernel above, us: 256 x 100352 x 32 27.4 -> 25.6, 8192^2 x 32 56.7 -> 53.7,
+// 4096 x 8192 x 25 30.1 -> 28.9, 1100 x 65536 x 32 63.6 -> 61.2; the same bits).  With stages of
+// 64 k it is 53 KB and three workgroups per CU against four: measured level with the kernel
+// above (256 x 100352 x 64: 39.5 against 39.3 us) and not instantiated.
+template <int BK>
+__device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As, float* B0, float* B1, float* Stg)
+{
+    using T = Tile<64, 64, BK, 32, 32>;
+    constexpr int PITCH = T::WN + 4;
+    constexpr int CPR = BK / 4;                      // 16-byte chunks per row of A
+    constexpr int B_LOADS = BK * 64 / 4 / 256;       // load instructions per thread and stage
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm0 = (wave / T::WAVES_N) * T::WM;
+    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
+    const int b_lane = wn0 + l32;
+    float* stg = Stg + wave * (8 * PITCH);
+
+    const int groups = (g.K + 7) >> 3;
+    const int tiles_all = g.tiles_m * g.tiles_n;
+    const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+    const int first = xcd * (tiles_all >> 3) + min(xcd, tiles_all & 7);
+    const int tiles = first + (tiles_all >> 3) + (xcd < (tiles_all & 7) ? 1 : 0);
+    int t = first + (blockIdx.x >> 3);
+    if (t >= tiles) return;
+
+    int a_off[T::A_ITERS], a_lds[T::A_ITERS], b_off[B_LOADS];
+#pragma unroll
+    for (int it = 0; it < T::A_ITERS; ++it) {
+        const int c = tid + it * T::THREADS, r = c / CPR, cc = c % CPR;
+        a_off[it] = cc * 4 < g.K ? (r * g.lda + cc * 4) * 4 : BUF_OOB;
+        a_lds[it] = r * BK + ((cc ^ (r & 7)) * 4);
+    }
+    // load instruction q = wave + 4 it of a stage fills rows 4 q .. 4 q + 3 of B's buffer
+#pragma unroll
+    for (int it = 0; it < B_LOADS; ++it) {
+        const int k = 4 * (wave + 4 * it) + (lane >> 4);
+        b_off[it] = k < g.K ? (k * g.ldb + (lane & 15) * 4) * 4 : BUF_OOB;
+    }
+    const bool ragged_k = (g.K & 3) != 0;
+    // rows at and past K of both buffers are never loaded: zero once (a value left there would
+    // meet a zero of A, but zero times a stray NaN is not zero)
+    for (int i = tid; i < BK * 64 / 4; i += T::THREADS) {
+        reinterpret_cast<f32x4*>(B0)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        reinterpret_cast<f32x4*>(B1)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();
+
+    struct Place {
+        int m0, n0;
+        const float* a;
+        const float* b;
+        float* c;
+        unsigned a_bytes, b_bytes;
+    };
+    auto place = [&](int tile) {
+        const int band_sz = g.group * g.tiles_n;
+        const int band = (int)g.by_band.div((unsigned)tile), rem = tile - band * band_sz;
+        const int row0 = band * g.group;
+        const bool whole_band = g.tiles_m - row0 >= g.group;
+        const int gsz = whole_band ? g.group : g.tiles_m - row0;
+        int tile_n = (int)(whole_band ? g.by_group.div((unsigned)rem) : g.by_last_group.div((unsigned)rem));
+        const int tile_m = row0 + rem - tile_n * gsz;
+        Place p;
+        p.b = g.B;
+        p.c = g.C;
+        if (g.tiles_n_per_image) {
+            const int img = (int)g.by_image_tiles.div((unsigned)tile_n);
+            tile_n -= img * g.tiles_n_per_image;
+            p.b += (size_t)img * g.b_batch_stride;
+            p.c += (size_t)img * g.c_batch_stride;
+        }
+        p.m0 = tile_m * T::BM;
+        p.n0 = tile_n * T::BN;
+        p.a = g.A + (size_t)p.m0 * g.lda;
+        p.b += p.n0;
+        p.a_bytes = records_left(clamp_elems((long long)(g.M - 1 - p.m0) * g.lda + g.K), 0u);
+        p.b_bytes = records_left(clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0), 0u);
+        return p;
+    };
+    f32x4 ra[T::A_ITERS];
+    auto load_a = [&](const Place& p) {
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) ra[it] = buffer_load_f32x4(p.a, a_off[it], p.a_bytes);
+    };
+    auto issue_b = [&](float* Bdst, const Place& p) {
+        __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.b), 0, (int)p.b_bytes, 0x00020000);
+#pragma unroll
+        for (int it = 0; it < B_LOADS; ++it)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(Bdst + (wave + 4 * it) * 256),
+                                                     16, b_off[it], 0, 0, 0);
+    };
+
+    Place cur = place(t), nxt = cur;
+    load_a(cur);
+    issue_b(B0, cur);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    bool a_fresh = true, more = true;
+
+    auto step = [&](const float* Bc, float* Bn) {
+        if (a_fresh) {
+            __syncthreads();   // every wave has read its last operands of A's previous rows
+#pragma unroll
+            for (int it = 0; it < T::A_ITERS; ++it) {
+                f32x4 v = ra[it];
+                if (ragged_k) v = a_chunk_below<T>(v, it, tid, 0, g.K);   // a chunk that straddles K was loaded whole
+                *reinterpret_cast<f32x4*>(As + a_lds[it]) = v;
+            }
+        }
+        // every wave's share of this tile's B has landed (each waited for its own loads), A is
+        // stored, and nobody reads the other buffer any more
+        __syncthreads();
+        const int t_next = t + stride;
+        more = t_next < tiles;
+        if (more) {
+            nxt = place(t_next);
+            a_fresh = nxt.m0 != cur.m0;
+            if (a_fresh) load_a(nxt);
+            issue_b(Bn, nxt);
+        }
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        f32x4 fa[2];
+        float fb[2][4];
+        auto fetch = [&](int kg, f32x4& a, float (&b)[4]) {
+            a = *reinterpret_cast<const f32x4*>(As + a_row + (((kg * 2 + lh) ^ a_swz) * 4));
+            const int kk = kg * 8 + lh * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = Bc[(kk + i) * 64 + b_lane];
+        };
+        fetch(0, fa[0], fb[0]);
+#pragma unroll
+        for (int kg = 0; kg < BK / 8; ++kg) {
+            if (kg < groups) {
+                if (kg + 1 < BK / 8) fetch(kg + 1, fa[(kg + 1) & 1], fb[(kg + 1) & 1]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kg & 1][i], fb[kg & 1][i], acc, 0, 0, 0);
+            }
+        }
+        // the next tile's operands have had the tile's MFMAs to arrive; no store is outstanding
+        // but the previous tile's
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        __builtin_amdgcn_sched_barrier(0);
+        // the wave's block, turned around in pieces of 8 rows through its own staging block
+        const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
+        const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+        float* dst = cur.c + (size_t)row * g.ldc + col;
+        const int rows = g.M - row, valid = min(4, g.N - col);
+        f32x4 v[4];
+#pragma unroll
+        for (int P = 0; P < 4; ++P) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) stg[(4 * lh + j) * PITCH + l32] = acc[4 * P + j];
+            v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int P = 0; P < 4; ++P) {
+            if (8 * P < rows && valid > 0) {
+                float* d = dst + (size_t)(8 * P) * g.ldc;
+                if (valid == 4) {
+                    *reinterpret_cast<f32x4_u*>(d) = v[P];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (e < valid) d[e] = v[P][e];
+                }
+            }
+        }
+    };
+    for (;;) {
+        step(B0, B1);
+        if (!more) break;
+        t += stride;
+        cur = nxt;
+        step(B1, B0);
+        if (!more) break;
+        t += stride;
+        cur = nxt;
+    }
+}
+
+// (the LDS arrays are separate objects on purpose: the compiler then knows that reads of one B
+// buffer need not wait for loads into the other)
+#define SHORTK_DIRECT_KERNEL(BK)                                                                    \
+    __global__ void __launch_bounds__(256) sgemm_shortk_direct_kernel_##BK(const GemmArgs g)        \
+    {                                                                                               \
+        __shared__ __align__(16) float As[64 * BK];                                                 \
+        __shared__ __align__(16) float B0[BK * 64];                                                 \
+        __shared__ __align__(16) float B1[BK * 64];                                                 \
+        __shared__ __align__(16) float Stg[4 * 8 * 36];                                             \
+        shortk_direct_body<BK>(g, As, B0, B1, Stg);                                                 \
+    }
+SHORTK_DIRECT_KERNEL(32)
+#undef SHORTK_DIRECT_KERNEL
+
 // K at most 64, 16-byte-loadable row-major operands, no K slices, and at least a 64 x 64 tile per
 // CU.  Measured against the macro-tile kernel's own choice at K = 16 to 64: 0.79-0.98 of its time
 // from 1 to 16 tiles per CU (1024^2 x 64: 5.3 -> 4.7 us, 3000^2 x 48: 20.1 -> 15.9 us,
@@ -274,7 +486,8 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
     if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
-    shortk_launch_shape(tiles, tile_n, cus, &grid, &lds);
+    const bool direct = args.K <= 32 && !args.accumulate && !args.col_bias;
+    shortk_launch_shape(tiles, tile_n, direct ? args.K : 64, cus, &grid, &lds);
     GemmArgs a2 = args;
     {
         const int group = args.group > 0 ? args.group : 1;
@@ -284,16 +497,22 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
         a2.by_last_group = FastDiv::make((unsigned)(args.tiles_m - (nbands - 1) * group));
         a2.by_image_tiles = FastDiv::make((unsigned)args.tiles_n_per_image);
     }
+    if (direct) {
+        hipLaunchKernelGGL(sgemm_shortk_direct_kernel_32, dim3(grid), dim3(256), 0, stream, a2);
+        return hipGetLastError();
+    }
     return launch_shortk<TileShortK64, LOAD_VEC4>(a2, grid, stream);
 }
 
-// Workgroups launched for `tiles` tiles of 64 x tile_n, and the LDS each of them takes
-void shortk_launch_shape(long tiles, int tile_n, int cus, int* grid, int* lds_bytes)
+// Workgroups launched for `tiles` tiles of 64 x tile_n of a product that overwrites C, and the LDS
+// each of them takes: K up to 32 runs on the kernel that loads B straight into LDS
+void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int* lds_bytes)
 {
     (void)tile_n;
-    const long slots = (long)cus * 4;   // what the LDS of a CU holds: 39.5 KB per workgroup
+    const bool direct = K <= 32;
+    const long slots = (long)cus * (direct ? 5 : 4);   // what the LDS of a CU holds: 28.5 or 39.5 KB per workgroup
     *grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
-    *lds_bytes = shortk_lds_bytes<TileShortK64>();
+    *lds_bytes = direct ? (64 * 32 + 2 * 32 * 64 + 4 * 8 * 36) * 4 : shortk_lds_bytes<TileShortK64>();
 }
 
 }  // namespace cake

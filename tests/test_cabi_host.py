@@ -154,7 +154,7 @@ def test_plan_covers_any_shape(M, N, K):
         assert pl.split_k >= 1 and pl.tail_split >= 1 and 0 <= pl.tail_tiles < tiles
         assert not (pl.split_k > 1 and pl.tail_tiles > 0)
         if pl.kernel == 4:   # short K: resident workgroups, as many as a CU's LDS holds, in whole rows of 8 XCDs
-            per_cu = 3 if pl.tile_n == 128 else 4
+            per_cu = 5 if pl.tile_k == 32 else 4
             assert pl.grid == (min(tiles, per_cu * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
         else:
             assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
@@ -332,6 +332,10 @@ def test_plan_names_the_kernel_family():
     assert (p.kernel, p.tile_m, p.tile_n, p.tile_k, p.threads, p.split_k, p.tail_tiles) == (4, 64, 64, 64, 256, 1, 0)
     assert (p.tiles_m, p.tiles_n) == (4, 1568) and p.grid == 4 * p.cus and p.grid % 8 == 0
     assert 4 * p.lds_bytes <= 160 * 1024
+    # K up to 32: stages of 32 k with B loaded straight into LDS, five workgroups per CU
+    q = cake.plan(250, 100352, 32)
+    assert (q.kernel, q.tile_m, q.tile_n, q.tile_k, q.threads) == (4, 64, 64, 32, 256)
+    assert q.grid == 5 * q.cus and 5 * q.lds_bytes <= 160 * 1024
     # (tiles 128 wide exist but lost every measurement: the choice never takes them)
     assert cake.plan(16384, 16384, 16).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
     # the tile sequence runs in bands: all tile rows of a product up to 16 of them, else 4, 8 or 16
