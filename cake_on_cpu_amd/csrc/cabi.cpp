@@ -520,8 +520,9 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     // (plain operands only: with a convolution's gathered B the integer divisions that place a
     // tile's columns in the image, paid per tile instead of once per workgroup, cost more than
     // the overlap gives -- 1 x 1, 64 -> 256 channels on 56 x 56: 56 us against 50 us)
+    // (beyond 64 k only where C is overwritten without a bias: that kernel has no other epilogue)
     if (vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, vec_plan, nullptr) &&
-        shortk_applies(M, N, K, cur().model.cus)) {
+        shortk_applies(M, N, K, cur().model.cus) && (K <= 64 || (!accumulate && !col_bias))) {
         GemmArgs g{};
         g.A = A; g.B = B; g.C = C;
         g.M = M; g.N = N; g.K = K;
@@ -858,7 +859,7 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
         // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
         // column blocks of B by the resident workgroups per CU
         const int tn = shortk_tile_n(M, N, K, model.cus);
-        out->tile_m = 64; out->tile_n = tn; out->tile_k = K <= 32 ? 32 : 64;
+        out->tile_m = 64; out->tile_n = tn; out->tile_k = K <= 32 || K > 64 ? 32 : 64;
         out->wave_m = 32; out->wave_n = tn / 2;
         out->threads = 256;
         out->split_k = 1; out->tail_tiles = 0; out->tail_split = 1;

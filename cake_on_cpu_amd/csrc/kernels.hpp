@@ -136,9 +136,12 @@ enum LoadMode {
 hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& args, int grid,
                         hipStream_t stream);
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
-// Products with K <= 64 and many 64 x 64 tiles: workgroups that walk over tiles with the next
+// Products with a short K and many 64 x 64 tiles: workgroups that walk over tiles with the next
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
+// K up to 64 of any kind; K from 65 to SHORTK_MAX_K when it is a multiple of 4, the product is a
+// single one (no batch) and C is overwritten without a bias (launch_sgemm_shortk refuses the rest).
 // shortk_tile_n: 0 when the kernel does not apply, else the width of its tiles (64)
+enum { SHORTK_MAX_K = 160 };
 // tile rows per band of the short-K kernel's tile sequence (group of the launch arguments)
 int shortk_band_rows(int tiles_m, int N);
 int shortk_tile_n(int M, int N, int K, int cus, int batch = 1);

@@ -457,6 +457,207 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
 SHORTK_DIRECT_KERNEL(32)
 #undef SHORTK_DIRECT_KERNEL
 
+// K from 65 to 160 (a multiple of 4), C overwritten, no bias: the walk over tiles continued into K.
+// A workgroup's work is a sequence of units -- (tile, stage of 32 k) -- and BOTH operands of a unit
+// go straight into LDS (A's rows swizzled as above, by the choice of which chunk a lane asks for);
+// each operand has two buffers, the loads of unit u + 1 are issued when unit u starts, across tile
+// borders, so a tile has no prologue of its own; one barrier per unit; the epilogue as above.
+// 37 KB of LDS and 76 registers: four workgroups per CU.  Nothing passes through registers, and
+// lanes past the operands' ends write zeros into LDS (the hardware does that for out-of-range
+// lanes of such loads).  K must be a multiple of 4: a chunk of A that straddled K would bring in
+// the next row's values where B holds zeros, and zero times a stray NaN is not zero.
+// Measured against the macro-tile kernel's choice for the same product (us): 1000 x 30000 x 128
+// 81.6 -> 72.1, 4096^2 x 128 46.8 -> 42.9, 8192^2 x 96 139 -> 129, 3000^2 x 100 27.4 -> 22.4,
+// 2000 x 20000 x 80 87.9 -> 70.2, 8192 x 2048 x 132 51.9 -> 44.1, 2048 x 8192 x 144 52.1 -> 46.4,
+// 4096^2 x 160 51.6 -> 49.5, 1024^2 x 128 6.7 -> 5.6; level at K = 192 (1024 x 16384: 57.7 / 57.2)
+// and behind at 256 (4096^2: 72.0 / 73.5), and behind the kernel at the top of this file at K = 64
+// (256 x 100352: 38.6 / 40.2).  With three buffers per operand and the loads two units ahead
+// (54 KB, three workgroups per CU) it was 2-8 % slower on all of them.
+template <int NSTAGE>
+__device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* const (&Ab)[NSTAGE], float* const (&Bb)[NSTAGE],
+                                                   float* Stg)
+{
+    constexpr int BK = 32, PITCH = 36, PF = NSTAGE - 1;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
+    const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
+    const int b_lane = wn0 + l32;
+    float* stg = Stg + wave * (8 * PITCH);
+
+    const int stages = (g.K + BK - 1) / BK;
+    const int tiles_all = g.tiles_m * g.tiles_n;
+    const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+    const int first = xcd * (tiles_all >> 3) + min(xcd, tiles_all & 7);
+    const int tiles = first + (tiles_all >> 3) + (xcd < (tiles_all & 7) ? 1 : 0);
+    const int t0 = first + (blockIdx.x >> 3);
+    if (t0 >= tiles) return;
+
+    // load instruction q = wave + 4 it fills rows 8 q .. 8 q + 7 of A's buffer (8 chunks of 16 bytes
+    // per row, chunk c of row r at place c ^ (r & 7)) and rows 4 q .. 4 q + 3 of B's
+    int a_off[2], a_off_last[2], b_off[2];
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int q = wave + 4 * it;
+        const int r = 8 * q + (lane >> 3), c = (lane & 7) ^ (r & 7);
+        a_off[it] = (r * g.lda + c * 4) * 4;
+        a_off_last[it] = (stages - 1) * BK + c * 4 < g.K ? a_off[it] : BUF_OOB;
+        b_off[it] = ((4 * q + (lane >> 4)) * g.ldb + (lane & 15) * 4) * 4;
+    }
+
+    struct Place {
+        int m0, n0;
+        const float* a;
+        const float* b;
+        float* c;
+        unsigned a_elems, b_elems;
+    };
+    auto place = [&](int tile) {
+        const int band_sz = g.group * g.tiles_n;
+        const int band = (int)g.by_band.div((unsigned)tile), rem = tile - band * band_sz;
+        const int row0 = band * g.group;
+        const bool whole_band = g.tiles_m - row0 >= g.group;
+        const int gsz = whole_band ? g.group : g.tiles_m - row0;
+        const int tile_n = (int)(whole_band ? g.by_group.div((unsigned)rem) : g.by_last_group.div((unsigned)rem));
+        const int tile_m = row0 + rem - tile_n * gsz;
+        Place p;
+        p.m0 = tile_m * 64;
+        p.n0 = tile_n * 64;
+        p.a = g.A + (size_t)p.m0 * g.lda;
+        p.b = g.B + p.n0;
+        p.c = g.C;
+        p.a_elems = clamp_elems((long long)(g.M - 1 - p.m0) * g.lda + g.K);
+        p.b_elems = clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0);
+        return p;
+    };
+    auto issue = [&](float* Ad, float* Bd, const Place& p, int ks) {
+        const unsigned ka = (unsigned)ks * BK, kb = (unsigned)ks * BK * (unsigned)g.ldb;
+        __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.a + ka), 0,
+                                                                      (int)records_left(p.a_elems, ka), 0x00020000);
+        __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.b + kb), 0,
+                                                                      (int)records_left(p.b_elems, kb), 0x00020000);
+        const bool last = ks == stages - 1;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(Ad + (wave + 4 * it) * 256), 16,
+                                                     last ? a_off_last[it] : a_off[it], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(Bd + (wave + 4 * it) * 256), 16,
+                                                     b_off[it], 0, 0, 0);
+        }
+    };
+
+    // consumer and producer positions in the unit sequence
+    int t = t0, ks = 0, tp = t0, kp = 0;
+    Place cur = place(t0), pp = cur;
+    bool producing = true;
+    auto produce = [&](float* Ad, float* Bd) {
+        if (!producing) return;
+        issue(Ad, Bd, pp, kp);
+        if (++kp == stages) {
+            kp = 0;
+            tp += stride;
+            producing = tp < tiles;
+            if (producing) pp = place(tp);
+        }
+    };
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+
+    // returns false after the workgroup's last unit
+    auto unit = [&](const float* Ac, const float* Bc, float* Ad, float* Bd) -> bool {
+        // this unit's loads have landed: at most the PF - 1 younger units' loads (4 instructions each) are outstanding
+        if (producing) {
+            if constexpr (PF == 1) __builtin_amdgcn_s_waitcnt(0x0F70);
+            else __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();   // everybody's share has landed, and nobody reads the buffer that is filled next
+        produce(Ad, Bd);
+        const int groups = min(4, (g.K - ks * BK + 7) >> 3);
+        f32x4 fa[2];
+        float fb[2][4];
+        auto fetch = [&](int kg, f32x4& a, float (&b)[4]) {
+            a = *reinterpret_cast<const f32x4*>(Ac + a_row + (((kg * 2 + lh) ^ a_swz) * 4));
+            const int kk = kg * 8 + lh * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = Bc[(kk + i) * 64 + b_lane];
+        };
+        fetch(0, fa[0], fb[0]);
+#pragma unroll
+        for (int kg = 0; kg < 4; ++kg) {
+            if (kg < groups) {
+                if (kg + 1 < 4) fetch(kg + 1, fa[(kg + 1) & 1], fb[(kg + 1) & 1]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kg & 1][i], fb[kg & 1][i], acc, 0, 0, 0);
+            }
+        }
+        if (++ks < stages) return true;
+        // the tile is finished: the wave's block, turned around in pieces of 8 rows through its own staging block
+        const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
+        const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+        float* dst = cur.c + (size_t)row * g.ldc + col;
+        const int rows = g.M - row, valid = min(4, g.N - col);
+        f32x4 v[4];
+#pragma unroll
+        for (int P = 0; P < 4; ++P) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) stg[(4 * lh + j) * PITCH + l32] = acc[4 * P + j];
+            v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int P = 0; P < 4; ++P) {
+            if (8 * P < rows && valid > 0) {
+                float* d = dst + (size_t)(8 * P) * g.ldc;
+                if (valid == 4) {
+                    *reinterpret_cast<f32x4_u*>(d) = v[P];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (e < valid) d[e] = v[P][e];
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        ks = 0;
+        t += stride;
+        if (t >= tiles) return false;
+        cur = place(t);
+        return true;
+    };
+
+    // the first PF units' loads
+#pragma unroll
+    for (int i = 0; i < PF; ++i) produce(Ab[i], Bb[i]);
+    for (;;) {
+        if constexpr (NSTAGE == 2) {
+            if (!unit(Ab[0], Bb[0], Ab[1], Bb[1])) break;
+            if (!unit(Ab[1], Bb[1], Ab[0], Bb[0])) break;
+        } else {
+            if (!unit(Ab[0], Bb[0], Ab[2], Bb[2])) break;
+            if (!unit(Ab[1], Bb[1], Ab[0], Bb[0])) break;
+            if (!unit(Ab[2], Bb[2], Ab[1], Bb[1])) break;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) sgemm_shortk_staged_kernel(const GemmArgs g)
+{
+    __shared__ __align__(16) float A0[2048];
+    __shared__ __align__(16) float A1[2048];
+    __shared__ __align__(16) float B0[2048];
+    __shared__ __align__(16) float B1[2048];
+    __shared__ __align__(16) float Stg[4 * 8 * 36];
+    float* const Ab[2] = {A0, A1};
+    float* const Bb[2] = {B0, B1};
+    shortk_staged_body<2>(g, Ab, Bb, Stg);
+}
+
 // K at most 64, 16-byte-loadable row-major operands, no K slices, and at least a 64 x 64 tile per
 // CU.  Measured against the macro-tile kernel's own choice at K = 16 to 64: 0.79-0.98 of its time
 // from 1 to 16 tiles per CU (1024^2 x 64: 5.3 -> 4.7 us, 3000^2 x 48: 20.1 -> 15.9 us,
@@ -467,7 +668,8 @@ SHORTK_DIRECT_KERNEL(32)
 // 256 x 100352 x 64: 58 against 46 us): the width is a parameter of the launch, with one value.
 int shortk_tile_n(int M, int N, int K, int cus, int batch)
 {
-    if (K < 1 || K > 64) return 0;
+    // beyond 64 k: stages of 32 k with both operands loaded straight into LDS, single products with K a multiple of 4
+    if (K < 1 || K > SHORTK_MAX_K || (K > 64 && (K % 4 != 0 || batch != 1))) return 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64) * batch;
     if (tiles < (long)cus) return 0;
     return 64;
@@ -483,11 +685,13 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
 {
     const long tiles = (long)args.tiles_m * args.tiles_n;
     if (tiles <= 0) return hipSuccess;
-    if (args.K > 64 || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
+    if (args.K > SHORTK_MAX_K || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
-    const bool direct = args.K <= 32 && !args.accumulate && !args.col_bias;
-    shortk_launch_shape(tiles, tile_n, direct ? args.K : 64, cus, &grid, &lds);
+    const bool plain = !args.accumulate && !args.col_bias;
+    if (args.K > 64 && (!plain || args.K % 4 != 0 || args.tiles_n_per_image)) return hipErrorInvalidValue;
+    const bool direct = args.K <= 32 && plain;
+    shortk_launch_shape(tiles, tile_n, direct || args.K > 64 ? args.K : 64, cus, &grid, &lds);
     GemmArgs a2 = args;
     {
         const int group = args.group > 0 ? args.group : 1;
@@ -497,8 +701,9 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
         a2.by_last_group = FastDiv::make((unsigned)(args.tiles_m - (nbands - 1) * group));
         a2.by_image_tiles = FastDiv::make((unsigned)args.tiles_n_per_image);
     }
-    if (direct) {
-        hipLaunchKernelGGL(sgemm_shortk_direct_kernel_32, dim3(grid), dim3(256), 0, stream, a2);
+    if (direct || args.K > 64) {
+        if (direct) hipLaunchKernelGGL(sgemm_shortk_direct_kernel_32, dim3(grid), dim3(256), 0, stream, a2);
+        else hipLaunchKernelGGL(sgemm_shortk_staged_kernel, dim3(grid), dim3(256), 0, stream, a2);
         return hipGetLastError();
     }
     return launch_shortk<TileShortK64, LOAD_VEC4>(a2, grid, stream);
@@ -510,9 +715,10 @@ void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int*
 {
     (void)tile_n;
     const bool direct = K <= 32;
-    const long slots = (long)cus * (direct ? 5 : 4);   // what the LDS of a CU holds: 28.5 or 39.5 KB per workgroup
+    const long slots = (long)cus * (direct ? 5 : 4);   // what the LDS of a CU holds: 28.5, 39.5 or (K above 64) 36.5 KB per workgroup
     *grid = (int)(((tiles < slots ? tiles : slots) + 7) / 8 * 8);   // whole rows of 8 XCDs
-    *lds_bytes = direct ? (64 * 32 + 2 * 32 * 64 + 4 * 8 * 36) * 4 : shortk_lds_bytes<TileShortK64>();
+    *lds_bytes = direct ? (64 * 32 + 2 * 32 * 64 + 4 * 8 * 36) * 4
+                        : K > 64 ? (4 * 2048 + 4 * 8 * 36) * 4 : shortk_lds_bytes<TileShortK64>();
 }
 
 }  // namespace cake

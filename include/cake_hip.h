@@ -75,14 +75,16 @@ typedef struct cake_hip_cpu_cntx_t {
  * as does one with 33 to 48 rows of A against a B of 48 million elements or more, 49 to 64
  * rows against 100 million, 65 to 80 against 30 million, 97 to 112 against 64 million,
  * one with K <= 64 and at least one tile of 64 x 64 per CU on workgroups that walk over tiles
- * (tile, grid and LDS fields then describe that launch),
+ * (tile, grid and LDS fields then describe that launch; K up to 32 and, when it is a multiple of 4,
+ * K from 65 to 160 in stages of 32 k loaded straight into LDS -- the latter only for a product
+ * that overwrites C, the plan of one that adds to C or carries a bias is the macro-tile's),
  * everything else on the macro-tile kernel the other fields describe. */
 enum {
     CAKE_HIP_KERNEL_TILE = 0,
     CAKE_HIP_KERNEL_GEMV = 1,
     CAKE_HIP_KERNEL_STREAM_ROWS = 2, /* few rows of A: B streamed once    */
     CAKE_HIP_KERNEL_STREAM_COLS = 3, /* few columns of B: A streamed once */
-    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K, many tiles: 64 x 64 tiles, next tile's operands in flight */
+    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K (up to 160), many tiles: 64 x 64 tiles, next tile's operands in flight */
 };
 
 /* What the GPU planner decided for one GEMM: the successor of

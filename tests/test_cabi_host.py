@@ -154,7 +154,7 @@ def test_plan_covers_any_shape(M, N, K):
         assert pl.split_k >= 1 and pl.tail_split >= 1 and 0 <= pl.tail_tiles < tiles
         assert not (pl.split_k > 1 and pl.tail_tiles > 0)
         if pl.kernel == 4:   # short K: resident workgroups, as many as a CU's LDS holds, in whole rows of 8 XCDs
-            per_cu = 5 if pl.tile_k == 32 else 4
+            per_cu = 5 if K <= 32 else 4
             assert pl.grid == (min(tiles, per_cu * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
         else:
             assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
@@ -324,6 +324,8 @@ def test_plan_names_the_kernel_family():
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 127) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
+    assert fam(4096, 4096, 68) == 4 and fam(4096, 4096, 160) == 4 and fam(4096, 4096, 164) == 0 and fam(4096, 4096, 130) == 0
+    assert fam(960, 960, 128) == 0
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
     # the plan of a short-K product describes that launch: 64 x 64 tiles holding the whole K, at most
@@ -336,6 +338,10 @@ def test_plan_names_the_kernel_family():
     q = cake.plan(250, 100352, 32)
     assert (q.kernel, q.tile_m, q.tile_n, q.tile_k, q.threads) == (4, 64, 64, 32, 256)
     assert q.grid == 5 * q.cus and 5 * q.lds_bytes <= 160 * 1024
+    # K from 65 to 160 (a multiple of 4): stages of 32 k, both operands straight into LDS, four workgroups per CU
+    q = cake.plan(250, 100352, 128)
+    assert (q.kernel, q.tile_m, q.tile_n, q.tile_k, q.threads) == (4, 64, 64, 32, 256)
+    assert q.grid == 4 * q.cus and 4 * q.lds_bytes <= 160 * 1024
     # (tiles 128 wide exist but lost every measurement: the choice never takes them)
     assert cake.plan(16384, 16384, 16).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
     # the tile sequence runs in bands: all tile rows of a product up to 16 of them, else 4, 8 or 16

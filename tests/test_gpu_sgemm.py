@@ -209,14 +209,19 @@ def test_tall_matrix_times_few_columns(shape):
                                    (4096, 16, 8200), (3333, 24, 7777), (8192, 25, 4096),
                                    # more than 16 tile rows against 12288 columns and more: bands of 4 tile rows,
                                    # 18 and 19 tile rows (neither a multiple of 4), ragged everything
-                                   (1100, 16, 12300), (1160, 24, 12417)],
+                                   (1100, 16, 12300), (1160, 24, 12417),
+                                   # K from 65 to 160, a multiple of 4: stages of 32 k straight into LDS (one to five
+                                   # stages, the last one partial); other K there stay on the macro-tile kernel
+                                   (1030, 68, 1100), (2048, 96, 2048), (1024, 128, 1024), (777, 132, 5000), (3001, 160, 1999),
+                                   (4096, 100, 4100), (1100, 101, 1100), (1024, 164, 1024), (1160, 72, 12417)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_short_k_many_tiles(shape):
     """K of at most 64 under at least one 64 x 64 tile per CU: workgroups that walk over tiles with
     the next tile's operands in flight (K = 65 and fewer tiles stay on the macro-tile kernel),
     ragged M, N and K, overwriting and accumulating, run-to-run identical."""
     M, K, N = shape
-    want = 4 if K <= 64 and ((M + 63) // 64) * ((N + 63) // 64) >= cake.device_info().cus else 0
+    short = K <= 64 or (K <= 160 and K % 4 == 0)
+    want = 4 if short and ((M + 63) // 64) * ((N + 63) // 64) >= cake.device_info().cus else 0
     assert cake.plan(M, N, K).kernel == want
     print(f"sgemm short K M={M} K={K} N={N}", flush=True)
     A, B, Cm = _run(M, K, N)
