@@ -1425,9 +1425,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // channels and many tiles the images are walked as a batch by the short-K kernel
     // (64 -> 256 channels on 32 x 56 x 56: 50 -> 43 us).
     const int HW = Hout * Wout;
+    // (up to 64 channels from 12 tiles per CU on; 65 to 256 channels -- the kernel whose operands go
+    // straight into LDS -- from 2 tiles per CU on, for a product that overwrites C, and beyond 160
+    // channels only where the planes fill their column tiles to 90 %)
+    const long batch_tiles = (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch;
+    const bool batch_pays = K <= 64 ? batch_tiles >= 12L * cur().model.cus
+                                    : !accumulate && batch_tiles >= 2L * cur().model.cus &&
+                                          (K <= SHORTK_MAX_K || 10L * ((HW + 63) / 64 * 64 - HW) <= (long)HW);
     if (!explicit_cols && Hf == 1 && Wf == 1 && stride == 1 && pad == 0 &&
-        shortk_applies(Cout, HW, K, cur().model.cus, batch) &&
-        (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch >= 12L * cur().model.cus &&   // measured from there on
+        shortk_applies(Cout, HW, K, cur().model.cus, batch, true) && batch_pays &&
         vec4_loadable(w.dev, i.dev, K, HW)) {
         GemmArgs g{};
         g.A = w.dev; g.B = i.dev; g.C = o.dev;
@@ -1436,7 +1442,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.ldc = out_nchw ? HW : N;                             // [batch][Cout][HW] or [Cout][batch*HW]
         g.b_batch_stride = (size_t)Cin * HW;
         g.c_batch_stride = out_nchw ? (size_t)Cout * HW : (size_t)HW;
-        const int tn = shortk_tile_n(Cout, HW, K, cur().model.cus, batch);
+        const int tn = shortk_tile_n(Cout, HW, K, cur().model.cus, batch, true);
         g.tiles_m = (Cout + 63) / 64;
         g.tiles_n_per_image = (HW + tn - 1) / tn;
         g.tiles_n = g.tiles_n_per_image * batch;

@@ -138,14 +138,19 @@ hipError_t launch_sgemm(int tile_id, int a_mode, int b_mode, const GemmArgs& arg
 hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t stream);
 // Products with a short K and many 64 x 64 tiles: workgroups that walk over tiles with the next
 // tile's operands in flight (sgemm_shortk.hip).  Both operands row-major and 16-byte-loadable.
-// K up to 64 of any kind; K from 65 to SHORTK_MAX_K when it is a multiple of 4, the product is a
-// single one (no batch) and C is overwritten without a bias (launch_sgemm_shortk refuses the rest).
+// K up to 64 of any kind; K from 65 to SHORTK_MAX_K (a batch of products with one A, i.e. a 1 x 1
+// convolution: to SHORTK_MAX_K_BATCH) when it is a multiple of 4 and C is overwritten without a
+// bias (launch_sgemm_shortk refuses the rest).
 // shortk_tile_n: 0 when the kernel does not apply, else the width of its tiles (64)
-enum { SHORTK_MAX_K = 160 };
+enum { SHORTK_MAX_K = 160, SHORTK_MAX_K_BATCH = 256 };
 // tile rows per band of the short-K kernel's tile sequence (group of the launch arguments)
 int shortk_band_rows(int tiles_m, int N);
-int shortk_tile_n(int M, int N, int K, int cus, int batch = 1);
-inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1) { return shortk_tile_n(M, N, K, cus, batch) != 0; }
+// batch >= 1 with shared_a: `batch` products M x K x N with one A (launched with tiles_n_per_image set)
+int shortk_tile_n(int M, int N, int K, int cus, int batch = 1, bool shared_a = false);
+inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1, bool shared_a = false)
+{
+    return shortk_tile_n(M, N, K, cus, batch, shared_a) != 0;
+}
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream);
 void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int* lds_bytes);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says

@@ -472,7 +472,16 @@ SHORTK_DIRECT_KERNEL(32)
 // 4096^2 x 160 51.6 -> 49.5, 1024^2 x 128 6.7 -> 5.6; level at K = 192 (1024 x 16384: 57.7 / 57.2)
 // and behind at 256 (4096^2: 72.0 / 73.5), and behind the kernel at the top of this file at K = 64
 // (256 x 100352: 38.6 / 40.2).  With three buffers per operand and the loads two units ahead
-// (54 KB, three workgroups per CU) it was 2-8 % slower on all of them.
+// (54 KB, three workgroups per CU) it was 2-8 % slower on all of them, and with the unit's barrier
+// moved in front of its last group of MFMAs (operands in registers, the next unit's first operands
+// read behind them) 0-8 % slower.
+// A batch of products with one A (a 1 x 1 convolution on the input as it lies) runs here up to
+// 256 channels: against the gather inside the macro-tile kernel, batch 32, us: 128 -> 512 on 28 x 28
+// 41.9 -> 37.3, 128 -> 256 on 56 x 56 74.1 -> 65.6, 80 -> 480 on 56 x 56 105 -> 84, 128 -> 128 on
+// 28 x 28 16.2 -> 13.9, 256 -> 128 on 56 x 56 63.3 -> 59.4, 256 -> 512 on 28 x 28 62.6 -> 59.8,
+// 128 -> 512 on 14 x 14 (196 pixels in four tiles of 64: a quarter of the columns is padding)
+// 15.7 -> 13.5, but 256 -> 1024 on 14 x 14 39.0 -> 41.7: with that much padding the gather stays
+// from 161 channels on.
 template <int NSTAGE>
 __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* const (&Ab)[NSTAGE], float* const (&Bb)[NSTAGE],
                                                    float* Stg)
@@ -519,14 +528,21 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         const int row0 = band * g.group;
         const bool whole_band = g.tiles_m - row0 >= g.group;
         const int gsz = whole_band ? g.group : g.tiles_m - row0;
-        const int tile_n = (int)(whole_band ? g.by_group.div((unsigned)rem) : g.by_last_group.div((unsigned)rem));
+        int tile_n = (int)(whole_band ? g.by_group.div((unsigned)rem) : g.by_last_group.div((unsigned)rem));
         const int tile_m = row0 + rem - tile_n * gsz;
         Place p;
+        p.b = g.B;
+        p.c = g.C;
+        if (g.tiles_n_per_image) {   // a batch of products with one A: the image's B and C
+            const int img = (int)g.by_image_tiles.div((unsigned)tile_n);
+            tile_n -= img * g.tiles_n_per_image;
+            p.b += (size_t)img * g.b_batch_stride;
+            p.c += (size_t)img * g.c_batch_stride;
+        }
         p.m0 = tile_m * 64;
         p.n0 = tile_n * 64;
         p.a = g.A + (size_t)p.m0 * g.lda;
-        p.b = g.B + p.n0;
-        p.c = g.C;
+        p.b += p.n0;
         p.a_elems = clamp_elems((long long)(g.M - 1 - p.m0) * g.lda + g.K);
         p.b_elems = clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0);
         return p;
@@ -666,10 +682,10 @@ __global__ void __launch_bounds__(256) sgemm_shortk_staged_kernel(const GemmArgs
 // Tiles 128 wide (four waves of 32 x 64, three workgroups per CU) were measured against these on
 // the same device from K = 16 to 64 and lost everywhere (16384^2 x 16: 260 against 231 us,
 // 256 x 100352 x 64: 58 against 46 us): the width is a parameter of the launch, with one value.
-int shortk_tile_n(int M, int N, int K, int cus, int batch)
+int shortk_tile_n(int M, int N, int K, int cus, int batch, bool shared_a)
 {
-    // beyond 64 k: stages of 32 k with both operands loaded straight into LDS, single products with K a multiple of 4
-    if (K < 1 || K > SHORTK_MAX_K || (K > 64 && (K % 4 != 0 || batch != 1))) return 0;
+    // beyond 64 k: stages of 32 k with both operands loaded straight into LDS, K a multiple of 4
+    if (K < 1 || K > (shared_a ? SHORTK_MAX_K_BATCH : SHORTK_MAX_K) || (K > 64 && K % 4 != 0)) return 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64) * batch;
     if (tiles < (long)cus) return 0;
     return 64;
@@ -685,11 +701,11 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
 {
     const long tiles = (long)args.tiles_m * args.tiles_n;
     if (tiles <= 0) return hipSuccess;
-    if (args.K > SHORTK_MAX_K || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
+    if (args.K > (args.tiles_n_per_image ? SHORTK_MAX_K_BATCH : SHORTK_MAX_K) || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
     const bool plain = !args.accumulate && !args.col_bias;
-    if (args.K > 64 && (!plain || args.K % 4 != 0 || args.tiles_n_per_image)) return hipErrorInvalidValue;
+    if (args.K > 64 && (!plain || args.K % 4 != 0)) return hipErrorInvalidValue;
     const bool direct = args.K <= 32 && plain;
     shortk_launch_shape(tiles, tile_n, direct || args.K > 64 ? args.K : 64, cus, &grid, &lds);
     GemmArgs a2 = args;
