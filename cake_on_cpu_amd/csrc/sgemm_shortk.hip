@@ -1,4 +1,11 @@
-// Products with a short K (at most 64) and many tiles of C: the macro-tile kernel spends a
+// Three kernels for products with a short K (up to 160; up to 256 for a batch that shares A) and
+// many tiles of C, in this order: K at most 64 with operands staged through registers (any
+// epilogue); K at most 32, C overwritten, B loaded straight into LDS; K from 65 up, C overwritten,
+// both operands loaded straight into LDS stage by stage.  What they share: a workgroup stays
+// resident and walks over 64 x 64 tiles, with the next tile's (or stage's) operands on their way
+// while the current one is multiplied.
+//
+// The first kernel.  With K at most 64 and many tiles of C the macro-tile kernel spends a
 // workgroup per tile, and with two k steps per tile the load latency of every tile sits in front
 // of its few MFMAs (measured 256 x 100352 x 64: 37 us for loads and arithmetic where the matrix
 // work alone takes 21 us, plus 6 us of stores).  Here a workgroup stays and walks over tiles: the
