@@ -1428,10 +1428,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     // (up to 64 channels from 12 tiles per CU on; 65 to 256 channels -- the kernel whose operands go
     // straight into LDS -- from 2 tiles per CU on, for a product that overwrites C, and beyond 160
     // channels only where the planes fill their column tiles to 90 %)
-    const long batch_tiles = (long)((Cout + 63) / 64) * ((HW + 63) / 64) * batch;
+    // Beyond 64 channels the column tiles run across image borders where that saves tiles (a plane's
+    // pixels a multiple of 4 but not of 64, the whole input below 2 GiB): 256 -> 1024 channels on
+    // 32 x 14 x 14 is 1568 tiles that way and 2048 with every image's last tile a quarter full.
+    const bool across_images = K > 64 && HW % 4 == 0 && HW % 64 != 0 && (double)batch * Cin * HW * 4.0 < 2147483648.0 &&
+                               fits_int((double)batch * HW);
+    const long batch_tiles = (long)((Cout + 63) / 64) * (across_images ? ((long)batch * HW + 63) / 64 : (long)((HW + 63) / 64) * batch);
     const bool batch_pays = K <= 64 ? batch_tiles >= 12L * cur().model.cus
                                     : !accumulate && batch_tiles >= 2L * cur().model.cus &&
-                                          (K <= SHORTK_MAX_K || 10L * ((HW + 63) / 64 * 64 - HW) <= (long)HW);
+                                          (K <= SHORTK_MAX_K || across_images || 10L * ((HW + 63) / 64 * 64 - HW) <= (long)HW);
     if (!explicit_cols && Hf == 1 && Wf == 1 && stride == 1 && pad == 0 &&
         shortk_applies(Cout, HW, K, cur().model.cus, batch, true) && batch_pays &&
         vec4_loadable(w.dev, i.dev, K, HW)) {
@@ -1444,8 +1449,14 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.c_batch_stride = out_nchw ? (size_t)Cout * HW : (size_t)HW;
         const int tn = shortk_tile_n(Cout, HW, K, cur().model.cus, batch, true);
         g.tiles_m = (Cout + 63) / 64;
-        g.tiles_n_per_image = (HW + tn - 1) / tn;
-        g.tiles_n = g.tiles_n_per_image * batch;
+        if (across_images) {
+            g.N = batch * HW;
+            g.batch_cols = HW;
+            g.tiles_n = (g.N + tn - 1) / tn;
+        } else {
+            g.tiles_n_per_image = (HW + tn - 1) / tn;
+            g.tiles_n = g.tiles_n_per_image * batch;
+        }
         g.split_k = 1; g.k_per_split = K;
         g.group = g.tiles_m; g.group_along_n = 0;
         g.accumulate = accumulate;

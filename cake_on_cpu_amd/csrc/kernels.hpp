@@ -95,9 +95,15 @@ struct GemmArgs {
     // all images, tiles_n_per_image of them per image.  0 = a single product.
     int tiles_n_per_image;
     size_t b_batch_stride, c_batch_stride;
+    // The same batch with its column tiles running across image borders (the kernel for K above 64
+    // only): column n of the product is pixel n % batch_cols of image n / batch_cols, N counts the
+    // columns of all images, tiles_n their tiles and tiles_n_per_image is 0.  Planes whose pixels
+    // do not fill whole tiles then cost no padding.  batch_cols is a multiple of 4 and all of B
+    // stays below 2^31 bytes.  0 = off.
+    int batch_cols;
     // sgemm_shortk.hip: divisions of the tile walk as multiplications (filled in by its launcher):
     // by tiles per band, by tile rows of a whole band, by those of the last band, by column tiles per image
-    FastDiv by_band, by_group, by_last_group, by_image_tiles;
+    FastDiv by_band, by_group, by_last_group, by_image_tiles, by_batch_cols;
 };
 
 // Macro-tile shapes the planner can choose from.

@@ -489,7 +489,16 @@ SHORTK_DIRECT_KERNEL(32)
 // 128 -> 512 on 14 x 14 (196 pixels in four tiles of 64: a quarter of the columns is padding)
 // 15.7 -> 13.5, but 256 -> 1024 on 14 x 14 39.0 -> 41.7: with that much padding the gather stays
 // from 161 channels on.
-template <int NSTAGE>
+// That padding goes away when the column tiles run across image borders (FLAT: the columns of all
+// images form one sequence, a lane's offset into B is recomputed per tile -- one division by the
+// plane size as a multiplication -- and a 16-byte chunk never spans two images because the plane
+// size is a multiple of 4): 256 -> 1024 on 14 x 14 is 1568 tiles instead of 2048, 38.5 -> 36.2 us
+// against the gather; 128 -> 512 on 14 x 14 16.7 -> 14.3, 192 -> 384 16.1 -> 14.4, 128 -> 512 on 28 x 28
+// 38.3 -> 33.8, 96 -> 256 on 28 x 28 19.5 -> 17.1, 128 -> 256 on 20 x 20 15.5 -> 13.3, batch 128
+// 256 -> 512 on 10 x 10 35.5 -> 34.0.  (The divisor of that division must stay in scalar
+// registers: a record count computed with an integer division of the arguments lands in a vector
+// register and the compiler then loops over every load.)
+template <int NSTAGE, bool FLAT>
 __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* const (&Ab)[NSTAGE], float* const (&Bb)[NSTAGE],
                                                    float* Stg)
 {
@@ -521,13 +530,28 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         a_off_last[it] = (stages - 1) * BK + c * 4 < g.K ? a_off[it] : BUF_OOB;
         b_off[it] = ((4 * q + (lane >> 4)) * g.ldb + (lane & 15) * 4) * 4;
     }
+    // A batch whose column tiles run across image borders: B's base stays the first image, the
+    // lane's offset moves with the tile (b_flat, below), and rows at and past K -- which the record
+    // count cannot cut off there, the next image follows -- are cut off per lane.
+    constexpr bool flat = FLAT;   // g.batch_cols != 0
+    const bool b_row_past_k[2] = {(stages - 1) * BK + 4 * wave + (lane >> 4) >= g.K,
+                                  (stages - 1) * BK + 4 * (wave + 4) + (lane >> 4) >= g.K};
 
+    // byte offset of the lane's first chunk of B in a tile that starts at column n0 of the whole batch
+    // (columns at and past N belong to images past the last one: out of range)
+    auto flat_offset = [&](int n0) {
+        const unsigned n = (unsigned)n0 + (lane & 15) * 4;
+        const unsigned img = g.by_batch_cols.div(n);
+        return (int)((img * (unsigned)g.b_batch_stride + (n - img * (unsigned)g.batch_cols) +
+                      (unsigned)(4 * wave + (lane >> 4)) * (unsigned)g.ldb) * 4u);
+    };
     struct Place {
         int m0, n0;
         const float* a;
         const float* b;
         float* c;
         unsigned a_elems, b_elems;
+        int b_flat;   // per lane: flat_offset(n0)
     };
     auto place = [&](int tile) {
         const int band_sz = g.group * g.tiles_n;
@@ -549,9 +573,15 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         p.m0 = tile_m * 64;
         p.n0 = tile_n * 64;
         p.a = g.A + (size_t)p.m0 * g.lda;
-        p.b += p.n0;
         p.a_elems = clamp_elems((long long)(g.M - 1 - p.m0) * g.lda + g.K);
-        p.b_elems = clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0);
+        p.b_flat = 0;
+        if (flat) {
+            p.b_elems = (unsigned)g.b_batch_stride * g.by_batch_cols.div((unsigned)g.N);   // all images: below 2^29 elements
+            p.b_flat = flat_offset(p.n0);
+        } else {
+            p.b += p.n0;
+            p.b_elems = clamp_elems((long long)(g.K - 1) * g.ldb + g.N - p.n0);
+        }
         return p;
     };
     auto issue = [&](float* Ad, float* Bd, const Place& p, int ks) {
@@ -565,8 +595,9 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         for (int it = 0; it < 2; ++it) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(Ad + (wave + 4 * it) * 256), 16,
                                                      last ? a_off_last[it] : a_off[it], 0, 0, 0);
+            const int bo = !flat ? b_off[it] : last && b_row_past_k[it] ? BUF_OOB : p.b_flat + it * (16 * 4) * g.ldb;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(Bd + (wave + 4 * it) * 256), 16,
-                                                     b_off[it], 0, 0, 0);
+                                                     bo, 0, 0, 0);
         }
     };
 
@@ -623,6 +654,10 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
         const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
         float* dst = cur.c + (size_t)row * g.ldc + col;
+        if (flat) {   // the chunk's image and pixel (a chunk never spans two images: batch_cols is a multiple of 4)
+            const unsigned img = g.by_batch_cols.div((unsigned)col);
+            dst = cur.c + (size_t)img * g.c_batch_stride + (size_t)row * g.ldc + ((unsigned)col - img * (unsigned)g.batch_cols);
+        }
         const int rows = g.M - row, valid = min(4, g.N - col);
         f32x4 v[4];
 #pragma unroll
@@ -669,17 +704,22 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
     }
 }
 
-__global__ void __launch_bounds__(256) sgemm_shortk_staged_kernel(const GemmArgs g)
-{
-    __shared__ __align__(16) float A0[2048];
-    __shared__ __align__(16) float A1[2048];
-    __shared__ __align__(16) float B0[2048];
-    __shared__ __align__(16) float B1[2048];
-    __shared__ __align__(16) float Stg[4 * 8 * 36];
-    float* const Ab[2] = {A0, A1};
-    float* const Bb[2] = {B0, B1};
-    shortk_staged_body<2>(g, Ab, Bb, Stg);
-}
+// (kernels by macro, not by template: with __shared__ arrays inside a kernel template the host
+// side of the launch did not link)
+#define SHORTK_STAGED_KERNEL(NAME, FLAT)                                                            \
+    __global__ void __launch_bounds__(256) NAME(const GemmArgs g)                                   \
+    {                                                                                               \
+        __shared__ __align__(16) float A0[2048];                                                    \
+        __shared__ __align__(16) float A1[2048];                                                    \
+        __shared__ __align__(16) float B0[2048];                                                    \
+        __shared__ __align__(16) float B1[2048];                                                    \
+        __shared__ __align__(16) float Stg[4 * 8 * 36];                                             \
+        float* const Ab[2] = {A0, A1};                                                              \
+        float* const Bb[2] = {B0, B1};                                                              \
+        shortk_staged_body<2, FLAT>(g, Ab, Bb, Stg);                                                \
+    }
+SHORTK_STAGED_KERNEL(sgemm_shortk_staged_kernel, false)
+SHORTK_STAGED_KERNEL(sgemm_shortk_staged_flat_kernel, true)   // a batch whose column tiles run across image borders
 
 // K at most 64, 16-byte-loadable row-major operands, no K slices, and at least a 64 x 64 tile per
 // CU.  Measured against the macro-tile kernel's own choice at K = 16 to 64: 0.79-0.98 of its time
@@ -708,7 +748,7 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
 {
     const long tiles = (long)args.tiles_m * args.tiles_n;
     if (tiles <= 0) return hipSuccess;
-    if (args.K > (args.tiles_n_per_image ? SHORTK_MAX_K_BATCH : SHORTK_MAX_K) || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
+    if (args.K > (args.tiles_n_per_image || args.batch_cols ? SHORTK_MAX_K_BATCH : SHORTK_MAX_K) || args.split_k != 1 || args.tail_tiles != 0 || args.partial) return hipErrorInvalidValue;
     int grid, lds;
     if (tile_n != 64) return hipErrorInvalidValue;
     const bool plain = !args.accumulate && !args.col_bias;
@@ -723,9 +763,14 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
         a2.by_group = FastDiv::make((unsigned)group);
         a2.by_last_group = FastDiv::make((unsigned)(args.tiles_m - (nbands - 1) * group));
         a2.by_image_tiles = FastDiv::make((unsigned)args.tiles_n_per_image);
+        a2.by_batch_cols = FastDiv::make((unsigned)args.batch_cols);
     }
+    if (args.batch_cols && (args.K <= 64 || args.batch_cols % 4 != 0 || args.tiles_n_per_image != 0 || args.N % args.batch_cols != 0 ||
+                            (double)args.b_batch_stride * (args.N / args.batch_cols) * 4.0 >= 2147483648.0))
+        return hipErrorInvalidValue;
     if (direct || args.K > 64) {
         if (direct) hipLaunchKernelGGL(sgemm_shortk_direct_kernel_32, dim3(grid), dim3(256), 0, stream, a2);
+        else if (args.batch_cols) hipLaunchKernelGGL(sgemm_shortk_staged_flat_kernel, dim3(grid), dim3(256), 0, stream, a2);
         else hipLaunchKernelGGL(sgemm_shortk_staged_kernel, dim3(grid), dim3(256), 0, stream, a2);
         return hipGetLastError();
     }

@@ -312,16 +312,19 @@ def test_cake_sconv_accumulates_the_direct_convolution(geom):
 @pytest.mark.parametrize("geom", [(16, 16, 56, 56, 256, 1, 1), (70, 7, 30, 30, 130, 1, 1), (256, 5, 21, 21, 100, 1, 1),
                                   (16, 64, 56, 56, 256, 1, 1), (16, 65, 56, 56, 256, 1, 1),
                                   # 65 to 256 channels, a multiple of 4: the batch runs in stages of 32 channels
-                                  (16, 128, 28, 28, 200, 1, 1), (12, 100, 30, 30, 130, 1, 1), (40, 68, 21, 21, 100, 1, 1),
-                                  (6, 256, 56, 56, 70, 1, 1), (32, 160, 14, 14, 512, 1, 1), (32, 192, 14, 14, 256, 1, 1)],
+                                  (16, 128, 28, 28, 200, 1, 1), (13, 100, 30, 30, 130, 1, 1), (40, 68, 21, 21, 100, 1, 1),
+                                  (6, 256, 56, 56, 70, 1, 1), (32, 160, 14, 14, 512, 1, 1), (32, 192, 14, 14, 256, 1, 1),
+                                  # planes that do not fill their last tile of 64 columns: tiles across image borders
+                                  (32, 256, 14, 14, 1024, 1, 1), (37, 192, 14, 14, 300, 1, 1), (150, 72, 10, 6, 200, 1, 1),
+                                  (13, 128, 26, 26, 640, 1, 1)],
                          ids=str)
 @pytest.mark.parametrize("nchw", [False, True])
 def test_conv2d_1x1_many_images(geom, nchw):
     """1 x 1 filters at stride 1 without padding and many tiles: every image is a plain product on
     the input as it lies, and the images are walked as a batch by the short-K kernels -- up to 64
     channels of any count, 65 to 256 when a multiple of 4 (65 stay on the gather path; so do 192
-    channels on 14 x 14 maps, whose 196 pixels leave a quarter of the column tiles empty) -- HW a
-    multiple of 64, of 4 only, and odd."""
+    channels on 32 maps of 14 x 14, fewer than two tiles per CU) -- HW a multiple of 64, of 4 only
+    (beyond 64 channels the column tiles then run across image borders), and odd."""
     Bn, Cin, Hin, Win, Cout, Hf, Wf = geom
     print(f"conv2d 1x1 geom={geom} nchw={nchw}", flush=True)
     inp = oracle.uniform((Bn, Cin, Hin, Win), 58)
@@ -333,7 +336,7 @@ def test_conv2d_1x1_many_images(geom, nchw):
     S = np.einsum("ok,bkp->bop", np.abs(w64), np.abs(x64))
     out = np.full((Bn, Cout, HW) if nchw else (Cout, Bn * HW), np.nan, np.float32)
     cake.conv2d(inp, wt, out, Bn, Cin, Hin, Win, Cout, 1, 1, 1, 0, out_nchw=nchw)
-    batch_route = Cin != 65 and not (Cin == 192 and HW == 196)
+    batch_route = Cin != 65 and not (Cin == 192 and HW == 196 and Bn == 32)
     assert cake.last_conv_route() == (cake.CONV_SHORTK_BATCH if batch_route else cake.CONV_GATHER)
     got = out if nchw else out.reshape(Cout, Bn, HW).transpose(1, 0, 2)
     assert np.max(np.abs(got - ref64) / np.maximum(S, 1e-30)) <= TIGHT
