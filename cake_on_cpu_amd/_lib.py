@@ -18,7 +18,8 @@ SCHED_NAMES = {KMN: "KMN", MKN: "MKN", NKM: "NKM", NA: "NA"}
 # Plan.kernel: which kernel family cake_hip_sgemm runs for a shape
 CONV_NONE, CONV_SHORTK_BATCH, CONV_PATCH, CONV_GATHER, CONV_TWO_STEP = range(5)   # cake_hip_last_conv_route
 KERNEL_NAMES = {0: "macro-tile", 1: "matrix-vector", 2: "streaming, few rows", 3: "streaming, few columns",
-                4: "short K, tiles walked by resident workgroups"}
+                4: "short K, tiles walked by resident workgroups",
+                5: "256 x 128 tiles walked by one resident workgroup per CU"}
 
 OK, ERR_ARG, ERR_NO_DEVICE, ERR_HIP, ERR_ALLOC, ERR_RANGE, ERR_ARCH = range(7)
 

@@ -573,6 +573,16 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
         st = scratch_space(cur().splitk, (size_t)plan.pub.split_k * M * N * sizeof(float), &g.partial);
         if (st) return st;
     }
+    // A plain product on 256 x 128 tiles with a K below 1024 and two tiles per CU or more: one
+    // workgroup per CU stays and walks over the tiles (sgemm_resident.hip).
+    // CAKE_HIP_GEMM_ROUTE=tile keeps the macro-tile kernel (for tests and measurements; read at every call).
+    if (plan.pub.tile_m == 256 && plan.pub.tile_n == 128 && plan.pub.split_k == 1 && plan.pub.tail_tiles == 0 && !conv &&
+        a_mode == LOAD_VEC4 && b_mode == LOAD_VEC4 &&
+        resident_applies(M, N, K, cur().model.cus, !accumulate && !col_bias, tile_override != nullptr)) {
+        const char* route = std::getenv("CAKE_HIP_GEMM_ROUTE");
+        if (!(route && !std::strcmp(route, "tile")))
+            return timer.family(0, [&] { return launch_sgemm_resident(g, cur().model.cus, stream); });
+    }
     st = timer.family(0, [&] { return launch_sgemm(plan.tile_id, a_mode, b_mode, g, plan.pub.grid, stream); });
     if (st) return st;
     if (plan.pub.split_k > 1)
@@ -866,6 +876,15 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
         out->tiles_m = (M + 63) / 64; out->tiles_n = (N + tn - 1) / tn;
         out->group = shortk_band_rows(out->tiles_m, N);
         shortk_launch_shape((long)out->tiles_m * out->tiles_n, tn, K, model.cus, &out->grid, &out->lds_bytes);
+    } else if (out->kernel == CAKE_HIP_KERNEL_TILE && vec && out->tile_m == 256 && out->tile_n == 128 && out->split_k == 1 &&
+               out->tail_tiles == 0 && resident_applies(M, N, K, model.cus, true, tile_override != nullptr)) {
+        // what launch_sgemm_resident does with the same tiles: one workgroup of 8 waves per CU
+        // that walks over them, its operands loaded straight into LDS
+        const long tiles = (long)out->tiles_m * out->tiles_n;
+        out->kernel = CAKE_HIP_KERNEL_RESIDENT;
+        out->threads = 512;
+        out->grid = (int)(((tiles < model.cus ? tiles : (long)model.cus) + 7) / 8 * 8);
+        out->lds_bytes = resident_lds_bytes();
     }
     return CAKE_HIP_OK;
 }

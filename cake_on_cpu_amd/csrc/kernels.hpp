@@ -158,6 +158,11 @@ inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1, bool sha
     return shortk_tile_n(M, N, K, cus, batch, shared_a) != 0;
 }
 hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStream_t stream);
+// sgemm_resident.hip: 256 x 128 tiles of a plain product walked by one resident workgroup per CU
+enum { RESIDENT_MAX_K = 1024 };   // from here on the macro-tile kernel
+bool resident_applies(int M, int N, int K, int cus, bool plain, bool forced);
+int resident_lds_bytes();
+hipError_t launch_sgemm_resident(const GemmArgs& args, int cus, hipStream_t stream);
 void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int* lds_bytes);
 // conv != nullptr: the columns are those of a convolution's product and go where conv_out_map says
 hipError_t launch_splitk_reduce(const float* partial, float* C, int M, int N, int ldc, int splits,

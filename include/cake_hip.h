@@ -84,7 +84,8 @@ enum {
     CAKE_HIP_KERNEL_GEMV = 1,
     CAKE_HIP_KERNEL_STREAM_ROWS = 2, /* few rows of A: B streamed once    */
     CAKE_HIP_KERNEL_STREAM_COLS = 3, /* few columns of B: A streamed once */
-    CAKE_HIP_KERNEL_SHORT_K = 4      /* short K (up to 160), many tiles: 64 x 64 tiles, next tile's operands in flight */
+    CAKE_HIP_KERNEL_SHORT_K = 4,     /* short K (up to 160), many tiles: 64 x 64 tiles, next tile's operands in flight */
+    CAKE_HIP_KERNEL_RESIDENT = 5     /* K below 1024 on 256 x 128 tiles, two or more per CU: one workgroup per CU walks over them */
 };
 
 /* What the GPU planner decided for one GEMM: the successor of

@@ -156,6 +156,8 @@ def test_plan_covers_any_shape(M, N, K):
         if pl.kernel == 4:   # short K: resident workgroups, as many as a CU's LDS holds, in whole rows of 8 XCDs
             per_cu = 5 if K <= 32 else 4
             assert pl.grid == (min(tiles, per_cu * pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
+        elif pl.kernel == 5:   # one resident workgroup per CU walks over the 256 x 128 tiles
+            assert pl.grid == (min(tiles, pl.cus) + 7) // 8 * 8 and pl.split_k == 1 and pl.tail_tiles == 0
         else:
             assert pl.grid == (tiles - pl.tail_tiles) * pl.split_k + pl.tail_tiles * pl.tail_split
         assert 1 <= pl.group <= max(pl.tiles_m, pl.tiles_n)
@@ -324,7 +326,7 @@ def test_plan_names_the_kernel_family():
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 127) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
-    assert fam(4096, 4096, 68) == 4 and fam(4096, 4096, 160) == 4 and fam(4096, 4096, 164) == 0 and fam(4096, 4096, 130) == 0
+    assert fam(4096, 4096, 68) == 4 and fam(4096, 4096, 160) == 4 and fam(4096, 4096, 164) == 5 and fam(4096, 4096, 130) == 0
     assert fam(960, 960, 128) == 0
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
@@ -342,6 +344,15 @@ def test_plan_names_the_kernel_family():
     q = cake.plan(250, 100352, 128)
     assert (q.kernel, q.tile_m, q.tile_n, q.tile_k, q.threads) == (4, 64, 64, 32, 256)
     assert q.grid == 4 * q.cus and 4 * q.lds_bytes <= 160 * 1024
+    # a K below 1024 (a multiple of 4) on 256 x 128 tiles, two or more per CU and no thin last round: one
+    # workgroup of 8 waves per CU walks over the tiles, 105 KB of LDS
+    r = cake.plan(8192, 8192, 256)
+    assert (r.kernel, r.tile_m, r.tile_n, r.tile_k, r.threads, r.split_k, r.tail_tiles) == (5, 256, 128, 32, 512, 1, 0)
+    assert r.grid == r.cus and r.lds_bytes == (2 * 256 * 32 + 2 * 32 * 128 + 8 * 8 * 36) * 4 <= 160 * 1024
+    assert fam(8192, 8192, 1020) == 5 and fam(8192, 8192, 1024) == 0 and fam(8192, 8192, 258) == 0
+    assert fam(2048, 2048, 256) == 0                                      # 128 tiles of 256 x 128: nothing to walk to
+    assert fam(700, 900, 520, tile=(256, 128, 32, 1)) == 5              # the caller named the tile (and no K slices): any tile count
+    assert fam(700, 900, 520, tile=(256, 128, 32, 3)) == 0              # K slices: the macro-tile kernel
     # (tiles 128 wide exist but lost every measurement: the choice never takes them)
     assert cake.plan(16384, 16384, 16).tile_n == 64 and cake.plan(2048, 2048, 16).tile_n == 64
     # the tile sequence runs in bands: all tile rows of a product up to 16 of them, else 4, 8 or 16

@@ -97,9 +97,10 @@ def test_large_b(big, M):
     _check(Cm[:, cols], A.double(), big[:, cols].double(), f"large B, M={M}")
 
 
-def test_large_c():
-    """C of 4.6 GB from a short K: the epilogue's addressing."""
-    K = 24
+@pytest.mark.parametrize("K", [24, 48, 100])
+def test_large_c(K):
+    """C of 4.6 GB from a short K: the epilogue's addressing in each of the three kernels that walk
+    over tiles (K up to 32, up to 64, beyond)."""
     A, B = _filled((R, K), 905), _filled((K, R), 906)
     Cm = torch.empty((R, R), dtype=torch.float32, device=_dev())
     Cm.fill_(float("nan"))

@@ -75,9 +75,10 @@ TILES = [(256, 256, 32), (256, 128, 32), (128, 256, 32), (128, 128, 32), (64, 64
                          ids=lambda s: "x".join(map(str, s)))
 def test_every_tile_shape(tile, shape):
     """Each macro-tile instantiation, on aligned (16-byte loader) and ragged
-    (scalar loader) operands, without and with split-K."""
+    (scalar loader) operands, with the planner's choice of K slices, a single one (on 256 x 128
+    tiles with K a multiple of 4 that is the kernel of resident workgroups) and three."""
     M, K, N = shape
-    for split in (0, 3):
+    for split in (0, 1, 3):
         print(f"sgemm tile={tile} split={split} M={M} K={K} N={N}", flush=True)
         A, B, Cm = _run(M, K, N, cake.KMN, tile=tile + (split,))
         _check(A, B, Cm, None, (tile, shape, split))
@@ -230,6 +231,42 @@ def test_short_k_many_tiles(shape):
     _, _, acc = _run(M, K, N, cake.MKN, C0=C0, beta=1.0)
     assert np.allclose(acc - Cm, C0, atol=2e-4)
     assert np.array_equal(_run(M, K, N)[2], Cm)
+
+
+@pytest.mark.parametrize("shape", [(4096, 256, 4096), (4000, 516, 4090), (6144, 388, 4096), (2048, 32, 8192 * 2), (8192, 1020, 4096),
+                                   (5000, 300, 4100), (4096, 1024, 4096), (4096, 258, 4096)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_resident_workgroups_walk_256x128_tiles(shape, monkeypatch):
+    """K below 1024 (a multiple of 4) on 256 x 128 tiles, two or more per CU: one workgroup per CU
+    walks over the tiles with both operands loaded straight into LDS.  Ragged last tile rows and
+    columns, a last stage of 4 k, rows of B that are not 16-byte aligned; the last three shapes stay
+    on (or may stay on) the macro-tile kernel.  Same bits as that kernel: both sum k in order."""
+    M, K, N = shape
+    pl = cake.plan(M, N, K)
+    if shape in [(4096, 256, 4096), (4000, 516, 4090), (6144, 388, 4096), (8192, 1020, 4096)]:
+        assert pl.kernel == 5, pl.as_dict()
+    if shape in [(4096, 1024, 4096), (4096, 258, 4096)]:
+        assert pl.kernel == 0, pl.as_dict()
+    print(f"sgemm resident M={M} K={K} N={N} kernel={pl.kernel}", flush=True)
+    import torch
+    A, B = oracle.uniform((M, K), 1), oracle.uniform((K, N), 2)
+    tA, tB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()     # on the device: host operands of this size go through in blocks of rows
+
+    def run(beta=0.0, sch=cake.NA, C0=None):
+        tC = torch.full((M, N), float("nan"), device="cuda") if C0 is None else torch.from_numpy(C0).cuda()
+        cake.cake_sgemm(tA, tB, tC, M, N, K, 4, None, None, False, False, 1.0, beta, sch)
+        torch.cuda.synchronize()
+        return tC.cpu().numpy()
+
+    Cm = run()
+    _check(A, B, Cm, None, shape)
+    assert np.array_equal(run(), Cm)
+    monkeypatch.setenv("CAKE_HIP_GEMM_ROUTE", "tile")
+    assert np.array_equal(run(), Cm)
+    monkeypatch.delenv("CAKE_HIP_GEMM_ROUTE")
+    C0 = oracle.uniform((M, N), 3)
+    acc = run(1.0, cake.MKN, C0)                               # accumulation: the macro-tile kernel
+    assert np.allclose(acc - Cm, C0, atol=2e-4)
 
 
 def test_random_shapes_against_fp64():
