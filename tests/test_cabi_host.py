@@ -349,7 +349,7 @@ def test_plan_names_the_kernel_family():
     r = cake.plan(8192, 8192, 256)
     assert (r.kernel, r.tile_m, r.tile_n, r.tile_k, r.threads, r.split_k, r.tail_tiles) == (5, 256, 128, 32, 512, 1, 0)
     assert r.grid == r.cus and r.lds_bytes == (2 * 256 * 32 + 2 * 32 * 128 + 8 * 8 * 36) * 4 <= 160 * 1024
-    assert fam(8192, 8192, 1020) == 5 and fam(8192, 8192, 1024) == 0 and fam(8192, 8192, 258) == 0
+    assert fam(8192, 8192, 1020) == 5 and fam(8192, 8192, 1024) == 0 and fam(8192, 8192, 258) == 0 and fam(8192, 8190, 256) == 0
     assert fam(2048, 2048, 256) == 0                                      # 128 tiles of 256 x 128: nothing to walk to
     assert fam(700, 900, 520, tile=(256, 128, 32, 1)) == 5              # the caller named the tile (and no K slices): any tile count
     assert fam(700, 900, 520, tile=(256, 128, 32, 3)) == 0              # K slices: the macro-tile kernel

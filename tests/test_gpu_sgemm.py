@@ -233,19 +233,21 @@ def test_short_k_many_tiles(shape):
     assert np.array_equal(_run(M, K, N)[2], Cm)
 
 
-@pytest.mark.parametrize("shape", [(4096, 256, 4096), (4000, 516, 4090), (6144, 388, 4096), (2048, 32, 8192 * 2), (8192, 1020, 4096),
-                                   (5000, 300, 4100), (4096, 1024, 4096), (4096, 258, 4096)],
+@pytest.mark.parametrize("shape", [(4096, 256, 4096), (4000, 516, 4092), (6144, 388, 4096), (2048, 32, 8192 * 2), (8192, 1020, 4096),
+                                   (4010, 36, 8100), (5000, 300, 4100), (4096, 1024, 4096), (4096, 258, 4096), (4000, 516, 4090)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_resident_workgroups_walk_256x128_tiles(shape, monkeypatch):
-    """K below 1024 (a multiple of 4) on 256 x 128 tiles, two or more per CU: one workgroup per CU
-    walks over the tiles with both operands loaded straight into LDS.  Ragged last tile rows and
-    columns, a last stage of 4 k, rows of B that are not 16-byte aligned; the last three shapes stay
-    on (or may stay on) the macro-tile kernel.  Same bits as that kernel: both sum k in order."""
+    """K below 1024 on 256 x 128 tiles, two or more per CU, K and N multiples of 4: one workgroup
+    per CU walks over the tiles with both operands loaded straight into LDS and writes a finished
+    tile out under the next one's first stage.  Ragged last tile rows and columns, a last stage of
+    4 k, a single stage per tile (every unit then starts a tile and writes one out), rows of B and
+    C that are not 16-byte aligned; the last four shapes stay on (or may stay on) the macro-tile
+    kernel.  Same bits as that kernel: both sum k in order."""
     M, K, N = shape
     pl = cake.plan(M, N, K)
-    if shape in [(4096, 256, 4096), (4000, 516, 4090), (6144, 388, 4096), (8192, 1020, 4096)]:
+    if shape in [(4096, 256, 4096), (4000, 516, 4092), (6144, 388, 4096), (8192, 1020, 4096)]:
         assert pl.kernel == 5, pl.as_dict()
-    if shape in [(4096, 1024, 4096), (4096, 258, 4096)]:
+    if shape in [(4096, 1024, 4096), (4096, 258, 4096), (4000, 516, 4090)]:
         assert pl.kernel == 0, pl.as_dict()
     print(f"sgemm resident M={M} K={K} N={N} kernel={pl.kernel}", flush=True)
     import torch
