@@ -521,8 +521,27 @@ int run_gemm(const float* A, const float* B, float* C, int M, int N, int K, int 
     // tile's columns in the image, paid per tile instead of once per workgroup, cost more than
     // the overlap gives -- 1 x 1, 64 -> 256 channels on 56 x 56: 56 us against 50 us)
     // (beyond 64 k only where C is overwritten without a bias: that kernel has no other epilogue)
-    if (vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, vec_plan, nullptr) &&
-        shortk_applies(M, N, K, cur().model.cus) && (K <= 64 || (!accumulate && !col_bias))) {
+    const bool shortk_ok = vec && !conv && !choice && !tile_override && !tune_lookup(M, N, K, vec_plan, nullptr) &&
+                           shortk_applies(M, N, K, cur().model.cus) && (K <= 64 || (!accumulate && !col_bias));
+    // (with very many tiles and K in whole stages of 32 the walk over 256 x 128 tiles is the faster one)
+    if (shortk_ok && !accumulate && !col_bias && b_mode == LOAD_VEC4 && resident_beats_shortk(M, N, K, cur().model.cus) &&
+        (double)256 * ldc * 4.0 < 2147483648.0) {
+        static const int big_tile[4] = {256, 128, 32, 1};
+        GemmPlan plan;
+        const char* route = std::getenv("CAKE_HIP_GEMM_ROUTE");
+        if (!(route && !std::strcmp(route, "tile")) && plan_gemm(M, N, K, sched, big_tile, vec_plan, cur().model, &plan) == CAKE_HIP_OK &&
+            plan.pub.split_k == 1 && plan.pub.tail_tiles == 0) {
+            GemmArgs g{};
+            g.A = A; g.B = B; g.C = C;
+            g.M = M; g.N = N; g.K = K;
+            g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+            g.tiles_m = plan.pub.tiles_m; g.tiles_n = plan.pub.tiles_n;
+            g.split_k = 1; g.k_per_split = plan.k_per_split;
+            g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
+            return timer.family(0, [&] { return launch_sgemm_resident(g, cur().model.cus, stream); });
+        }
+    }
+    if (shortk_ok) {
         GemmArgs g{};
         g.A = A; g.B = B; g.C = C;
         g.M = M; g.N = N; g.K = K;
@@ -865,6 +884,15 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
     if (st) return fail(st, "cake_hip_plan: bad shape, schedule or tile override");
     *out = plan.pub;
     out->kernel = kernel_family(M, N, K, tile_override != nullptr, vec);
+    if (out->kernel == CAKE_HIP_KERNEL_SHORT_K && resident_beats_shortk(M, N, K, model.cus)) {
+        // very many tiles, K in whole stages of 32: the walk over 256 x 128 tiles instead
+        static const int big_tile[4] = {256, 128, 32, 1};
+        GemmPlan big;
+        if (plan_gemm(M, N, K, sched, big_tile, vec, model, &big) == CAKE_HIP_OK && big.pub.split_k == 1 && big.pub.tail_tiles == 0) {
+            *out = big.pub;
+            out->kernel = CAKE_HIP_KERNEL_TILE;   // (named below)
+        }
+    }
     if (out->kernel == CAKE_HIP_KERNEL_SHORT_K) {
         // what launch_sgemm_shortk does: 64 x 64 tiles with the whole K in one LDS stage, walked in
         // column blocks of B by the resident workgroups per CU
@@ -877,7 +905,8 @@ int cake_hip_plan(int M, int N, int K, int sched, const int* tile_override, cake
         out->group = shortk_band_rows(out->tiles_m, N);
         shortk_launch_shape((long)out->tiles_m * out->tiles_n, tn, K, model.cus, &out->grid, &out->lds_bytes);
     } else if (out->kernel == CAKE_HIP_KERNEL_TILE && vec && out->tile_m == 256 && out->tile_n == 128 && out->split_k == 1 &&
-               out->tail_tiles == 0 && resident_applies(M, N, K, model.cus, true, tile_override != nullptr)) {
+               out->tail_tiles == 0 &&
+               (resident_applies(M, N, K, model.cus, true, tile_override != nullptr) || (!tile_override && resident_beats_shortk(M, N, K, model.cus)))) {
         // what launch_sgemm_resident does with the same tiles: one workgroup of 8 waves per CU
         // that walks over them, its operands loaded straight into LDS
         const long tiles = (long)out->tiles_m * out->tiles_n;

@@ -161,6 +161,7 @@ hipError_t launch_sgemm_shortk(const GemmArgs& args, int tile_n, int cus, hipStr
 // sgemm_resident.hip: 256 x 128 tiles of a plain product walked by one resident workgroup per CU
 enum { RESIDENT_MAX_K = 1024 };   // from here on the macro-tile kernel
 bool resident_applies(int M, int N, int K, int cus, bool plain, bool forced);
+bool resident_beats_shortk(int M, int N, int K, int cus);   // where sgemm_shortk.hip applies as well
 int resident_lds_bytes();
 hipError_t launch_sgemm_resident(const GemmArgs& args, int cus, hipStream_t stream);
 void shortk_launch_shape(long tiles, int tile_n, int K, int cus, int* grid, int* lds_bytes);

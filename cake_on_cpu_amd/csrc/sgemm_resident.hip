@@ -362,6 +362,26 @@ bool resident_applies(int M, int N, int K, int cus, bool plain, bool forced)
     return forced || tiles >= 2L * cus;
 }
 
+// A short K (32 to 160) under very many tiles, where the 64 x 64 walks of sgemm_shortk.hip apply:
+// this kernel's larger tiles win when K is whole stages (those kernels multiply only the groups
+// of 8 k that exist, this one whole stages of 32), the tiles fill their rounds and the matrix to
+// 90 %, and there are three rounds or more -- two from K = 96 on.  Measured, same device and run,
+// us 64 x 64 walk -> this kernel: 8192^2 x 32 59.1 -> 53.5, x 64 91.3 -> 85.3, x 96 128.1 -> 109.3,
+// x 128 163.5 -> 136.5, x 160 192.9 -> 163.8; 12288^2 x 64 206.1 -> 182.4; 16384^2 x 64 365.3 -> 326.2;
+// 4096 x 16384 x 96 129.3 -> 113.2; 3072 x 8192 x 128 62.0 -> 55.7; 7000 x 9000 x 64 87.8 -> 80.5;
+// 4096^2 x 128 41.7 -> 39.7 (two rounds); against it: 8192^2 x 48 75.3 -> 81.9 (a stage half
+// empty), 5120^2 x 64 35.6 -> 40.8 (3.1 rounds cost 4), 4096^2 x 64 27.9 -> 28.2 and x 32 18.4 ->
+// 19.6 (two rounds), 256 x 100352 x 64 36.9 -> 42.2 (3.06 rounds), 2048^2 x 64 9.7 -> 13.8.
+bool resident_beats_shortk(int M, int N, int K, int cus)
+{
+    if (K < RES_BK || K > SHORTK_MAX_K || K % RES_BK != 0 || N % 4 != 0) return false;
+    const long tiles_m = (M + RES_BM - 1) / RES_BM, tiles_n = (N + RES_BN - 1) / RES_BN, tiles = tiles_m * tiles_n;
+    const long rounds = (tiles + cus - 1) / cus;
+    if (10 * tiles < 9 * rounds * cus) return false;                                           // the rounds filled to 90 %
+    if (10.0 * M * N < 9.0 * (double)(tiles_m * RES_BM) * (double)(tiles_n * RES_BN)) return false;   // and the tiles
+    return tiles >= 3L * cus || (K >= 96 && tiles >= 2L * cus);
+}
+
 int resident_lds_bytes() { return (2 * RES_BM * RES_BK + 2 * RES_BK * RES_BN + 8 * 8 * RES_STG_PITCH) * 4; }
 
 // args: tiles_m, tiles_n, group, group_along_n set for 256 x 128 tiles; split_k = 1, no tail tiles

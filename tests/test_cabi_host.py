@@ -326,7 +326,7 @@ def test_plan_names_the_kernel_family():
     assert fam(16, 511, 4096) == 0 and fam(16, 4096, 127) == 0 and fam(16, 16, 100000) == 0
     assert fam(1024, 1024, 1024) == 0
     assert fam(4096, 4096, 64) == 4 and fam(4096, 4096, 65) == 0 and fam(1024, 1024, 64) == 4 and fam(960, 960, 64) == 0   # short K, a tile per CU
-    assert fam(4096, 4096, 68) == 4 and fam(4096, 4096, 160) == 4 and fam(4096, 4096, 164) == 5 and fam(4096, 4096, 130) == 0
+    assert fam(4096, 4096, 68) == 4 and fam(4096, 4096, 144) == 4 and fam(4096, 4096, 164) == 5 and fam(4096, 4096, 130) == 0
     assert fam(960, 960, 128) == 0
     assert fam(16, 16384, 16384, tile=(64, 64, 64)) == 0
     assert cake.KERNEL_NAMES[fam(8, 2048, 2048)] == "streaming, few rows"
@@ -351,6 +351,12 @@ def test_plan_names_the_kernel_family():
     assert r.grid == r.cus and r.lds_bytes == (2 * 256 * 32 + 2 * 32 * 128 + 8 * 8 * 36) * 4 <= 160 * 1024
     assert fam(8192, 8192, 1020) == 5 and fam(8192, 8192, 1024) == 0 and fam(8192, 8192, 258) == 0 and fam(8192, 8190, 256) == 0
     assert fam(2048, 2048, 256) == 0                                      # 128 tiles of 256 x 128: nothing to walk to
+    # where the 64 x 64 walks apply as well (K up to 160): the large tiles when K is whole stages of 32 and the
+    # tiles fill three rounds or more (two from K = 96 on) to 90 %
+    assert fam(8192, 8192, 64) == 5 and fam(8192, 8192, 32) == 5 and fam(4096, 4096, 160) == 5 and fam(4096, 4096, 96) == 5
+    assert fam(4096, 4096, 64) == 4 and fam(8192, 8192, 48) == 4 and fam(5120, 5120, 64) == 4 and fam(8192, 8192, 16) == 4
+    r = cake.plan(8192, 8192, 64)
+    assert (r.tile_m, r.tile_n, r.threads, r.grid, r.split_k, r.tail_tiles) == (256, 128, 512, r.cus, 1, 0)
     assert fam(700, 900, 520, tile=(256, 128, 32, 1)) == 5              # the caller named the tile (and no K slices): any tile count
     assert fam(700, 900, 520, tile=(256, 128, 32, 3)) == 0              # K slices: the macro-tile kernel
     # (tiles 128 wide exist but lost every measurement: the choice never takes them)
@@ -358,7 +364,7 @@ def test_plan_names_the_kernel_family():
     # the tile sequence runs in bands: all tile rows of a product up to 16 of them, else 4, 8 or 16
     # tile rows, lower for wider products
     assert p.group == 4 and cake.plan(1024, 50176, 64).group == 16
-    assert cake.plan(16384, 16384, 16).group == 4 and cake.plan(8192, 8192, 32).group == 8
+    assert cake.plan(16384, 16384, 16).group == 4 and cake.plan(8192, 8192, 24).group == 8
     assert cake.plan(16384, 4096, 16).group == 16
 
 

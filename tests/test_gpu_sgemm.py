@@ -234,6 +234,8 @@ def test_short_k_many_tiles(shape):
 
 
 @pytest.mark.parametrize("shape", [(4096, 256, 4096), (4000, 516, 4092), (6144, 388, 4096), (2048, 32, 8192 * 2), (8192, 1020, 4096),
+                                   # K up to 160 in whole stages of 32 under three rounds of tiles or more: taken from the 64 x 64 walks
+                                   (8192, 64, 8192), (8192, 32, 8192), (6000, 96, 8192), (4096, 160, 4096),
                                    (4010, 36, 8100), (5000, 300, 4100), (4096, 1024, 4096), (4096, 258, 4096), (4000, 516, 4090)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_resident_workgroups_walk_256x128_tiles(shape, monkeypatch):
@@ -245,7 +247,7 @@ def test_resident_workgroups_walk_256x128_tiles(shape, monkeypatch):
     kernel.  Same bits as that kernel: both sum k in order."""
     M, K, N = shape
     pl = cake.plan(M, N, K)
-    if shape in [(4096, 256, 4096), (4000, 516, 4092), (6144, 388, 4096), (8192, 1020, 4096)]:
+    if shape in [(4096, 256, 4096), (4000, 516, 4092), (6144, 388, 4096), (8192, 1020, 4096), (8192, 64, 8192), (8192, 32, 8192), (6000, 96, 8192), (4096, 160, 4096)]:
         assert pl.kernel == 5, pl.as_dict()
     if shape in [(4096, 1024, 4096), (4096, 258, 4096), (4000, 516, 4090)]:
         assert pl.kernel == 0, pl.as_dict()
