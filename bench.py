@@ -405,8 +405,8 @@ def main() -> int:
             other_extras.append(gemm_extra("sgemm short K, many tiles: M=256 K=64 N=100352", 256, 100352, 64, "shortk_256x64x100352"))
             other_extras.append(gemm_extra("sgemm mid K on 256 x 128 tiles walked by resident workgroups: M=8192 K=256 N=8192",
                                            8192, 8192, 256, "resident_8192x256x8192", bound="mfma"))
-            other_extras.append(gemm_extra("sgemm mid K, resident workgroups: M=4096 K=512 N=4096", 4096, 4096, 512, bound="mfma"))
-            other_extras.append(gemm_extra("sgemm K = 128, 64 x 64 tiles walked stage by stage: M=4096 K=128 N=4096", 4096, 4096, 128, bound="mfma"))
+            other_extras.append(gemm_extra("sgemm K = 100, 64 x 64 tiles walked stage by stage: M=3000 K=100 N=3000", 3000, 3000, 100,
+                                           "staged_3000x100x3000", bound="mfma"))
             other_extras.append(gemm_extra("sgemm 16 rows: M=16 K=16384 N=16384", 16, 16384, 16384, "fewrows_nn",
                                            "sgemm_fewrows_nn_kernel + splitk_reduce_kernel", rotate="B"))
             other_extras.append(gemm_extra("sgemm 16 columns: M=16384 K=16384 N=16", 16384, 16, 16384, "fewrows_nt",

@@ -25,6 +25,29 @@ namespace cake {
 // 64 x 64 tiles of C, 4 waves of 32 x 32; BK is the longest K it takes
 using TileShortK64 = Tile<64, 64, 64, 32, 32>;
 
+// The four pieces of a wave's 32 x 32 block (8 rows x 32 columns each, a lane holding 16 bytes of a
+// row) stored into a tile whose rows of C are whole 16-byte chunks: through a buffer resource that
+// starts at the tile's first element and ends with C, so rows past M are out of range by
+// themselves, a lane past N gets an out-of-range offset, and the rest of a piece's address is a
+// scalar -- no vector arithmetic per piece (every regular vector instruction costs the matrix
+// pipe four cycles on this hardware: none is issued beside an MFMA).
+// c_lane: bytes from a piece's first element to the lane's 16 bytes, (row in piece * ldc + column) * 4.
+__device__ __forceinline__ void store_block_pieces(const GemmArgs& g, float* c, int m0, int n0, int wm0, int wn0, int rd_col, int c_lane,
+                                                   const f32x4 (&v)[4])
+{
+    const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(
+        c + (size_t)m0 * g.ldc + n0, 0, (int)records_left(clamp_elems((long long)(g.M - 1 - m0) * g.ldc + g.N - n0), 0u), 0x00020000);
+    const int off = n0 + wn0 + rd_col < g.N ? c_lane : BUF_OOB;
+#pragma unroll
+    for (int P = 0; P < 4; ++P)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v[P]), rc, off, ((wm0 + 8 * P) * g.ldc + wn0) * 4, 0);
+}
+// whole 16-byte chunks per row of C, and offsets within a tile that fit 31 bits
+__device__ __forceinline__ bool c_in_whole_chunks(const GemmArgs& g, int tile_rows)
+{
+    return (g.N & 3) == 0 && (long long)tile_rows * g.ldc * 4 < 2147483647ll;
+}
+
 // one stage of each operand and, behind them, 8 rows of staging per wave for the epilogue that overwrites C
 template <class T>
 static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE + T::WAVES_M * T::WAVES_N * 8 * (T::WN + 4)) * 4; }
@@ -47,7 +70,7 @@ static constexpr int shortk_lds_bytes() { return (T::A_STAGE + T::B_STAGE + T::W
 //     are issued: loads and stores share one counter of outstanding operations, so a wait placed
 //     after the stores would wait for their round trip to memory as well.
 template <class T, int B_MODE, bool PLAIN>
-__global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs g)
+__global__ void __launch_bounds__(T::THREADS) __attribute__((amdgpu_waves_per_eu(4))) sgemm_shortk_kernel(const GemmArgs g)
 {
     static_assert(B_MODE == LOAD_VEC4, "row-major operands");
     static_assert(T::KSPLIT == 1, "one wave per block of C");
@@ -88,6 +111,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
         b_off[it] = k < g.K ? (k * g.ldb + (c % (T::BN / 4)) * 4) * 4 : BUF_OOB;
     }
     const bool ragged_k = (g.K & 3) != 0;     // then an A chunk can straddle K and is masked when it is stored
+    const bool c_whole_chunks = c_in_whole_chunks(g, T::BM);
+    const int c_lane = (((tid & 63) >> 3) * g.ldc + (tid & 7) * 4) * 4;   // bytes from a piece's first element to the lane's 16 bytes
 
     // tile number -> origin of the tile, the operands' base addresses and record counts
     struct Place {
@@ -165,20 +190,33 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
             load_b(nxt);
         }
 
+        // (the tile's first MFMA starts from a constant zero: nothing is cleared.  Every regular
+        // vector instruction costs the matrix pipe four cycles on this hardware -- none is issued
+        // beside an MFMA -- and a tile has only 32 MFMAs per wave to set against them.)
         f32x16 acc[T::TM][T::TN];
-#pragma unroll
-        for (int tm = 0; tm < T::TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < T::TN; ++tn)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         Frag<T> frag[2];
         load_frag<T>(As, Bs, a_lane, b_lane, lh, 0, frag[0]);
 #pragma unroll
         for (int kg = 0; kg < T::BK / 8; ++kg) {
             if (kg < groups) {   // uniform: K is the same for everyone
                 if (kg + 1 < T::BK / 8) load_frag<T>(As, Bs, a_lane, b_lane, lh, kg + 1, frag[(kg + 1) & 1]);
-                mma_frag<T>(frag[kg & 1], acc);
+                if (kg == 0) {
+#pragma unroll
+                    for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+                        for (int tn = 0; tn < T::TN; ++tn)
+                            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag[0].a[tm][0], frag[0].b[tn][0], zero, 0, 0, 0);
+#pragma unroll
+                    for (int i = 1; i < 4; ++i)
+#pragma unroll
+                        for (int tm = 0; tm < T::TM; ++tm)
+#pragma unroll
+                            for (int tn = 0; tn < T::TN; ++tn)
+                                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag[0].a[tm][i], frag[0].b[tn][i], acc[tm][tn], 0, 0, 0);
+                } else {
+                    mma_frag<T>(frag[kg & 1], acc);
+                }
             }
         }
         if (PLAIN) {
@@ -196,9 +234,6 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
             constexpr int PITCH = T::WN + 4;
             float* stg = smem + T::A_STAGE + T::B_STAGE + wave * (8 * PITCH);
             const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
-            const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
-            float* dst = cur.c + (size_t)row * g.ldc + col;
-            const int rows = g.M - row, valid = min(4, g.N - col);
             // LDS serves a wave's requests in order: a piece's read sees its writes, and the next
             // piece's writes come after it.  All four pieces are therefore issued back to back and
             // the stores follow as the reads return.
@@ -210,16 +245,23 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_shortk_kernel(const GemmArgs
                 v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (c_whole_chunks) {
+                store_block_pieces(g, cur.c, cur.m0, cur.n0, wm0, wn0, rd_col, c_lane, v);
+            } else {
+                const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+                float* dst = cur.c + (size_t)row * g.ldc + col;
+                const int rows = g.M - row, valid = min(4, g.N - col);
 #pragma unroll
-            for (int P = 0; P < 4; ++P) {
-                if (8 * P < rows && valid > 0) {
-                    float* d = dst + (size_t)(8 * P) * g.ldc;
-                    if (valid == 4) {
-                        *reinterpret_cast<f32x4_u*>(d) = v[P];
-                    } else {
+                for (int P = 0; P < 4; ++P) {
+                    if (8 * P < rows && valid > 0) {
+                        float* d = dst + (size_t)(8 * P) * g.ldc;
+                        if (valid == 4) {
+                            *reinterpret_cast<f32x4_u*>(d) = v[P];
+                        } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (e < valid) d[e] = v[P][e];
+                            for (int e = 0; e < 4; ++e)
+                                if (e < valid) d[e] = v[P][e];
+                        }
                     }
                 }
             }
@@ -282,6 +324,8 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
     const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
     const int b_lane = wn0 + l32;
     float* stg = Stg + wave * (8 * PITCH);
+    const bool c_whole_chunks = c_in_whole_chunks(g, 64);
+    const int c_lane = ((lane >> 3) * g.ldc + (lane & 7) * 4) * 4;
 
     const int groups = (g.K + 7) >> 3;
     const int tiles_all = g.tiles_m * g.tiles_n;
@@ -385,9 +429,8 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
             if (a_fresh) load_a(nxt);
             issue_b(Bn, nxt);
         }
-        f32x16 acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        f32x16 acc;   // (the tile's first MFMA starts from a constant zero: nothing is cleared)
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         f32x4 fa[2];
         float fb[2][4];
         auto fetch = [&](int kg, f32x4& a, float (&b)[4]) {
@@ -403,7 +446,7 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
                 if (kg + 1 < BK / 8) fetch(kg + 1, fa[(kg + 1) & 1], fb[(kg + 1) & 1]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kg & 1][i], fb[kg & 1][i], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kg & 1][i], fb[kg & 1][i], kg == 0 && i == 0 ? zero : acc, 0, 0, 0);
             }
         }
         // the next tile's operands have had the tile's MFMAs to arrive; no store is outstanding
@@ -413,9 +456,6 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
         __builtin_amdgcn_sched_barrier(0);
         // the wave's block, turned around in pieces of 8 rows through its own staging block
         const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
-        const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
-        float* dst = cur.c + (size_t)row * g.ldc + col;
-        const int rows = g.M - row, valid = min(4, g.N - col);
         f32x4 v[4];
 #pragma unroll
         for (int P = 0; P < 4; ++P) {
@@ -424,6 +464,13 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
             v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (c_whole_chunks) {
+            store_block_pieces(g, cur.c, cur.m0, cur.n0, wm0, wn0, rd_col, c_lane, v);
+            return;
+        }
+        const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+        float* dst = cur.c + (size_t)row * g.ldc + col;
+        const int rows = g.M - row, valid = min(4, g.N - col);
 #pragma unroll
         for (int P = 0; P < 4; ++P) {
             if (8 * P < rows && valid > 0) {
@@ -453,7 +500,7 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
 // (the LDS arrays are separate objects on purpose: the compiler then knows that reads of one B
 // buffer need not wait for loads into the other)
 #define SHORTK_DIRECT_KERNEL(BK)                                                                    \
-    __global__ void __launch_bounds__(256) sgemm_shortk_direct_kernel_##BK(const GemmArgs g)        \
+    __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) sgemm_shortk_direct_kernel_##BK(const GemmArgs g)        \
     {                                                                                               \
         __shared__ __align__(16) float As[64 * BK];                                                 \
         __shared__ __align__(16) float B0[BK * 64];                                                 \
@@ -510,6 +557,8 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
     const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
     const int b_lane = wn0 + l32;
     float* stg = Stg + wave * (8 * PITCH);
+    const bool c_whole_chunks = !FLAT && c_in_whole_chunks(g, 64);   // (across image borders a lane's place in C is not the tile's plus a constant)
+    const int c_lane = ((lane >> 3) * g.ldc + (lane & 7) * 4) * 4;
 
     const int stages = (g.K + BK - 1) / BK;
     const int tiles_all = g.tiles_m * g.tiles_n;
@@ -652,13 +701,6 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
         if (++ks < stages) return true;
         // the tile is finished: the wave's block, turned around in pieces of 8 rows through its own staging block
         const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;
-        const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
-        float* dst = cur.c + (size_t)row * g.ldc + col;
-        if (flat) {   // the chunk's image and pixel (a chunk never spans two images: batch_cols is a multiple of 4)
-            const unsigned img = g.by_batch_cols.div((unsigned)col);
-            dst = cur.c + (size_t)img * g.c_batch_stride + (size_t)row * g.ldc + ((unsigned)col - img * (unsigned)g.batch_cols);
-        }
-        const int rows = g.M - row, valid = min(4, g.N - col);
         f32x4 v[4];
 #pragma unroll
         for (int P = 0; P < 4; ++P) {
@@ -667,16 +709,27 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
             v[P] = *reinterpret_cast<const f32x4*>(stg + rd_row * PITCH + rd_col);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (c_whole_chunks) {
+            store_block_pieces(g, cur.c, cur.m0, cur.n0, wm0, wn0, rd_col, c_lane, v);
+        } else {
+            const int row = cur.m0 + wm0 + rd_row, col = cur.n0 + wn0 + rd_col;
+            float* dst = cur.c + (size_t)row * g.ldc + col;
+            if (flat) {   // the chunk's image and pixel (a chunk never spans two images: batch_cols is a multiple of 4)
+                const unsigned img = g.by_batch_cols.div((unsigned)col);
+                dst = cur.c + (size_t)img * g.c_batch_stride + (size_t)row * g.ldc + ((unsigned)col - img * (unsigned)g.batch_cols);
+            }
+            const int rows = g.M - row, valid = min(4, g.N - col);
 #pragma unroll
-        for (int P = 0; P < 4; ++P) {
-            if (8 * P < rows && valid > 0) {
-                float* d = dst + (size_t)(8 * P) * g.ldc;
-                if (valid == 4) {
-                    *reinterpret_cast<f32x4_u*>(d) = v[P];
-                } else {
+            for (int P = 0; P < 4; ++P) {
+                if (8 * P < rows && valid > 0) {
+                    float* d = dst + (size_t)(8 * P) * g.ldc;
+                    if (valid == 4) {
+                        *reinterpret_cast<f32x4_u*>(d) = v[P];
+                    } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (e < valid) d[e] = v[P][e];
+                        for (int e = 0; e < 4; ++e)
+                            if (e < valid) d[e] = v[P][e];
+                    }
                 }
             }
         }
@@ -707,7 +760,7 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
 // (kernels by macro, not by template: with __shared__ arrays inside a kernel template the host
 // side of the launch did not link)
 #define SHORTK_STAGED_KERNEL(NAME, FLAT)                                                            \
-    __global__ void __launch_bounds__(256) NAME(const GemmArgs g)                                   \
+    __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) NAME(const GemmArgs g)                                   \
     {                                                                                               \
         __shared__ __align__(16) float A0[2048];                                                    \
         __shared__ __align__(16) float A1[2048];                                                    \
