@@ -1554,8 +1554,22 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         // tiles of a thin last round are cut along K in whole channel blocks, or -- when the plan asks
         // for more slices than there are blocks and half a block still has the three taps a walk
         // needs -- in halves of a block's taps (config 5: 16 tiles in 16 slices of 5 and 4 taps)
+        // -- or, under 3 x 3 filters, not cut along K at all: 16 workgroups per tail tile compute
+        // 64 rows x 32 pixels each over the whole K, no partial sums in memory and no second kernel
+        // (CAKE_HIP_CONV_TAIL=slices|subtiles overrides the choice; for tests and measurements)
         int grid = g.tiles_m * g.tiles_n;
-        if (plan.pub.tail_tiles > 0) {
+        const char* tail_env = std::getenv("CAKE_HIP_CONV_TAIL");
+        const bool subtiles_fit = taps == 9 && plan.pub.tail_tiles > 0;
+        const bool subtiles = tail_env && !std::strcmp(tail_env, "slices") ? false
+                              : tail_env && !std::strcmp(tail_env, "subtiles") ? subtiles_fit
+                              : subtiles_fit && plan.pub.tail_tiles * CONV_TAIL_SUBTILES_PER_TILE <= 2 * cur().model.cus;
+        if (subtiles) {
+            g.tail_tiles = plan.pub.tail_tiles;
+            g.tail_split = CONV_TAIL_SUBTILES_PER_TILE;
+            g.tail_k_per_split = Kp;
+            g.conv.tail_mode = CONV_TAIL_SUBTILES;
+            grid += g.tail_tiles * (CONV_TAIL_SUBTILES_PER_TILE - 1);
+        } else if (plan.pub.tail_tiles > 0) {
             const int block_k = 32 * taps, blocks = Kp / block_k;
             const bool halves = plan.pub.tail_split > blocks && taps >= 6;
             const int per = halves ? 1 : (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
@@ -1564,7 +1578,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
                 g.tail_tiles = plan.pub.tail_tiles;
                 g.tail_split = slices;
                 g.tail_k_per_split = per * block_k;    // (not read for halves: the kernel places them itself)
-                g.conv.tail_halves = halves ? 1 : 0;
+                g.conv.tail_mode = halves ? CONV_TAIL_HALVES : CONV_TAIL_BLOCKS;
                 if ((st = scratch_space(cur().splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
                     return st;
                 grid += g.tail_tiles * (slices - 1);
@@ -1583,7 +1597,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         if ((st = timer.start())) return st;
         if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, taps, stream); }))) return st;
         if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;
-        if (g.tail_tiles > 0 && (st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); }))) return st;
+        if (g.tail_partial && (st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); }))) return st;
         if ((st = timer.stop())) return st;
         return stage_out(o, stream);
     }

@@ -47,6 +47,13 @@ struct FastDiv {
 
 // k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
 // B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
+// Tail tiles of the patch kernel: K slices of whole channel blocks; slice s = half h = s & 1 of the
+// taps of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest); or no slices in memory at
+// all: 16 workgroups per tile, each computing 64 rows x 32 pixels over the whole K with the K
+// quarters of every stage dealt to its waves and summed through LDS (3 x 3 taps only).
+enum { CONV_TAIL_BLOCKS = 0, CONV_TAIL_HALVES = 1, CONV_TAIL_SUBTILES = 2 };
+enum { CONV_TAIL_SUBTILES_PER_TILE = 16 };
+
 struct ConvGeom {
     const float* in;        // the staged input (the input itself for stride 1 without padding)
     unsigned in_bytes;      // its size: loads past it read as zero
@@ -67,8 +74,7 @@ struct ConvGeom {
     FastDiv by_row_n, by_hout, by_vrows, by_channel_chunks, by_row_chunks;
     int stream_out;                // sgemm_conv_patch.hip: the output's rows are whole 128-byte lines, so it may leave
                                    // with non-temporal stores (partial lines written that way cost 35-45 %)
-    int tail_halves;               // sgemm_conv_patch.hip: slice s of a tail tile is half h = s & 1 of the taps
-                                   // of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest)
+    int tail_mode;                 // sgemm_conv_patch.hip, how the tiles of a thin last round are cut (CONV_TAIL_*)
 };
 
 struct GemmArgs {

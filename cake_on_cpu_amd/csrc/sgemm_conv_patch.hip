@@ -38,14 +38,11 @@ constexpr int PATCH_FLOATS = PATCH_PLANE_FLOATS * PATCH_CHANNELS;
 template <class T>
 constexpr int patch_smem_bytes() { return (2 * T::A_STAGE + PATCH_FLOATS) * 4; }
 
-// Everything about the operands that is fixed per thread for a whole tile.
-template <class T>
-struct PatchLoader {
-    static constexpr int PATCH_ITERS = PATCH_FLOATS / 4 / T::THREADS;   // 16-byte chunks of a patch per thread
-    static_assert(PATCH_FLOATS / 4 % T::THREADS == 0, "patch chunks are dealt evenly");
-    int a_off[T::A_ITERS];      // byte offset from the A tile origin, or BUF_OOB for rows >= M
-    const float* a_base;        // Wt + m0 * lda
-    unsigned a_elems;
+// A thread's share of a patch: where its 16-byte chunks come from and where they go.
+template <int THREADS>
+struct PatchFetch {
+    static constexpr int PATCH_ITERS = PATCH_FLOATS / 4 / THREADS;   // 16-byte chunks of a patch per thread
+    static_assert(PATCH_FLOATS / 4 % THREADS == 0, "patch chunks are dealt evenly");
     int p_off[PATCH_ITERS];     // byte offset of the chunk inside channel block 0 of the input, or BUF_OOB
     int p_lds[PATCH_ITERS];     // where it goes in the patch (floats, a multiple of 4), or -1; the two low bits
                                 // say how many of its 4 floats hang over the end of the row (the last chunk may)
@@ -53,31 +50,20 @@ struct PatchLoader {
     const float* in;
     unsigned in_bytes;
     unsigned block_bytes;       // bytes of the input between channel blocks
-    float* patch;
 
     // v0: virtual row the patch starts at; rows_used: how many of its rows this tile's pixels reach
-    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid, float* patch_)
+    __device__ __forceinline__ void init_patch(const ConvGeom& cv, int v0, int rows_used, int tid)
     {
-        const ConvGeom& cv = g.conv;
-        a_base = g.A + (size_t)m0 * g.lda;
-        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
-#pragma unroll
-        for (int it = 0; it < T::A_ITERS; ++it) {
-            const int c = tid + it * T::THREADS;
-            const int r = c / (T::BK / 4);
-            a_off[it] = (m0 + r < g.M) ? (r * g.lda + (c % (T::BK / 4)) * 4) * 4 : BUF_OOB;
-        }
         in = cv.in;
         in_bytes = cv.in_bytes;
         block_bytes = (unsigned)PATCH_CHANNELS * cv.Hin * cv.Win * 4u;
-        patch = patch_;
         const int wc = (cv.Win + 3) >> 2;                 // chunks per input row
         const int per_channel = cv.patch_rows * wc;
         const int total = PATCH_CHANNELS * per_channel;
         const int vrows = cv.Hin + 2 * cv.pad;            // rows of a padded image
 #pragma unroll
         for (int it = 0; it < PATCH_ITERS; ++it) {
-            const int q = tid + it * T::THREADS;
+            const int q = tid + it * THREADS;
             const int c = (int)cv.by_channel_chunks.div(q), rem = q - c * per_channel;
             const int r = (int)cv.by_row_chunks.div(rem), j = rem - r * wc;
             const int v = v0 + r;
@@ -86,11 +72,6 @@ struct PatchLoader {
             p_off[it] = data ? (((b * cv.Cin + c) * cv.Hin + hi) * cv.Win + 4 * j) * 4 : BUF_OOB;
             p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : -1;
         }
-    }
-
-    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
-    {
-        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
     }
 
     // chunk `it` of channel block cb's patch (rows outside an image read as zero).  cb must be a
@@ -113,7 +94,7 @@ struct PatchLoader {
         }
     }
 
-    __device__ __forceinline__ void store_patch()
+    __device__ __forceinline__ void store_patch_to(float* patch)
     {
 #pragma unroll
         for (int it = 0; it < PATCH_ITERS; ++it) {
@@ -125,6 +106,37 @@ struct PatchLoader {
             if (p_lds[it] >= 0) *reinterpret_cast<f32x4*>(patch + (p_lds[it] & ~3)) = v;
         }
     }
+};
+
+// Everything about the operands that is fixed per thread for a whole tile.
+template <class T>
+struct PatchLoader : PatchFetch<T::THREADS> {
+    using PatchFetch<T::THREADS>::PATCH_ITERS;
+    int a_off[T::A_ITERS];      // byte offset from the A tile origin, or BUF_OOB for rows >= M
+    const float* a_base;        // Wt + m0 * lda
+    unsigned a_elems;
+    float* patch;
+
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid, float* patch_)
+    {
+        a_base = g.A + (size_t)m0 * g.lda;
+        a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
+#pragma unroll
+        for (int it = 0; it < T::A_ITERS; ++it) {
+            const int c = tid + it * T::THREADS;
+            const int r = c / (T::BK / 4);
+            a_off[it] = (m0 + r < g.M) ? (r * g.lda + (c % (T::BK / 4)) * 4) * 4 : BUF_OOB;
+        }
+        patch = patch_;
+        this->init_patch(g.conv, v0, rows_used, tid);
+    }
+
+    __device__ __forceinline__ f32x4 load_a(int k0, int off) const
+    {
+        return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
+    }
+
+    __device__ __forceinline__ void store_patch() { this->store_patch_to(patch); }
 };
 
 // One K step as the slot machinery of sgemm_tile.hpp sees it.
@@ -160,6 +172,147 @@ struct PatchStep {
     __device__ __forceinline__ void swap_patch() const { pl.store_patch(); }
 };
 
+// A tail tile without K slices in memory.  A thin last round (config 5: 16 tiles for 256 CUs) used
+// to be cut along K into one slice per CU, each slice paying a tile's whole prologue for four or
+// five steps, writing its 128 KB of partial sums and leaving them to a second kernel.  Here a tile
+// is cut into 16 sub-tiles of 64 rows x 32 pixels instead, one workgroup each, over the whole K:
+//   * wave (blk, kq) of the 8 owns 32 x 32 block blk and quarter kq (8 channels) of every stage,
+//     so each SIMD holds two independent chains of MFMAs, and the four quarters meet in LDS at the
+//     end, summed in quarter order;
+//   * A never touches LDS: a lane's 16 bytes of filters per stage (row blk * 32 + lane % 32, four
+//     consecutive channels) are exactly its MFMA operands, loaded a whole channel block ahead
+//     into a ring of TAPS registers;
+//   * the patch (32 pixels' worth of rows, same layout and loader as the large tile's) is double
+//     buffered, so a channel block ends with one barrier and no swap;
+//   * the result goes to C from the summing pass, 32 consecutive pixels per row.
+// TAPS is a template argument because the ring is indexed by tap and because the compiler can
+// only count how many younger loads may stay in flight at each wait when the block is unrolled.
+template <class T, int TAPS>
+__device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* smem, const WorkItem& w)
+{
+    static_assert(T::THREADS == 512 && T::BM == 256 && T::BN == 128, "16 sub-tiles of 64 x 32, 8 waves each");
+    static_assert(2 * PATCH_FLOATS * 4 <= patch_smem_bytes<T>(), "two patches fit the kernel's LDS");
+    using PF = PatchFetch<T::THREADS>;
+    const ConvGeom& cv = g.conv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int blk = wave & 1, kq = wave >> 1;
+    const int m0 = w.tile_m * T::BM + (w.slice & 3) * 64;
+    const int n0 = w.tile_n * T::BN + (w.slice >> 2) * 32;
+    if (m0 >= g.M || n0 >= g.N) return;                   // the whole workgroup
+
+    // the patch: as for the large tile, for 32 pixels
+    const int vrows = cv.Hin + 2 * cv.pad;
+    const int g0 = (int)cv.by_row_n.div(n0), img0 = (int)cv.by_hout.div(g0);
+    const int v0 = img0 * vrows + (g0 - img0 * cv.Hout);
+    int pix;
+    {
+        int n = n0 + l32;
+        if (n >= g.N) n = n0;                              // computed and dropped
+        const int gr = (int)cv.by_row_n.div(n), wo = n - gr * cv.row_n;
+        const int b = (int)cv.by_hout.div(gr), ho = gr - b * cv.Hout;
+        pix = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + (kq * 8 + lh * 4) * PATCH_PLANE_FLOATS;
+    }
+    const int n_last = min(n0 + 32, g.N) - 1;
+    const int g_last = (int)cv.by_row_n.div(n_last), img_last = (int)cv.by_hout.div(g_last);
+    const int rows_used = img_last * vrows + (g_last - img_last * cv.Hout) - v0 + cv.Hf;
+    PF pf;
+    pf.init_patch(cv, v0, rows_used, tid);
+    // (the two patches are addressed by offsets into the one LDS array: pointers picked from a table
+    // would lose their address space and become flat accesses)
+
+    // A: the lane's row of the filters, its 4 channels of the wave's quarter
+    const float* a_base = g.A + (size_t)m0 * g.lda;
+    const unsigned a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
+    const int a_row = blk * 32 + l32;
+    const int a_off = (m0 + a_row < g.M) ? (a_row * g.lda + kq * 8 + lh * 4) * 4 : BUF_OOB;
+    auto load_a = [&](int step) {
+        return buffer_load_f32x4(a_base + step * PATCH_CHANNELS, a_off, records_left(a_elems, (unsigned)(step * PATCH_CHANNELS)));
+    };
+
+    int toff[TAPS];
+    {
+        int th = 0, tw = 0;
+#pragma unroll
+        for (int t = 0; t < TAPS; ++t) {
+            toff[t] = th * cv.patch_pitch + tw;
+            if (++tw == cv.Wf) { tw = 0; ++th; }
+        }
+    }
+    const int blocks = cv.Cin / PATCH_CHANNELS, last_block = blocks - 1;
+
+    pf.load_patch(0);
+    f32x4 ring[TAPS];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) ring[t] = load_a(t);
+    // margins (and rows no chunk writes) are zero for the whole walk, in both patches
+    for (int i = tid; i < 2 * PATCH_FLOATS / 4; i += T::THREADS)
+        reinterpret_cast<f32x4*>(smem)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    pf.store_patch_to(smem);
+    pf.load_patch(min(1, last_block));
+    __syncthreads();
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+
+    auto read_b = [&](float (&b)[4], int patch, int off) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b[i] = smem[i * PATCH_PLANE_FLOATS + pix + patch + off];
+    };
+    // one channel block out of `patch`; with PREFETCH the filters of the block after it follow
+    // their predecessors into the ring
+    auto block = [&](int cb, int patch, auto prefetch) {
+        float bq[2][4];
+        read_b(bq[0], patch, toff[0]);
+#pragma unroll
+        for (int t = 0; t < TAPS; ++t) {
+            const f32x4 a = ring[t];
+            if constexpr (decltype(prefetch)::value) ring[t] = load_a((cb + 1) * TAPS + t);
+            if (t + 1 < TAPS) read_b(bq[(t + 1) & 1], patch, toff[t + 1]);
+            // (pinned: left to itself the compiler reads each operand right in front of its MFMA and
+            // the chain waits out an LDS round trip per pair)
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bq[t & 1][i], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int cb = 0; cb < last_block; ++cb) {
+        block(cb, (cb & 1) * PATCH_FLOATS, std::true_type{});
+        // (the other patch was last read a block ago, before the barrier that ended that block)
+        pf.store_patch_to(smem + ((cb + 1) & 1) * PATCH_FLOATS);
+        __syncthreads();
+        pf.load_patch(min(cb + 2, last_block));
+    }
+    block(last_block, (last_block & 1) * PATCH_FLOATS, std::false_type{});
+
+    // the four K quarters of each block meet in LDS; register r of a 32 x 32 block holds row
+    // 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+    __syncthreads();                                       // nobody reads a patch any more
+    float* red = smem;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    const int n = n0 + l32;
+    size_t off = 0, row_stride = 0;
+    const int valid = n < g.N ? conv_out_map(cv, g.M, g.ldc, n, 1, off, row_stride) : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + i * T::THREADS;
+        const int b = e >> 10, r = (e >> 6) & 15;
+        float s = red[((0 * 2 + b) * 16 + r) * 64 + lane];
+#pragma unroll
+        for (int q = 1; q < 4; ++q) s += red[((q * 2 + b) * 16 + r) * 64 + lane];
+        const int m = m0 + b * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (valid > 0 && m < g.M) {
+            float* dst = g.C + (size_t)m * row_stride + off;
+            *dst = g.accumulate ? *dst + s : s;
+        }
+    }
+}
+
 template <class T>
 __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const GemmArgs g)
 {
@@ -180,9 +333,13 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     const WorkItem w = decode_tile(g, blockIdx.x);
     const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
     const int taps = cv.Hf * cv.Wf;
-    // K slices are whole channel blocks, or (tail_halves) the first or second half of one block's taps
+    if (w.tail_tile >= 0 && cv.tail_mode == CONV_TAIL_SUBTILES) {
+        patch_tail_subtile<T, 9>(g, smem, w);
+        return;
+    }
+    // K slices are whole channel blocks, or the first or second half of one block's taps
     int kbeg = w.kbeg, kend = w.kend;
-    if (w.tail_tile >= 0 && cv.tail_halves) {
+    if (w.tail_tile >= 0 && cv.tail_mode == CONV_TAIL_HALVES) {
         const int first = (taps + 1) >> 1, cb = w.slice >> 1;
         kbeg = (cb * taps + (w.slice & 1) * first) * T::BK;
         kend = (w.slice & 1) ? (cb + 1) * taps * T::BK : kbeg + first * T::BK;
