@@ -1551,9 +1551,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         g.split_k = 1; g.k_per_split = Kp;
         g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
         g.accumulate = accumulate;
-        // tiles of a thin last round are cut along K in whole channel blocks, or -- when the plan asks
-        // for more slices than there are blocks and half a block still has the three taps a walk
-        // needs -- in halves of a block's taps (config 5: 16 tiles in 16 slices of 5 and 4 taps)
+        // tiles of a thin last round are cut along K in whole channel blocks
         // -- or, under 3 x 3 filters, not cut along K at all: 16 workgroups per tail tile compute
         // 64 rows x 32 pixels each over the whole K, no partial sums in memory and no second kernel
         // (CAKE_HIP_CONV_TAIL=slices|subtiles overrides the choice; for tests and measurements)
@@ -1571,14 +1569,13 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             grid += g.tail_tiles * (CONV_TAIL_SUBTILES_PER_TILE - 1);
         } else if (plan.pub.tail_tiles > 0) {
             const int block_k = 32 * taps, blocks = Kp / block_k;
-            const bool halves = plan.pub.tail_split > blocks && taps >= 6;
-            const int per = halves ? 1 : (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
-            const int slices = halves ? 2 * blocks : (blocks + per - 1) / per;
+            const int per = (blocks + plan.pub.tail_split - 1) / plan.pub.tail_split;
+            const int slices = (blocks + per - 1) / per;
             if (slices > 1) {
                 g.tail_tiles = plan.pub.tail_tiles;
                 g.tail_split = slices;
-                g.tail_k_per_split = per * block_k;    // (not read for halves: the kernel places them itself)
-                g.conv.tail_mode = halves ? CONV_TAIL_HALVES : CONV_TAIL_BLOCKS;
+                g.tail_k_per_split = per * block_k;
+                g.conv.tail_mode = CONV_TAIL_BLOCKS;
                 if ((st = scratch_space(cur().splitk, (size_t)g.tail_tiles * slices * 256 * 128 * sizeof(float), &g.tail_partial)))
                     return st;
                 grid += g.tail_tiles * (slices - 1);

@@ -47,11 +47,10 @@ struct FastDiv {
 
 // k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
 // B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
-// Tail tiles of the patch kernel: K slices of whole channel blocks; slice s = half h = s & 1 of the
-// taps of channel block s >> 1 (taps [0, (taps + 1) / 2) or the rest); or no slices in memory at
+// Tail tiles of the patch kernel: K slices of whole channel blocks, or no slices in memory at
 // all: 16 workgroups per tile, each computing 64 rows x 32 pixels over the whole K with the K
-// quarters of every stage dealt to its waves and summed through LDS (3 x 3 taps only).
-enum { CONV_TAIL_BLOCKS = 0, CONV_TAIL_HALVES = 1, CONV_TAIL_SUBTILES = 2 };
+// quarters of every block dealt to its waves and summed through LDS (3 x 3 taps only).
+enum { CONV_TAIL_BLOCKS = 0, CONV_TAIL_SUBTILES = 2 };
 enum { CONV_TAIL_SUBTILES_PER_TILE = 16 };
 
 struct ConvGeom {
@@ -224,8 +223,8 @@ hipError_t launch_cn_to_nchw(const float* src, float* dst, int batch, int Cout, 
                              hipStream_t stream);
 
 // Stride-1 convolutions that read the input where it lies (sgemm_conv_patch.hip).  The product is
-// out[Cout][n] = Wt[Cout][K'] . B with K' = conv_patch_k(...) walked as (channel block of 32, tap,
-// channel); Wt is the filters re-laid to that order by launch_conv_filter_relayout.
+// out[Cout][n] = Wt[Cout][K'] . B with K' = conv_patch_k(...) walked as (half block of 16
+// channels, tap, channel); Wt is the filters re-laid to that order by launch_conv_filter_relayout.
 // conv_patch_geometry: false when the kernel does not take the geometry, else the patch's shape.
 enum { CONV_PATCH_PLANE = 512 };   // floats per channel of the LDS patch: rows x pitch must fit
 bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout,

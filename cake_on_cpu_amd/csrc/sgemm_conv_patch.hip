@@ -2,25 +2,29 @@
 // where it lies (the direct convolution of examples/cake_conv.cpp:31-258,614-716 on the MFMA
 // macro-tile): no padded copy, no column matrix, no table of tap offsets.
 //
-// out[co][n] = sum_k' Wt[co][k'] * B[k'][n] with the sum walked channel block by channel block:
-//     k' = (cb * taps + tap) * 32 + c,   channel = cb * 32 + c,   tap = h * Wf + w
+// out[co][n] = sum_k' Wt[co][k'] * B[k'][n] with the sum walked in half blocks of 16 channels:
+//     k' = (hb * taps + tap) * 16 + c,   channel = hb * 16 + c,   tap = h * Wf + w
 // (the order of a sum is free as long as both operands agree; the filters are re-laid to it by
-// conv_filter_relayout_kernel, 2 MB for 256 x 256 x 3 x 3).  A K stage of 32 is then 32 channels
-// under ONE filter tap, so B[k'][n] = patch[c][row(n) + h][col(n) + w] for a patch of the input
-// that stays in LDS for all taps of a channel block:
-//   * the patch holds, for 32 channels, the R input rows the tile's pixels can reach and whole
+// conv_filter_relayout_kernel, 2 MB for 256 x 256 x 3 x 3).  A K stage of 32 is then two *pairs*
+// of operand groups, each pair 16 channels under ONE filter tap, so
+// B[k'][n] = patch[c][row(n) + h][col(n) + w] for a patch of the input that stays in LDS for all
+// taps of its half block:
+//   * a patch holds, for 16 channels, the R input rows the tile's pixels can reach and whole
 //     rows of P floats: 4 + Win + pad columns, the image's own starting at column 4 so that the
 //     16-byte global loads land 16-byte aligned in LDS.  Rows above and below an image and the
 //     margins left and right of a row are zero: the padding exists in LDS only.  Rows come from
 //     the "virtual" sequence image 0 padded, image 1 padded, ...: a tile whose pixels straddle two
 //     images sees the lower margin of one and the upper margin of the next as distinct rows;
-//   * the MFMA's B operand of lane n for stage (tap, group of 8 channels) is a 4-byte LDS read at
+//   * the MFMA's B operand of lane n for a group (tap, 8 channels) is a 4-byte LDS read at
 //     pixel(n) + tap offset + channel * PLANE: the pixel part is fixed per lane, the tap part per
-//     stage, the channel part an immediate -- no integer work between the MFMAs;
-//   * A (the filters) walks through the usual double-buffered stages; the patch is loaded once per
-//     channel block (8 x 16 bytes per thread for 9 stages, where the gather from a staged copy
-//     issued 2 per stage), at the start of the block's second-to-last stage, and swapped in
-//     between the last stage's barrier and its last operand group.
+//     pair, the channel part an immediate -- no integer work between the MFMAs;
+//   * LDS has room for two such patches, and half blocks alternate between them: while the taps
+//     of half block hb are walked out of one, half block hb + 1 waits in the other and hb + 2 is
+//     fetched (4 x 16 bytes per thread) and written over hb's predecessor -- behind a stage's
+//     barrier, two stages after its loads were issued, with no barrier of its own.  (One patch of
+//     32 channels, swapped between two barriers at the end of its taps, stalled every wave of the
+//     workgroup once per 9 stages: 11 us of config 5's 841.)
+//   * A (the filters) walks through the usual double-buffered stages.
 // Everything else -- tile raster, tail tiles cut along K, epilogue with the NCHW layout -- is the
 // macro-tile kernel's (sgemm_tile.hpp).
 #include "sgemm_tile.hpp"
@@ -32,34 +36,38 @@ namespace {
 using TilePatch = Tile<256, 128, 32, 64, 64, 2, 1, 1>;   // 8 waves of 64 x 64, two register stages for A
 
 constexpr int PATCH_PLANE_FLOATS = CONV_PATCH_PLANE;      // floats per channel of the patch (rows x pitch fit in it)
-constexpr int PATCH_CHANNELS = 32;                        // = BK: one tap of 32 channels per K stage
-constexpr int PATCH_FLOATS = PATCH_PLANE_FLOATS * PATCH_CHANNELS;
+constexpr int PATCH_CHANNELS = 32;                        // channels per block: two patches of 16, a whole number of K stages
+constexpr int HALF_CHANNELS = 16;                         // channels per patch: a pair of operand groups per tap
+constexpr int PATCH_FLOATS = PATCH_PLANE_FLOATS * PATCH_CHANNELS;   // both patches
+constexpr int HALF_FLOATS = PATCH_PLANE_FLOATS * HALF_CHANNELS;
 
 template <class T>
 constexpr int patch_smem_bytes() { return (2 * T::A_STAGE + PATCH_FLOATS) * 4; }
 
 // A thread's share of a patch: where its 16-byte chunks come from and where they go.
-template <int THREADS>
+template <int THREADS, int CHANNELS>
 struct PatchFetch {
-    static constexpr int PATCH_ITERS = PATCH_FLOATS / 4 / THREADS;   // 16-byte chunks of a patch per thread
-    static_assert(PATCH_FLOATS / 4 % THREADS == 0, "patch chunks are dealt evenly");
-    int p_off[PATCH_ITERS];     // byte offset of the chunk inside channel block 0 of the input, or BUF_OOB
-    int p_lds[PATCH_ITERS];     // where it goes in the patch (floats, a multiple of 4), or -1; the two low bits
-                                // say how many of its 4 floats hang over the end of the row (the last chunk may)
-    f32x4 pr[PATCH_ITERS];      // the next block's patch on its way
+    static constexpr int PATCH_ITERS = PATCH_PLANE_FLOATS * CHANNELS / 4 / THREADS;   // 16-byte chunks of a patch per thread
+    static_assert(PATCH_PLANE_FLOATS * CHANNELS / 4 % THREADS == 0, "patch chunks are dealt evenly");
+    int p_off[PATCH_ITERS];     // byte offset of the chunk inside the first CHANNELS channels of the input, or BUF_OOB
+    int p_lds[PATCH_ITERS];     // where it goes in the patch (floats, a multiple of 4); the two low bits say how
+                                // many of its 4 floats hang over the end of the row (the last chunk may).  A
+                                // chunk that does not exist is fetched as zeros and goes to the left margin
+                                // of the patch's first row, which is zero anyway: no branch around the store
+    f32x4 pr[PATCH_ITERS];      // a patch on its way
     const float* in;
     unsigned in_bytes;
-    unsigned block_bytes;       // bytes of the input between channel blocks
+    unsigned block_bytes;       // bytes of the input between blocks of CHANNELS channels
 
     // v0: virtual row the patch starts at; rows_used: how many of its rows this tile's pixels reach
     __device__ __forceinline__ void init_patch(const ConvGeom& cv, int v0, int rows_used, int tid)
     {
         in = cv.in;
         in_bytes = cv.in_bytes;
-        block_bytes = (unsigned)PATCH_CHANNELS * cv.Hin * cv.Win * 4u;
+        block_bytes = (unsigned)CHANNELS * cv.Hin * cv.Win * 4u;
         const int wc = (cv.Win + 3) >> 2;                 // chunks per input row
         const int per_channel = cv.patch_rows * wc;
-        const int total = PATCH_CHANNELS * per_channel;
+        const int total = CHANNELS * per_channel;
         const int vrows = cv.Hin + 2 * cv.pad;            // rows of a padded image
 #pragma unroll
         for (int it = 0; it < PATCH_ITERS; ++it) {
@@ -70,12 +78,12 @@ struct PatchFetch {
             const int b = (int)cv.by_vrows.div(v), hi = v - b * vrows - cv.pad;
             const bool data = q < total && r < rows_used && b < cv.batch && hi >= 0 && hi < cv.Hin;
             p_off[it] = data ? (((b * cv.Cin + c) * cv.Hin + hi) * cv.Win + 4 * j) * 4 : BUF_OOB;
-            p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : -1;
+            p_lds[it] = q < total ? c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + 4 + 4 * j + max(0, 4 * j + 4 - cv.Win) : 0;
         }
     }
 
-    // chunk `it` of channel block cb's patch (rows outside an image read as zero).  cb must be a
-    // block of the input: the record count is a plain difference on purpose (a saturating one only
+    // chunk `it` of the patch of block cb of CHANNELS channels (rows outside an image read as zero).
+    // cb must be a block of the input: the record count is a plain difference on purpose (a saturating one only
     // exists as a vector instruction, and a record count in a vector register makes the compiler
     // loop over the load).
     template <int IT>
@@ -94,30 +102,35 @@ struct PatchFetch {
         }
     }
 
+    template <int IT>
+    __device__ __forceinline__ void store_patch_chunk_to(float* patch)
+    {
+        f32x4 v = pr[IT];
+        const int over = p_lds[IT] & 3;
+        if (over > 0) v[3] = 0.f;
+        if (over > 1) v[2] = 0.f;
+        if (over > 2) v[1] = 0.f;
+        *reinterpret_cast<f32x4*>(patch + (p_lds[IT] & ~3)) = v;
+    }
+    template <int IT = 0>
     __device__ __forceinline__ void store_patch_to(float* patch)
     {
-#pragma unroll
-        for (int it = 0; it < PATCH_ITERS; ++it) {
-            f32x4 v = pr[it];
-            const int over = p_lds[it] & 3;
-            if (over > 0) v[3] = 0.f;
-            if (over > 1) v[2] = 0.f;
-            if (over > 2) v[1] = 0.f;
-            if (p_lds[it] >= 0) *reinterpret_cast<f32x4*>(patch + (p_lds[it] & ~3)) = v;
+        if constexpr (IT < PATCH_ITERS) {
+            store_patch_chunk_to<IT>(patch);
+            store_patch_to<IT + 1>(patch);
         }
     }
 };
 
 // Everything about the operands that is fixed per thread for a whole tile.
 template <class T>
-struct PatchLoader : PatchFetch<T::THREADS> {
-    using PatchFetch<T::THREADS>::PATCH_ITERS;
+struct PatchLoader : PatchFetch<T::THREADS, HALF_CHANNELS> {
+    using PatchFetch<T::THREADS, HALF_CHANNELS>::PATCH_ITERS;
     int a_off[T::A_ITERS];      // byte offset from the A tile origin, or BUF_OOB for rows >= M
     const float* a_base;        // Wt + m0 * lda
     unsigned a_elems;
-    float* patch;
 
-    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid, float* patch_)
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid)
     {
         a_base = g.A + (size_t)m0 * g.lda;
         a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
@@ -127,7 +140,6 @@ struct PatchLoader : PatchFetch<T::THREADS> {
             const int r = c / (T::BK / 4);
             a_off[it] = (m0 + r < g.M) ? (r * g.lda + (c % (T::BK / 4)) * 4) * 4 : BUF_OOB;
         }
-        patch = patch_;
         this->init_patch(g.conv, v0, rows_used, tid);
     }
 
@@ -135,41 +147,37 @@ struct PatchLoader : PatchFetch<T::THREADS> {
     {
         return buffer_load_f32x4(a_base + k0, off, records_left(a_elems, (unsigned)k0));
     }
-
-    __device__ __forceinline__ void store_patch() { this->store_patch_to(patch); }
 };
 
-// One K step as the slot machinery of sgemm_tile.hpp sees it.
-// PAIRED: one of two consecutive taps inside a channel block, which alternate between the two
-// register stages of A so that their loads are dealt over the whole step.
-// PAIRED_FETCH: the second tap of a block's last pair; it also fetches the next block's patch, in
-// its first operand group, so that the patch has a whole step and more to arrive.
-// SINGLE: a tap on its own (a block with an even number of taps starts with one): its loads of A
-// follow its stores, into the registers just stored.
-// LAST: the last tap of a channel block, as SINGLE; it swaps the fetched patch in between its
-// barrier and its last operand group.
-enum PatchStepKind { PATCH_PAIRED, PATCH_PAIRED_FETCH, PATCH_SINGLE, PATCH_LAST };
-template <class T, int KIND>
+// One K step as the slot machinery of sgemm_tile.hpp sees it.  Steps come in pairs that alternate
+// between the two register stages of A, so that their loads are dealt over the whole step; a
+// SINGLE step stands alone (a block with an odd number of steps ends with one): its loads of A
+// follow its stores, into the registers just stored.  FETCH: the step also issues the loads of a
+// patch (half block `hb`), in its first operand group.  STORE: the step writes the patch fetched
+// two or three steps earlier to `dst`, chunk by chunk between the MFMAs of its last group.
+template <class T, bool SINGLE, bool FETCH, bool STORE>
 struct PatchStep {
     using PL = PatchLoader<T>;
     static constexpr int NUM_LOADS = T::A_ITERS;
-    static constexpr int EARLY_LOADS = KIND == PATCH_PAIRED_FETCH ? PL::PATCH_ITERS : 0;
-    static constexpr bool SINGLE_STAGE = KIND == PATCH_SINGLE || KIND == PATCH_LAST;
+    static constexpr int EARLY_LOADS = FETCH ? PL::PATCH_ITERS : 0;
+    static constexpr bool SINGLE_STAGE = SINGLE;
     static constexpr bool MASK_A_STORES = false;   // K' is a whole number of stages
     static constexpr bool B_ALONG_K = false;
     static constexpr int PATCH_PLANE = PATCH_PLANE_FLOATS;
-    static constexpr bool END_OF_BLOCK = KIND == PATCH_LAST;
+    static constexpr int PATCH_STORES = STORE ? PL::PATCH_ITERS : 0;
     PL& pl;
-    int next_block;
+    int hb;          // FETCH: the half block whose patch this step fetches
+    float* dst;      // STORE: where the fetched patch goes
     template <int OP, class RA, class RB>
     __device__ __forceinline__ void load_one(int k0, int /*kend*/, RA& ra, RB& /*rb*/) const
     {
         if constexpr (OP < T::A_ITERS)
             ra[OP] = pl.load_a(k0, pl.a_off[OP]);
         else
-            pl.template load_patch_chunk<OP - T::A_ITERS>(next_block);
+            pl.template load_patch_chunk<OP - T::A_ITERS>(hb);
     }
-    __device__ __forceinline__ void swap_patch() const { pl.store_patch(); }
+    template <int IT>
+    __device__ __forceinline__ void store_patch_chunk() const { pl.template store_patch_chunk_to<IT>(dst); }
 };
 
 // A tail tile without K slices in memory.  A thin last round (config 5: 16 tiles for 256 CUs) used
@@ -192,7 +200,7 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
 {
     static_assert(T::THREADS == 512 && T::BM == 256 && T::BN == 128, "16 sub-tiles of 64 x 32, 8 waves each");
     static_assert(2 * PATCH_FLOATS * 4 <= patch_smem_bytes<T>(), "two patches fit the kernel's LDS");
-    using PF = PatchFetch<T::THREADS>;
+    using PF = PatchFetch<T::THREADS, PATCH_CHANNELS>;
     const ConvGeom& cv = g.conv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
@@ -221,13 +229,15 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     // (the two patches are addressed by offsets into the one LDS array: pointers picked from a table
     // would lose their address space and become flat accesses)
 
-    // A: the lane's row of the filters, its 4 channels of the wave's quarter
+    // A: the lane's row of the filters, its 4 channels of the wave's quarter -- quarter kq is
+    // channels (kq & 1) * 8 .. + 7 of the block's half block kq >> 1, whose taps lie 16 floats apart
     const float* a_base = g.A + (size_t)m0 * g.lda;
     const unsigned a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
     const int a_row = blk * 32 + l32;
-    const int a_off = (m0 + a_row < g.M) ? (a_row * g.lda + kq * 8 + lh * 4) * 4 : BUF_OOB;
-    auto load_a = [&](int step) {
-        return buffer_load_f32x4(a_base + step * PATCH_CHANNELS, a_off, records_left(a_elems, (unsigned)(step * PATCH_CHANNELS)));
+    const int a_off = (m0 + a_row < g.M) ? (a_row * g.lda + (kq >> 1) * TAPS * HALF_CHANNELS + (kq & 1) * 8 + lh * 4) * 4 : BUF_OOB;
+    auto load_a = [&](int cb, int tap) {
+        const int k0 = (2 * cb * TAPS + tap) * HALF_CHANNELS;
+        return buffer_load_f32x4(a_base + k0, a_off, records_left(a_elems, (unsigned)k0));
     };
 
     int toff[TAPS];
@@ -244,7 +254,7 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     pf.load_patch(0);
     f32x4 ring[TAPS];
 #pragma unroll
-    for (int t = 0; t < TAPS; ++t) ring[t] = load_a(t);
+    for (int t = 0; t < TAPS; ++t) ring[t] = load_a(0, t);
     // margins (and rows no chunk writes) are zero for the whole walk, in both patches
     for (int i = tid; i < 2 * PATCH_FLOATS / 4; i += T::THREADS)
         reinterpret_cast<f32x4*>(smem)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -269,7 +279,7 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
 #pragma unroll
         for (int t = 0; t < TAPS; ++t) {
             const f32x4 a = ring[t];
-            if constexpr (decltype(prefetch)::value) ring[t] = load_a((cb + 1) * TAPS + t);
+            if constexpr (decltype(prefetch)::value) ring[t] = load_a(cb + 1, t);
             if (t + 1 < TAPS) read_b(bq[(t + 1) & 1], patch, toff[t + 1]);
             // (pinned: left to itself the compiler reads each operand right in front of its MFMA and
             // the chain waits out an LDS round trip per pair)
@@ -313,7 +323,8 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     }
 }
 
-template <class T>
+// HF x WF: the filter's shape when the kernel is built for one (3 x 3), 0 x 0: any, read from the arguments
+template <class T, int HF, int WF>
 __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const GemmArgs g)
 {
     static_assert(T::KSPLIT == 1 && T::REG_STAGES == 2 && T::BK == PATCH_CHANNELS && T::TN <= 2, "tile shape");
@@ -337,26 +348,18 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         patch_tail_subtile<T, 9>(g, smem, w);
         return;
     }
-    // K slices are whole channel blocks, or the first or second half of one block's taps
-    int kbeg = w.kbeg, kend = w.kend;
-    if (w.tail_tile >= 0 && cv.tail_mode == CONV_TAIL_HALVES) {
-        const int first = (taps + 1) >> 1, cb = w.slice >> 1;
-        kbeg = (cb * taps + (w.slice & 1) * first) * T::BK;
-        kend = (w.slice & 1) ? (cb + 1) * taps * T::BK : kbeg + first * T::BK;
-    }
-    const int steps = (kend - kbeg) / T::BK;
-    const int cb0 = kbeg / (T::BK * taps);
-    const int tap_lo = kbeg / T::BK - cb0 * taps;         // the first tap of the walk (0 unless half a block)
-    const int tap_n = steps < taps ? steps : taps;        // taps walked per channel block
-    const int th0 = tap_lo / cv.Wf, tw0 = tap_lo - th0 * cv.Wf;
-    const int off0 = th0 * cv.patch_pitch + tw0;
-    const int last_block = cv.Cin / PATCH_CHANNELS - 1;
+    // K slices are whole channel blocks
+    const int kbeg = w.kbeg, kend = w.kend;
+    const int block_k = PATCH_CHANNELS * taps;             // k' per channel block: `taps` steps
+    const int blocks = (kend - kbeg) / block_k;
+    const int cb0 = kbeg / block_k;
+    const int last_half = cv.Cin / HALF_CHANNELS - 1;
 
-    // the tile's first pixel fixes which virtual row the patch starts at
+    // the tile's first pixel fixes which virtual row the patches start at
     const int vrows = cv.Hin + 2 * cv.pad;
     const int g0 = (int)cv.by_row_n.div(n0), img0 = (int)cv.by_hout.div(g0);
     const int v0 = img0 * vrows + (g0 - img0 * cv.Hout);
-    // where the lane's pixels (one per 32-column block of the wave) sit in the patch under tap (0, 0);
+    // where the lane's pixels (one per 32-column block of the wave) sit in a patch under tap (0, 0);
     // the lane's half of an operand group (channels 0..3 or 4..7) is folded in
     int pix[2] = {0, 0};
 #pragma unroll
@@ -376,81 +379,145 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.f;
 
-    if (steps > 0) {
+    if (blocks > 0) {
         // the rows below the last pixel's window are never read: not fetched either
         const int n_last = min(n0 + T::BN, g.N) - 1;
         const int g_last = (int)cv.by_row_n.div(n_last), img_last = (int)cv.by_hout.div(g_last);
         const int rows_used = img_last * vrows + (g_last - img_last * cv.Hout) - v0 + cv.Hf;
         PL pl;
-        pl.init(g, m0, v0, rows_used, tid, patch);
+        pl.init(g, m0, v0, rows_used, tid);
         // ra[1] holds the stage that the next step stores, at every step that is not the second of a pair
         f32x4 ra[2][T::A_ITERS], rb_unused[T::B_ITERS];
         Frag<T> frag[2];
-        // prologue: the first block's patch and the first stage of A
-        pl.load_patch(cb0);
+        // prologue: the first half block's patch, the second one's on its way, the first stage of A
+        pl.load_patch(2 * cb0);
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(kbeg, pl.a_off[it]);
-        // margins (and rows no chunk writes) are zero for the whole walk
+        // margins (and rows no chunk writes) are zero for the whole walk, in both patches
         for (int i = tid; i < PATCH_FLOATS / 4; i += T::THREADS)
             reinterpret_cast<f32x4*>(patch)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
-        pl.store_patch();
+        pl.store_patch_to(patch);
+        pl.load_patch(2 * cb0 + 1);
         store_stage_a<T>(As, tid, ra[1]);
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(kbeg + T::BK, pl.a_off[it]);
         __syncthreads();
-        // operands of the first group: A from stage 0, B from the patch under the first tap
+        // operands of the first group: A from stage 0, B from the first patch under the first tap
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
             frag[0].a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + lh * 4);
 #pragma unroll
         for (int tn = 0; tn < T::TN; ++tn)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn] + off0];
+            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn]];
 
-        // One loop per kind of step: two step bodies chosen inside one loop would make the compiler
-        // copy the accumulators wherever the bodies' register assignments meet, i.e. after every step.
+        // A step is two pairs of operand groups; a pair is (half block, tap), and pairs follow each
+        // other tap by tap, half block by half block, alternating between the two patches: pair p
+        // of a block is tap p % taps of half block p / taps and reads at
+        // (p / taps) * HALF_FLOATS + (tap / Wf) * pitch + tap % Wf.
+        // One code copy per kind of step and place in the block: two step bodies chosen inside one
+        // loop would make the compiler copy the accumulators wherever the bodies' register
+        // assignments meet, i.e. after every step.
         int cur = 0, s = 0;
-        auto step_with = [&](const auto& loader, int off_cur, int off_next, f32x4 (&sa)[T::A_ITERS], f32x4 (&fa)[T::A_ITERS]) {
+        auto step_with = [&](const auto& loader, f32x4 (&sa)[T::A_ITERS], f32x4 (&fa)[T::A_ITERS], int off0, int off1, int off2) {
             using LD = std::remove_cv_t<std::remove_reference_t<decltype(loader)>>;
             const WalkCtx<T, LD> c{loader, kbeg + (s + 2) * T::BK, kend,
-                                   As + cur * T::A_STAGE, patch + off_cur,
-                                   As + (cur ^ 1) * T::A_STAGE, patch + off_next,
-                                   tid, a_lane, pix[0], lh, sa, rb_unused, fa, rb_unused, pix[T::TN - 1]};
+                                   As + cur * T::A_STAGE, patch + off0,
+                                   As + (cur ^ 1) * T::A_STAGE, patch + off2,
+                                   tid, a_lane, pix[0], lh, sa, rb_unused, fa, rb_unused, pix[T::TN - 1], patch + off1};
             __builtin_amdgcn_sched_barrier(0);
             step_groups<T, LD>(c, frag, acc);
             cur ^= 1;
             ++s;
         };
-        const int blocks = steps < taps ? 1 : steps / taps;
-        for (int cb = cb0; cb < cb0 + blocks; ++cb) {
-            int th = th0, tw = tw0, off = off0;
-            // offset of the next stage's tap, whose first operands a step reads
-            auto next_tap = [&] {
-                if (++tw == cv.Wf) { tw = 0; ++th; }
-                return th * cv.patch_pitch + tw;
+        using Plain = PatchStep<T, false, false, false>;
+        using Fetch = PatchStep<T, false, true, false>;
+        using Store = PatchStep<T, false, false, true>;
+        using Single = PatchStep<T, true, false, false>;
+        using SingleFetch = PatchStep<T, true, true, false>;
+        // Block cb walks half blocks 2 cb (out of the first patch) and 2 cb + 1 (out of the second).
+        // The second one's patch is on its way when the block starts and is written in the block's
+        // second step (third, with an even number of taps), which nothing reads before the step
+        // after it; the next block's first patch is fetched five steps before the block ends and
+        // written three steps before it ends, when the first half block's last tap is two steps or
+        // more behind; its second patch is fetched in the last step.  (Half blocks past the last
+        // are fetched as the last one again and never used.)
+        if constexpr (HF > 0) {
+            // The filter's shape is known: every pair's place is th * pitch + a constant, so the
+            // lanes' read addresses are three registers (one per filter row) for the whole tile and
+            // everything else an immediate -- no address arithmetic between the MFMAs at all.
+            // (Kept up at run time, the places cost 40 scalar and 6 vector instructions per step in
+            // front of its first MFMA: 20 us of config 5's 840.)
+            constexpr int TAPS = HF * WF;
+            static_assert(TAPS >= 7 && TAPS % 2 == 1, "the block's steps are written out for an odd number of taps");
+            int row_off[HF];
+#pragma unroll
+            for (int h = 0; h < HF; ++h) row_off[h] = h * cv.patch_pitch;
+            auto place = [&](auto P) {
+                constexpr int p = decltype(P)::value % (2 * TAPS);
+                constexpr int tap = p % TAPS;
+                return (p / TAPS) * HALF_FLOATS + tap % WF + row_off[tap / WF];
             };
-            int tap = 0;
-            if ((tap_n - 1) & 1) {
-                const int off_next = next_tap();
-                step_with(PatchStep<T, PATCH_SINGLE>{pl, cb}, off, off_next, ra[1], ra[1]);
-                off = off_next;
-                ++tap;
+            auto step_at = [&](auto J, const auto& loader) {
+                constexpr int j = decltype(J)::value;
+                const int off0 = place(std::integral_constant<int, 2 * j>{}), off1 = place(std::integral_constant<int, 2 * j + 1>{}),
+                          off2 = place(std::integral_constant<int, 2 * j + 2>{});
+                if constexpr (j == TAPS - 1) step_with(loader, ra[1], ra[1], off0, off1, off2);
+                else if constexpr (j % 2 == 0) step_with(loader, ra[1], ra[0], off0, off1, off2);
+                else step_with(loader, ra[0], ra[1], off0, off1, off2);
+            };
+            auto plain_steps = [&](auto self, auto J, auto END) {
+                if constexpr (decltype(J)::value < decltype(END)::value) {
+                    step_at(J, Plain{pl, 0, nullptr});
+                    self(self, std::integral_constant<int, decltype(J)::value + 1>{}, END);
+                }
+            };
+            for (int cb = cb0; cb < cb0 + blocks; ++cb) {
+                const int hx = min(2 * cb + 2, last_half), hy = min(2 * cb + 3, last_half);
+                step_at(std::integral_constant<int, 0>{}, Plain{pl, 0, nullptr});
+                step_at(std::integral_constant<int, 1>{}, Store{pl, 0, patch + HALF_FLOATS});
+                plain_steps(plain_steps, std::integral_constant<int, 2>{}, std::integral_constant<int, TAPS - 5>{});
+                step_at(std::integral_constant<int, TAPS - 5>{}, Fetch{pl, hx, nullptr});
+                step_at(std::integral_constant<int, TAPS - 4>{}, Plain{pl, 0, nullptr});
+                step_at(std::integral_constant<int, TAPS - 3>{}, Store{pl, 0, patch});
+                step_at(std::integral_constant<int, TAPS - 2>{}, Plain{pl, 0, nullptr});
+                step_at(std::integral_constant<int, TAPS - 1>{}, SingleFetch{pl, hy, nullptr});
             }
-            // (after the last channel block its own patch is fetched once more and never used)
-            const int fetch = min(cb + 1, last_block);
-            for (; tap < tap_n - 3; tap += 2) {
-                const int off1 = next_tap();
-                step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
-                const int off2 = next_tap();
-                step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off1, off2, ra[0], ra[1]);
-                off = off2;
+        } else {
+            // `where` is the place in LDS of the pair that the next step starts with
+            int th = 0, tw = 0, half = 0, where = 0;
+            auto next_pair = [&] {
+                if (++tw == cv.Wf) {
+                    tw = 0;
+                    if (++th == cv.Hf) { th = 0; half ^= 1; }
+                }
+                where = half * HALF_FLOATS + th * cv.patch_pitch + tw;
+                return where;
+            };
+            auto step_next = [&](const auto& loader, f32x4 (&sa)[T::A_ITERS], f32x4 (&fa)[T::A_ITERS]) {
+                const int off0 = where, off1 = next_pair(), off2 = next_pair();
+                step_with(loader, sa, fa, off0, off1, off2);
+            };
+            auto first_of_pair = [&](const auto& loader) { step_next(loader, ra[1], ra[0]); };
+            auto second_of_pair = [&](const auto& loader) { step_next(loader, ra[0], ra[1]); };
+            auto single = [&](const auto& loader) { step_next(loader, ra[1], ra[1]); };
+            const int middle_pairs = (taps - 7) >> 1;
+            for (int cb = cb0; cb < cb0 + blocks; ++cb) {
+                const int hx = min(2 * cb + 2, last_half), hy = min(2 * cb + 3, last_half);
+                if (!(taps & 1)) single(Single{pl, 0, nullptr});
+                first_of_pair(Plain{pl, 0, nullptr});
+                second_of_pair(Store{pl, 0, patch + HALF_FLOATS});
+                for (int i = 0; i < middle_pairs; ++i) {
+                    first_of_pair(Plain{pl, 0, nullptr});
+                    second_of_pair(Plain{pl, 0, nullptr});
+                }
+                first_of_pair(Fetch{pl, hx, nullptr});
+                second_of_pair(Plain{pl, 0, nullptr});
+                first_of_pair(Store{pl, 0, patch});
+                second_of_pair(Plain{pl, 0, nullptr});
+                single(SingleFetch{pl, hy, nullptr});
             }
-            const int off1 = next_tap();
-            step_with(PatchStep<T, PATCH_PAIRED>{pl, cb}, off, off1, ra[1], ra[0]);
-            const int off2 = next_tap();
-            step_with(PatchStep<T, PATCH_PAIRED_FETCH>{pl, fetch}, off1, off2, ra[0], ra[1]);
-            step_with(PatchStep<T, PATCH_LAST>{pl, fetch}, off2, 0, ra[1], ra[1]);
         }
     }
 
@@ -471,28 +538,29 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     store_c_tile<T, LOAD_IM2COL_ROW, false, true>(g, smem, acc, m0, n0, w.slice, wave, wm0, wn0, lane, l32, lh);
 }
 
-// Wt[co][(cb * taps + tap) * 32 + c] = W[co][(cb * 32 + c) * taps + tap], zero for channels past Cin
+// Wt[co][(hb * taps + tap) * 16 + c] = W[co][(hb * 16 + c) * taps + tap], zero for channels past Cin
 __global__ void __launch_bounds__(256) conv_filter_relayout_kernel(const float* __restrict__ W, float* __restrict__ Wt,
                                                                    int Cout, int Cin, int taps, int kp)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)Cout * kp) return;
     const int co = (int)(i / kp), k = (int)(i - (size_t)co * kp);
-    const int c = k & 31, bt = k >> 5;
-    const int cb = bt / taps, tap = bt - cb * taps;
-    const int ch = cb * 32 + c;
+    const int c = k & 15, bt = k >> 4;
+    const int hb = bt / taps, tap = bt - hb * taps;
+    const int ch = hb * 16 + c;
     Wt[i] = ch < Cin ? W[((size_t)co * Cin + ch) * taps + tap] : 0.f;
 }
 
 }  // namespace
 
 // Rows and row pitch of the patch for this geometry, or false when the kernel does not take it:
-// stride 1 only, at least three taps, padding of at most 4, whole blocks of 32 channels, and a patch plane of at most 512 floats
+// stride 1 only, at least seven taps (the walk fetches and writes its patches at fixed steps of a block), padding of at most 4,
+// whole blocks of 32 channels, and a patch plane of at most 512 floats
 // (56 x 56 maps under a 3 x 3 filter use all of it; wider images keep the staged-copy path).
 bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout, int Wout,
                          int* rows, int* pitch)
 {
-    if (stride != 1 || Hf * Wf < 3 || pad > 4 || Cin % 32 != 0) return false;
+    if (stride != 1 || Hf * Wf < 7 || pad > 4 || Cin % 32 != 0) return false;
     const int row_n = (Wout + 3) & ~3;
     const int bn = TilePatch::BN;
     const int out_rows = (row_n - 1 + bn - 1) / row_n + 1;               // output rows a tile's pixels can lie in
@@ -525,11 +593,18 @@ hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int 
 hipError_t launch_sgemm_conv_patch(const GemmArgs& args, int grid, hipStream_t stream)
 {
     using T = TilePatch;
-    auto kern = sgemm_conv_patch_kernel<T>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, patch_smem_bytes<T>());
-    if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::THREADS), patch_smem_bytes<T>(), stream, args);
+    auto any = sgemm_conv_patch_kernel<T, 0, 0>;
+    auto k3x3 = sgemm_conv_patch_kernel<T, 3, 3>;
+    static const hipError_t attr_any = hipFuncSetAttribute(reinterpret_cast<const void*>(any),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, patch_smem_bytes<T>());
+    static const hipError_t attr_3x3 = hipFuncSetAttribute(reinterpret_cast<const void*>(k3x3),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, patch_smem_bytes<T>());
+    if (attr_any != hipSuccess) return attr_any;
+    if (attr_3x3 != hipSuccess) return attr_3x3;
+    if (args.conv.Hf == 3 && args.conv.Wf == 3)
+        hipLaunchKernelGGL(k3x3, dim3(grid), dim3(T::THREADS), patch_smem_bytes<T>(), stream, args);
+    else
+        hipLaunchKernelGGL(any, dim3(grid), dim3(T::THREADS), patch_smem_bytes<T>(), stream, args);
     return hipGetLastError();
 }
 

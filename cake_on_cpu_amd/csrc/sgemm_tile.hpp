@@ -735,10 +735,14 @@ __device__ __forceinline__ int conv_out_map(const ConvGeom& cv, int M, int ldc, 
 // first operands of the new stage come in from LDS, instead of the pipe
 // draining after every barrier.  (By then nobody reads the current buffer any
 // more, and it is only overwritten a whole step later.)
-// Loaders whose B operand is not staged per K step: B is read from a patch of the convolution's
-// input that stays in LDS for a whole block of channels (sgemm_conv_patch.hip).  Such a loader
-// declares PATCH_PLANE, the distance in floats between the planes of two consecutive k of a stage,
-// and may declare END_OF_BLOCK: the step then swaps the patch between its barrier and its last group.
+// Loaders whose B operand is not staged per K step: B is read from patches of the convolution's
+// input that stay in LDS for a whole block of channels (sgemm_conv_patch.hip).  Such a loader
+// declares PATCH_PLANE, the distance in floats between the planes of two consecutive k of an
+// operand group.  A stage is then two pairs of groups, each pair 16 channels under one filter tap
+// with a place of its own in LDS (WalkCtx::Bc for groups 0 and 1, Bc2 for groups 2 and 3).  The
+// loader may declare PATCH_STORES: the step then writes that many 16-byte chunks of a fetched
+// patch to LDS between the MFMAs of its last group, i.e. behind its barrier, into a place that
+// nobody reads before the next step's barrier.
 template <class L, class = void>
 struct patch_plane : std::integral_constant<int, 0> {};
 template <class L>
@@ -756,9 +760,9 @@ struct single_stage : std::false_type {};
 template <class L>
 struct single_stage<L, std::void_t<decltype(L::SINGLE_STAGE)>> : std::bool_constant<L::SINGLE_STAGE> {};
 template <class L, class = void>
-struct ends_block : std::false_type {};
+struct patch_stores : std::integral_constant<int, 0> {};
 template <class L>
-struct ends_block<L, std::void_t<decltype(L::END_OF_BLOCK)>> : std::bool_constant<L::END_OF_BLOCK> {};
+struct patch_stores<L, std::void_t<decltype(L::PATCH_STORES)>> : std::integral_constant<int, L::PATCH_STORES> {};
 
 template <class T, class L>
 struct Slots {
@@ -787,8 +791,10 @@ struct Slots {
     static constexpr int loads_in(int kg) { return own_in(kg) + (kg == 0 ? EARLY : 0); }
     // number (as the loader counts them) of load j of group kg: the early ones follow the stage's own
     static constexpr int load_index(int kg, int j) { return j < own_in(kg) ? own_begin(kg) + j : LOAD_OPS + j - own_in(kg); }
+    static constexpr int stage_stores_in(int kg) { return kg == STORE_KG ? STORE_OPS : 0; }
+    static constexpr int patch_stores_in(int kg) { return kg == NKG - 1 ? patch_stores<L>::value : 0; }
     // memory instructions riding in group kg: operand reads, then loads, then stores
-    static constexpr int ops(int kg) { return FRAG_OPS + loads_in(kg) + (kg == STORE_KG ? STORE_OPS : 0); }
+    static constexpr int ops(int kg) { return FRAG_OPS + loads_in(kg) + stage_stores_in(kg) + patch_stores_in(kg); }
 };
 
 // A loader seen through this wrapper fetches stages that lie wholly below kend,
@@ -822,6 +828,7 @@ struct WalkCtx {
     f32x4 (&la)[T::A_ITERS];  // register stage that this step's global loads fill
     f32x4 (&lb)[T::B_ITERS];
     int b_lane2 = 0;          // patch loaders: where the lane's second column block starts (b_lane: the first)
+    const float* Bc2 = nullptr;   // patch loaders: where the stage's groups 2 and 3 read (Bc: groups 0 and 1)
 };
 
 // Memory instruction number OP of group KG (compile-time indices, so every
@@ -848,14 +855,18 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
         } else if constexpr (S::PLANE > 0) {
             // k = plane of the patch; the lane's half (k 0..3 or 4..7 of the group) is part of b_lane
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
-            static_assert(T::TN <= 2, "two column blocks per wave at most");
-            next.b[tn][i] = B[((wrap ? 0 : KG + 1) * 8 + i) * S::PLANE + (tn == 0 ? c.b_lane : c.b_lane2)];
+            static_assert(T::TN <= 2 && S::NKG == 4, "two column blocks per wave at most, two pairs of groups per stage");
+            constexpr int ng = wrap ? 0 : KG + 1;          // the group these operands belong to
+            const float* P = wrap ? c.Bn : (ng < 2 ? c.Bc : c.Bc2);
+            next.b[tn][i] = P[((ng & 1) * 8 + i) * S::PLANE + (tn == 0 ? c.b_lane : c.b_lane2)];
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
         }
     } else if constexpr (OP < N_FRAG + N_LOAD) {
         c.ld.template load_one<S::load_index(KG, OP - N_FRAG)>(c.k_next, c.kend, c.la, c.lb);
+    } else if constexpr (OP >= N_FRAG + N_LOAD + S::stage_stores_in(KG)) {
+        c.ld.template store_patch_chunk<OP - N_FRAG - N_LOAD - S::stage_stores_in(KG)>();
     } else {
         constexpr int W = OP - N_FRAG - N_LOAD;  // store number W of the stage
         if constexpr (W < T::A_ITERS) {
@@ -917,12 +928,6 @@ __device__ __forceinline__ void step_groups(const WalkCtx<T, L>& c, Frag<T> (&fr
         if constexpr (KG == Slots<T, L>::NKG - 1) {
             __syncthreads();  // every wave has stored its share of the next stage
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (ends_block<L>::value) {
-                // nobody reads the old patch any more (the last group's operands are in registers)
-                c.ld.swap_patch();
-                __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
-            }
         }
         mfma_group<T, L, KG>(c, frag[KG & 1], frag[(KG + 1) & 1], acc);
         __builtin_amdgcn_sched_barrier(0);

@@ -151,10 +151,13 @@ CONV_GEOMS = [
     (5, 64, 7, 7, 300, 3, 3, 1, 1),      # 7 x 7 maps: a tile spans three images; two row tiles of filters
     (2, 32, 13, 9, 33, 3, 3, 1, 0),      # no padding, Win = 9: the last 16 bytes of a row hang over its end
     (2, 96, 12, 20, 70, 5, 3, 1, 2),     # 5 x 3 filter, pad 2 (the left margin holds 2 zero columns)
-    (2, 32, 30, 30, 16, 2, 2, 1, 1),     # 2 x 2 filter: Wout = 31
+    (2, 32, 30, 30, 16, 2, 4, 1, 1),     # 2 x 4 filter (an even number of taps: the block starts with a step on its own): Wout = 29
+    (2, 32, 12, 20, 20, 1, 7, 1, 3),     # 1 x 7 and
+    (2, 64, 20, 12, 20, 7, 1, 1, 3),     # 7 x 1: the fewest taps that kernel's walk takes
     (1, 32, 56, 56, 24, 3, 3, 1, 1),     # a full-width plane of 56 x 56: every row and column of the patch in use
-    (34, 32, 32, 32, 72, 3, 3, 1, 1),    # 272 tiles: the 16 of the thin last round are cut in halves of the block's 9 taps
-    (34, 64, 32, 32, 40, 5, 3, 1, 2),    # the same with two channel blocks of 15 taps: four slices of 8 and 7 taps
+    (34, 32, 32, 32, 72, 3, 3, 1, 1),    # 272 tiles: the 16 of the thin last round are computed in sub-tiles of 64 x 32 (two of the four row blocks in use)
+    (34, 64, 32, 32, 40, 5, 3, 1, 2),    # the same with two channel blocks of 15 taps: two K slices per tile of the last round
+    (34, 96, 32, 32, 300, 3, 3, 1, 1),   # 544 tiles in two rows, 32 in the last round: sub-tiles of both tile rows, the second 44 rows high
     (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
     (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
     (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
@@ -202,7 +205,7 @@ def test_conv2d_random_geometries():
 def test_conv2d_random_geometries_whole_channel_blocks(monkeypatch):
     """Seeded random stride-1 geometries with 32, 64 or 96 input channels on the kernel that reads
     the input where it lies, a patch per channel block in LDS (CAKE_HIP_CONV_ROUTE=patch takes it
-    wherever the geometry allows; by default only large layers do): filters of 3 to 25 taps, square or not, padding 0 to 4
+    wherever the geometry allows; by default only large layers do): filters of 8 to 25 taps, square or not, padding 0 to 4
     (also wider than the filter needs), maps from the filter's size to 60 pixels wide, tiles that
     straddle image rows and images, against the naive fp64 convolution; NCHW and matrix output,
     and the same result twice."""
@@ -211,7 +214,7 @@ def test_conv2d_random_geometries_whole_channel_blocks(monkeypatch):
     done = refused = 0
     while done < 40:
         Hf, Wf = int(rng.integers(1, 6)), int(rng.integers(1, 6))
-        if Hf * Wf < 3:
+        if Hf * Wf < 7:
             continue
         pad = int(rng.integers(0, 5))
         Hin, Win = int(rng.integers(max(1, Hf - 2 * pad), 40)), int(rng.integers(max(1, Wf - 2 * pad), 61))
