@@ -1534,11 +1534,11 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     const char* route = std::getenv("CAKE_HIP_CONV_ROUTE");
     const bool patch_wanted = route && !std::strcmp(route, "patch") ? true
                               : route && !std::strcmp(route, "staged") ? false : patch_pays;
-    if (!explicit_cols && patch_wanted && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_k(Cin, Hf, Wf)) &&
+    if (!explicit_cols && patch_wanted && fits_int((double)Cout * batch * Hout * row_n) && fits_int((double)Cout * conv_patch_lda(Cin, Hf, Wf)) &&
         conv_patch_geometry(batch, Cin, Hin, Win, Hf, Wf, stride, pad, Hout, Wout, &patch_rows, &patch_pitch)) {
-        const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n;
+        const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n, ldw = conv_patch_lda(Cin, Hf, Wf);
         g_last_conv_route = CAKE_HIP_CONV_PATCH;
-        if ((st = cur().conv_filters.reserve((size_t)Cout * Kp * sizeof(float)))) return st;
+        if ((st = cur().conv_filters.reserve((size_t)Cout * ldw * sizeof(float)))) return st;
         float* wt = static_cast<float*>(cur().conv_filters.ptr);
         const int tile[4] = {256, 128, 32, 0};
         GemmPlan plan;
@@ -1546,7 +1546,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         GemmArgs g{};
         g.A = wt; g.B = nullptr; g.C = o.dev;
         g.M = Cout; g.N = Np; g.K = Kp;
-        g.lda = Kp; g.ldb = Np; g.ldc = N;
+        g.lda = ldw; g.ldb = Np; g.ldc = N;
         g.tiles_m = plan.pub.tiles_m; g.tiles_n = plan.pub.tiles_n;
         g.split_k = 1; g.k_per_split = Kp;
         g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
@@ -1592,7 +1592,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.by_row_n = FastDiv::make(row_n); cv.by_hout = FastDiv::make(Hout); cv.by_vrows = FastDiv::make(Hin + 2 * pad);
         cv.by_channel_chunks = FastDiv::make(patch_rows * ((Win + 3) / 4)); cv.by_row_chunks = FastDiv::make((Win + 3) / 4);
         if ((st = timer.start())) return st;
-        if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, taps, stream); }))) return st;
+        if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, Hf, Wf, stream); }))) return st;
         if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;
         if (g.tail_partial && (st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); }))) return st;
         if ((st = timer.stop())) return st;

@@ -230,7 +230,8 @@ enum { CONV_PATCH_PLANE = 512 };   // floats per channel of the LDS patch: rows 
 bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, int stride, int pad, int Hout,
                          int Wout, int* rows, int* pitch);
 int conv_patch_k(int Cin, int Hf, int Wf);
-hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int taps, hipStream_t stream);
+int conv_patch_lda(int Cin, int Hf, int Wf);   // floats between rows of Wt (>= K')
+hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int Hf, int Wf, hipStream_t stream);
 // args as for launch_sgemm with the 256 x 128 x 32 tile; K slices (tail tiles) must be whole channel
 // blocks of 32 * Hf * Wf
 hipError_t launch_sgemm_conv_patch(const GemmArgs& args, int grid, hipStream_t stream);

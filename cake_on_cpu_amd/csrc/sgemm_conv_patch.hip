@@ -184,23 +184,30 @@ struct PatchStep {
 // to be cut along K into one slice per CU, each slice paying a tile's whole prologue for four or
 // five steps, writing its 128 KB of partial sums and leaving them to a second kernel.  Here a tile
 // is cut into 16 sub-tiles of 64 rows x 32 pixels instead, one workgroup each, over the whole K:
-//   * wave (blk, kq) of the 8 owns 32 x 32 block blk and quarter kq (8 channels) of every stage,
-//     so each SIMD holds two independent chains of MFMAs, and the four quarters meet in LDS at the
-//     end, summed in quarter order;
-//   * A never touches LDS: a lane's 16 bytes of filters per stage (row blk * 32 + lane % 32, four
+//   * wave (blk, kq) of the 8 owns 32 x 32 block blk and quarter kq (8 channels) of every channel
+//     block, so each SIMD holds two independent chains of MFMAs, and the four quarters meet in
+//     LDS at the end, summed in quarter order;
+//   * A never touches LDS: a lane's 16 bytes of filters per tap (row blk * 32 + lane % 32, four
 //     consecutive channels) are exactly its MFMA operands, loaded a whole channel block ahead
 //     into a ring of TAPS registers;
-//   * the patch (32 pixels' worth of rows, same layout and loader as the large tile's) is double
-//     buffered, so a channel block ends with one barrier and no swap;
+//   * the patch (32 channels, 32 pixels' worth of rows, same layout and loader as the large
+//     tile's) is double buffered: block cb + 1's is written during the first taps of block cb,
+//     between the MFMAs, most of a block after its loads were issued, so a block ends with one
+//     barrier;
 //   * the result goes to C from the summing pass, 32 consecutive pixels per row.
 // TAPS is a template argument because the ring is indexed by tap and because the compiler can
 // only count how many younger loads may stay in flight at each wait when the block is unrolled.
-template <class T, int TAPS>
+// With the filter's shape known as well (HF x WF > 0) a lane's read addresses are one register
+// per patch and filter row plus immediates.
+template <class T, int TAPS, int HF, int WF>
 __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* smem, const WorkItem& w)
 {
     static_assert(T::THREADS == 512 && T::BM == 256 && T::BN == 128, "16 sub-tiles of 64 x 32, 8 waves each");
     static_assert(2 * PATCH_FLOATS * 4 <= patch_smem_bytes<T>(), "two patches fit the kernel's LDS");
+    static_assert(HF == 0 || HF * WF == TAPS, "filter shape");
     using PF = PatchFetch<T::THREADS, PATCH_CHANNELS>;
+    static_assert(PF::PATCH_ITERS == 8 && TAPS >= 4, "the patch's chunks are written four per tap in taps 0 and 1, the next ones fetched four per tap in taps 2 and 3");
+    constexpr int ROWS = HF > 0 ? HF : 1;
     const ConvGeom& cv = g.conv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
@@ -240,8 +247,13 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
         return buffer_load_f32x4(a_base + k0, a_off, records_left(a_elems, (unsigned)k0));
     };
 
-    int toff[TAPS];
-    {
+    // where the lane reads under tap t in patch number p: place[p][row] + column (+ plane)
+    int place[2][ROWS], toff[TAPS];
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int h = 0; h < ROWS; ++h) place[p][h] = p * PATCH_FLOATS + pix + h * cv.patch_pitch;
+    if constexpr (HF == 0) {
         int th = 0, tw = 0;
 #pragma unroll
         for (int t = 0; t < TAPS; ++t) {
@@ -249,7 +261,7 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
             if (++tw == cv.Wf) { tw = 0; ++th; }
         }
     }
-    const int blocks = cv.Cin / PATCH_CHANNELS, last_block = blocks - 1;
+    const int last_block = cv.Cin / PATCH_CHANNELS - 1;
 
     pf.load_patch(0);
     f32x4 ring[TAPS];
@@ -267,36 +279,57 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 
-    auto read_b = [&](float (&b)[4], int patch, int off) {
+    auto read_b = [&](float (&b)[4], auto P, int t) {     // (t is a constant once the taps are unrolled)
+        constexpr int p = decltype(P)::value;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b[i] = smem[i * PATCH_PLANE_FLOATS + pix + patch + off];
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (HF > 0) b[i] = smem[place[p][t / WF] + t % WF + i * PATCH_PLANE_FLOATS];
+            else b[i] = smem[place[p][0] + toff[t] + i * PATCH_PLANE_FLOATS];
+        }
     };
-    // one channel block out of `patch`; with PREFETCH the filters of the block after it follow
-    // their predecessors into the ring
-    auto block = [&](int cb, int patch, auto prefetch) {
+    // One channel block out of patch P.  With MORE, the filters of the block after it follow their
+    // predecessors into the ring, the next block's patch (fetched a block ago) is written into the
+    // other patch and the one after that is fetched.
+    auto block = [&](int cb, auto P, auto more) {
+        constexpr int p = decltype(P)::value;
+        constexpr bool MORE = decltype(more)::value;
         float bq[2][4];
-        read_b(bq[0], patch, toff[0]);
+        read_b(bq[0], P, 0);
 #pragma unroll
         for (int t = 0; t < TAPS; ++t) {
-            const f32x4 a = ring[t];
-            if constexpr (decltype(prefetch)::value) ring[t] = load_a(cb + 1, t);
-            if (t + 1 < TAPS) read_b(bq[(t + 1) & 1], patch, toff[t + 1]);
+            if (t + 1 < TAPS) read_b(bq[(t + 1) & 1], P, t + 1);
             // (pinned: left to itself the compiler reads each operand right in front of its MFMA and
             // the chain waits out an LDS round trip per pair)
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bq[t & 1][i], acc, 0, 0, 0);
+            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ring[t][i], bq[t & 1][i], acc, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MORE) {
+                ring[t] = load_a(cb + 1, t);
+                float* other = smem + (1 - p) * PATCH_FLOATS;
+                if (t == 0) { pf.template store_patch_chunk_to<0>(other); pf.template store_patch_chunk_to<1>(other); pf.template store_patch_chunk_to<2>(other); pf.template store_patch_chunk_to<3>(other); }
+                if (t == 1) { pf.template store_patch_chunk_to<4>(other); pf.template store_patch_chunk_to<5>(other); pf.template store_patch_chunk_to<6>(other); pf.template store_patch_chunk_to<7>(other); }
+                const int fetch = min(cb + 2, last_block);
+                if (t == 2) { pf.template load_patch_chunk<0>(fetch); pf.template load_patch_chunk<1>(fetch); pf.template load_patch_chunk<2>(fetch); pf.template load_patch_chunk<3>(fetch); }
+                if (t == 3) { pf.template load_patch_chunk<4>(fetch); pf.template load_patch_chunk<5>(fetch); pf.template load_patch_chunk<6>(fetch); pf.template load_patch_chunk<7>(fetch); }
+            }
         }
+        // the other patch is complete, and nobody reads this one any more
+        if constexpr (MORE) __syncthreads();
     };
-    for (int cb = 0; cb < last_block; ++cb) {
-        block(cb, (cb & 1) * PATCH_FLOATS, std::true_type{});
-        // (the other patch was last read a block ago, before the barrier that ended that block)
-        pf.store_patch_to(smem + ((cb + 1) & 1) * PATCH_FLOATS);
-        __syncthreads();
-        pf.load_patch(min(cb + 2, last_block));
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    int cb = 0;
+    for (; cb + 2 <= last_block; cb += 2) {
+        block(cb, P0{}, std::true_type{});
+        block(cb + 1, P1{}, std::true_type{});
     }
-    block(last_block, (last_block & 1) * PATCH_FLOATS, std::false_type{});
+    if (cb < last_block) {
+        block(cb, P0{}, std::true_type{});
+        block(cb + 1, P1{}, std::false_type{});
+    } else {
+        block(cb, P0{}, std::false_type{});
+    }
 
     // the four K quarters of each block meet in LDS; register r of a 32 x 32 block holds row
     // 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
@@ -345,7 +378,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     const int m0 = w.tile_m * T::BM, n0 = w.tile_n * T::BN;
     const int taps = cv.Hf * cv.Wf;
     if (w.tail_tile >= 0 && cv.tail_mode == CONV_TAIL_SUBTILES) {
-        patch_tail_subtile<T, 9>(g, smem, w);
+        patch_tail_subtile<T, 9, HF, WF>(g, smem, w);
         return;
     }
     // K slices are whole channel blocks
@@ -540,7 +573,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
 
 // Wt[co][(hb * taps + tap) * 16 + c] = W[co][(hb * 16 + c) * taps + tap], zero for channels past Cin
 __global__ void __launch_bounds__(256) conv_filter_relayout_kernel(const float* __restrict__ W, float* __restrict__ Wt,
-                                                                   int Cout, int Cin, int taps, int kp)
+                                                                   int Cout, int Cin, int taps, int kp, int ld)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)Cout * kp) return;
@@ -548,7 +581,7 @@ __global__ void __launch_bounds__(256) conv_filter_relayout_kernel(const float* 
     const int c = k & 15, bt = k >> 4;
     const int hb = bt / taps, tap = bt - hb * taps;
     const int ch = hb * 16 + c;
-    Wt[i] = ch < Cin ? W[((size_t)co * Cin + ch) * taps + tap] : 0.f;
+    Wt[(size_t)co * ld + k] = ch < Cin ? W[((size_t)co * Cin + ch) * taps + tap] : 0.f;
 }
 
 }  // namespace
@@ -581,12 +614,21 @@ bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, i
 
 int conv_patch_k(int Cin, int Hf, int Wf) { return (Cin + 31) / 32 * 32 * Hf * Wf; }
 
-hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int taps, hipStream_t stream)
+// Floats between the rows of the re-laid filters: an odd number of 128-byte lines.  With an even
+// number (config 5: 72) the same k' of 64 consecutive rows, which the sub-tiles of a last round
+// load straight into MFMA operands, falls into 8 sets of the vector cache and every load misses.
+int conv_patch_lda(int Cin, int Hf, int Wf)
 {
-    const int kp = (Cin + 31) / 32 * 32 * taps;
+    const int kp = conv_patch_k(Cin, Hf, Wf);
+    return (kp / 32) % 2 ? kp : kp + 32;
+}
+
+hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int Hf, int Wf, hipStream_t stream)
+{
+    const int kp = conv_patch_k(Cin, Hf, Wf);
     const size_t n = (size_t)Cout * kp;
     hipLaunchKernelGGL(conv_filter_relayout_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, W, Wt, Cout,
-                       Cin, taps, kp);
+                       Cin, Hf * Wf, kp, conv_patch_lda(Cin, Hf, Wf));
     return hipGetLastError();
 }
 
