@@ -1591,6 +1591,8 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.stream_out = (reinterpret_cast<uintptr_t>(o.dev) & 127) == 0 && (out_nchw ? (Hout * Wout) % 32 == 0 : N % 32 == 0);
         cv.by_row_n = FastDiv::make(row_n); cv.by_hout = FastDiv::make(Hout); cv.by_vrows = FastDiv::make(Hin + 2 * pad);
         cv.by_channel_chunks = FastDiv::make(patch_rows * ((Win + 3) / 4)); cv.by_row_chunks = FastDiv::make((Win + 3) / 4);
+        cv.margin_chunks = patch_pitch / 4 - (Win + 3) / 4;
+        cv.by_margin_chunks = FastDiv::make(cv.margin_chunks); cv.by_channel_margin_chunks = FastDiv::make(patch_rows * cv.margin_chunks);
         if ((st = timer.start())) return st;
         if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, Hf, Wf, stream); }))) return st;
         if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;

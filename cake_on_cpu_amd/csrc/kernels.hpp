@@ -45,14 +45,14 @@ struct FastDiv {
     __device__ __forceinline__ unsigned div(unsigned n) const { return (unsigned)(((unsigned long long)n * m) >> sh); }
 };
 
-// k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
-// B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
 // Tail tiles of the patch kernel: K slices of whole channel blocks, or no slices in memory at
 // all: 16 workgroups per tile, each computing 64 rows x 32 pixels over the whole K with the K
 // quarters of every block dealt to its waves and summed through LDS (3 x 3 taps only).
 enum { CONV_TAIL_BLOCKS = 0, CONV_TAIL_SUBTILES = 2 };
 enum { CONV_TAIL_SUBTILES_PER_TILE = 16 };
 
+// k = c*Hf*Wf + h*Wf + w, n = (b*Hout + ho)*row_n + wo,
+// B[k][n] = in[((b*Cin*plane_rows + ho*row_step)*pitch + wo) + tap_table[k] / 4].
 struct ConvGeom {
     const float* in;        // the staged input (the input itself for stride 1 without padding)
     unsigned in_bytes;      // its size: loads past it read as zero
@@ -71,6 +71,10 @@ struct ConvGeom {
     // divisions by row_n, Hout, rows of a padded image (Hin + 2 pad), 16-byte chunks per patch
     // channel (patch_rows * ceil(Win / 4)) and chunks per input row
     FastDiv by_row_n, by_hout, by_vrows, by_channel_chunks, by_row_chunks;
+    // the 16-byte chunks of a patch row that no load ever writes (one left of the image's columns,
+    // the rest right of them): how many per row, and divisions by that and by the count per channel
+    int margin_chunks;
+    FastDiv by_margin_chunks, by_channel_margin_chunks;
     int stream_out;                // sgemm_conv_patch.hip: the output's rows are whole 128-byte lines, so it may leave
                                    // with non-temporal stores (partial lines written that way cost 35-45 %)
     int tail_mode;                 // sgemm_conv_patch.hip, how the tiles of a thin last round are cut (CONV_TAIL_*)

@@ -44,6 +44,22 @@ constexpr int HALF_FLOATS = PATCH_PLANE_FLOATS * HALF_CHANNELS;
 template <class T>
 constexpr int patch_smem_bytes() { return (2 * T::A_STAGE + PATCH_FLOATS) * 4; }
 
+// Zeroes what the walk reads of `planes` channel planes but never writes: per row, the 16 bytes left
+// of the image's columns and the chunks right of them (the zero padding lives there; every other
+// chunk of a row, rows outside an image included, is written anew with each patch).
+template <int THREADS>
+__device__ __forceinline__ void zero_patch_margins(const ConvGeom& cv, float* patch, int planes, int tid)
+{
+    const int per_channel = cv.patch_rows * cv.margin_chunks;
+    const int first_right = 4 + 4 * ((cv.Win + 3) >> 2);
+    for (int q = tid; q < planes * per_channel; q += THREADS) {
+        const int c = (int)cv.by_channel_margin_chunks.div(q), rem = q - c * per_channel;
+        const int r = (int)cv.by_margin_chunks.div(rem), m = rem - r * cv.margin_chunks;
+        const int col = m == 0 ? 0 : first_right + 4 * (m - 1);
+        *reinterpret_cast<f32x4*>(patch + c * PATCH_PLANE_FLOATS + r * cv.patch_pitch + col) = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+}
+
 // A thread's share of a patch: where its 16-byte chunks come from and where they go.
 template <int THREADS, int CHANNELS>
 struct PatchFetch {
@@ -267,9 +283,8 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     f32x4 ring[TAPS];
 #pragma unroll
     for (int t = 0; t < TAPS; ++t) ring[t] = load_a(0, t);
-    // margins (and rows no chunk writes) are zero for the whole walk, in both patches
-    for (int i = tid; i < 2 * PATCH_FLOATS / 4; i += T::THREADS)
-        reinterpret_cast<f32x4*>(smem)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // margins are zero for the whole walk, in both patches
+    zero_patch_margins<T::THREADS>(cv, smem, 2 * PATCH_CHANNELS, tid);
     __syncthreads();
     pf.store_patch_to(smem);
     pf.load_patch(min(1, last_block));
@@ -426,9 +441,8 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         pl.load_patch(2 * cb0);
 #pragma unroll
         for (int it = 0; it < T::A_ITERS; ++it) ra[1][it] = pl.load_a(kbeg, pl.a_off[it]);
-        // margins (and rows no chunk writes) are zero for the whole walk, in both patches
-        for (int i = tid; i < PATCH_FLOATS / 4; i += T::THREADS)
-            reinterpret_cast<f32x4*>(patch)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // margins are zero for the whole walk, in both patches
+        zero_patch_margins<T::THREADS>(cv, patch, PATCH_CHANNELS, tid);
         __syncthreads();
         pl.store_patch_to(patch);
         pl.load_patch(2 * cb0 + 1);
