@@ -1538,15 +1538,17 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         conv_patch_geometry(batch, Cin, Hin, Win, Hf, Wf, stride, pad, Hout, Wout, &patch_rows, &patch_pitch)) {
         const int taps = Hf * Wf, Kp = conv_patch_k(Cin, Hf, Wf), Np = batch * Hout * row_n, ldw = conv_patch_lda(Cin, Hf, Wf);
         g_last_conv_route = CAKE_HIP_CONV_PATCH;
-        if ((st = cur().conv_filters.reserve((size_t)Cout * ldw * sizeof(float)))) return st;
-        float* wt = static_cast<float*>(cur().conv_filters.ptr);
+        // (the kernel built for 3 x 3 filters walks K in the filters' own order and reads them where they lie)
+        const bool relay = !conv_patch_reads_filters_in_place(Hf, Wf);
+        if (relay && (st = cur().conv_filters.reserve((size_t)Cout * ldw * sizeof(float)))) return st;
+        const float* wt = relay ? static_cast<const float*>(cur().conv_filters.ptr) : w.dev;
         const int tile[4] = {256, 128, 32, 0};
         GemmPlan plan;
         if ((st = plan_gemm(Cout, Np, Kp, CAKE_HIP_NA, tile, true, cur().model, &plan))) return fail(st, "conv2d: no plan");
         GemmArgs g{};
         g.A = wt; g.B = nullptr; g.C = o.dev;
         g.M = Cout; g.N = Np; g.K = Kp;
-        g.lda = ldw; g.ldb = Np; g.ldc = N;
+        g.lda = relay ? ldw : Kp; g.ldb = Np; g.ldc = N;
         g.tiles_m = plan.pub.tiles_m; g.tiles_n = plan.pub.tiles_n;
         g.split_k = 1; g.k_per_split = Kp;
         g.group = plan.pub.group; g.group_along_n = plan.group_along_n;
@@ -1594,7 +1596,7 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         cv.margin_chunks = patch_pitch / 4 - (Win + 3) / 4;
         cv.by_margin_chunks = FastDiv::make(cv.margin_chunks); cv.by_channel_margin_chunks = FastDiv::make(patch_rows * cv.margin_chunks);
         if ((st = timer.start())) return st;
-        if ((st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, wt, Cout, Cin, Hf, Wf, stream); }))) return st;
+        if (relay && (st = timer.family(3, [&] { return launch_conv_filter_relayout(w.dev, static_cast<float*>(cur().conv_filters.ptr), Cout, Cin, Hf, Wf, stream); }))) return st;
         if ((st = timer.family(0, [&] { return launch_sgemm_conv_patch(g, grid, stream); }))) return st;
         if (g.tail_partial && (st = timer.family(1, [&] { return launch_tail_reduce(plan.tile_id, g, stream); }))) return st;
         if ((st = timer.stop())) return st;

@@ -235,6 +235,7 @@ bool conv_patch_geometry(int batch, int Cin, int Hin, int Win, int Hf, int Wf, i
                          int Wout, int* rows, int* pitch);
 int conv_patch_k(int Cin, int Hf, int Wf);
 int conv_patch_lda(int Cin, int Hf, int Wf);   // floats between rows of Wt (>= K')
+bool conv_patch_reads_filters_in_place(int Hf, int Wf);   // no re-laying: A is the filters themselves, lda = K'
 hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int Hf, int Wf, hipStream_t stream);
 // args as for launch_sgemm with the 256 x 128 x 32 tile; K slices (tail tiles) must be whole channel
 // blocks of 32 * Hf * Wf

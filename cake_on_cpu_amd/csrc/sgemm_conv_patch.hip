@@ -25,6 +25,13 @@
 //     32 channels, swapped between two barriers at the end of its taps, stalled every wave of the
 //     workgroup once per 9 stages: 11 us of config 5's 841.)
 //   * A (the filters) walks through the usual double-buffered stages.
+// Built for a known filter shape (3 x 3), the kernel walks K in the filters' own order instead,
+// k = channel * taps + tap, and reads them where they lie as well: a pair of groups is then 16
+// consecutive k, i.e. one or two channels under runs of taps, and since everything about a k is
+// known when the code is compiled, a lane's read address is a register per filter tap of its
+// first k (where its pixel sits under that tap's row, with the difference to the tap four k
+// further on folded in for the upper half of the lanes) plus an immediate.  Half blocks of 16
+// channels are still 16 * taps consecutive k, so the patches take turns exactly as above.
 // Everything else -- tile raster, tail tiles cut along K, epilogue with the NCHW layout -- is the
 // macro-tile kernel's (sgemm_tile.hpp).
 #include "sgemm_tile.hpp"
@@ -138,15 +145,32 @@ struct PatchFetch {
     }
 };
 
-// Everything about the operands that is fixed per thread for a whole tile.
-template <class T>
+// Where lane half lh (k + 4 lh of a group) reads under the tap of the group's k in the filters'
+// own order, relative to the lane's pixel under tap (0, 0) and apart from the immediate part
+// channel(k) * PLANE + column(tap(k)): the lower lanes read in the row of tap(k); the upper lanes
+// four k further on, which is another tap and possibly the next channel.
+template <int HF, int WF>
+__device__ __forceinline__ int natural_place(int tap, int lh, int pitch)
+{
+    constexpr int TAPS = HF * WF;
+    const int tap_b = (tap + 4) % TAPS, ch_b = (tap + 4) / TAPS;
+    const int lower = (tap / WF) * pitch;
+    const int upper = (tap_b / WF) * pitch + ch_b * PATCH_PLANE_FLOATS + tap_b % WF - tap % WF;
+    return lh ? upper : lower;
+}
+
+// Everything about the operands that is fixed per thread for a whole tile.  NPLACE > 0: the
+// filters' own K order; place[tn][tap] then says where the lane reads for a k under that tap.
+template <class T, int NPLACE = 0>
 struct PatchLoader : PatchFetch<T::THREADS, HALF_CHANNELS> {
     using PatchFetch<T::THREADS, HALF_CHANNELS>::PATCH_ITERS;
     int a_off[T::A_ITERS];      // byte offset from the A tile origin, or BUF_OOB for rows >= M
-    const float* a_base;        // Wt + m0 * lda
+    const float* a_base;        // the filters (re-laid or not) + m0 * lda
     unsigned a_elems;
+    const float* patch;
+    int place[T::TN][NPLACE > 0 ? NPLACE : 1];
 
-    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid)
+    __device__ __forceinline__ void init(const GemmArgs& g, int m0, int v0, int rows_used, int tid, const float* patch_)
     {
         a_base = g.A + (size_t)m0 * g.lda;
         a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
@@ -156,6 +180,7 @@ struct PatchLoader : PatchFetch<T::THREADS, HALF_CHANNELS> {
             const int r = c / (T::BK / 4);
             a_off[it] = (m0 + r < g.M) ? (r * g.lda + (c % (T::BK / 4)) * 4) * 4 : BUF_OOB;
         }
+        patch = patch_;
         this->init_patch(g.conv, v0, rows_used, tid);
     }
 
@@ -171,9 +196,10 @@ struct PatchLoader : PatchFetch<T::THREADS, HALF_CHANNELS> {
 // follow its stores, into the registers just stored.  FETCH: the step also issues the loads of a
 // patch (half block `hb`), in its first operand group.  STORE: the step writes the patch fetched
 // two or three steps earlier to `dst`, chunk by chunk between the MFMAs of its last group.
-template <class T, bool SINGLE, bool FETCH, bool STORE>
+// HF x WF > 0: the filters' own K order, and J is the step's number in its channel block.
+template <class T, bool SINGLE, bool FETCH, bool STORE, int HF = 0, int WF = 0, int J = 0>
 struct PatchStep {
-    using PL = PatchLoader<T>;
+    using PL = PatchLoader<T, HF * WF>;
     static constexpr int NUM_LOADS = T::A_ITERS;
     static constexpr int EARLY_LOADS = FETCH ? PL::PATCH_ITERS : 0;
     static constexpr bool SINGLE_STAGE = SINGLE;
@@ -181,6 +207,7 @@ struct PatchStep {
     static constexpr bool B_ALONG_K = false;
     static constexpr int PATCH_PLANE = PATCH_PLANE_FLOATS;
     static constexpr int PATCH_STORES = STORE ? PL::PATCH_ITERS : 0;
+    static constexpr bool READS_PATCH_ITSELF = HF > 0;
     PL& pl;
     int hb;          // FETCH: the half block whose patch this step fetches
     float* dst;      // STORE: where the fetched patch goes
@@ -194,6 +221,16 @@ struct PatchStep {
     }
     template <int IT>
     __device__ __forceinline__ void store_patch_chunk() const { pl.template store_patch_chunk_to<IT>(dst); }
+    // operand i of the lane for column block TN_ and group NG of this step (WRAP: of the next step):
+    // k = 8 * group + 4 * (lane / 32) + i, counted from the start of the channel block
+    template <int NG, bool WRAP, int TN_, int I>
+    __device__ __forceinline__ float patch_read() const
+    {
+        constexpr int TAPS = HF * WF;
+        constexpr int G = (4 * (WRAP ? J + 1 : J) + NG) % (4 * TAPS);
+        constexpr int k = 8 * G + I, ch = k / TAPS, tap = k % TAPS;
+        return pl.patch[pl.place[TN_][tap] + ch * PATCH_PLANE_FLOATS + tap % WF];
+    }
 };
 
 // A tail tile without K slices in memory.  A thin last round (config 5: 16 tiles for 256 CUs) used
@@ -213,8 +250,9 @@ struct PatchStep {
 //   * the result goes to C from the summing pass, 32 consecutive pixels per row.
 // TAPS is a template argument because the ring is indexed by tap and because the compiler can
 // only count how many younger loads may stay in flight at each wait when the block is unrolled.
-// With the filter's shape known as well (HF x WF > 0) a lane's read addresses are one register
-// per patch and filter row plus immediates.
+// With the filter's shape known as well (HF x WF > 0) K runs in the filters' own order, a quarter
+// is 8 * TAPS consecutive k, and a lane's read addresses are a register per patch and tap plus
+// immediates (natural_place).
 template <class T, int TAPS, int HF, int WF>
 __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* smem, const WorkItem& w)
 {
@@ -223,7 +261,6 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     static_assert(HF == 0 || HF * WF == TAPS, "filter shape");
     using PF = PatchFetch<T::THREADS, PATCH_CHANNELS>;
     static_assert(PF::PATCH_ITERS == 8 && TAPS >= 4, "the patch's chunks are written four per tap in taps 0 and 1, the next ones fetched four per tap in taps 2 and 3");
-    constexpr int ROWS = HF > 0 ? HF : 1;
     const ConvGeom& cv = g.conv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
@@ -242,7 +279,7 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
         if (n >= g.N) n = n0;                              // computed and dropped
         const int gr = (int)cv.by_row_n.div(n), wo = n - gr * cv.row_n;
         const int b = (int)cv.by_hout.div(gr), ho = gr - b * cv.Hout;
-        pix = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + (kq * 8 + lh * 4) * PATCH_PLANE_FLOATS;
+        pix = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + (kq * 8 + (HF > 0 ? 0 : lh * 4)) * PATCH_PLANE_FLOATS;
     }
     const int n_last = min(n0 + 32, g.N) - 1;
     const int g_last = (int)cv.by_row_n.div(n_last), img_last = (int)cv.by_hout.div(g_last);
@@ -252,23 +289,31 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
     // (the two patches are addressed by offsets into the one LDS array: pointers picked from a table
     // would lose their address space and become flat accesses)
 
-    // A: the lane's row of the filters, its 4 channels of the wave's quarter -- quarter kq is
-    // channels (kq & 1) * 8 .. + 7 of the block's half block kq >> 1, whose taps lie 16 floats apart
+    // A: the lane's row of the filters, 4 consecutive k of the wave's quarter.  Quarter kq is channels
+    // 8 kq .. 8 kq + 7 of the block.  In the re-laid order these are channels (kq & 1) * 8 .. + 7 of
+    // half block kq >> 1, whose taps lie 16 floats apart, and load t is tap t; in the filters' own
+    // order they are 8 * TAPS consecutive k, and load t is the t-th group of 8.
     const float* a_base = g.A + (size_t)m0 * g.lda;
     const unsigned a_elems = clamp_elems((long long)(g.M - 1 - m0) * g.lda + g.K);
     const int a_row = blk * 32 + l32;
-    const int a_off = (m0 + a_row < g.M) ? (a_row * g.lda + (kq >> 1) * TAPS * HALF_CHANNELS + (kq & 1) * 8 + lh * 4) * 4 : BUF_OOB;
-    auto load_a = [&](int cb, int tap) {
-        const int k0 = (2 * cb * TAPS + tap) * HALF_CHANNELS;
+    const int a_first = HF > 0 ? kq * 8 * TAPS + lh * 4 : (kq >> 1) * TAPS * HALF_CHANNELS + (kq & 1) * 8 + lh * 4;
+    const int a_off = (m0 + a_row < g.M) ? (a_row * g.lda + a_first) * 4 : BUF_OOB;
+    auto load_a = [&](int cb, int t) {
+        const int k0 = cb * PATCH_CHANNELS * TAPS + t * (HF > 0 ? 8 : HALF_CHANNELS);
         return buffer_load_f32x4(a_base + k0, a_off, records_left(a_elems, (unsigned)k0));
     };
 
-    // where the lane reads under tap t in patch number p: place[p][row] + column (+ plane)
-    int place[2][ROWS], toff[TAPS];
+    // where the lane reads in patch number p: in the filters' own order place[p][tap of the first of
+    // its 4 k] + channel * PLANE + column; in the re-laid order place[p][0] + the tap's offset + i * PLANE
+    constexpr int NPLACE = HF > 0 ? TAPS : 1;
+    int place[2][NPLACE], toff[TAPS];
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-        for (int h = 0; h < ROWS; ++h) place[p][h] = p * PATCH_FLOATS + pix + h * cv.patch_pitch;
+        for (int e = 0; e < NPLACE; ++e) {
+            if constexpr (HF > 0) place[p][e] = p * PATCH_FLOATS + pix + natural_place<HF, WF>(e, lh, cv.patch_pitch);
+            else place[p][e] = p * PATCH_FLOATS + pix;
+        }
     if constexpr (HF == 0) {
         int th = 0, tw = 0;
 #pragma unroll
@@ -298,8 +343,12 @@ __device__ __forceinline__ void patch_tail_subtile(const GemmArgs& g, float* sme
         constexpr int p = decltype(P)::value;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if constexpr (HF > 0) b[i] = smem[place[p][t / WF] + t % WF + i * PATCH_PLANE_FLOATS];
-            else b[i] = smem[place[p][0] + toff[t] + i * PATCH_PLANE_FLOATS];
+            if constexpr (HF > 0) {
+                const int k = 8 * t + i, tap = k % TAPS;   // counted from the quarter's first k
+                b[i] = smem[place[p][tap] + (k / TAPS) * PATCH_PLANE_FLOATS + tap % WF];
+            } else {
+                b[i] = smem[place[p][0] + toff[t] + i * PATCH_PLANE_FLOATS];
+            }
         }
     };
     // One channel block out of patch P.  With MORE, the filters of the block after it follow their
@@ -376,7 +425,7 @@ template <class T, int HF, int WF>
 __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const GemmArgs g)
 {
     static_assert(T::KSPLIT == 1 && T::REG_STAGES == 2 && T::BK == PATCH_CHANNELS && T::TN <= 2, "tile shape");
-    using PL = PatchLoader<T>;
+    using PL = PatchLoader<T, HF * WF>;
     extern __shared__ __align__(16) float smem[];
     float* As = smem;
     float* patch = smem + 2 * T::A_STAGE;
@@ -408,7 +457,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
     const int g0 = (int)cv.by_row_n.div(n0), img0 = (int)cv.by_hout.div(g0);
     const int v0 = img0 * vrows + (g0 - img0 * cv.Hout);
     // where the lane's pixels (one per 32-column block of the wave) sit in a patch under tap (0, 0);
-    // the lane's half of an operand group (channels 0..3 or 4..7) is folded in
+    // in the re-laid K order the lane's half of an operand group (channels 0..3 or 4..7) is folded in
     int pix[2] = {0, 0};
 #pragma unroll
     for (int tn = 0; tn < T::TN; ++tn) {
@@ -416,7 +465,7 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         if (n >= g.N) n = n0;                              // computed and dropped
         const int gr = (int)cv.by_row_n.div(n), wo = n - gr * cv.row_n;
         const int b = (int)cv.by_hout.div(gr), ho = gr - b * cv.Hout;
-        pix[tn] = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + lh * 4 * PATCH_PLANE_FLOATS;
+        pix[tn] = (b * vrows + ho - v0) * cv.patch_pitch + (4 - cv.pad) + wo + (HF > 0 ? 0 : lh * 4 * PATCH_PLANE_FLOATS);
     }
 
     f32x16 acc[T::TM][T::TN];
@@ -433,7 +482,13 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         const int g_last = (int)cv.by_row_n.div(n_last), img_last = (int)cv.by_hout.div(g_last);
         const int rows_used = img_last * vrows + (g_last - img_last * cv.Hout) - v0 + cv.Hf;
         PL pl;
-        pl.init(g, m0, v0, rows_used, tid);
+        pl.init(g, m0, v0, rows_used, tid, patch);
+        if constexpr (HF > 0) {
+#pragma unroll
+            for (int tn = 0; tn < T::TN; ++tn)
+#pragma unroll
+                for (int tap = 0; tap < HF * WF; ++tap) pl.place[tn][tap] = pix[tn] + natural_place<HF, WF>(tap, lh, cv.patch_pitch);
+        }
         // ra[1] holds the stage that the next step stores, at every step that is not the second of a pair
         f32x4 ra[2][T::A_ITERS], rb_unused[T::B_ITERS];
         Frag<T> frag[2];
@@ -454,15 +509,31 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
 #pragma unroll
         for (int tm = 0; tm < T::TM; ++tm)
             frag[0].a[tm] = *reinterpret_cast<const f32x4*>(As + a_lane + tm * 32 * T::LDA + lh * 4);
+        if constexpr (HF > 0) {
+            const PatchStep<T, false, false, false, HF, WF, 0> first{pl, 0, nullptr};
+            frag[0].b[0][0] = first.template patch_read<0, false, 0, 0>();
+            frag[0].b[0][1] = first.template patch_read<0, false, 0, 1>();
+            frag[0].b[0][2] = first.template patch_read<0, false, 0, 2>();
+            frag[0].b[0][3] = first.template patch_read<0, false, 0, 3>();
+            if constexpr (T::TN > 1) {
+                frag[0].b[T::TN - 1][0] = first.template patch_read<0, false, T::TN - 1, 0>();
+                frag[0].b[T::TN - 1][1] = first.template patch_read<0, false, T::TN - 1, 1>();
+                frag[0].b[T::TN - 1][2] = first.template patch_read<0, false, T::TN - 1, 2>();
+                frag[0].b[T::TN - 1][3] = first.template patch_read<0, false, T::TN - 1, 3>();
+            }
+        } else {
 #pragma unroll
-        for (int tn = 0; tn < T::TN; ++tn)
+            for (int tn = 0; tn < T::TN; ++tn)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn]];
+                for (int i = 0; i < 4; ++i) frag[0].b[tn][i] = patch[i * PATCH_PLANE_FLOATS + pix[tn]];
+        }
 
-        // A step is two pairs of operand groups; a pair is (half block, tap), and pairs follow each
-        // other tap by tap, half block by half block, alternating between the two patches: pair p
-        // of a block is tap p % taps of half block p / taps and reads at
-        // (p / taps) * HALF_FLOATS + (tap / Wf) * pitch + tap % Wf.
+        // A step is two pairs of operand groups.  In the re-laid order a pair is (half block, tap),
+        // and pairs follow each other tap by tap, half block by half block, alternating between
+        // the two patches: pair p of a block is tap p % taps of half block p / taps and reads at
+        // (p / taps) * HALF_FLOATS + (tap / Wf) * pitch + tap % Wf (off0 for the step's first pair,
+        // off1 for its second, off2 for the next step's first).  In the filters' own order the
+        // step's loader knows the places itself.
         // One code copy per kind of step and place in the block: two step bodies chosen inside one
         // loop would make the compiler copy the accumulators wherever the bodies' register
         // assignments meet, i.e. after every step.
@@ -478,11 +549,6 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
             cur ^= 1;
             ++s;
         };
-        using Plain = PatchStep<T, false, false, false>;
-        using Fetch = PatchStep<T, false, true, false>;
-        using Store = PatchStep<T, false, false, true>;
-        using Single = PatchStep<T, true, false, false>;
-        using SingleFetch = PatchStep<T, true, true, false>;
         // Block cb walks half blocks 2 cb (out of the first patch) and 2 cb + 1 (out of the second).
         // The second one's patch is on its way when the block starts and is written in the block's
         // second step (third, with an even number of taps), which nothing reads before the step
@@ -491,47 +557,46 @@ __global__ void __launch_bounds__(T::THREADS) sgemm_conv_patch_kernel(const Gemm
         // more behind; its second patch is fetched in the last step.  (Half blocks past the last
         // are fetched as the last one again and never used.)
         if constexpr (HF > 0) {
-            // The filter's shape is known: every pair's place is th * pitch + a constant, so the
-            // lanes' read addresses are three registers (one per filter row) for the whole tile and
-            // everything else an immediate -- no address arithmetic between the MFMAs at all.
-            // (Kept up at run time, the places cost 40 scalar and 6 vector instructions per step in
-            // front of its first MFMA: 20 us of config 5's 840.)
+            // The filter's shape is known: the steps of a block are written out, each knowing its
+            // number in the block and with it the channel and tap of every k it multiplies; the
+            // lanes' read addresses are registers computed once per tile plus immediates -- no
+            // address arithmetic between the MFMAs at all.  (Kept up at run time, the places of a
+            // step's operand groups cost 40 scalar and 6 vector instructions in front of its first
+            // MFMA: 20 us of config 5's 840.)
             constexpr int TAPS = HF * WF;
             static_assert(TAPS >= 7 && TAPS % 2 == 1, "the block's steps are written out for an odd number of taps");
-            int row_off[HF];
-#pragma unroll
-            for (int h = 0; h < HF; ++h) row_off[h] = h * cv.patch_pitch;
-            auto place = [&](auto P) {
-                constexpr int p = decltype(P)::value % (2 * TAPS);
-                constexpr int tap = p % TAPS;
-                return (p / TAPS) * HALF_FLOATS + tap % WF + row_off[tap / WF];
-            };
-            auto step_at = [&](auto J, const auto& loader) {
+            auto step_at = [&](auto J, auto single, auto fetch, auto store, int hb, float* dst) {
                 constexpr int j = decltype(J)::value;
-                const int off0 = place(std::integral_constant<int, 2 * j>{}), off1 = place(std::integral_constant<int, 2 * j + 1>{}),
-                          off2 = place(std::integral_constant<int, 2 * j + 2>{});
-                if constexpr (j == TAPS - 1) step_with(loader, ra[1], ra[1], off0, off1, off2);
-                else if constexpr (j % 2 == 0) step_with(loader, ra[1], ra[0], off0, off1, off2);
-                else step_with(loader, ra[0], ra[1], off0, off1, off2);
+                const PatchStep<T, decltype(single)::value, decltype(fetch)::value, decltype(store)::value, HF, WF, j> loader{pl, hb, dst};
+                if constexpr (decltype(single)::value) step_with(loader, ra[1], ra[1], 0, 0, 0);
+                else if constexpr (j % 2 == 0) step_with(loader, ra[1], ra[0], 0, 0, 0);
+                else step_with(loader, ra[0], ra[1], 0, 0, 0);
             };
+            constexpr std::false_type no{};
+            constexpr std::true_type yes{};
             auto plain_steps = [&](auto self, auto J, auto END) {
                 if constexpr (decltype(J)::value < decltype(END)::value) {
-                    step_at(J, Plain{pl, 0, nullptr});
+                    step_at(J, no, no, no, 0, nullptr);
                     self(self, std::integral_constant<int, decltype(J)::value + 1>{}, END);
                 }
             };
             for (int cb = cb0; cb < cb0 + blocks; ++cb) {
                 const int hx = min(2 * cb + 2, last_half), hy = min(2 * cb + 3, last_half);
-                step_at(std::integral_constant<int, 0>{}, Plain{pl, 0, nullptr});
-                step_at(std::integral_constant<int, 1>{}, Store{pl, 0, patch + HALF_FLOATS});
+                step_at(std::integral_constant<int, 0>{}, no, no, no, 0, nullptr);
+                step_at(std::integral_constant<int, 1>{}, no, no, yes, 0, patch + HALF_FLOATS);
                 plain_steps(plain_steps, std::integral_constant<int, 2>{}, std::integral_constant<int, TAPS - 5>{});
-                step_at(std::integral_constant<int, TAPS - 5>{}, Fetch{pl, hx, nullptr});
-                step_at(std::integral_constant<int, TAPS - 4>{}, Plain{pl, 0, nullptr});
-                step_at(std::integral_constant<int, TAPS - 3>{}, Store{pl, 0, patch});
-                step_at(std::integral_constant<int, TAPS - 2>{}, Plain{pl, 0, nullptr});
-                step_at(std::integral_constant<int, TAPS - 1>{}, SingleFetch{pl, hy, nullptr});
+                step_at(std::integral_constant<int, TAPS - 5>{}, no, yes, no, hx, nullptr);
+                step_at(std::integral_constant<int, TAPS - 4>{}, no, no, no, 0, nullptr);
+                step_at(std::integral_constant<int, TAPS - 3>{}, no, no, yes, 0, patch);
+                step_at(std::integral_constant<int, TAPS - 2>{}, no, no, no, 0, nullptr);
+                step_at(std::integral_constant<int, TAPS - 1>{}, yes, yes, no, hy, nullptr);
             }
         } else {
+            using Plain = PatchStep<T, false, false, false>;
+            using Fetch = PatchStep<T, false, true, false>;
+            using Store = PatchStep<T, false, false, true>;
+            using Single = PatchStep<T, true, false, false>;
+            using SingleFetch = PatchStep<T, true, true, false>;
             // `where` is the place in LDS of the pair that the next step starts with
             int th = 0, tw = 0, half = 0, where = 0;
             auto next_pair = [&] {
@@ -636,6 +701,8 @@ int conv_patch_lda(int Cin, int Hf, int Wf)
     const int kp = conv_patch_k(Cin, Hf, Wf);
     return (kp / 32) % 2 ? kp : kp + 32;
 }
+
+bool conv_patch_reads_filters_in_place(int Hf, int Wf) { return Hf == 3 && Wf == 3; }
 
 hipError_t launch_conv_filter_relayout(const float* W, float* Wt, int Cout, int Cin, int Hf, int Wf, hipStream_t stream)
 {

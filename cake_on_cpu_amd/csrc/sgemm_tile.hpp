@@ -759,6 +759,12 @@ template <class L, class = void>
 struct single_stage : std::false_type {};
 template <class L>
 struct single_stage<L, std::void_t<decltype(L::SINGLE_STAGE)>> : std::bool_constant<L::SINGLE_STAGE> {};
+// READS_PATCH_ITSELF: the loader knows where each operand of a group lies in its patches
+// (patch_read<group, wrap, column block, i>()) and the step's Bc, Bc2 and Bn are not used.
+template <class L, class = void>
+struct reads_patch_itself : std::false_type {};
+template <class L>
+struct reads_patch_itself<L, std::void_t<decltype(L::READS_PATCH_ITSELF)>> : std::bool_constant<L::READS_PATCH_ITSELF> {};
 template <class L, class = void>
 struct patch_stores : std::integral_constant<int, 0> {};
 template <class L>
@@ -857,8 +863,12 @@ __device__ __forceinline__ void slot_op(const WalkCtx<T, L>& c, Frag<T>& next)
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
             static_assert(T::TN <= 2 && S::NKG == 4, "two column blocks per wave at most, two pairs of groups per stage");
             constexpr int ng = wrap ? 0 : KG + 1;          // the group these operands belong to
-            const float* P = wrap ? c.Bn : (ng < 2 ? c.Bc : c.Bc2);
-            next.b[tn][i] = P[((ng & 1) * 8 + i) * S::PLANE + (tn == 0 ? c.b_lane : c.b_lane2)];
+            if constexpr (reads_patch_itself<L>::value) {
+                next.b[tn][i] = c.ld.template patch_read<ng, wrap, tn, i>();
+            } else {
+                const float* P = wrap ? c.Bn : (ng < 2 ? c.Bc : c.Bc2);
+                next.b[tn][i] = P[((ng & 1) * 8 + i) * S::PLANE + (tn == 0 ? c.b_lane : c.b_lane2)];
+            }
         } else {
             constexpr int tn = (OP - T::TM) / 4, i = (OP - T::TM) % 4;
             next.b[tn][i] = B[(kk + i) * T::LDB + c.b_lane + tn * 32];
