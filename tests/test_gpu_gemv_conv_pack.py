@@ -158,6 +158,7 @@ CONV_GEOMS = [
     (34, 32, 32, 32, 72, 3, 3, 1, 1),    # 272 tiles: the 16 of the thin last round are computed in sub-tiles of 64 x 32 (two of the four row blocks in use)
     (34, 64, 32, 32, 40, 5, 3, 1, 2),    # the same with two channel blocks of 15 taps: two K slices per tile of the last round
     (34, 96, 32, 32, 300, 3, 3, 1, 1),   # 544 tiles in two rows, 32 in the last round: sub-tiles of both tile rows, the second 44 rows high
+    (35, 32, 30, 30, 72, 3, 3, 1, 1),    # Wout = 30 in rows of 32, 263 tiles: the last of the 7 sub-tiled ones is half full
     (1, 3, 9, 8, 6, 9, 9, 1, 4),         # pad 4: stride 1 but past the row gather's limit
     (2, 16, 8, 8, 260, 3, 3, 1, 1),      # Cout over one tile with the row gather
     (2, 3, 12, 12, 16, 3, 3, 1, 1),      # RGB first layer: K = 27 is not a multiple of 4
@@ -310,6 +311,36 @@ def test_cake_sconv_accumulates_the_direct_convolution(geom):
         assert np.max(np.abs(dev - C0 - cpu) / (S + np.abs(C0))) <= TOL
     with pytest.raises(cake.CakeHipError):
         cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout - 1, Hout, Cin, Cout, s, 4)
+
+
+@pytest.mark.parametrize("filt", [(3, 3), (5, 3)], ids=str)
+def test_cake_sconv_accumulates_through_the_last_round_of_the_patch_kernel(filt, monkeypatch):
+    """cake_sconv on one tall image (32 channels, 700 x 50, no padding) through the kernel that
+    reads the input where it lies: 262 tiles of 256 x 128, so the last 6 -- the last of them half
+    full, 72 of the tile's 256 rows in use -- run as sub-tiles of 64 x 32 under the 3 x 3 filter
+    and as K slices under the 5 x 3 one (two channel blocks), and both add to what C holds."""
+    Hf, Wf = filt
+    Cin, Hin, Win, Cout = 32 if filt == (3, 3) else 64, 700, 50, 72
+    Hout, Wout = Hin - Hf + 1, Win - Wf + 1
+    monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")
+    print(f"cake_sconv on the patch kernel: {Cin} x {Hin} x {Win} -> {Cout}, {Hf} x {Wf}", flush=True)
+    inp = oracle.uniform((Cin, Hin, Win), 71)
+    wt = oracle.uniform((Cout, Cin, Hf, Wf), 72)
+    C0 = oracle.uniform((Cout, Hout, Wout), 73)
+    ref64, S = oracle.conv_naive_f64(inp[None], wt, 1, 0)
+    ref64, S = ref64[0], S[0]
+    out = C0.copy()
+    cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, 1, 4)
+    assert cake.last_conv_route() == cake.CONV_PATCH
+    assert np.max(np.abs(out.astype(np.float64) - C0 - ref64) / (S + np.abs(C0))) <= TIGHT
+    cake.cake_sconv(wt, inp, out, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, 1, 4)
+    assert np.max(np.abs(out.astype(np.float64) - C0 - 2 * ref64) / (2 * S + np.abs(C0))) <= TIGHT
+    if filt == (3, 3):
+        # the same last round cut along K instead: the same sums in another order
+        monkeypatch.setenv("CAKE_HIP_CONV_TAIL", "slices")
+        sliced = C0.copy()
+        cake.cake_sconv(wt, inp, sliced, Wf, Hf, Win, Hin, Wout, Hout, Cin, Cout, 1, 4)
+        assert np.max(np.abs(sliced.astype(np.float64) - C0 - ref64) / (S + np.abs(C0))) <= TIGHT
 
 
 @pytest.mark.parametrize("geom", [(16, 16, 56, 56, 256, 1, 1), (70, 7, 30, 30, 130, 1, 1), (256, 5, 21, 21, 100, 1, 1),
