@@ -290,14 +290,16 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * without padding needs neither: a plane is then one row of Hin * Win pixels,
  * gathered from the input as it lies, and with at most 64 input channels and
  * enough tiles the images run as one batch of plain products on the short-K
- * kernel.  Stride-1 layers with whole blocks of 32 input channels, up to 4
- * columns of padding and maps up to about 60 pixels wide have a kernel that
- * reads the input where it lies (no staged copy: a patch of the input per
- * workgroup and channel block in LDS, zero padding in place); it has a single
- * 256 x 128 tile and is taken where that pays -- 64 K steps or more, tile rows
- * at least three quarters full, two rounds of tiles or more.  The environment
- * variable CAKE_HIP_CONV_ROUTE (read at every call) overrides that choice:
- * "patch" takes this kernel wherever its geometry allows, "staged" never.
+ * kernel.  Stride-1 layers with whole blocks of 32 input channels, a filter of
+ * 7 taps or more, up to 4 columns of padding and maps up to about 60 pixels
+ * wide have a kernel that reads the input where it lies (no staged copy:
+ * patches of the input per workgroup in LDS, zero padding in place; under a
+ * 3 x 3 filter the filters are read where they lie as well and the call is
+ * that one kernel); it has a single 256 x 128 tile and is taken where that
+ * pays -- 64 K steps or more, tile rows at least three quarters full, two
+ * rounds of tiles or more.  The environment variable CAKE_HIP_CONV_ROUTE (read
+ * at every call) overrides that choice: "patch" takes this kernel wherever
+ * its geometry allows, "staged" never.
  * A batch whose staged input
  * would reach 2 GiB, or whose product 2^31 elements, is run in chunks of whole
  * images through the same staged buffer, so input and output may be as large
@@ -324,7 +326,7 @@ int cake_hip_conv2d_im2col(const float* in, const float* weights, float* out,
 enum {
     CAKE_HIP_CONV_NONE = 0,
     CAKE_HIP_CONV_SHORTK_BATCH = 1, /* 1 x 1 layer as a batch of plain products on the short-K kernel */
-    CAKE_HIP_CONV_PATCH = 2,        /* input read where it lies, a patch per channel block in LDS     */
+    CAKE_HIP_CONV_PATCH = 2,        /* input read where it lies, patches of 16 channels in LDS        */
     CAKE_HIP_CONV_GATHER = 3,       /* columns gathered inside the product (staged copy where needed) */
     CAKE_HIP_CONV_TWO_STEP = 4      /* column matrix written out, then the product                    */
 };
