@@ -151,6 +151,7 @@ CONV_GEOMS = [
     (5, 64, 7, 7, 300, 3, 3, 1, 1),      # 7 x 7 maps: a tile spans three images; two row tiles of filters
     (2, 32, 13, 9, 33, 3, 3, 1, 0),      # no padding, Win = 9: the last 16 bytes of a row hang over its end
     (2, 96, 12, 20, 70, 5, 3, 1, 2),     # 5 x 3 filter, pad 2 (the left margin holds 2 zero columns)
+    (2, 32, 30, 30, 16, 2, 2, 1, 1),     # 2 x 2 filter: Wout = 31; fewer taps than that kernel's walk takes, so the staged gather runs
     (2, 32, 30, 30, 16, 2, 4, 1, 1),     # 2 x 4 filter (an even number of taps: the block starts with a step on its own): Wout = 29
     (2, 32, 12, 20, 20, 1, 7, 1, 3),     # 1 x 7 and
     (2, 64, 20, 12, 20, 7, 1, 1, 3),     # 7 x 1: the fewest taps that kernel's walk takes
