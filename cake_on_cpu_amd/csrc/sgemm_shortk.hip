@@ -82,8 +82,10 @@ __global__ void __launch_bounds__(T::THREADS) __attribute__((amdgpu_waves_per_eu
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int wm0 = (wave / T::WAVES_N) * T::WM;
-    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    // (through readfirstlane: derived from the thread id, the compiler would take the wave's place in
+    // the tile for a per-lane value and loop over every store whose scalar offset it enters)
+    const int wm0 = __builtin_amdgcn_readfirstlane((wave / T::WAVES_N) * T::WM);
+    const int wn0 = __builtin_amdgcn_readfirstlane((wave % T::WAVES_N) * T::WN);
     const int a_lane = (wm0 + l32) * T::LDA;
     const int b_lane = wn0 + l32;
 
@@ -319,8 +321,8 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int wm0 = (wave / T::WAVES_N) * T::WM;
-    const int wn0 = (wave % T::WAVES_N) * T::WN;
+    const int wm0 = __builtin_amdgcn_readfirstlane((wave / T::WAVES_N) * T::WM);   // (scalars: see sgemm_shortk_kernel)
+    const int wn0 = __builtin_amdgcn_readfirstlane((wave % T::WAVES_N) * T::WN);
     const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
     const int b_lane = wn0 + l32;
     float* stg = Stg + wave * (8 * PITCH);
@@ -553,7 +555,7 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
+    const int wm0 = __builtin_amdgcn_readfirstlane((wave >> 1) * 32), wn0 = __builtin_amdgcn_readfirstlane((wave & 1) * 32);   // (scalars: see sgemm_shortk_kernel)
     const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
     const int b_lane = wn0 + l32;
     float* stg = Stg + wave * (8 * PITCH);
