@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(T::THREADS) __attribute__((amdgpu_waves_per_eu
     float* Bs = smem + T::A_STAGE;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar for the compiler too
     const int l32 = lane & 31, lh = lane >> 5;
     // (through readfirstlane: derived from the thread id, the compiler would take the wave's place in
     // the tile for a per-lane value and loop over every store whose scalar offset it enters)
@@ -319,7 +319,7 @@ __device__ __forceinline__ void shortk_direct_body(const GemmArgs& g, float* As,
     constexpr int B_LOADS = BK * 64 / 4 / 256;       // load instructions per thread and stage
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar for the compiler too
     const int l32 = lane & 31, lh = lane >> 5;
     const int wm0 = __builtin_amdgcn_readfirstlane((wave / T::WAVES_N) * T::WM);   // (scalars: see sgemm_shortk_kernel)
     const int wn0 = __builtin_amdgcn_readfirstlane((wave % T::WAVES_N) * T::WN);
@@ -553,7 +553,7 @@ __device__ __forceinline__ void shortk_staged_body(const GemmArgs& g, float* con
 {
     constexpr int BK = 32, PITCH = 36, PF = NSTAGE - 1;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar for the compiler too
     const int l32 = lane & 31, lh = lane >> 5;
     const int wm0 = __builtin_amdgcn_readfirstlane((wave >> 1) * 32), wn0 = __builtin_amdgcn_readfirstlane((wave & 1) * 32);   // (scalars: see sgemm_shortk_kernel)
     const int a_row = (wm0 + l32) * BK, a_swz = l32 & 7;
