@@ -1516,19 +1516,41 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         return stage_out(o, stream);
     }
     // Stride 1 with whole blocks of 32 channels and maps up to about 60 pixels wide: the input is
-    // read where it lies, a patch of it per workgroup and channel block kept in LDS with the zero
-    // padding around it (sgemm_conv_patch.hip) -- no padded copy, no table of tap offsets.
-    // That kernel has one tile shape, 256 x 128, and one workgroup per CU, so nothing hides a tile's
-    // prologue and epilogue: it is taken where those are small against the tile's K walk and the
-    // tiles fill their rows and the machine -- 64 steps or more, at least three quarters of the
-    // tile rows in use, two rounds of tiles or more (config 5: 840 against 856 us from the staged
-    // copy).  Elsewhere the staged gather with the planner's choice of tile is faster, often by far
-    // (32 x 128 x 56 x 56 -> 256: 440 against 449 us; 64 x 256 x 28 x 28 -> 256: 450 against 538 us;
-    // 32 x 512 x 7 x 7 -> 512: 88 against 534 us).
+    // read where it lies, patches of it per workgroup kept in LDS with the zero padding around them
+    // (sgemm_conv_patch.hip) -- no padded copy, no table of tap offsets.
+    // That kernel has one tile shape, 256 x 128, and one workgroup per CU.  Where its tiles fill
+    // their rows and the machine it is 5-7 % ahead of the staged gather with the planner's choice
+    // of tile, from 18 K steps on (batch 32 on 56 x 56 maps, us patch / staged: 64 -> 256 channels
+    // 223 / 239, 128 -> 256 418 / 439, 256 -> 256 807 / 856, 256 -> 512 1614 / 1656); where they do not
+    // it loses by what is left empty (256 -> 192: 805 / 661; batch 16, 1.5 rounds: 518 / 437; batch
+    // 48, 4.6 rounds: 1302 / 1276).  So it is taken when 95 % of the tile rows are in use and its
+    // rounds -- whole ones, plus what the planner's cut of a thin last round costs: sub-tiles at a
+    // tenth of a round per 256 of them, K slices at a slice's share and a tenth -- come to no more
+    // than 1.06 times (1.03 for filters other than 3 x 3, whose K walk keeps its places at run time)
+    // the tiles' own count in rounds.
     int patch_rows = 0, patch_pitch = 0;
-    const long patch_tiles_m = (Cout + 255) / 256, patch_tiles_n = ((long)batch * Hout * row_n + 127) / 128;
-    const bool patch_pays = conv_patch_k(Cin, Hf, Wf) / 32 >= 64 && 4L * Cout >= 3L * 256 * patch_tiles_m &&
-                            patch_tiles_m * patch_tiles_n >= 2L * cur().model.cus;
+    bool patch_pays = false;
+    {
+        const int cus = cur().model.cus;
+        const long tiles_m = (Cout + 255) / 256, tiles_n = ((long)batch * Hout * row_n + 127) / 128, tiles = tiles_m * tiles_n;
+        const int taps = Hf * Wf, steps = conv_patch_k(Cin, Hf, Wf) / 32;
+        const int tile[4] = {256, 128, 32, 0};
+        GemmPlan pp;
+        if (steps >= 18 && 20L * Cout >= 19L * 256 * tiles_m && tiles >= cus && fits_int((double)batch * Hout * row_n) &&
+            plan_gemm(Cout, batch * Hout * row_n, steps * 32, CAKE_HIP_NA, tile, true, cur().model, &pp) == CAKE_HIP_OK) {
+            const int tail = pp.pub.tail_tiles;
+            double rounds = (double)((tiles - tail + cus - 1) / cus);
+            if (tail > 0) {
+                const int blocks = steps / taps;                  // K slices are whole blocks of 32 channels
+                const int slices = std::min(blocks, std::max(1, pp.pub.tail_split));
+                if (taps == 9 && tail * CONV_TAIL_SUBTILES_PER_TILE <= 2 * cus)
+                    rounds += 0.1 * ((tail * CONV_TAIL_SUBTILES_PER_TILE + cus - 1) / cus);
+                else
+                    rounds += slices > 1 ? 1.0 / slices + 0.1 : 1.0;
+            }
+            patch_pays = rounds <= (Hf == 3 && Wf == 3 ? 1.06 : 1.03) * (double)tiles / cus;
+        }
+    }
     // CAKE_HIP_CONV_ROUTE=patch takes that kernel wherever its geometry allows, =staged never
     // (for tests and measurements; read at every call)
     const char* route = std::getenv("CAKE_HIP_CONV_ROUTE");

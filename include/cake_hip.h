@@ -296,8 +296,9 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * patches of the input per workgroup in LDS, zero padding in place; under a
  * 3 x 3 filter the filters are read where they lie as well and the call is
  * that one kernel); it has a single 256 x 128 tile and is taken where that
- * pays -- 64 K steps or more, tile rows at least three quarters full, two
- * rounds of tiles or more.  The environment variable CAKE_HIP_CONV_ROUTE (read
+ * pays -- 18 K steps or more, 95 % of the tile rows in use, and rounds of tiles
+ * that fill the device (a thin last round cut into sub-tiles or K slices
+ * counted for what it costs).  The environment variable CAKE_HIP_CONV_ROUTE (read
  * at every call) overrides that choice: "patch" takes this kernel wherever
  * its geometry allows, "staged" never.
  * A batch whose staged input
