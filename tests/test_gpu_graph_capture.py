@@ -93,7 +93,7 @@ def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
     monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")   # layers this small would take the staged copy by themselves
     dev = torch.device("cuda:0")
     lib = cake.load()
-    geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: 16 tail tiles in 2 slices
+    geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: the 16 of the last round as sub-tiles
              (3, 16, 12, 12, 32, 3, 3, 2, 1, lib.cake_hip_conv2d),         # staged copy
              (2, 8, 16, 16, 24, 3, 3, 1, 1, lib.cake_hip_conv2d_im2col)]   # column matrix first
     ins, wts = [], []
