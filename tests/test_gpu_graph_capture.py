@@ -86,14 +86,16 @@ def test_captured_sequence_replays_like_eager_calls():
 
 
 def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
-    """The convolution routes under capture: the input read where it lies (re-laid filters, tail
-    slices summed by a second kernel), the gather from a staged copy (stride 2: staging kernel,
-    tap table) and the reference's two steps (column matrix in a workspace).  A larger eager
+    """The convolution routes under capture: the input read where it lies (under a 3 x 3 filter one
+    kernel with the last round in sub-tiles; under a 5 x 3 one re-laid filters and tail slices
+    summed by a second kernel), the gather from a staged copy (stride 2: staging kernel, tap
+    table) and the reference's two steps (column matrix in a workspace).  A larger eager
     convolution between the replays grows every one of those workspaces."""
     monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")   # layers this small would take the staged copy by themselves
     dev = torch.device("cuda:0")
     lib = cake.load()
     geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: the 16 of the last round as sub-tiles
+             (34, 64, 32, 32, 40, 5, 3, 1, 2, lib.cake_hip_conv2d),        # the same under 15 taps: re-laid filters, K slices
              (3, 16, 12, 12, 32, 3, 3, 2, 1, lib.cake_hip_conv2d),         # staged copy
              (2, 8, 16, 16, 24, 3, 3, 1, 1, lib.cake_hip_conv2d_im2col)]   # column matrix first
     ins, wts = [], []
@@ -124,13 +126,15 @@ def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
         run(captured, torch.cuda.current_stream().cuda_stream)
 
     def grow_every_workspace():
-        for b, cin, h, w, cout, s, fn in ((70, 64, 32, 32, 300, 1, lib.cake_hip_conv2d), (8, 32, 40, 40, 64, 2, lib.cake_hip_conv2d),
-                                          (8, 16, 32, 32, 48, 1, lib.cake_hip_conv2d_im2col)):
+        # (the first one under 15 taps: more re-laid filters and more K slices of a last round than captured)
+        for b, cin, h, w, cout, hf, wf, s, p, fn in ((70, 96, 32, 32, 300, 5, 3, 1, 2, lib.cake_hip_conv2d),
+                                                     (8, 32, 40, 40, 64, 3, 3, 2, 1, lib.cake_hip_conv2d),
+                                                     (8, 16, 32, 32, 48, 3, 3, 1, 1, lib.cake_hip_conv2d_im2col)):
             x = torch.empty((b, cin, h, w), dtype=torch.float32, device=dev)
-            f = torch.empty((cout, cin, 3, 3), dtype=torch.float32, device=dev)
-            ho = (h + 2 - 3) // s + 1
-            o = torch.empty((b, cout, ho, ho), dtype=torch.float32, device=dev)
-            assert fn(x.data_ptr(), f.data_ptr(), o.data_ptr(), b, cin, h, w, cout, 3, 3, s, 1, 1, None, None, None) == 0
+            f = torch.empty((cout, cin, hf, wf), dtype=torch.float32, device=dev)
+            ho, wo = (h + 2 * p - hf) // s + 1, (w + 2 * p - wf) // s + 1
+            o = torch.empty((b, cout, ho, wo), dtype=torch.float32, device=dev)
+            assert fn(x.data_ptr(), f.data_ptr(), o.data_ptr(), b, cin, h, w, cout, hf, wf, s, p, 1, None, None, None) == 0
         torch.cuda.synchronize()
 
     for replay in range(4):
