@@ -618,98 +618,128 @@ static dim3 rowwise_grid(int rows, int cols)
 // packed layouts a micro-panel is stored with its short axis fastest: A as [k][mr rows], B and C
 // as [k or row][nr columns].  A thread per row-major element therefore scatters 4-byte stores
 // `fast` floats apart (A) or writes 64-byte pieces (B, C).  Here a workgroup takes a tile of up
-// to 64 x 64 elements whose short-axis extent is a whole number of panels, moves it between the
-// row-major side and LDS with rows of 256 bytes, and walks the packed side in packed order
+// to TR x TC elements whose short-axis extent is a whole number of panels, moves it between the
+// row-major side and LDS in rows of TC floats, and walks the packed side in packed order
 // (short axis fastest, then the long axis, then the next panel), which is ascending addresses
 // wherever the tile lies inside one block of the schedule.  Offsets still come from the index
 // tables, so a tile that straddles blocks or starts off a panel boundary is only slower.
-static constexpr int PT = 64;
+// Tiles of 16 to 32 rows of 512 bytes: with 64 x 64 tiles (256-byte rows) 8192 x 8192 took 115-130 us,
+// with these 96-110 us, where a plain copy of as many bytes takes 99 us; 32 x 256 and 64 x 128
+// (twice the elements per thread) were 10 % slower than 64 x 64, 16-byte accesses on either
+// side changed nothing.  STREAM: both sides bypass the caches' keep-for-later policy; it pays from
+// about 100 MB per side on (8192 x 8192: 104 -> 96 us) and costs 10 % where both sides fit the
+// memory-side cache (4096 x 4096: 28 -> 31 us).
+template <bool STREAM>
+__device__ __forceinline__ float pack_load(const float* p)
+{
+    return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
 
-template <bool UNPACK>
+template <bool STREAM>
+__device__ __forceinline__ void pack_store(float v, float* p)
+{
+    if (STREAM) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
+// TC and the long axis of the packed walk (TC when rows are the fast axis, else TR) are powers of two.
+template <bool UNPACK, int TR, int TC, bool STREAM>
 __global__ void __launch_bounds__(256) pack_tile_kernel(const float* __restrict__ src, float* __restrict__ dst,
                                                         int rows, int cols, int ld, int rows_p, int cols_p,
-                                                        IndexTables tab, int fast, int rows_fast, int tr, int tc)
+                                                        IndexTables tab, int fast, int rows_fast, int tr, int tc,
+                                                        int pitch, int lshift)
 {
-    // Row pitch 64 + ceil(64 / fast): a wave walking the packed order touches `fast` short-axis
-    // positions times 64 / fast long-axis positions, which this pitch spreads over all banks
-    __shared__ float tile[PT * 2 * PT];
-    __shared__ int4 Rt[PT], Ct[PT];
-    const int pitch = PT + (PT + fast - 1) / fast;
+    constexpr int N = TR * TC / 256;      // elements per thread
+    constexpr int RPP = 256 / TC;         // rows per pass of the row-major side
+    static_assert(TR * TC % 256 == 0 && 256 % TC == 0, "a pass of the row-major side covers whole rows");
+    __shared__ float tile[TR * (TC + 64)];
+    __shared__ int4 Rt[TR], Ct[TC];
     const int tid = threadIdx.x;
     const int r0 = blockIdx.y * tr, c0 = blockIdx.x * tc;
-    if (tid < PT) {
-        if (tid < tr && r0 + tid < rows_p) Rt[tid] = tab.row[r0 + tid];
-    } else if (tid < 2 * PT) {
-        const int i = tid - PT;
-        if (i < tc && c0 + i < cols_p) Ct[i] = tab.col[c0 + i];
+    for (int i = tid; i < TR + TC; i += 256) {
+        if (i < TR) {
+            if (i < tr && r0 + i < rows_p) Rt[i] = tab.row[r0 + i];
+        } else {
+            const int c = i - TR;
+            if (c < tc && c0 + c < cols_p) Ct[c] = tab.col[c0 + c];
+        }
     }
     const int lim_r = UNPACK ? rows : rows_p, lim_c = UNPACK ? cols : cols_p;  // extent of the packed-side walk
-    const int dc_rm = tid & 63;   // row-major side: a wave per row of the tile
+    const int dc_rm = tid % TC, dr_rm = tid / TC;
     const float inv_fast = 1.0f / (float)fast;
     const int count = tr * tc;
+    const int lmask = (1 << lshift) - 1;
 
-    // Fixed trip counts and full unrolling: all 16 loads of a thread are in flight together
+    // Fixed trip counts and full unrolling: all N loads of a thread are in flight together
     // (with a run-time bound the compiler keeps one load per thread in flight, and the kernel
-    // runs at the speed of 16 memory latencies per tile).
+    // runs at the speed of N memory latencies per tile).
     if (!UNPACK) {
-        float v[PT / 4];
+        float v[N];
 #pragma unroll
-        for (int i = 0; i < PT / 4; ++i) {
-            const int dr = (tid >> 6) + 4 * i;
+        for (int i = 0; i < N; ++i) {
+            const int dr = dr_rm + RPP * i;
             const int r = r0 + dr, c = c0 + dc_rm;
-            v[i] = (dr < tr && dc_rm < tc && r < rows && c < cols) ? src[(size_t)r * ld + c] : 0.f;
+            v[i] = (dr < tr && dc_rm < tc && r < rows && c < cols) ? pack_load<STREAM>(src + (size_t)r * ld + c) : 0.f;
         }
 #pragma unroll
-        for (int i = 0; i < PT / 4; ++i) tile[((tid >> 6) + 4 * i) * pitch + dc_rm] = v[i];
+        for (int i = 0; i < N; ++i) tile[(dr_rm + RPP * i) * pitch + dc_rm] = v[i];
     }
     __syncthreads();
     {
-        float v[PT * PT / 256];
-        size_t off[PT * PT / 256];
-        int at[PT * PT / 256];
-        bool live[PT * PT / 256];
+        float v[N];
+        size_t off[N];
+        int at[N];
+        bool live[N];
 #pragma unroll
-        for (int i = 0; i < PT * PT / 256; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int e = tid + 256 * i;
             // e = (panel * long + l) * fast + j; exact for e < 2^22: (e + 0.5) / fast is at least
             // 0.5 / fast away from an integer
             const int q = (int)(((float)e + 0.5f) * inv_fast);
             const int j = e - q * fast;
-            const int panel = q >> 6, l = q & 63;      // the long axis of a tile is 64
+            const int panel = q >> lshift, l = q & lmask;
             const int dr = rows_fast ? panel * fast + j : l;
             const int dc = rows_fast ? l : panel * fast + j;
             const int r = r0 + dr, c = c0 + dc;
             live[i] = e < count && dr < tr && dc < tc && r < lim_r && c < lim_c;
             off[i] = live[i] ? table_offset(Rt[dr], Ct[dc]) : 0;
             at[i] = dr * pitch + dc;
-            if (UNPACK) v[i] = live[i] ? src[off[i]] : 0.f;
+            if (UNPACK) v[i] = live[i] ? pack_load<STREAM>(src + off[i]) : 0.f;
             else v[i] = live[i] ? tile[at[i]] : 0.f;
         }
 #pragma unroll
-        for (int i = 0; i < PT * PT / 256; ++i) {
+        for (int i = 0; i < N; ++i) {
             if (!live[i]) continue;
             if (UNPACK) tile[at[i]] = v[i];
-            else dst[off[i]] = v[i];
+            else pack_store<STREAM>(v[i], dst + off[i]);
         }
     }
     if (UNPACK) {
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PT / 4; ++i) {
-            const int dr = (tid >> 6) + 4 * i;
+        for (int i = 0; i < N; ++i) {
+            const int dr = dr_rm + RPP * i;
             const int r = r0 + dr, c = c0 + dc_rm;
-            if (dr < tr && dc_rm < tc && r < rows && c < cols) dst[(size_t)r * ld + c] = tile[dr * pitch + dc_rm];
+            if (dr < tr && dc_rm < tc && r < rows && c < cols)
+                pack_store<STREAM>(tile[dr * pitch + dc_rm], dst + (size_t)r * ld + c);
         }
     }
 }
 
-// fast = rows (rows_fast) or columns of a micro-panel; 0 or more than 64: the element-wise kernels
-template <bool UNPACK>
-static hipError_t launch_pack_tiles(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
-                                    int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
+static constexpr int PACK_TC = 128;        // floats per row of a tile
+static constexpr int PACK_STREAM_BYTES = 100 << 20;
+
+template <bool UNPACK, int TR, int TC, bool STREAM>
+static hipError_t launch_pack_tiles_as(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
+                                       int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
 {
-    const int whole = fast * (PT / fast);   // a whole number of panels, at most 64
-    const int tr = rows_fast ? whole : PT, tc = rows_fast ? PT : whole;
+    const int tr = rows_fast ? fast * (TR / fast) : TR, tc = rows_fast ? TC : fast * (TC / fast);
+    // LDS pitch: a wave walking the packed order touches `fast` short-axis positions times 64 / fast
+    // long-axis positions; with rows fast, consecutive rows are ceil(64 / fast) banks apart, with
+    // columns fast, consecutive rows are `fast` banks apart
+    const int pitch = rows_fast ? TC + (64 + fast - 1) / fast : TC + (fast & 63);
+    int lshift = 0;
+    while ((1 << lshift) < (rows_fast ? TC : TR)) ++lshift;
     const int ext_r = UNPACK ? rows : rows_p, ext_c = UNPACK ? cols : cols_p;
     const int tiles_c = (ext_c + tc - 1) / tc;
     const int tiles_r = (ext_r + tr - 1) / tr;
@@ -720,19 +750,55 @@ static hipError_t launch_pack_tiles(const float* src, float* dst, int rows, int 
         const float* s = UNPACK ? src : src + (size_t)r0 * ld;
         float* d = UNPACK ? dst + (size_t)r0 * ld : dst;
         const int live = rows - r0 < 0 ? 0 : rows - r0;
-        hipLaunchKernelGGL(pack_tile_kernel<UNPACK>, dim3(tiles_c, nt), dim3(256), 0, stream, s, d, live, cols, ld,
-                           rows_p - r0, cols_p, t, fast, rows_fast ? 1 : 0, tr, tc);
+        hipLaunchKernelGGL((pack_tile_kernel<UNPACK, TR, TC, STREAM>), dim3(tiles_c, nt), dim3(256), 0, stream, s, d,
+                           live, cols, ld, rows_p - r0, cols_p, t, fast, rows_fast ? 1 : 0, tr, tc, pitch, lshift);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
 }
 
+// Largest short-axis extent a tile kernel takes: rows of a micro-panel of A up to 64, columns of one of B or C up to 128.
+static bool pack_tiles_take(int fast, bool rows_fast)
+{
+    return fast >= 1 && fast <= (rows_fast ? 64 : PACK_TC);
+}
+
+// fast = rows (rows_fast) or columns of a micro-panel.  Tile height: 16 rows, or with rows fast the one of
+// 16, 24 and 32 that whole panels fill best (m_r = 6: 24), 64 x 64 tiles for panels of more than 32 rows.
+template <bool UNPACK>
+static hipError_t launch_pack_tiles(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
+                                    int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
+{
+    const bool big = (size_t)rows * (size_t)cols * sizeof(float) >= (size_t)PACK_STREAM_BYTES;
+    int tr = 16;
+    if (rows_fast) {
+        if (fast > 32) tr = 64;
+        else {
+            int best = 0;
+            for (int cand : {16, 24, 32}) {
+                const int used = 1000 * (fast * (cand / fast)) / cand;
+                if (used > best) { best = used; tr = cand; }
+            }
+        }
+    }
+#define CAKE_PACK_TILES(TR, TC) \
+    return big ? launch_pack_tiles_as<UNPACK, TR, TC, true>(src, dst, rows, cols, ld, rows_p, cols_p, tab, fast, rows_fast, stream) \
+               : launch_pack_tiles_as<UNPACK, TR, TC, false>(src, dst, rows, cols, ld, rows_p, cols_p, tab, fast, rows_fast, stream)
+    switch (tr) {
+        case 16: CAKE_PACK_TILES(16, PACK_TC);
+        case 24: CAKE_PACK_TILES(24, PACK_TC);
+        case 32: CAKE_PACK_TILES(32, PACK_TC);
+        default: CAKE_PACK_TILES(64, 64);
+    }
+#undef CAKE_PACK_TILES
+}
+
 hipError_t launch_pack(const float* src, float* dst, int rows, int cols, int ld, int rows_p,
                        int cols_p, IndexTables tab, int fast, bool rows_fast, hipStream_t stream)
 {
     if (rows_p <= 0 || cols_p <= 0) return hipSuccess;
-    if (fast >= 1 && fast <= PT)
+    if (pack_tiles_take(fast, rows_fast))
         return launch_pack_tiles<false>(src, dst, rows, cols, ld, rows_p, cols_p, tab, fast, rows_fast, stream);
     // grid.y is limited to 65535 rows per launch
     for (int r0 = 0; r0 < rows_p; r0 += 65535) {
@@ -751,7 +817,7 @@ hipError_t launch_unpack(const float* src, float* dst, int rows, int cols, int l
                          int fast, bool rows_fast, hipStream_t stream)
 {
     if (rows <= 0 || cols <= 0) return hipSuccess;
-    if (fast >= 1 && fast <= PT)
+    if (pack_tiles_take(fast, rows_fast))
         return launch_pack_tiles<true>(src, dst, rows, cols, ld, rows, cols, tab, fast, rows_fast, stream);
     for (int r0 = 0; r0 < rows; r0 += 65535) {
         const int nr = rows - r0 < 65535 ? rows - r0 : 65535;

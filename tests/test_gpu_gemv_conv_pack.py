@@ -485,6 +485,51 @@ def test_pack_unpack_bit_exact(shape, sch, p):
         assert oracle.max_rel_err(out, C64, S) <= TIGHT, (pa, pb)
 
 
+def _pack_round_trip(M, K, N, p, sch, ocx, ccx, device=False):
+    """pack_A, pack_B, pack_C against the oracle bit for bit, unpack_C back to the values packed."""
+    xo = oracle.init_block_dims(M, N, K, p, ocx, sch)
+    xc = cake.init_block_dims(M, N, K, p, ccx, sch)
+    A, B, Cm = oracle.uniform((M, K), 21), oracle.uniform((K, N), 22), oracle.uniform((M, N), 23)
+    sizes = (cake.cake_sgemm_packed_A_size(M, K, p, xc, ccx, sch) // 4, cake.cake_sgemm_packed_B_size(K, N, p, xc, ccx) // 4,
+             cake.cake_sgemm_packed_C_size(M, N, p, xc, ccx, sch) // 4)
+    if device:
+        import torch
+        dev = torch.device("cuda:0")
+        up = lambda a: torch.from_numpy(a).to(dev)
+        dn = lambda t: t.cpu().numpy()
+        new = lambda shape: torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+    else:
+        up = dn = lambda a: a
+        new = lambda shape: np.full(shape, np.nan, np.float32)
+    Ap, Bp, Cp, back = new((sizes[0],)), new((sizes[1],)), new((sizes[2],)), new((M, N))
+    cake.pack_A(up(A), Ap, M, K, p, xc, ccx, sch)
+    assert np.array_equal(dn(Ap), oracle.pack_A(A, p, xo, ocx, sch))
+    cake.pack_B(up(B), Bp, K, N, p, xc, ccx, sch)
+    assert np.array_equal(dn(Bp), oracle.pack_B(B, p, xo, ocx, sch))
+    cake.pack_C(up(Cm), Cp, M, N, p, xc, ccx, sch)
+    assert np.array_equal(dn(Cp), oracle.pack_C(Cm, p, xo, ocx, sch))
+    cake.unpack_C(back, Cp, M, N, p, xc, ccx, sch)
+    assert np.array_equal(dn(back), Cm)
+
+
+# micro-panels of every tile height of the copy kernels (16, 24, 32 and 64 rows), panels wider than a
+# tile row is long (one thread per element instead), sizes that are no multiple of 4
+@pytest.mark.parametrize("sch", [cake.KMN, cake.MKN, cake.NKM])
+@pytest.mark.parametrize("mr,nr", [(8, 12), (4, 48), (14, 24), (30, 8), (12, 64), (40, 100), (64, 128), (6, 160), (70, 16),
+                                   (5, 7), (1, 1)])
+def test_pack_unpack_other_micro_panels(mr, nr, sch):
+    print(f"pack mr={mr} nr={nr} sch={sch}", flush=True)
+    ocx, ccx = _cx(mr=mr, nr=nr, L2=256 << 10, L3=2 << 20)
+    for (M, K, N), p in (((333, 270, 401), 3), ((130, 515, 259), 8)):
+        _pack_round_trip(M, K, N, p, sch, ocx, ccx)
+
+
+def test_pack_unpack_operands_past_the_streaming_threshold():
+    """From 100 MB per operand on the copy kernels read and write past the caches; device operands."""
+    ocx, ccx = _cx()
+    _pack_round_trip(5200, 5200, 5200, 8, cake.KMN, ocx, ccx, device=True)
+
+
 def test_packed_sgemm_through_reference_call_sequence():
     """examples/cake_conv.cpp:1028-1055: init_block_dims -> pack_A, pack_B -> cake_sgemm(..., 1, 1, 1, 0, KMN)."""
     M, K, N, p = 96, 8 * 9, 30 * 28, 10
