@@ -108,6 +108,13 @@ def test_sgemv_deterministic():
 @pytest.mark.parametrize("geom", [
     (1, 3, 18, 18, 3, 3, 1, 0), (2, 5, 9, 13, 3, 3, 1, 1), (3, 4, 12, 12, 3, 3, 2, 1),
     (1, 2, 6, 7, 1, 1, 1, 0), (2, 4, 8, 8, 5, 3, 1, 2), (4, 16, 14, 14, 3, 3, 1, 1), (1, 1, 7, 30, 3, 3, 3, 0),
+    # workgroups of 1024 columns that span many small images, columns that are no multiple of 4,
+    # padding beyond the filter's reach, strides with padding, a filter width without an unrolled kernel
+    (40, 3, 7, 7, 3, 3, 1, 1), (9, 2, 14, 14, 3, 3, 1, 1), (3, 2, 5, 5, 3, 3, 1, 0), (23, 2, 9, 11, 3, 3, 1, 2),
+    (7, 3, 31, 29, 5, 5, 2, 2), (5, 2, 33, 40, 7, 7, 3, 3), (6, 2, 20, 21, 2, 4, 1, 1), (3, 1, 64, 64, 3, 3, 2, 0),
+    (2, 3, 224, 224, 7, 7, 2, 3), (300, 1, 3, 3, 3, 3, 1, 1), (1500, 1, 1, 1, 1, 1, 1, 0), (2, 2, 40, 5, 11, 3, 4, 1),
+    # rows too wide for the staged kernel's LDS: the kernel that loads every window from memory
+    (1, 2, 5, 4100, 3, 3, 1, 1), (2, 1, 9, 2500, 5, 5, 2, 2),
 ], ids=str)
 def test_im2col_bit_exact(geom):
     Bn, Cin, Hin, Win, Hf, Wf, stride, pad = geom
