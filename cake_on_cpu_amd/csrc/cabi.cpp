@@ -1641,11 +1641,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
         int* taps = static_cast<int*>(cur().conv_taps.ptr);
         if ((st = timer.start())) return st;
         const bool one_by_one = Hf == 1 && Wf == 1;   // row k is channel k: no table of tap offsets
-        if (!one_by_one) {
+        // the table of tap offsets is written by the launch that stages the first chunk of images,
+        // or by a launch of its own where the input is read as it lies
+        bool table_due = !one_by_one;
+        if (table_due && !sg.copy) {
             st = timer.family(3, [&] {
                 return launch_conv_tap_table(taps, K, CONV_TAP_TABLE_EXTRA, sg.Hs, sg.pitch, sg.Wq, Hf, Wf, stride, sg.RH, stream);
             });
             if (st) return st;
+            table_due = false;
         }
         const size_t HW = (size_t)Hout * Wout;
         for (int b0 = 0; b0 < batch; b0 += chunk) {
@@ -1653,12 +1657,11 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
             const float* src = i.dev + (size_t)b0 * Cin * Hin * Win;
             if (sg.copy) {
                 st = timer.family(3, [&] {
-                    // stride 1: the plain zero-padded copy has a kernel of its own (a workgroup per plane)
-                    return stride == 1 ? launch_pad_planes(src, staged, (size_t)nb * Cin, Hin, Win, pad, sg.pitch, stream)
-                                       : launch_conv_stage_input(src, staged, (size_t)nb * Cin, Hin, Win, pad, stride,
-                                                                 sg.RH, sg.PW, sg.Hs, sg.Wq, stream);
+                    return launch_conv_stage_input(src, staged, (size_t)nb * Cin, Hin, Win, pad, stride, sg.RH, sg.PW, sg.Hs,
+                                                   sg.Wq, table_due ? taps : nullptr, K, CONV_TAP_TABLE_EXTRA, Hf, Wf, stream);
                 });
                 if (st) return st;
+                table_due = false;
             }
             ConvGeom cv{};
             cv.in = sg.copy ? staged : src;

@@ -210,14 +210,12 @@ hipError_t launch_sgemv_colmajor(const float* A, const float* x, float* y, int M
 hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int Hin, int Win,
                          int Hf, int Wf, int Hout, int Wout, int stride, int pad,
                          hipStream_t stream);
-// out[plane][y][x] = in[plane][y - pad][x - pad], zero in the border and in the row tail; out planes
-// are (Hin+2pad) rows of `pitch` floats (pitch % 4 == 0, pitch >= Win+2pad, out 16-byte aligned)
-hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                             int pitch, hipStream_t stream);
 // The input of a convolution staged for the gather: see conv_stage_input_kernel.  `out` holds
 // planes * Hs * PW * Wq floats (Wq % 4 == 0, 16-byte aligned).
+// `table` (may be nullptr) is filled in the same launch: launch_conv_tap_table's K + extra entries.
 hipError_t launch_conv_stage_input(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                                   int stride, int RH, int PW, int Hs, int Wq, hipStream_t stream);
+                                   int stride, int RH, int PW, int Hs, int Wq, int* table, int K, int extra,
+                                   int Hf, int Wf, hipStream_t stream);
 // table[k] = byte offset of filter tap k inside one staged image; `extra` zero entries follow
 enum { CONV_TAP_TABLE_EXTRA = 256 };
 hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch, int Wq, int Hf, int Wf,

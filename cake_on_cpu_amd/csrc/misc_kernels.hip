@@ -133,45 +133,12 @@ hipError_t launch_filter_layout(const float* src, float* dst, const PackGeom& g,
     return hipGetLastError();
 }
 
-// ---------------------------------------------------------------------------
-// zero padding of image planes: the convolution's gather then needs no edge
-// tests.  Output rows are `pitch` floats apart (a multiple of 4, >= Win + 2 pad),
-// so every thread writes one aligned float4; reads run along image rows.  One
-// workgroup per plane: 16 lanes along a row, 16 rows at a time.
-// ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) pad_planes_kernel(const float* __restrict__ in,
-                                                         float* __restrict__ out, size_t planes,
-                                                         int Hin, int Win, int pad, int pitch)
+__device__ __forceinline__ int conv_tap_offset(int k, int Hs, int pitch, int Wq, int Hf, int Wf, int stride, int RH)
 {
-    const int Hp = Hin + 2 * pad;
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    for (size_t plane = blockIdx.x; plane < planes; plane += gridDim.x) {
-        const float* src = in + plane * Hin * Win;
-        float* dst = out + plane * Hp * pitch;
-        for (int y = ty; y < Hp; y += 16) {
-            const int yi = y - pad;
-            const bool row_in = (unsigned)yi < (unsigned)Hin;
-            for (int x = tx * 4; x < pitch; x += 64) {
-                f32x4 v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int xi = x + e - pad;
-                    v[e] = (row_in && (unsigned)xi < (unsigned)Win) ? src[yi * Win + xi] : 0.f;
-                }
-                *reinterpret_cast<f32x4*>(dst + y * pitch + x) = v;
-            }
-        }
-    }
-}
-
-hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                             int pitch, hipStream_t stream)
-{
-    if (planes == 0) return hipSuccess;
-    if (pitch % 4 != 0 || pitch < Win + 2 * pad) return hipErrorInvalidValue;
-    const unsigned blocks = (unsigned)(planes < (1u << 20) ? planes : (1u << 20));
-    hipLaunchKernelGGL(pad_planes_kernel, dim3(blocks), dim3(256), 0, stream, in, out, planes, Hin, Win, pad, pitch);
-    return hipGetLastError();
+    const int c = k / (Hf * Wf), tap = k - c * (Hf * Wf);
+    const int h = tap / Wf, w = tap - h * Wf;
+    const int row = (h / stride) * RH + h % stride;
+    return ((c * Hs + row) * pitch + (w % stride) * Wq + w / stride) * 4;
 }
 
 // The input of a strided convolution, staged so that the gather reads consecutive floats: a row
@@ -183,14 +150,24 @@ hipError_t launch_pad_planes(const float* in, float* out, size_t planes, int Hin
 //     plane[(ho + h / s) * RH + h % s][w % s][wo + w / s]
 // whose address splits into a pixel part (ho * RH * pitch + wo, pitch = PW * Wq) and a tap part,
 // and 4 consecutive wo are 4 consecutive floats.  stride 1 is the plain zero-padded copy.
-// One thread per float4 of the staged image.
+// One thread per float4 of the staged image; at stride 1 the four values are one 16-byte load
+// wherever they lie inside a row of the image (any 4-byte alignment).  The workgroups past
+// `stage_blocks` write the table of tap offsets (conv_tap_table_kernel below) in the same launch,
+// so a convolution has one launch in front of its product, not two (table == nullptr: none).
 __global__ void __launch_bounds__(256) conv_stage_input_kernel(const float* __restrict__ in,
                                                                float* __restrict__ out, unsigned total4,
                                                                int Hin, int Win, int pad, int stride, int RH,
                                                                int PW, int Hs, int Wq, FastDiv by_wq4,
-                                                               FastDiv by_pw, FastDiv by_hs, FastDiv by_rh)
+                                                               FastDiv by_pw, FastDiv by_hs, FastDiv by_rh,
+                                                               unsigned stage_blocks, int* __restrict__ table, int K,
+                                                               int extra, int Hf, int Wf)
 {
-    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < total4; i += gridDim.x * 256) {
+    if (blockIdx.x >= stage_blocks) {
+        const int k = (blockIdx.x - stage_blocks) * 256 + threadIdx.x;
+        if (k < K + extra) table[k] = k < K ? conv_tap_offset(k, Hs, PW * Wq, Wq, Hf, Wf, stride, RH) : 0;
+        return;
+    }
+    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < total4; i += stage_blocks * 256) {
         unsigned t = by_wq4.div(i);
         const int wq = (int)(i - t * by_wq4.d) * 4;
         unsigned u = by_pw.div(t);
@@ -202,26 +179,34 @@ __global__ void __launch_bounds__(256) conv_stage_input_kernel(const float* __re
         const float* src = in + ((size_t)plane * Hin + yi) * Win;
         const bool row_in = (unsigned)yi < (unsigned)Hin;
         f32x4 v;
+        const int x0 = wq - pad;
+        if (stride == 1 && row_in && x0 >= 0 && x0 + 3 < Win) {
+            v = *reinterpret_cast<const f32x4_u*>(src + x0);
+        } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int xi = (wq + e) * stride + ph - pad;
-            v[e] = (row_in && (unsigned)xi < (unsigned)Win) ? src[xi] : 0.f;
+            for (int e = 0; e < 4; ++e) {
+                const int xi = (wq + e) * stride + ph - pad;
+                v[e] = (row_in && (unsigned)xi < (unsigned)Win) ? src[xi] : 0.f;
+            }
         }
         *reinterpret_cast<f32x4*>(out + (size_t)i * 4) = v;
     }
 }
 
 hipError_t launch_conv_stage_input(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
-                                   int stride, int RH, int PW, int Hs, int Wq, hipStream_t stream)
+                                   int stride, int RH, int PW, int Hs, int Wq, int* table, int K, int extra,
+                                   int Hf, int Wf, hipStream_t stream)
 {
     const size_t total4 = planes * Hs * PW * (Wq / 4);
     if (total4 == 0) return hipSuccess;
     if (Wq % 4 != 0 || total4 >= (1ull << 31)) return hipErrorInvalidValue;
     size_t blocks = (total4 + 255) / 256;
     if (blocks > (1u << 20)) blocks = 1u << 20;
-    hipLaunchKernelGGL(conv_stage_input_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, in, out,
+    const unsigned table_blocks = table ? (unsigned)((K + extra + 255) / 256) : 0u;
+    hipLaunchKernelGGL(conv_stage_input_kernel, dim3((unsigned)blocks + table_blocks), dim3(256), 0, stream, in, out,
                        (unsigned)total4, Hin, Win, pad, stride, RH, PW, Hs, Wq, FastDiv::make((unsigned)(Wq / 4)),
-                       FastDiv::make((unsigned)PW), FastDiv::make((unsigned)Hs), FastDiv::make((unsigned)RH));
+                       FastDiv::make((unsigned)PW), FastDiv::make((unsigned)Hs), FastDiv::make((unsigned)RH),
+                       (unsigned)blocks, table, K, extra, Hf, Wf);
     return hipGetLastError();
 }
 
@@ -234,10 +219,7 @@ __global__ void __launch_bounds__(256) conv_tap_table_kernel(int* __restrict__ t
 {
     const int k = blockIdx.x * 256 + threadIdx.x;
     if (k >= K + extra) return;
-    const int c = k / (Hf * Wf), tap = k - c * (Hf * Wf);
-    const int h = tap / Wf, w = tap - h * Wf;
-    const int row = (h / stride) * RH + h % stride;
-    table[k] = k < K ? ((c * Hs + row) * pitch + (w % stride) * Wq + w / stride) * 4 : 0;
+    table[k] = k < K ? conv_tap_offset(k, Hs, pitch, Wq, Hf, Wf, stride, RH) : 0;
 }
 
 hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch, int Wq, int Hf, int Wf,
