@@ -52,23 +52,23 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563234669, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_8192": (4563255275, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
     "sgemm_1024": (29500957, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
     "sgemm_tall_skinny": (306412911, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
-    "sgemv_16384_rowmajor": (1074454808, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
-    "sgemv_16384_colmajor": (1075872903, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (278905814, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 3, 3>` grid 524288"),
-    "conv_c5_two_step": (2206526220, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129061250, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (42917801, "row `sgemm_shortk_staged_flat_kernel` grid 262144"),
-    "resident_8192x256x8192": (400698411, "row `sgemm_resident_kernel` grid 131072"),
-    "staged_3000x100x3000": (44742434, "row `sgemm_shortk_staged_kernel` grid 262144"),
-    "fewrows_nn": (1087400124, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nn_64rows": (1128387616, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
-    "narrow_tile_32cols": (288883396, "row `sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0>` grid 131072"),
-    "fewrows_nt": (1083225768, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_16x16384x16384": (1083225768, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_8192x4096x4096": (1208270602, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "sgemv_16384_rowmajor": (1074454809, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
+    "sgemv_16384_colmajor": (1075873031, "row `sgemv_colmajor_kernel<true>` grid 196608"),
+    "conv_c5_gather": (278904781, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 3, 3>` grid 524288"),
+    "conv_c5_two_step": (2212091572, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129060149, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (43105781, "row `sgemm_shortk_staged_flat_kernel` grid 262144"),
+    "resident_8192x256x8192": (400705391, "row `sgemm_resident_kernel` grid 131072"),
+    "staged_3000x100x3000": (44978223, "row `sgemm_shortk_staged_kernel` grid 262144"),
+    "fewrows_nn": (1087400122, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nn_64rows": (1128387618, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
+    "narrow_tile_32cols": (288997411, "row `sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0>` grid 131072"),
+    "fewrows_nt": (1083225769, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083225769, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_8192x4096x4096": (1208264117, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
