@@ -216,6 +216,10 @@ hipError_t launch_im2col(const float* in, float* cols, int batch, int Cin, int H
 hipError_t launch_conv_stage_input(const float* in, float* out, size_t planes, int Hin, int Win, int pad,
                                    int stride, int RH, int PW, int Hs, int Wq, int* table, int K, int extra,
                                    int Hf, int Wf, hipStream_t stream);
+// out[plane][ho][wo] = in[plane][ho * stride][wo * stride], out dense and 16-byte aligned,
+// planes * Hout * Wout < 2^31
+hipError_t launch_subsample_planes(const float* in, float* out, size_t planes, int Hin, int Win, int Hout, int Wout,
+                                   int stride, hipStream_t stream);
 // table[k] = byte offset of filter tap k inside one staged image; `extra` zero entries follow
 enum { CONV_TAP_TABLE_EXTRA = 256 };
 hipError_t launch_conv_tap_table(int* table, int K, int extra, int Hs, int pitch, int Wq, int Hf, int Wf,

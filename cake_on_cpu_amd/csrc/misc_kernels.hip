@@ -133,6 +133,58 @@ hipError_t launch_filter_layout(const float* src, float* dst, const PackGeom& g,
     return hipGetLastError();
 }
 
+// Every stride-th pixel of every stride-th row of each plane, densely: the input of a 1 x 1
+// convolution at that stride.  A thread per 4 consecutive outputs (one 16-byte store), their
+// (plane, row, column) carried from one to the next.
+__global__ void __launch_bounds__(256) subsample_planes_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                               unsigned total, int Hin, int Win, int Hout, int Wout,
+                                                               int stride, FastDiv by_hw, FastDiv by_wout)
+{
+    for (unsigned j = (blockIdx.x * 256 + threadIdx.x) * 4; j < total; j += gridDim.x * 1024) {
+        unsigned plane = by_hw.div(j);
+        const unsigned r = j - plane * by_hw.d;
+        int ho = (int)by_wout.div(r);
+        int wo = (int)(r - ho * Wout);
+        const int valid = (int)min(4u, total - j);
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (stride == 2 && valid == 4 && wo + 3 < Wout && 2 * wo + 7 < Win) {
+            // four outputs of one row under stride 2: eight consecutive input values, two 16-byte loads
+            const float* src = in + ((size_t)plane * Hin + (size_t)ho * 2) * Win + 2 * wo;
+            const f32x4_u a = *reinterpret_cast<const f32x4_u*>(src), b = *reinterpret_cast<const f32x4_u*>(src + 4);
+            v = f32x4{a[0], a[2], b[0], b[2]};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (e < valid) v[e] = in[((size_t)plane * Hin + (size_t)ho * stride) * Win + (size_t)wo * stride];
+                if (++wo == Wout) {
+                    wo = 0;
+                    if (++ho == Hout) { ho = 0; ++plane; }
+                }
+            }
+        }
+        if (valid == 4) {
+            *reinterpret_cast<f32x4*>(out + j) = v;
+        } else {
+            for (int e = 0; e < valid; ++e) out[j + e] = v[e];
+        }
+    }
+}
+
+hipError_t launch_subsample_planes(const float* in, float* out, size_t planes, int Hin, int Win, int Hout, int Wout,
+                                   int stride, hipStream_t stream)
+{
+    const size_t total = planes * Hout * Wout;
+    if (total == 0) return hipSuccess;
+    if (total >= (1ull << 31) || (reinterpret_cast<uintptr_t>(out) & 15) || (Hout - 1) * (long)stride >= Hin ||
+        (Wout - 1) * (long)stride >= Win)
+        return hipErrorInvalidValue;
+    size_t blocks = (total + 1023) / 1024;
+    if (blocks > (1u << 20)) blocks = 1u << 20;
+    hipLaunchKernelGGL(subsample_planes_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, in, out, (unsigned)total,
+                       Hin, Win, Hout, Wout, stride, FastDiv::make((unsigned)(Hout * Wout)), FastDiv::make((unsigned)Wout));
+    return hipGetLastError();
+}
+
 __device__ __forceinline__ int conv_tap_offset(int k, int Hs, int pitch, int Wq, int Hf, int Wf, int stride, int RH)
 {
     const int c = k / (Hf * Wf), tap = k - c * (Hf * Wf);

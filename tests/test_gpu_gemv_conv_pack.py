@@ -173,7 +173,11 @@ CONV_GEOMS = [
     (3, 5, 8, 8, 7, 1, 1, 1, 0),         # 1x1, K = 5
     (2, 3, 17, 17, 33, 3, 3, 2, 1),      # stride 2, K = 27, Wout = 9 (two-step) ...
     (2, 3, 15, 16, 33, 3, 3, 2, 1),      # ... and Wout = 8 (gathered from the phase-split copy)
-    (2, 8, 16, 16, 12, 1, 1, 2, 0),      # 1x1 stride 2: one row in two and one column phase are staged
+    (2, 8, 16, 16, 12, 1, 1, 2, 0),      # 1x1 stride 2: the pixels it reads are copied out densely, then a 1x1 layer at stride 1
+    (3, 20, 15, 13, 70, 1, 1, 2, 0),     # ... odd sizes: 8 x 7 outputs a plane, 56 a multiple of 4, planes across tile borders
+    (5, 7, 10, 11, 9, 1, 1, 3, 0),       # ... stride 3, 4 x 4 outputs, K = 7
+    (4, 96, 28, 28, 128, 1, 1, 2, 0),    # ... 14 x 14 outputs on 96 channels: the kernels with a short K
+    (2, 6, 9, 9, 5, 1, 1, 2, 1),         # 1x1 stride 2 with padding: staged like any other filter
     (2, 3, 32, 32, 16, 7, 7, 2, 3),      # 7x7 stride 2 pad 3 (a first layer), Wout = 16
     (1, 4, 33, 29, 6, 3, 3, 4, 1),       # stride 4 over a 3x3 filter: rows and phases skipped, Wout = 8
     (2, 2, 21, 27, 5, 2, 5, 3, 0),       # 2x5 filter, stride 3: Hf below and Wf above the stride, Wout = 8
