@@ -290,7 +290,9 @@ int cake_hip_im2col(const float* in, float* cols, int batch, int Cin, int Hin, i
  * without padding needs neither: a plane is then one row of Hin * Win pixels,
  * gathered from the input as it lies, and with at most 64 input channels and
  * enough tiles the images run as one batch of plain products on the short-K
- * kernel.  Stride-1 layers with whole blocks of 32 input channels, a filter of
+ * kernel.  A 1 x 1 filter at a stride above 1 without padding has the pixels
+ * it reads copied out densely first and then runs as such a layer on the copy.
+ * Stride-1 layers with whole blocks of 32 input channels, a filter of
  * 7 taps or more, up to 4 columns of padding and maps up to about 60 pixels
  * wide have a kernel that reads the input where it lies (no staged copy:
  * patches of the input per workgroup in LDS, zero padding in place; under a
