@@ -127,6 +127,48 @@ def test_transpose(big):
     torch.cuda.empty_cache()
 
 
+def test_im2col_columns_past_4_gb():
+    """A column matrix of 576 x 2 000 000 floats (4.6 GB): sampled rows, the last ones among them,
+    equal the shifted planes they are copies of, bit for bit."""
+    Bn, Cin, H, W, Hf, Wf, pad = 32, 64, 250, 250, 3, 3, 1
+    K, N = Cin * Hf * Wf, Bn * H * W
+    inp = _filled((Bn, Cin, H, W), 977)
+    cols = torch.full((K, N), float("nan"), dtype=torch.float32, device=_dev())
+    print(f"im2col {K}x{N}: {K * N * 4 / 1e9:.2f} GB", flush=True)
+    cake.im2col(inp, cols, Bn, Cin, H, W, Hf, Wf, 1, pad)
+    for k in (0, 1, 4, 8, 9, K // 2, K - 10, K - 9, K - 2, K - 1):
+        c, h, w = k // (Hf * Wf), (k % (Hf * Wf)) // Wf, k % Wf
+        padded = torch.nn.functional.pad(inp[:, c], (pad, pad, pad, pad))
+        assert torch.equal(cols[k], padded[:, h:h + H, w:w + W].reshape(-1)), k
+    del cols, inp
+    torch.cuda.empty_cache()
+
+
+def test_pack_and_unpack(big):
+    """pack_A and pack_C of the large matrix: sampled elements, the last rows among them, sit at the
+    offsets of the packed index map (evaluated on the host), and unpack_C brings every bit back."""
+    p = 8
+    ccx = cake.CpuCntx(1.0, 6, 16, 48 << 10, 2 << 20, 105 << 20, 8)
+    x = cake.init_block_dims(R, R, R, p, ccx, cake.KMN)
+    picks = [(0, 0), (5, 17), (R // 2 + 1, R // 3), (R - 7, 11), (R - 1, R - 1), (R - 2, 3), (12345, R - 1)]
+    for which, size, pack in ((0, cake.cake_sgemm_packed_A_size(R, R, p, x, ccx, cake.KMN), cake.pack_A),
+                              (2, cake.cake_sgemm_packed_C_size(R, R, p, x, ccx, cake.KMN), cake.pack_C)):
+        print(f"pack {'AC'[which // 2]} {R}x{R}: {size / 1e9:.2f} GB packed", flush=True)
+        packed = torch.full((size // 4,), float("nan"), dtype=torch.float32, device=_dev())
+        pack(big, packed, R, R, p, x, ccx, cake.KMN)
+        for r, c in picks:
+            off = cake.packed_offset(which, r, c, R, R, R, p, x, ccx, cake.KMN)
+            assert 0 <= off < size // 4
+            assert float(packed[off]) == float(big[r, c]), (which, r, c, off)
+        if which == 2:
+            back = torch.full((R, R), float("nan"), dtype=torch.float32, device=_dev())
+            cake.unpack_C(back, packed, R, R, p, x, ccx, cake.KMN)
+            assert torch.equal(back, big)
+            del back
+        del packed
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("batch", [1, 2, 16, 40], ids=lambda b: f"batch{b}")
 def test_linear_forward(big, batch):
     """y = x . big^T + b: matrix-vector sweep, its two-vector form, the streaming kernel, and the
