@@ -1744,14 +1744,15 @@ static int conv2d_common(const float* in, const float* weights, float* out, int 
     if (accumulate) out_nchw = 0;   // a single image: [Cout][HW] is its NCHW layout
     const bool vec = vec4_loadable(w.dev, cols, K, N);
     const int mode = vec ? LOAD_VEC4 : LOAD_SCALAR;
-    // NCHW output: with rows of the product a multiple of 4 long the GEMM's epilogue (and its
-    // slice reductions) write the layout themselves, as on the gather path; otherwise the product
+    // NCHW output: where an image's pixels are a multiple of 4 (its 16-byte chunks of columns then
+    // never run from one image into the next) the GEMM's epilogue (and its slice reductions) write
+    // the layout themselves, an image seen as one row of Hout * Wout pixels; otherwise the product
     // goes to [Cout][N] first and a layout pass follows
     ConvGeom nchw{};
-    const bool fused_nchw = out_nchw && vec && Wout % 4 == 0 && Cout > 48 && K > 64;   // (the macro-tile kernel's shapes)
+    const bool fused_nchw = out_nchw && vec && (Hout * Wout) % 4 == 0 && Cout > 48 && K > 64;   // (the macro-tile kernel's shapes)
     if (fused_nchw) {
         nchw.in = cols;
-        nchw.Hout = Hout; nchw.Wout = Wout; nchw.row_n = Wout;
+        nchw.Hout = 1; nchw.Wout = Hout * Wout; nchw.row_n = Hout * Wout;
         nchw.out_nchw = 1;
         out_nchw = 0;
     }
