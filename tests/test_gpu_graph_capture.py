@@ -89,7 +89,8 @@ def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
     """The convolution routes under capture: the input read where it lies (under a 3 x 3 filter one
     kernel with the last round in sub-tiles; under a 5 x 3 one re-laid filters and tail slices
     summed by a second kernel), the gather from a staged copy (stride 2: staging kernel, tap
-    table) and the reference's two steps (column matrix in a workspace).  A larger eager
+    table), a 1 x 1 layer at stride 2 (dense copy first) and the reference's two steps (column
+    matrix in a workspace).  A larger eager
     convolution between the replays grows every one of those workspaces."""
     monkeypatch.setenv("CAKE_HIP_CONV_ROUTE", "patch")   # layers this small would take the staged copy by themselves
     dev = torch.device("cuda:0")
@@ -97,6 +98,7 @@ def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
     geoms = [(34, 32, 32, 32, 72, 3, 3, 1, 1, lib.cake_hip_conv2d),        # 272 tiles: the 16 of the last round as sub-tiles
              (34, 64, 32, 32, 40, 5, 3, 1, 2, lib.cake_hip_conv2d),        # the same under 15 taps: re-laid filters, K slices
              (3, 16, 12, 12, 32, 3, 3, 2, 1, lib.cake_hip_conv2d),         # staged copy
+             (4, 32, 16, 16, 48, 1, 1, 2, 0, lib.cake_hip_conv2d),         # 1 x 1 at stride 2: dense copy of the pixels it reads
              (2, 8, 16, 16, 24, 3, 3, 1, 1, lib.cake_hip_conv2d_im2col)]   # column matrix first
     ins, wts = [], []
     for i, (b, cin, h, w, cout, hf, wf, s, p, _) in enumerate(geoms):
@@ -152,3 +154,61 @@ def test_captured_convolutions_replay_like_eager_calls(monkeypatch):
         torch.cuda.synchronize()
         for got, want in zip(captured, eager):
             assert torch.equal(got, want), f"replay {replay}"
+
+
+def test_captured_packing_and_im2col_replay_like_eager_calls():
+    """pack_A, pack_B, pack_C, unpack_C (index tables in a workspace, then the copy kernels) and im2col."""
+    dev = torch.device("cuda:0")
+    lib = cake.load()
+    M, K, N, p = 333, 270, 401, 3
+    ccx = cake.CpuCntx(1.0, 6, 16, 48 << 10, 256 << 10, 2 << 20, 8)
+    x = cake.init_block_dims(M, N, K, p, ccx, cake.KMN)
+    A = torch.empty((M, K), dtype=torch.float32, device=dev)
+    B = torch.empty((K, N), dtype=torch.float32, device=dev)
+    Cm = torch.empty((M, N), dtype=torch.float32, device=dev)
+    img = torch.empty((5, 6, 13, 14), dtype=torch.float32, device=dev)
+    sizes = (cake.cake_sgemm_packed_A_size(M, K, p, x, ccx, cake.KMN) // 4, cake.cake_sgemm_packed_B_size(K, N, p, x, ccx) // 4,
+             cake.cake_sgemm_packed_C_size(M, N, p, x, ccx, cake.KMN) // 4)
+    bx, bc = ctypes.byref(x), ctypes.byref(ccx)
+
+    def outputs():
+        return tuple(torch.zeros(shape, dtype=torch.float32, device=dev)
+                     for shape in ((sizes[0],), (sizes[1],), (sizes[2],), (M, N), (6 * 9, 5 * 13 * 14)))
+
+    def run(out, stream):
+        ap, bp, cp, back, cols = out
+        assert lib.cake_hip_pack_a(A.data_ptr(), ap.data_ptr(), M, K, p, bx, bc, cake.KMN, stream, None) == 0
+        assert lib.cake_hip_pack_b(B.data_ptr(), bp.data_ptr(), K, N, p, bx, bc, cake.KMN, stream, None) == 0
+        assert lib.cake_hip_pack_c(Cm.data_ptr(), cp.data_ptr(), M, N, p, bx, bc, cake.KMN, stream, None) == 0
+        assert lib.cake_hip_unpack_c(back.data_ptr(), cp.data_ptr(), M, N, p, bx, bc, cake.KMN, stream, None) == 0
+        assert lib.cake_hip_im2col(img.data_ptr(), cols.data_ptr(), 5, 6, 13, 14, 3, 3, 1, 1, stream, None) == 0
+
+    side = torch.cuda.Stream()
+    captured = outputs()
+    with torch.cuda.stream(side):
+        run(captured, side.cuda_stream)          # warm: the index tables' workspace is allocated before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(captured, torch.cuda.current_stream().cuda_stream)
+
+    for replay in range(4):
+        if replay == 2:   # larger index tables between the replays: the workspace grows, the graph keeps its addresses
+            big = torch.empty((3000, 2000), dtype=torch.float32, device=dev)
+            bx2 = cake.init_block_dims(3000, 2000, 2000, p, ccx, cake.KMN)
+            bp2 = torch.empty((cake.cake_sgemm_packed_A_size(3000, 2000, p, bx2, ccx, cake.KMN) // 4,), dtype=torch.float32, device=dev)
+            cake.pack_A(big, bp2, 3000, 2000, p, bx2, ccx, cake.KMN)
+            torch.cuda.synchronize()
+        for i, t in enumerate((A, B, Cm, img)):
+            cake.fill_uniform(t, 500 + 10 * replay + i)
+        for t in captured:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = outputs()
+        run(eager, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), f"replay {replay}"
+        assert torch.equal(captured[3], Cm)
