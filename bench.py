@@ -52,23 +52,28 @@ HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E peak
 # names the row of profiles/all_kernels_hbm_traffic_pmc.md it was read from.
 # The figure is the column "with its helper kernels" of that file's workload table, in bytes.
 MEASURED_TRAFFIC = {
-    "sgemm_8192": (4563255275, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
+    "sgemm_8192": (4563256106, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 1048576"),
     "sgemm_1024": (29500957, "row `sgemm_tile_kernel<Tile<64, 64, 64, 32, 32, 2, 2, 2>, 0, 0>` grid 131072"),
     "sgemm_tall_skinny": (306412911, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 0>` grid 131072"),
     "sgemv_16384_rowmajor": (1074454809, "row `sgemv_rowmajor_wg_kernel<2, 8>` grid 4194304"),
-    "sgemv_16384_colmajor": (1075873031, "row `sgemv_colmajor_kernel<true>` grid 196608"),
-    "conv_c5_gather": (278904781, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 3, 3>` grid 524288"),
-    "conv_c5_two_step": (2212091572, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
-    "shortk_256x64x100352": (129060149, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
-    "conv_1x1_14x14": (43105781, "row `sgemm_shortk_staged_flat_kernel` grid 262144"),
-    "resident_8192x256x8192": (400705391, "row `sgemm_resident_kernel` grid 131072"),
-    "staged_3000x100x3000": (44978223, "row `sgemm_shortk_staged_kernel` grid 262144"),
-    "fewrows_nn": (1087400122, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
-    "fewrows_nn_64rows": (1128387618, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
-    "narrow_tile_32cols": (288997411, "row `sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0>` grid 131072"),
-    "fewrows_nt": (1083225769, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_16x16384x16384": (1083225769, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
-    "linear_fwd_8192x4096x4096": (1208264117, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
+    "sgemv_16384_colmajor": (1075873287, "row `sgemv_colmajor_kernel<true>` grid 196608"),
+    "conv_c5_gather": (278924379, "row `sgemm_conv_patch_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 3, 3>` grid 524288"),
+    "conv_c5_two_step": (2212324492, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 6>` grid 516096"),
+    "shortk_256x64x100352": (129060273, "row `sgemm_shortk_kernel<Tile<64, 64, 64, 32, 32, 1, 1, 1>, 0, true>` grid 262144"),
+    "conv_1x1_14x14": (43096930, "row `sgemm_shortk_staged_flat_kernel` grid 262144"),
+    "resident_8192x256x8192": (400702558, "row `sgemm_resident_kernel` grid 131072"),
+    "staged_3000x100x3000": (44956993, "row `sgemm_shortk_staged_kernel` grid 262144"),
+    "fewrows_nn": (1087400124, "row `sgemm_fewrows_nn_kernel<1, 2>` grid 65536"),
+    "fewrows_nn_64rows": (1128387615, "row `sgemm_fewrows_nn_kernel<4, 2>` grid 65536"),
+    "narrow_tile_32cols": (289075043, "row `sgemm_tile_kernel<Tile<128, 32, 32, 32, 32, 2, 1, 1>, 0, 0>` grid 131072"),
+    "fewrows_nt": (1083225759, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "linear_fwd_16x16384x16384": (1083225759, "row `sgemm_fewrows_nt_kernel<false, 1, 64, 32, 1>` grid 65536"),
+    "pack_a_8192": (542362035, "row `pack_tile_kernel<false, 24, 128, true>` grid 5603328"),
+    "pack_b_8192": (538087108, "row `pack_tile_kernel<false, 16, 128, true>` grid 8388608"),
+    "pack_c_8192": (538227331, "row `pack_tile_kernel<false, 16, 128, true>` grid 8404992"),
+    "unpack_c_8192": (538110727, "row `pack_tile_kernel<true, 16, 128, true>` grid 8388608"),
+    "im2col_c5": (1046053869, "row `im2col_rows_kernel<3>` grid 6422528"),
+    "linear_fwd_8192x4096x4096": (1208263337, "row `sgemm_tile_kernel<Tile<256, 128, 32, 64, 64, 2, 1, 1>, 0, 2>` grid 524288"),
 }
 
 
@@ -347,6 +352,52 @@ def main() -> int:
                        "roofline": roofline("hbm", sby, avg, "linear_fwd_16x16384x16384",
                                             timed_on=f"{ROTATE} rotating weight matrices",
                                             frac_same_buffer=round(sby / same / 1e9 / HBM_PEAK_GBPS, 4))})
+
+        # The copies of the path: pack_A / pack_B / pack_C / unpack_C (8192^2 operands in the reference's
+        # panel layout for m_r = 6, n_r = 16; each call builds its two index tables first) and im2col
+        # of config 5's input.  Algorithmic bytes: every element read once and written once.
+        import ctypes as C
+        Pn, Pp = 8192, 8
+        pcx = cake.CpuCntx(1.0, 6, 16, 48 << 10, 2 << 20, 105 << 20, 8)
+        pdims = cake.init_block_dims(Pn, Pn, Pn, Pp, pcx, cake.KMN)
+        plain = dev_uniform((Pn, Pn), 21)
+        sizes = {"a": cake.cake_sgemm_packed_A_size(Pn, Pn, Pp, pdims, pcx, cake.KMN), "b": cake.cake_sgemm_packed_B_size(Pn, Pn, Pp, pdims, pcx),
+                 "c": cake.cake_sgemm_packed_C_size(Pn, Pn, Pp, pdims, pcx, cake.KMN)}
+        packed = torch.empty((max(sizes.values()) // 4,), dtype=torch.float32, device=dev)
+        back = torch.empty((Pn, Pn), dtype=torch.float32, device=dev)
+        bd, bc = C.byref(pdims), C.byref(pcx)
+        calls = (("pack_A", "a", lambda: lib.cake_hip_pack_a(plain.data_ptr(), packed.data_ptr(), Pn, Pn, Pp, bd, bc, cake.KMN, stream, None)),
+                 ("pack_B", "b", lambda: lib.cake_hip_pack_b(plain.data_ptr(), packed.data_ptr(), Pn, Pn, Pp, bd, bc, cake.KMN, stream, None)),
+                 ("pack_C", "c", lambda: lib.cake_hip_pack_c(plain.data_ptr(), packed.data_ptr(), Pn, Pn, Pp, bd, bc, cake.KMN, stream, None)),
+                 ("unpack_C", "c", lambda: lib.cake_hip_unpack_c(back.data_ptr(), packed.data_ptr(), Pn, Pn, Pp, bd, bc, cake.KMN, stream, None)))
+        for name, which, call in calls:
+            _, avg, _ = time_steps(lambda: _lib.check(call(), name), 20, 3, 20.0)
+            pby = 4.0 * Pn * Pn + sizes[which]
+            extras.append({"workload": f"{name} of an 8192 x 8192 operand (index tables included)", "us": round(avg * 1e6, 2),
+                           "roofline": roofline("hbm", pby, avg, {"pack_A": "pack_a_8192", "pack_B": "pack_b_8192", "pack_C": "pack_c_8192",
+                                                                  "unpack_C": "unpack_c_8192"}[name])})
+        del plain, packed, back
+        Bn, Cc, H = 32, 256, 56
+        iin = dev_uniform((Bn, Cc, H, H), 22)
+        icols = torch.empty((Cc * 9, Bn * H * H), dtype=torch.float32, device=dev)
+        other_a, other_b = torch.empty((8192, 8192), dtype=torch.float32, device=dev), torch.empty((8192, 8192), dtype=torch.float32, device=dev)
+        iby = 4.0 * (iin.numel() + icols.numel())
+        im = lambda: _lib.check(lib.cake_hip_im2col(iin.data_ptr(), icols.data_ptr(), Bn, Cc, H, H, 3, 3, 1, 1, stream, None), "im2col")
+        _, alone, _ = time_steps(im, 20, 3, 20.0)
+        # ... and with a 256 MB copy between the launches, so that neither the input nor the end of the
+        # previous launch's columns wait in the memory-side cache: what the kernel costs inside a convolution
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+        for a, b in evs:
+            other_b.copy_(other_a)
+            a.record()
+            im()
+            b.record()
+        torch.cuda.synchronize()
+        between = float(np.mean([a.elapsed_time(b) for a, b in evs])) * 1e-3
+        extras.append({"workload": "im2col of config 5's input (32 x 256 x 56 x 56, 3 x 3, pad 1): 925 MB of columns",
+                       "us": round(between * 1e6, 2), "us_in_a_loop_of_its_own": round(alone * 1e6, 2),
+                       "roofline": roofline("hbm", iby, between, "im2col_c5", timed_on="launches with a 256 MB copy between them")})
+        del iin, icols, other_a, other_b
 
     if not args.no_extras:
 
