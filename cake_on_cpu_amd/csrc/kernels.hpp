@@ -160,6 +160,19 @@ hipError_t launch_tail_reduce(int tile_id, const GemmArgs& args, hipStream_t str
 enum { SHORTK_MAX_K = 160, SHORTK_MAX_K_BATCH = 256 };
 // tile rows per band of the short-K kernel's tile sequence (group of the launch arguments)
 int shortk_band_rows(int tiles_m, int N);
+// A product that is all stores (K up to 32) into a C of more than the memory-side cache holds,
+// with rows that are no whole cache lines apart: every row of a tile then ends in pieces of
+// lines, which this memory writes far more slowly than whole ones, and what counts is how the
+// pieces of neighbouring tiles meet in the L2.  Measured, us, short-K kernel / macro-tile kernel
+// on 64 x 64 / on 96 x 128 / on 256 x 128 tiles: 8548 x 24 x 13421 161 / 144 / 140 / 149,
+// 16384 x 16 x 16383 390 / 308 / 278 / 400, 8192 x 24 x 13420 147 / 154 / 122 / 175, 16384 x 16 x 16400
+// 297 / 365 / 280 / 395, 9000 x 12 x 9001 102 / 92 / 91 / 103 (with rows 128 bytes apart, 8548 x 24 x 13440,
+// the short-K kernel takes 96).  Such products run on the macro-tile kernel's 96 x 128 x 32 tile,
+// the best or within 3 % of it on 14 shapes.
+inline bool stores_in_pieces_of_lines(int M, int N, int K)
+{
+    return K <= 32 && N % 32 != 0 && (double)M * N * 4.0 > 256e6;
+}
 // batch >= 1 with shared_a: `batch` products M x K x N with one A (launched with tiles_n_per_image set)
 int shortk_tile_n(int M, int N, int K, int cus, int batch = 1, bool shared_a = false);
 inline bool shortk_applies(int M, int N, int K, int cus, int batch = 1, bool shared_a = false)

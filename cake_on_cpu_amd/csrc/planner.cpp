@@ -295,6 +295,9 @@ int plan_gemm(int M, int N, int K, int sched, const int* ov, bool vector_ok, con
     if (!ov && tune_lookup(M, N, K, vector_ok, &tuned) && tile_info(tuned.tile_id).lds_bytes <= dev.lds_per_cu)
         return finish_plan(M, N, K, sched, tuned.tile_id, tuned.split_k, tuned.tail_ok != 0, vector_ok, dev, out);
 
+    if (!want_m && !want_n && !want_k && !want_split && stores_in_pieces_of_lines(M, N, K)) {   // (kernels.hpp)
+        want_m = 96; want_n = 128; want_k = 32; want_split = 1;
+    }
     Candidate best = {-1, 1, 1e30};
     for (int id = 0; id < TILE_COUNT; ++id) {
         const TileInfo& t = tile_info(id);

@@ -790,6 +790,7 @@ int shortk_tile_n(int M, int N, int K, int cus, int batch, bool shared_a)
     if (K < 1 || K > (shared_a ? SHORTK_MAX_K_BATCH : SHORTK_MAX_K) || (K > 64 && K % 4 != 0)) return 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64) * batch;
     if (tiles < (long)cus) return 0;
+    if (!shared_a && stores_in_pieces_of_lines(M, N, K)) return 0;
     return 64;
 }
 

@@ -127,6 +127,27 @@ def test_transpose(big):
     torch.cuda.empty_cache()
 
 
+def test_store_bound_product_with_rows_off_cache_lines():
+    """K = 12 into a C of 324 MB whose rows are 36004 bytes apart: the planner leaves the short-K
+    kernel for the 96 x 128 macro-tile; the whole result against fp64 on the device."""
+    M, K, N = 9000, 12, 9001
+    plan = cake.plan(M, N, K)
+    assert (plan.tile_m, plan.tile_n, plan.tile_k, plan.split_k) == (96, 128, 32, 1)
+    assert (cake.plan(M, 9024, K).tile_m, cake.plan(M, 9024, K).tile_n) == (64, 64)   # rows of whole lines: the short-K kernel
+    A, B = _filled((M, K), 961), _filled((K, N), 962)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device=_dev())
+    lib = cake.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    print(f"sgemm {M}x{K}x{N}", flush=True)
+    assert lib.cake_hip_sgemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, cake.NA, 0, None, stream, None) == 0
+    _check(C, A.double(), B.double(), "store-bound product")
+    first = C.clone()
+    assert lib.cake_hip_sgemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, cake.NA, 1, None, stream, None) == 0
+    assert torch.equal(C, first + first)       # accumulating once more doubles every element exactly
+    del A, B, C, first
+    torch.cuda.empty_cache()
+
+
 def test_im2col_columns_past_4_gb():
     """A column matrix of 576 x 2 000 000 floats (4.6 GB): sampled rows, the last ones among them,
     equal the shifted planes they are copies of, bit for bit."""
